@@ -1,0 +1,56 @@
+"""ctypes binding of libdifflogic_hip.so.  The library is the only implementation of the GPU
+path: if it is missing or a symbol is absent, importing this module's users fails loudly."""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libdifflogic_hip.so")
+
+DL_OK = 0
+DL_ERR_INVALID_ARGUMENT = 1
+DL_ERR_BIT_COUNT = 2
+DL_ERR_NOT_DIVISIBLE = 3
+DL_ERR_DTYPE = 4
+DL_ERR_LAUNCH = 5
+DL_ERR_TOO_LARGE = 6
+
+DL_F16, DL_F32, DL_F64 = 0, 1, 2
+
+_vp, _i64, _int, _dbl = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_double
+
+# name -> argument types; every function returns int (dl_status) unless listed in _RESTYPES.
+SIGNATURES = {
+    "dl_version": [],
+    "dl_status_string": [_int],
+    "dl_logic_forward": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
+    "dl_logic_backward_w": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
+    "dl_logic_backward_x": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _dbl, _int, _vp],
+    "dl_logic_eval": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
+    "dl_tensor_packbits": [_vp, _vp, _i64, _i64, _int, ctypes.POINTER(_i64), _vp],
+    "dl_groupbitsum": [_vp, _vp, _i64, _i64, _int, _i64, _i64, _vp],
+}
+_RESTYPES = {"dl_status_string": ctypes.c_char_p}
+
+_lib = None
+
+
+def load():
+    """Loads the library once and declares every prototype of include/difflogic_hip.h."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: the HIP kernel library has not been built. "
+            "Run `python -m difflogic_amd.build` (needs hipcc); there is no fallback implementation.")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)          # AttributeError if the symbol is not exported
+        fn.argtypes = argtypes
+        fn.restype = _RESTYPES.get(name, ctypes.c_int)
+    _lib = lib
+    return lib
+
+
+def status_string(status: int) -> str:
+    return load().dl_status_string(int(status)).decode()

@@ -1,0 +1,367 @@
+// Packed-bit inference kernels for gfx950: gate evaluation on bit-packed words, bool -> word
+// packing, and the per-class vertical bit count.
+//
+// All three treat a packed matrix as rows of BYTES: with little-endian words, sample s of a
+// row is bit (s % 8) of byte (s / 8) whatever the word width, so one code path serves the
+// 8/16/32/64-bit word types and the widest vector access the row length allows is used.
+#include "dl_common.h"
+
+namespace {
+
+// ------------------------------------------------------------------------------------------
+// Gate evaluation.  Gate id = 4-bit truth table (f(0,0) f(0,1) f(1,0) f(1,1)), MSB first.
+// Branch-free: two levels of bitwise select driven by b then a, with the four table bits
+// expanded to all-ones / all-zero masks (wave-uniform, they live in scalar registers).
+// ------------------------------------------------------------------------------------------
+
+struct GateMasks { uint32_t m00, m01, m10, m11; };
+
+__device__ __forceinline__ GateMasks gate_masks(uint32_t op) {
+    GateMasks m;
+    m.m00 = 0u - ((op >> 3) & 1u);
+    m.m01 = 0u - ((op >> 2) & 1u);
+    m.m10 = 0u - ((op >> 1) & 1u);
+    m.m11 = 0u - (op & 1u);
+    return m;
+}
+
+template <typename V> struct Splat;
+template <> struct Splat<dl_u32x4> { static __device__ __forceinline__ dl_u32x4 of(uint32_t v) { return dl_u32x4{v, v, v, v}; } };
+template <> struct Splat<dl_u32x2> { static __device__ __forceinline__ dl_u32x2 of(uint32_t v) { return dl_u32x2{v, v}; } };
+template <> struct Splat<uint32_t> { static __device__ __forceinline__ uint32_t of(uint32_t v) { return v; } };
+template <> struct Splat<uint16_t> { static __device__ __forceinline__ uint16_t of(uint32_t v) { return (uint16_t) v; } };
+template <> struct Splat<uint8_t> { static __device__ __forceinline__ uint8_t of(uint32_t v) { return (uint8_t) v; } };
+
+template <typename V> __device__ __forceinline__ V gate_apply(V a, V b, const GateMasks &m) {
+    const V hi = (b & Splat<V>::of(m.m11)) | (~b & Splat<V>::of(m.m10));  // value if a = 1
+    const V lo = (b & Splat<V>::of(m.m01)) | (~b & Splat<V>::of(m.m00));  // value if a = 0
+    return (V) ((a & hi) | (~a & lo));
+}
+
+// One wave owns NPW neurons x 64 consecutive vectors of the row; a workgroup owns
+// 4 * NPW * ITERS consecutive neurons.  blockIdx.x walks neuron tiles, blockIdx.y column
+// tiles: workgroups are dispatched x-fastest, so the chip sweeps all neurons of one column
+// tile before the next and the input rows of that tile (in_dim * 64 * sizeof(V) bytes) are
+// what has to stay cache-resident between a row's uses.
+template <typename V, int NPW, int ITERS>
+__global__ __launch_bounds__(DL_BLOCK) void eval_kernel(const V *__restrict__ x, const int64_t *__restrict__ a,
+                                                        const int64_t *__restrict__ b,
+                                                        const uint8_t *__restrict__ w, V *__restrict__ y,
+                                                        int64_t out_dim, int64_t ncols) {
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t n_first = ((int64_t) blockIdx.x * 4 + wave) * (NPW * ITERS);
+
+    for (int64_t ct = blockIdx.y; ct * DL_WAVE < ncols; ct += gridDim.y) {
+        const int64_t col = ct * DL_WAVE + lane;
+        const bool live = col < ncols;
+#pragma unroll 1
+        for (int it = 0; it < ITERS; ++it) {
+            const int64_t n0 = n_first + (int64_t) it * NPW;
+            if (n0 >= out_dim) break;
+            int64_t ia[NPW], ib[NPW];
+            uint32_t op[NPW];
+#pragma unroll
+            for (int j = 0; j < NPW; ++j) {
+                const int64_t n = (n0 + j < out_dim) ? n0 + j : out_dim - 1;
+                ia[j] = a[n];
+                ib[j] = b[n];
+                op[j] = w[n];
+            }
+            if (live) {
+                V va[NPW], vb[NPW];
+#pragma unroll
+                for (int j = 0; j < NPW; ++j) {
+                    va[j] = x[ia[j] * ncols + col];
+                    vb[j] = x[ib[j] * ncols + col];
+                }
+#pragma unroll
+                for (int j = 0; j < NPW; ++j) {
+                    if (n0 + j < out_dim) {
+                        const V r = gate_apply<V>(va[j], vb[j], gate_masks(op[j]));
+                        __builtin_nontemporal_store(r, &y[(n0 + j) * ncols + col]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <typename V, int NPW, int ITERS>
+int launch_eval(const void *x, const int64_t *a, const int64_t *b, const uint8_t *w, void *y, int64_t out_dim,
+                int64_t row_bytes, hipStream_t stream) {
+    const int64_t ncols = row_bytes / (int64_t) sizeof(V);
+    const int64_t ntiles = dl_ceil_div(out_dim, 4 * NPW * ITERS);
+    int64_t ctiles = dl_ceil_div(ncols, DL_WAVE);
+    if (ntiles > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    if (ctiles > 65535) ctiles = 65535;
+    dim3 grid((unsigned) ntiles, (unsigned) ctiles);
+    hipLaunchKernelGGL((eval_kernel<V, NPW, ITERS>), grid, dim3(DL_BLOCK), 0, stream, (const V *) x, a, b, w, (V *) y,
+                       out_dim, ncols);
+    return dl_launch_status();
+}
+
+// ------------------------------------------------------------------------------------------
+// bool -> packed bytes.  Output byte j of a row holds samples 8j .. 8j+7, lowest sample in
+// bit 0; bytes past the batch are zero.
+// ------------------------------------------------------------------------------------------
+
+// 8 bool bytes (any non-zero value counts as true) -> 8 bits, byte i -> bit i.
+__device__ __forceinline__ uint32_t squeeze8(uint64_t v) {
+    const uint64_t k7f = 0x7f7f7f7f7f7f7f7fULL;
+    v = (((v & k7f) + k7f) | v) & ~k7f;                          // 0x80 in every non-zero byte
+    return (uint32_t) (((v >> 7) * 0x0102040810204080ULL) >> 56);  // gather the eight flags
+}
+
+// Rows whose length is a multiple of 16 bools and 16-byte aligned: one 16-byte load and one
+// 2-byte store per lane, both coalesced.
+__global__ __launch_bounds__(DL_BLOCK) void packbits_vec16_kernel(const uint8_t *__restrict__ t,
+                                                                  uint8_t *__restrict__ out, int64_t features,
+                                                                  int64_t batch, int64_t out_row_bytes) {
+    const int64_t chunks = batch / 16;                  // 16 samples -> 2 output bytes
+    const int64_t out_pairs = out_row_bytes / 2;        // out_row_bytes is even here
+    for (int64_t f = blockIdx.y; f < features; f += gridDim.y) {
+        const dl_u32x4 *src = reinterpret_cast<const dl_u32x4 *>(t + f * batch);
+        uint16_t *dst = reinterpret_cast<uint16_t *>(out + f * out_row_bytes);
+        for (int64_t i = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x; i < out_pairs;
+             i += (int64_t) gridDim.x * DL_BLOCK) {
+            uint32_t r = 0;
+            if (i < chunks) {
+                const dl_u32x4 v = __builtin_nontemporal_load(&src[i]);
+                const uint64_t lo = ((uint64_t) v.y << 32) | v.x, hi = ((uint64_t) v.w << 32) | v.z;
+                r = squeeze8(lo) | (squeeze8(hi) << 8);
+            }
+            dst[i] = (uint16_t) r;
+        }
+    }
+}
+
+// Any batch length: one output byte per thread from up to 8 single-byte loads.
+__global__ __launch_bounds__(DL_BLOCK) void packbits_generic_kernel(const uint8_t *__restrict__ t,
+                                                                    uint8_t *__restrict__ out, int64_t features,
+                                                                    int64_t batch, int64_t out_row_bytes) {
+    for (int64_t f = blockIdx.y; f < features; f += gridDim.y) {
+        const uint8_t *src = t + f * batch;
+        uint8_t *dst = out + f * out_row_bytes;
+        for (int64_t j = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x; j < out_row_bytes;
+             j += (int64_t) gridDim.x * DL_BLOCK) {
+            uint32_t r = 0;
+            const int64_t s0 = j * 8;
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (s0 + i < batch) r |= (uint32_t) (src[s0 + i] != 0) << i;
+            dst[j] = (uint8_t) r;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Vertical bit count (GroupSum on packed words).  For each class (a contiguous block of
+// per_class neuron rows) and each sample bit, the number of rows with that bit set.
+//
+// Lanes run along 64-bit word columns (coalesced row reads); each wave takes a quarter of the
+// class's rows and keeps bit-sliced counters: 16 rows at a time are compressed by a
+// carry-save-adder tree into planes of weight 1, 2, 4, 8 and a carry of weight 16 that is
+// rippled into NPH higher planes.  The four waves' planes are exchanged through LDS, each
+// wave expands 16 of the 64 sample bits to integers, and the [column][sample] tile is written
+// out with lanes along samples.
+// ------------------------------------------------------------------------------------------
+
+__device__ __forceinline__ void csa(uint64_t &carry, uint64_t &sum, uint64_t a, uint64_t b, uint64_t c) {
+    const uint64_t u = a ^ b;
+    carry = (a & b) | (u & c);
+    sum = u ^ c;
+}
+
+template <int NPH>
+__global__ __launch_bounds__(DL_BLOCK) void groupbitsum_kernel(const uint64_t *__restrict__ bits,
+                                                               int32_t *__restrict__ out, int64_t words,
+                                                               int64_t per_class, int64_t k, int64_t batch) {
+    constexpr int NP = NPH + 4;
+    __shared__ uint64_t planes_lds[4][NP][DL_WAVE];
+    __shared__ int32_t tile[DL_WAVE][DL_WAVE + 1];   // [column][sample], padded against bank conflicts
+
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t cls = blockIdx.y;
+    const int64_t c0 = (int64_t) blockIdx.x * DL_WAVE;
+    const int64_t col = c0 + lane;
+    const bool live = col < words;
+
+    const int64_t chunk = (per_class + 3) / 4;
+    int64_t r_begin = (int64_t) wave * chunk;
+    if (r_begin > per_class) r_begin = per_class;
+    int64_t r_end = r_begin + chunk;
+    if (r_end > per_class) r_end = per_class;
+
+    uint64_t ones = 0, twos = 0, fours = 0, eights = 0;
+    uint64_t high[NPH];
+#pragma unroll
+    for (int p = 0; p < NPH; ++p) high[p] = 0;
+
+    const uint64_t *row = bits + (cls * per_class + r_begin) * words + (live ? col : 0);
+    for (int64_t r = r_begin; r < r_end; r += 16) {
+        uint64_t v[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            v[j] = (live && r + j < r_end) ? __builtin_nontemporal_load(row + (int64_t) j * words) : 0;
+        }
+        row += 16 * words;
+        uint64_t t2a, t2b, t4a, t4b, t8a, t8b, t16;
+        csa(t2a, ones, ones, v[0], v[1]);
+        csa(t2b, ones, ones, v[2], v[3]);
+        csa(t4a, twos, twos, t2a, t2b);
+        csa(t2a, ones, ones, v[4], v[5]);
+        csa(t2b, ones, ones, v[6], v[7]);
+        csa(t4b, twos, twos, t2a, t2b);
+        csa(t8a, fours, fours, t4a, t4b);
+        csa(t2a, ones, ones, v[8], v[9]);
+        csa(t2b, ones, ones, v[10], v[11]);
+        csa(t4a, twos, twos, t2a, t2b);
+        csa(t2a, ones, ones, v[12], v[13]);
+        csa(t2b, ones, ones, v[14], v[15]);
+        csa(t4b, twos, twos, t2a, t2b);
+        csa(t8b, fours, fours, t4a, t4b);
+        csa(t16, eights, eights, t8a, t8b);
+#pragma unroll
+        for (int p = 0; p < NPH; ++p) {
+            const uint64_t old = high[p];
+            high[p] = old ^ t16;
+            t16 = old & t16;
+        }
+    }
+
+    planes_lds[wave][0][lane] = ones;
+    planes_lds[wave][1][lane] = twos;
+    planes_lds[wave][2][lane] = fours;
+    planes_lds[wave][3][lane] = eights;
+#pragma unroll
+    for (int p = 0; p < NPH; ++p) planes_lds[wave][4 + p][lane] = high[p];
+    __syncthreads();
+
+    // This wave expands sample bits [16*wave, 16*wave + 16) of every column.
+    int32_t cnt[16];
+#pragma unroll
+    for (int s = 0; s < 16; ++s) cnt[s] = 0;
+    const int shift = 16 * wave;
+    for (int q = 0; q < 4; ++q) {
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const uint32_t slice = (uint32_t) (planes_lds[q][p][lane] >> shift) & 0xffffu;
+#pragma unroll
+            for (int s = 0; s < 16; ++s) cnt[s] += (int32_t) (((slice >> s) & 1u) << p);
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < 16; ++s) tile[lane][shift + s] = cnt[s];
+    __syncthreads();
+
+    // Lanes along samples: thread t writes sample (t % 64) of columns t/64, t/64 + 4, ...
+    const int s = lane;
+    for (int cc = wave; cc < DL_WAVE; cc += 4) {
+        const int64_t c = c0 + cc;
+        const int64_t sample = c * 64 + s;
+        if (c < words && sample < batch) out[sample * k + cls] = tile[cc][s];
+    }
+}
+
+// Any word width / row length: one thread per (sample, class), like the reference, but with
+// lanes on consecutive samples of the sample-major output.
+__global__ __launch_bounds__(DL_BLOCK) void groupbitsum_generic_kernel(const uint8_t *__restrict__ bits,
+                                                                       int32_t *__restrict__ out, int64_t row_bytes,
+                                                                       int64_t per_class, int64_t k, int64_t batch) {
+    for (int64_t cls = blockIdx.y; cls < k; cls += gridDim.y) {
+        for (int64_t s = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x; s < batch;
+             s += (int64_t) gridDim.x * DL_BLOCK) {
+            const uint8_t *p = bits + cls * per_class * row_bytes + (s >> 3);
+            const int sh = (int) (s & 7);
+            int32_t acc = 0;
+            for (int64_t r = 0; r < per_class; ++r) acc += (p[r * row_bytes] >> sh) & 1;
+            out[s * k + cls] = acc;
+        }
+    }
+}
+
+bool valid_bit_count(int bit_count) { return bit_count == 8 || bit_count == 16 || bit_count == 32 || bit_count == 64; }
+
+}  // namespace
+
+extern "C" int dl_logic_eval(const void *x, const int64_t *a, const int64_t *b, const uint8_t *w, void *y,
+                             int64_t in_dim, int64_t out_dim, int64_t words, int bit_count, void *stream) {
+    if (!valid_bit_count(bit_count)) return DL_ERR_BIT_COUNT;
+    if (in_dim < 0 || out_dim < 0 || words < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim == 0 || words == 0) return DL_OK;
+    if (!x || !a || !b || !w || !y || in_dim == 0) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    const int64_t row_bytes = words * (bit_count / 8);
+    const uintptr_t mis = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) | (uintptr_t) row_bytes;
+    if (mis % 16 == 0) return launch_eval<dl_u32x4, 4, 4>(x, a, b, w, y, out_dim, row_bytes, s);
+    if (mis % 8 == 0) return launch_eval<dl_u32x2, 4, 4>(x, a, b, w, y, out_dim, row_bytes, s);
+    if (mis % 4 == 0) return launch_eval<uint32_t, 4, 4>(x, a, b, w, y, out_dim, row_bytes, s);
+    if (mis % 2 == 0) return launch_eval<uint16_t, 4, 4>(x, a, b, w, y, out_dim, row_bytes, s);
+    return launch_eval<uint8_t, 4, 4>(x, a, b, w, y, out_dim, row_bytes, s);
+}
+
+extern "C" int dl_tensor_packbits(const uint8_t *t, void *out, int64_t features, int64_t batch, int bit_count,
+                                  int64_t *pad_len, void *stream) {
+    if (!valid_bit_count(bit_count)) return DL_ERR_BIT_COUNT;
+    if (features < 0 || batch < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (pad_len) *pad_len = (bit_count - batch % bit_count) % bit_count;
+    if (features == 0 || batch == 0) return DL_OK;
+    if (!t || !out) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    const int64_t words = dl_ceil_div(batch, bit_count);
+    const int64_t out_row_bytes = words * (bit_count / 8);
+    const unsigned gy = (unsigned) (features < 65535 ? features : 65535);
+    const bool vec = batch % 16 == 0 && dl_aligned(t, 16) && out_row_bytes % 2 == 0 && dl_aligned(out, 2);
+    if (vec) {
+        int64_t gx = dl_ceil_div(out_row_bytes / 2, DL_BLOCK);
+        if (gx > 65535) gx = 65535;
+        hipLaunchKernelGGL(packbits_vec16_kernel, dim3((unsigned) gx, gy), dim3(DL_BLOCK), 0, s, t, (uint8_t *) out,
+                           features, batch, out_row_bytes);
+    } else {
+        int64_t gx = dl_ceil_div(out_row_bytes, DL_BLOCK);
+        if (gx > 65535) gx = 65535;
+        hipLaunchKernelGGL(packbits_generic_kernel, dim3((unsigned) gx, gy), dim3(DL_BLOCK), 0, s, t,
+                           (uint8_t *) out, features, batch, out_row_bytes);
+    }
+    return dl_launch_status();
+}
+
+extern "C" int dl_groupbitsum(const void *b, int32_t *out, int64_t in_dim, int64_t words, int bit_count,
+                              int64_t pad_len, int64_t k, void *stream) {
+    if (!valid_bit_count(bit_count)) return DL_ERR_BIT_COUNT;
+    if (in_dim < 0 || words < 0 || k <= 0 || pad_len < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (in_dim % k != 0) return DL_ERR_NOT_DIVISIBLE;
+    const int64_t batch = words * bit_count - pad_len;
+    if (batch < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (batch == 0) return DL_OK;
+    if (!out || (!b && in_dim > 0)) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    const int64_t per_class = in_dim / k;
+    const int64_t row_bytes = words * (bit_count / 8);
+    if (per_class > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+
+    if (row_bytes % 8 == 0 && dl_aligned(b, 8) && k <= 65535) {
+        const int64_t words64 = row_bytes / 8;
+        const int64_t gx = dl_ceil_div(words64, DL_WAVE);
+        if (gx > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+        const dim3 grid((unsigned) gx, (unsigned) k);
+        const int64_t chunk = (per_class + 3) / 4;      // rows one wave counts
+        const uint64_t *bw = (const uint64_t *) b;
+        // NPH planes above weight 8 hold counts up to 16 * 2^NPH - 1.
+        if (chunk < (16LL << 8))
+            hipLaunchKernelGGL(groupbitsum_kernel<8>, grid, dim3(DL_BLOCK), 0, s, bw, out, words64, per_class, k, batch);
+        else if (chunk < (16LL << 14))
+            hipLaunchKernelGGL(groupbitsum_kernel<14>, grid, dim3(DL_BLOCK), 0, s, bw, out, words64, per_class, k, batch);
+        else
+            hipLaunchKernelGGL(groupbitsum_kernel<27>, grid, dim3(DL_BLOCK), 0, s, bw, out, words64, per_class, k, batch);
+    } else {
+        int64_t gx = dl_ceil_div(batch, DL_BLOCK);
+        if (gx > 0x7fffffffLL) gx = 0x7fffffffLL;
+        const unsigned gy = (unsigned) (k < 65535 ? k : 65535);
+        hipLaunchKernelGGL(groupbitsum_generic_kernel, dim3((unsigned) gx, gy), dim3(DL_BLOCK), 0, s,
+                           (const uint8_t *) b, out, row_bytes, per_class, k, batch);
+    }
+    return dl_launch_status();
+}

@@ -1,0 +1,419 @@
+// Training-mode kernels for gfx950: relaxed forward, backward_w, backward_x.
+//
+// Layout: activations are feature-major [features, batch]; lanes run along the batch so that
+// every gathered row segment is one coalesced access (16 bytes per lane where the batch length
+// and the base addresses allow it).  Everything indexed by the neuron (connection indices, the
+// 16 gate weights) is wave-uniform and read through the scalar cache.
+//
+// The mixture of the 16 relaxed gates is bilinear in (a, b).  With
+//     P_st = sum_i w_i * [gate i is true at (s, t)]            (four sums of eight weights)
+// it is  y = (1-a)(1-b) P00 + (1-a) b P01 + a (1-b) P10 + a b P11, evaluated as two
+// interpolations along b followed by one along a.
+#include <hip/hip_fp16.h>
+
+#include "dl_common.h"
+
+namespace {
+
+template <typename T> struct Acc { typedef float type; };
+template <> struct Acc<double> { typedef double type; };
+
+template <typename T, int N> struct alignas(sizeof(T) * N) Pack { T v[N]; };
+
+template <typename T> __device__ __forceinline__ typename Acc<T>::type up(T v) { return (typename Acc<T>::type) v; }
+template <> __device__ __forceinline__ float up<__half>(__half v) { return __half2float(v); }
+template <typename T, typename C> __device__ __forceinline__ T down(C v) { return (T) v; }
+template <> __device__ __forceinline__ __half down<__half, float>(float v) { return __float2half(v); }
+
+// The four corner values of neuron n's gate mixture.
+template <typename C> struct Corners { C p00, p01, p10, p11; };
+
+template <typename T> __device__ __forceinline__ Corners<typename Acc<T>::type> corners(const T *__restrict__ w, int64_t n) {
+    typedef typename Acc<T>::type C;
+    C g[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) g[i] = up<T>(w[n * 16 + i]);
+    Corners<C> c;
+    c.p00 = ((g[8] + g[9]) + (g[10] + g[11])) + ((g[12] + g[13]) + (g[14] + g[15]));
+    c.p01 = ((g[4] + g[5]) + (g[6] + g[7])) + ((g[12] + g[13]) + (g[14] + g[15]));
+    c.p10 = ((g[2] + g[3]) + (g[6] + g[7])) + ((g[10] + g[11]) + (g[14] + g[15]));
+    c.p11 = ((g[1] + g[3]) + (g[5] + g[7])) + ((g[9] + g[11]) + (g[13] + g[15]));
+    return c;
+}
+
+// ------------------------------------------------------------------------------------------
+// forward: one wave = NPW neurons x 64 vectors of the batch.
+// ------------------------------------------------------------------------------------------
+template <typename T, int VEC, int NPW>
+__global__ __launch_bounds__(DL_BLOCK) void forward_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
+                                                           const int64_t *__restrict__ b, const T *__restrict__ w,
+                                                           T *__restrict__ y, int64_t out_dim, int64_t ncols) {
+    typedef typename Acc<T>::type C;
+    typedef Pack<T, VEC> P;
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t n0 = ((int64_t) blockIdx.x * 4 + wave) * NPW;
+    if (n0 >= out_dim) return;
+
+    int64_t ia[NPW], ib[NPW];
+    C p00[NPW], p10[NPW], d0[NPW], d1[NPW];
+#pragma unroll
+    for (int j = 0; j < NPW; ++j) {
+        const int64_t n = (n0 + j < out_dim) ? n0 + j : out_dim - 1;
+        ia[j] = a[n];
+        ib[j] = b[n];
+        const Corners<C> c = corners<T>(w, n);
+        p00[j] = c.p00;
+        p10[j] = c.p10;
+        d0[j] = c.p01 - c.p00;
+        d1[j] = c.p11 - c.p10;
+    }
+    const P *xv = reinterpret_cast<const P *>(x);
+    P *yv = reinterpret_cast<P *>(y);
+    for (int64_t col = (int64_t) blockIdx.y * DL_WAVE + lane; col < ncols; col += (int64_t) gridDim.y * DL_WAVE) {
+        P va[NPW], vb[NPW];
+#pragma unroll
+        for (int j = 0; j < NPW; ++j) {
+            va[j] = xv[ia[j] * ncols + col];
+            vb[j] = xv[ib[j] * ncols + col];
+        }
+#pragma unroll
+        for (int j = 0; j < NPW; ++j) {
+            if (n0 + j < out_dim) {
+                P r;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const C av = up<T>(va[j].v[e]), bv = up<T>(vb[j].v[e]);
+                    const C lo = p00[j] + bv * d0[j];
+                    const C hi = p10[j] + bv * d1[j];
+                    r.v[e] = down<T, C>(lo + av * (hi - lo));
+                }
+                yv[(n0 + j) * ncols + col] = r;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Wave-wide sums with a fixed association order (deterministic).
+// ------------------------------------------------------------------------------------------
+template <int CTRL> __device__ __forceinline__ float dpp_f32(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]  : lane ^ 1
+    v += dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]  : lane ^ 2
+    v += dpp_f32<0x141>(v);  // row_half_mirror      : the other quad of the 8-lane half row
+    v += dpp_f32<0x140>(v);  // row_mirror           : the other half of the 16-lane row
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+    for (int m = 1; m < DL_WAVE; m <<= 1) v += __shfl_xor(v, m, DL_WAVE);
+    return v;
+}
+
+// ------------------------------------------------------------------------------------------
+// backward_w: per neuron, the four corner-weighted batch sums
+//     S_st = sum_r g[r] * a^s (1-a)^(1-s) * b^t (1-b)^(1-t)
+// and grad_w[n, i] = sum of the S_st at which gate i is true.
+// WPN = waves that share one neuron's batch (1: a wave owns NPW neurons; 4: the workgroup's
+// four waves split the batch of NPW neurons and combine through LDS in wave order).
+// ------------------------------------------------------------------------------------------
+template <typename T, int VEC, int NPW, int WPN>
+__global__ __launch_bounds__(DL_BLOCK) void backward_w_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
+                                                              const int64_t *__restrict__ b,
+                                                              const T *__restrict__ gy, T *__restrict__ gw,
+                                                              int64_t out_dim, int64_t ncols) {
+    typedef typename Acc<T>::type C;
+    typedef Pack<T, VEC> P;
+    __shared__ C partial[4][NPW][4];
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t n0 = (WPN == 1) ? ((int64_t) blockIdx.x * 4 + wave) * NPW : (int64_t) blockIdx.x * NPW;
+    const int part = (WPN == 1) ? 0 : wave;
+
+    C s00[NPW], s01[NPW], s10[NPW], s11[NPW];
+#pragma unroll
+    for (int j = 0; j < NPW; ++j) s00[j] = s01[j] = s10[j] = s11[j] = (C) 0;
+
+    if (n0 < out_dim) {
+        int64_t ia[NPW], ib[NPW], nn[NPW];
+#pragma unroll
+        for (int j = 0; j < NPW; ++j) {
+            nn[j] = (n0 + j < out_dim) ? n0 + j : out_dim - 1;
+            ia[j] = a[nn[j]];
+            ib[j] = b[nn[j]];
+        }
+        const P *xv = reinterpret_cast<const P *>(x);
+        const P *gv = reinterpret_cast<const P *>(gy);
+        for (int64_t base = (int64_t) part * DL_WAVE; base < ncols; base += (int64_t) WPN * DL_WAVE) {
+            const int64_t col = base + lane;
+            if (col < ncols) {
+                P va[NPW], vb[NPW], vg[NPW];
+#pragma unroll
+                for (int j = 0; j < NPW; ++j) {
+                    va[j] = xv[ia[j] * ncols + col];
+                    vb[j] = xv[ib[j] * ncols + col];
+                    vg[j] = gv[nn[j] * ncols + col];
+                }
+#pragma unroll
+                for (int j = 0; j < NPW; ++j) {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        const C av = up<T>(va[j].v[e]), bv = up<T>(vb[j].v[e]), g = up<T>(vg[j].v[e]);
+                        const C ga = g * av, gna = g - ga;       // g*a, g*(1-a)
+                        const C t11 = ga * bv, t01 = gna * bv;
+                        s11[j] += t11;
+                        s10[j] += ga - t11;
+                        s01[j] += t01;
+                        s00[j] += gna - t01;
+                    }
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int j = 0; j < NPW; ++j) {
+        s00[j] = wave_sum(s00[j]);
+        s01[j] = wave_sum(s01[j]);
+        s10[j] = wave_sum(s10[j]);
+        s11[j] = wave_sum(s11[j]);
+    }
+
+    if (WPN != 1) {
+        if (lane == 0) {
+#pragma unroll
+            for (int j = 0; j < NPW; ++j) {
+                partial[wave][j][0] = s00[j];
+                partial[wave][j][1] = s01[j];
+                partial[wave][j][2] = s10[j];
+                partial[wave][j][3] = s11[j];
+            }
+        }
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int j = 0; j < NPW; ++j) {
+            s00[j] = (partial[0][j][0] + partial[1][j][0]) + (partial[2][j][0] + partial[3][j][0]);
+            s01[j] = (partial[0][j][1] + partial[1][j][1]) + (partial[2][j][1] + partial[3][j][1]);
+            s10[j] = (partial[0][j][2] + partial[1][j][2]) + (partial[2][j][2] + partial[3][j][2]);
+            s11[j] = (partial[0][j][3] + partial[1][j][3]) + (partial[2][j][3] + partial[3][j][3]);
+        }
+    }
+
+    // lane i < 16 holds gate i: add the corners whose truth-table bit is set.
+    if (lane < 16) {
+#pragma unroll
+        for (int j = 0; j < NPW; ++j) {
+            if (n0 + j < out_dim) {
+                C r = (C) 0;
+                if (lane & 8) r += s00[j];
+                if (lane & 4) r += s01[j];
+                if (lane & 2) r += s10[j];
+                if (lane & 1) r += s11[j];
+                gw[(n0 + j) * 16 + lane] = down<T, C>(r);
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// backward_x: one wave = one input row x 64 vectors of the batch; it walks the row's fan-out
+// list (reverse index) and gathers, so every grad_x element has a single writer.
+//     dy/da = (P10 - P00) + b * ((P11 - P10) - (P01 - P00))
+//     dy/db = (P01 - P00) + a * ((P11 - P10) - (P01 - P00))
+// A neuron wired twice to this input appears twice in the list; each visit adds half of
+// dy/da + dy/db.
+// ------------------------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ __launch_bounds__(DL_BLOCK) void backward_x_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
+                                                              const int64_t *__restrict__ b, const T *__restrict__ w,
+                                                              const T *__restrict__ gy,
+                                                              const int64_t *__restrict__ start,
+                                                              const int64_t *__restrict__ idx, T *__restrict__ gx,
+                                                              int64_t in_dim, int64_t ncols,
+                                                              typename Acc<T>::type scale) {
+    typedef typename Acc<T>::type C;
+    typedef Pack<T, VEC> P;
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t c = (int64_t) blockIdx.x * 4 + wave;
+    if (c >= in_dim) return;
+    const int64_t e0 = start[c], e1 = start[c + 1];
+    const P *xv = reinterpret_cast<const P *>(x);
+    const P *gv = reinterpret_cast<const P *>(gy);
+    P *ov = reinterpret_cast<P *>(gx);
+
+    for (int64_t col = (int64_t) blockIdx.y * DL_WAVE + lane; col < ncols; col += (int64_t) gridDim.y * DL_WAVE) {
+        C acc[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = (C) 0;
+        for (int64_t e = e0; e < e1; e += 2) {
+            // two fan-out entries per trip so that their loads overlap
+            const bool two = e + 1 < e1;
+            const int64_t nA = idx[e], nB = two ? idx[e + 1] : nA;
+            const int64_t iaA = a[nA], ibA = b[nA], iaB = a[nB], ibB = b[nB];
+            const bool isaA = iaA == c, isaB = iaB == c;
+            const P gA = gv[nA * ncols + col], oA = xv[(isaA ? ibA : iaA) * ncols + col];
+            const P gB = gv[nB * ncols + col], oB = xv[(isaB ? ibB : iaB) * ncols + col];
+            const Corners<C> kA = corners<T>(w, nA), kB = corners<T>(w, nB);
+            {
+                const C d0 = kA.p01 - kA.p00, d1 = kA.p11 - kA.p10, dd = d1 - d0, da = kA.p10 - kA.p00;
+                const C k0 = (isaA && ibA == c) ? (C) 0.5 * (da + d0) : (isaA ? da : d0);
+#pragma unroll
+                for (int q = 0; q < VEC; ++q) acc[q] += up<T>(gA.v[q]) * (k0 + up<T>(oA.v[q]) * dd);
+            }
+            if (two) {
+                const C d0 = kB.p01 - kB.p00, d1 = kB.p11 - kB.p10, dd = d1 - d0, da = kB.p10 - kB.p00;
+                const C k0 = (isaB && ibB == c) ? (C) 0.5 * (da + d0) : (isaB ? da : d0);
+#pragma unroll
+                for (int q = 0; q < VEC; ++q) acc[q] += up<T>(gB.v[q]) * (k0 + up<T>(oB.v[q]) * dd);
+            }
+        }
+        P r;
+#pragma unroll
+        for (int q = 0; q < VEC; ++q) r.v[q] = down<T, C>(acc[q] * scale);
+        ov[c * ncols + col] = r;
+    }
+}
+
+template <typename T> struct Vec16 { static constexpr int n = 16 / (int) sizeof(T); };
+
+unsigned col_tiles(int64_t ncols) {
+    int64_t t = dl_ceil_div(ncols, DL_WAVE);
+    return (unsigned) (t > 65535 ? 65535 : t);
+}
+
+template <typename T>
+int forward_t(const void *x, const int64_t *a, const int64_t *b, const void *w, void *y, int64_t out_dim,
+              int64_t batch, hipStream_t s) {
+    constexpr int NPW = 4;
+    const int64_t blocks = dl_ceil_div(out_dim, 4 * NPW);
+    if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    constexpr int V = Vec16<T>::n;
+    if (batch % V == 0 && dl_aligned(x, 16) && dl_aligned(y, 16)) {
+        hipLaunchKernelGGL((forward_kernel<T, V, NPW>), dim3((unsigned) blocks, col_tiles(batch / V)), dim3(DL_BLOCK), 0, s,
+                           (const T *) x, a, b, (const T *) w, (T *) y, out_dim, batch / V);
+    } else {
+        hipLaunchKernelGGL((forward_kernel<T, 1, NPW>), dim3((unsigned) blocks, col_tiles(batch)), dim3(DL_BLOCK), 0, s,
+                           (const T *) x, a, b, (const T *) w, (T *) y, out_dim, batch);
+    }
+    return dl_launch_status();
+}
+
+template <typename T>
+int backward_w_t(const void *x, const int64_t *a, const int64_t *b, const void *gy, void *gw, int64_t out_dim,
+                 int64_t batch, hipStream_t s) {
+    constexpr int NPW = 2;
+    constexpr int V = Vec16<T>::n;
+    const bool vec = batch % V == 0 && dl_aligned(x, 16) && dl_aligned(gy, 16);
+    const int64_t ncols = vec ? batch / V : batch;
+    // Split one neuron's batch over the four waves once every wave still gets whole segments.
+    const bool split = ncols >= 8 * DL_WAVE;
+    const int64_t blocks = split ? dl_ceil_div(out_dim, NPW) : dl_ceil_div(out_dim, 4 * NPW);
+    if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    const dim3 grid((unsigned) blocks), block(DL_BLOCK);
+    const T *xp = (const T *) x, *gp = (const T *) gy;
+    T *wp = (T *) gw;
+    if (vec && split)
+        hipLaunchKernelGGL((backward_w_kernel<T, V, NPW, 4>), grid, block, 0, s, xp, a, b, gp, wp, out_dim, ncols);
+    else if (vec)
+        hipLaunchKernelGGL((backward_w_kernel<T, V, NPW, 1>), grid, block, 0, s, xp, a, b, gp, wp, out_dim, ncols);
+    else if (split)
+        hipLaunchKernelGGL((backward_w_kernel<T, 1, NPW, 4>), grid, block, 0, s, xp, a, b, gp, wp, out_dim, ncols);
+    else
+        hipLaunchKernelGGL((backward_w_kernel<T, 1, NPW, 1>), grid, block, 0, s, xp, a, b, gp, wp, out_dim, ncols);
+    return dl_launch_status();
+}
+
+template <typename T>
+int backward_x_t(const void *x, const int64_t *a, const int64_t *b, const void *w, const void *gy,
+                 const int64_t *start, const int64_t *idx, void *gx, int64_t in_dim, int64_t batch, double scale,
+                 hipStream_t s) {
+    typedef typename Acc<T>::type C;
+    constexpr int V = Vec16<T>::n;
+    const int64_t blocks = dl_ceil_div(in_dim, 4);
+    if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    if (batch % V == 0 && dl_aligned(x, 16) && dl_aligned(gy, 16) && dl_aligned(gx, 16)) {
+        hipLaunchKernelGGL((backward_x_kernel<T, V>), dim3((unsigned) blocks, col_tiles(batch / V)), dim3(DL_BLOCK), 0, s,
+                           (const T *) x, a, b, (const T *) w, (const T *) gy, start, idx, (T *) gx, in_dim, batch / V,
+                           (C) scale);
+    } else {
+        hipLaunchKernelGGL((backward_x_kernel<T, 1>), dim3((unsigned) blocks, col_tiles(batch)), dim3(DL_BLOCK), 0, s,
+                           (const T *) x, a, b, (const T *) w, (const T *) gy, start, idx, (T *) gx, in_dim, batch,
+                           (C) scale);
+    }
+    return dl_launch_status();
+}
+
+}  // namespace
+
+extern "C" int dl_logic_forward(const void *x, const int64_t *a, const int64_t *b, const void *w, void *y,
+                                int64_t in_dim, int64_t out_dim, int64_t batch, int dtype, void *stream) {
+    if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
+    if (in_dim < 0 || out_dim < 0 || batch < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim == 0 || batch == 0) return DL_OK;
+    if (!x || !a || !b || !w || !y || in_dim == 0) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    switch (dtype) {
+    case DL_F16: return forward_t<__half>(x, a, b, w, y, out_dim, batch, s);
+    case DL_F32: return forward_t<float>(x, a, b, w, y, out_dim, batch, s);
+    default: return forward_t<double>(x, a, b, w, y, out_dim, batch, s);
+    }
+}
+
+extern "C" int dl_logic_backward_w(const void *x, const int64_t *a, const int64_t *b, const void *grad_y,
+                                   void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch, int dtype,
+                                   void *stream) {
+    if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
+    if (in_dim < 0 || out_dim < 0 || batch < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim == 0) return DL_OK;
+    if (!a || !b || !grad_w || in_dim == 0) return DL_ERR_INVALID_ARGUMENT;
+    if (batch > 0 && (!x || !grad_y)) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    switch (dtype) {
+    case DL_F16: return backward_w_t<__half>(x, a, b, grad_y, grad_w, out_dim, batch, s);
+    case DL_F32: return backward_w_t<float>(x, a, b, grad_y, grad_w, out_dim, batch, s);
+    default: return backward_w_t<double>(x, a, b, grad_y, grad_w, out_dim, batch, s);
+    }
+}
+
+extern "C" int dl_logic_backward_x(const void *x, const int64_t *a, const int64_t *b, const void *w,
+                                   const void *grad_y, const int64_t *start, const int64_t *idx, void *grad_x,
+                                   int64_t in_dim, int64_t out_dim, int64_t batch, double scale, int dtype,
+                                   void *stream) {
+    if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
+    if (in_dim < 0 || out_dim < 0 || batch < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (in_dim == 0 || batch == 0) return DL_OK;
+    if (!x || !grad_x || !start) return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim > 0 && (!a || !b || !w || !grad_y || !idx)) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    switch (dtype) {
+    case DL_F16: return backward_x_t<__half>(x, a, b, w, grad_y, start, idx, grad_x, in_dim, batch, scale, s);
+    case DL_F32: return backward_x_t<float>(x, a, b, w, grad_y, start, idx, grad_x, in_dim, batch, scale, s);
+    default: return backward_x_t<double>(x, a, b, w, grad_y, start, idx, grad_x, in_dim, batch, scale, s);
+    }
+}
+
+extern "C" int dl_version(void) { return 100; }
+
+extern "C" const char *dl_status_string(int status) {
+    switch (status) {
+    case DL_OK: return "ok";
+    case DL_ERR_INVALID_ARGUMENT: return "invalid argument (null pointer, negative size or misaligned buffer)";
+    case DL_ERR_BIT_COUNT: return "`bit_count` has to be in { 8, 16, 32, 64 }";
+    case DL_ERR_NOT_DIVISIBLE: return "in_dim has to be divisible by k";
+    case DL_ERR_DTYPE: return "dtype has to be DL_F16, DL_F32 or DL_F64";
+    case DL_ERR_LAUNCH: return "HIP refused the kernel launch";
+    case DL_ERR_TOO_LARGE: return "size exceeds what this entry point supports";
+    default: return "unknown status";
+    }
+}

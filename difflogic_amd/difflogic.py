@@ -1,0 +1,170 @@
+"""LogicLayer, GroupSum and the autograd glue (reference: difflogic/difflogic.py), running on
+the gfx950 kernels through ``difflogic_cuda``."""
+import torch
+
+from . import difflogic_cuda
+from .functional import (GradFactor, bin_op_s, build_reverse_index, get_random_connections,
+                         get_unique_connections)
+from .packbitstensor import PackBitsTensor
+
+
+class LogicLayer(torch.nn.Module):
+    """A layer of ``out_dim`` two-input logic gates, each a learnable mixture of the 16 gates
+    over two fixed inputs (difflogic/difflogic.py:11-169).
+
+    :param in_dim:      number of inputs
+    :param out_dim:     number of gates
+    :param device:      'cuda' (the MI355X; torch-ROCm names it cuda) or 'cpu'
+    :param grad_factor: scales the gradient passed to the layer's input (use >1 for deep nets)
+    :param implementation: 'cuda' (HIP kernels, default on 'cuda') or 'python' (eager torch,
+                        default on 'cpu'); never chosen implicitly for a 'cuda' layer
+    :param connections: 'random' or 'unique'
+    """
+
+    def __init__(self, in_dim: int, out_dim: int, device: str = "cuda", grad_factor: float = 1.,
+                 implementation: str = None, connections: str = "random"):
+        super().__init__()
+        # drawn before the connections, from the device's generator (difflogic.py:33)
+        self.weights = torch.nn.parameter.Parameter(torch.randn(out_dim, 16, device=device))
+        self.in_dim = in_dim
+        self.out_dim = out_dim
+        self.device = device
+        self.grad_factor = grad_factor
+
+        if implementation is None:
+            implementation = {"cuda": "cuda", "cpu": "python"}.get(device)
+        assert implementation in ["cuda", "python"], implementation
+        self.implementation = implementation
+
+        assert connections in ["random", "unique"], connections
+        self.connections = connections
+        self.set_connections(*self.get_connections(connections, device))
+
+        self.num_neurons = out_dim
+        self.num_weights = out_dim
+
+    def set_connections(self, a, b):
+        """Installs the wiring ``a, b`` ([out_dim] integer tensors with values in [0, in_dim))
+        and rebuilds the reverse index the backward pass walks.  The wiring is not part of the
+        state_dict (only ``weights`` is), so a model restored from a state_dict needs the
+        wiring of the model that was saved: same seed, or this method."""
+        a = torch.as_tensor(a).to(torch.int64).to(self.device).contiguous()
+        b = torch.as_tensor(b).to(torch.int64).to(self.device).contiguous()
+        if a.shape != (self.out_dim,) or b.shape != (self.out_dim,):
+            raise ValueError(f"expected two index tensors of shape ({self.out_dim},), got {tuple(a.shape)}, "
+                             f"{tuple(b.shape)}")
+        if self.out_dim and (min(int(a.min()), int(b.min())) < 0 or max(int(a.max()), int(b.max())) >= self.in_dim):
+            raise ValueError(f"connection indices have to lie in [0, {self.in_dim})")
+        self.indices = (a, b)
+        if self.implementation == "cuda":
+            # reverse index for backward_x (difflogic.py:56-69)
+            start, idx = build_reverse_index(a, b, self.in_dim)
+            self.given_x_indices_of_y_start = start.to(self.device)
+            self.given_x_indices_of_y = idx.to(self.device)
+
+    def forward(self, x):
+        if isinstance(x, PackBitsTensor):
+            assert not self.training, "PackBitsTensor is not supported for the differentiable training mode."
+            assert self.device == "cuda", (
+                "PackBitsTensor is only supported for CUDA, not for {}. If you want fast inference on CPU, "
+                "please use CompiledDiffLogicModel.".format(self.device))
+            assert self.implementation == "cuda", self.implementation
+            return self.forward_cuda_eval(x)
+        if self.implementation == "cuda":
+            return self.forward_cuda(x)
+        if self.implementation == "python":
+            if self.grad_factor != 1.:
+                x = GradFactor.apply(x, self.grad_factor)
+            return self.forward_python(x)
+        raise ValueError(self.implementation)
+
+    def forward_python(self, x):
+        assert x.shape[-1] == self.in_dim, (x.shape[-1], self.in_dim)
+        a, b = x[..., self.indices[0]], x[..., self.indices[1]]
+        if self.training:
+            w = torch.nn.functional.softmax(self.weights, dim=-1)
+        else:
+            w = torch.nn.functional.one_hot(self.weights.argmax(-1), 16).to(torch.float32)
+        return bin_op_s(a, b, w.to(x.dtype))
+
+    def forward_cuda(self, x):
+        if self.training:
+            assert x.device.type == "cuda", x.device
+        assert x.ndim == 2, x.ndim
+        x = x.transpose(0, 1).contiguous()                  # feature-major [in, B]
+        assert x.shape[0] == self.in_dim, (x.shape, self.in_dim)
+        a, b = self.indices
+        tail = (self.given_x_indices_of_y_start, self.given_x_indices_of_y, float(self.grad_factor))
+        if self.training:
+            w = torch.nn.functional.softmax(self.weights, dim=-1).to(x.dtype)
+            return LogicLayerCudaFunction.apply(x, a, b, w, *tail).transpose(0, 1)
+        w = torch.nn.functional.one_hot(self.weights.argmax(-1), 16).to(x.dtype)
+        with torch.no_grad():
+            return LogicLayerCudaFunction.apply(x, a, b, w, *tail).transpose(0, 1)
+
+    def forward_cuda_eval(self, x: PackBitsTensor):
+        """Packed inference.  Rebinds ``x.t`` and returns ``x`` (in place on the wrapper)."""
+        assert not self.training
+        assert isinstance(x, PackBitsTensor)
+        assert x.t.shape[0] == self.in_dim, (x.t.shape, self.in_dim)
+        a, b = self.indices
+        w = self.weights.argmax(-1).to(torch.uint8)
+        x.t = difflogic_cuda.eval(x.t, a, b, w)
+        return x
+
+    def extra_repr(self):
+        return "{}, {}, {}".format(self.in_dim, self.out_dim, "train" if self.training else "eval")
+
+    def get_connections(self, connections, device="cuda"):
+        assert self.out_dim * 2 >= self.in_dim, (
+            "The number of neurons ({}) must not be smaller than half of the number of inputs ({}) because "
+            "otherwise not all inputs could be used or considered.".format(self.out_dim, self.in_dim))
+        if connections == "random":
+            return get_random_connections(self.in_dim, self.out_dim, device)
+        if connections == "unique":
+            return get_unique_connections(self.in_dim, self.out_dim, device)
+        raise ValueError(connections)
+
+
+class GroupSum(torch.nn.Module):
+    """Sums contiguous groups of out/k neurons into k scores and divides by tau
+    (difflogic/difflogic.py:175-199).  On a PackBitsTensor: undivided int32 bit counts."""
+
+    def __init__(self, k: int, tau: float = 1., device="cuda"):
+        super().__init__()
+        self.k = k
+        self.tau = tau
+        self.device = device
+
+    def forward(self, x):
+        if isinstance(x, PackBitsTensor):
+            return x.group_sum(self.k)
+        assert x.shape[-1] % self.k == 0, (x.shape, self.k)
+        return x.reshape(*x.shape[:-1], self.k, x.shape[-1] // self.k).sum(-1) / self.tau
+
+    def extra_repr(self):
+        return "k={}, tau={}".format(self.k, self.tau)
+
+
+class LogicLayerCudaFunction(torch.autograd.Function):
+    """Feature-major forward/backward of one layer (difflogic/difflogic.py:205-221).  The
+    optional trailing ``grad_factor`` is folded into backward_x instead of a separate
+    elementwise pass over the input gradient."""
+
+    @staticmethod
+    def forward(ctx, x, a, b, w, given_x_indices_of_y_start, given_x_indices_of_y, grad_factor=1.0):
+        ctx.save_for_backward(x, a, b, w, given_x_indices_of_y_start, given_x_indices_of_y)
+        ctx.grad_factor = grad_factor
+        return difflogic_cuda.forward(x, a, b, w)
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        x, a, b, w, given_x_indices_of_y_start, given_x_indices_of_y = ctx.saved_tensors
+        grad_y = grad_y.contiguous()
+        grad_w = grad_x = None
+        if ctx.needs_input_grad[0]:
+            grad_x = difflogic_cuda.backward_x(x, a, b, w, grad_y, given_x_indices_of_y_start,
+                                               given_x_indices_of_y, ctx.grad_factor)
+        if ctx.needs_input_grad[3]:
+            grad_w = difflogic_cuda.backward_w(x, a, b, grad_y)
+        return grad_x, None, None, grad_w, None, None, None

@@ -1,0 +1,201 @@
+"""Drop-in for the reference's extension module ``difflogic_cuda``
+(difflogic/cuda/difflogic.cpp:45-84): the same six functions on torch tensors, implemented by
+the gfx950 kernels of libdifflogic_hip.so.
+
+Differences from the reference that callers can observe:
+* work is enqueued on torch's current stream for the tensors' device and the call returns
+  without a device-wide synchronisation (the reference blocks after every kernel);
+* HIP errors raise RuntimeError instead of terminating the process
+  (difflogic/cuda/difflogic_kernel.cu:22-28 calls exit());
+* ``backward_x`` gives a neuron with a[n] == b[n] the derivative d/da + d/db, as autograd does
+  for the python implementation (the reference's kernel counts d/da twice,
+  difflogic_kernel.cu:215-218).
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+
+_FLOAT_CODES = {torch.float16: _lib.DL_F16, torch.float32: _lib.DL_F32, torch.float64: _lib.DL_F64}
+_WORD_BITS = {torch.int8: 8, torch.uint8: 8, torch.int16: 16, torch.int32: 32, torch.int64: 64}
+_BITS_TO_DTYPE = {8: torch.int8, 16: torch.int16, 32: torch.int32, 64: torch.int64}
+
+
+def _check_input(t, name):
+    # difflogic_kernel.cu:13-17 (CHECK_CUDA, CHECK_CONTIGUOUS)
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+def _check_index(t, name, numel=None):
+    _check_input(t, name)
+    if t.dtype != torch.int64 or t.dim() != 1:
+        raise RuntimeError(f"expected {name} to be a 1-D int64 tensor, got {t.dtype} with {t.dim()} dims")
+    if numel is not None and t.numel() != numel:
+        raise RuntimeError(f"{name} has {t.numel()} elements, expected {numel}")
+
+
+def _float_code(t, name):
+    code = _FLOAT_CODES.get(t.dtype)
+    if code is None:
+        raise RuntimeError(f'"{name}" not implemented for \'{t.dtype}\'')
+    return code
+
+
+def _same_device(*tensors):
+    dev = tensors[0].device
+    for t in tensors[1:]:
+        if t.device != dev:
+            raise RuntimeError(f"all tensors must be on the same device, got {dev} and {t.device}")
+    return dev
+
+
+def _stream(dev):
+    return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def _raise(status, what):
+    msg = f"{what}: {_lib.status_string(status)}"
+    if status in (_lib.DL_ERR_BIT_COUNT, _lib.DL_ERR_NOT_DIVISIBLE):
+        raise ValueError(msg)
+    raise RuntimeError(msg)
+
+
+def _p(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def forward(x, a, b, w):
+    """x [in,B], a/b [out] int64, w [out,16] -> y [out,B]   (difflogic.cpp:46-51)."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w")):
+        _check_input(t, n)
+    code = _float_code(x, "logic_layer_cuda_forward")
+    if x.dim() != 2 or w.dim() != 2 or w.shape[1] != 16 or w.dtype != x.dtype:
+        raise RuntimeError(f"expected x [in,B] and w [out,16] of one dtype, got {tuple(x.shape)} {x.dtype}, "
+                           f"{tuple(w.shape)} {w.dtype}")
+    out_dim = w.shape[0]
+    _check_index(a, "a", out_dim)
+    _check_index(b, "b", out_dim)
+    dev = _same_device(x, a, b, w)
+    in_dim, batch = x.shape
+    y = torch.empty((out_dim, batch), dtype=x.dtype, device=dev)
+    with torch.cuda.device(dev):
+        st = _lib.load().dl_logic_forward(_p(x), _p(a), _p(b), _p(w), _p(y), in_dim, out_dim, batch, code, _stream(dev))
+    if st:
+        _raise(st, "logic_layer_cuda_forward")
+    return y
+
+
+def backward_w(x, a, b, grad_y):
+    """-> grad_w [out,16]   (difflogic.cpp:52-56)."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (grad_y, "grad_y")):
+        _check_input(t, n)
+    code = _float_code(x, "logic_layer_cuda_backward_w")
+    if x.dim() != 2 or grad_y.dim() != 2 or grad_y.shape[1] != x.shape[1] or grad_y.dtype != x.dtype:
+        raise RuntimeError(f"expected x [in,B] and grad_y [out,B] of one dtype, got {tuple(x.shape)} {x.dtype}, "
+                           f"{tuple(grad_y.shape)} {grad_y.dtype}")
+    out_dim = grad_y.shape[0]
+    _check_index(a, "a", out_dim)
+    _check_index(b, "b", out_dim)
+    dev = _same_device(x, a, b, grad_y)
+    in_dim, batch = x.shape
+    grad_w = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
+    with torch.cuda.device(dev):
+        st = _lib.load().dl_logic_backward_w(_p(x), _p(a), _p(b), _p(grad_y), _p(grad_w), in_dim, out_dim, batch, code,
+                                             _stream(dev))
+    if st:
+        _raise(st, "logic_layer_cuda_backward_w")
+    return grad_w
+
+
+def backward_x(x, a, b, w, grad_y, given_x_indices_of_y_start, given_x_indices_of_y, scale=1.0):
+    """-> grad_x [in,B]   (difflogic.cpp:57-62).  ``scale`` multiplies the result (1.0 = the
+    reference's function); LogicLayer passes its grad_factor here."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w"), (grad_y, "grad_y"),
+                 (given_x_indices_of_y_start, "given_x_indices_of_y_start"),
+                 (given_x_indices_of_y, "given_x_indices_of_y")):
+        _check_input(t, n)
+    code = _float_code(x, "logic_layer_cuda_backward_x")
+    if (x.dim() != 2 or grad_y.dim() != 2 or grad_y.shape[1] != x.shape[1] or grad_y.dtype != x.dtype
+            or w.dim() != 2 or w.shape != (grad_y.shape[0], 16) or w.dtype != x.dtype):
+        raise RuntimeError(f"expected x [in,B], w [out,16], grad_y [out,B] of one dtype, got {tuple(x.shape)}, "
+                           f"{tuple(w.shape)}, {tuple(grad_y.shape)}")
+    in_dim, batch = x.shape
+    out_dim = grad_y.shape[0]
+    _check_index(a, "a", out_dim)
+    _check_index(b, "b", out_dim)
+    _check_index(given_x_indices_of_y_start, "given_x_indices_of_y_start", in_dim + 1)
+    _check_index(given_x_indices_of_y, "given_x_indices_of_y", 2 * out_dim)
+    dev = _same_device(x, a, b, w, grad_y, given_x_indices_of_y_start, given_x_indices_of_y)
+    grad_x = torch.empty_like(x)
+    with torch.cuda.device(dev):
+        st = _lib.load().dl_logic_backward_x(_p(x), _p(a), _p(b), _p(w), _p(grad_y), _p(given_x_indices_of_y_start),
+                                             _p(given_x_indices_of_y), _p(grad_x), in_dim, out_dim, batch,
+                                             float(scale), code, _stream(dev))
+    if st:
+        _raise(st, "logic_layer_cuda_backward_x")
+    return grad_x
+
+
+def eval(x, a, b, w):  # noqa: A001  (the reference's name)
+    """x [in,W] int words, w [out] uint8 gate ids -> y [out,W]   (difflogic.cpp:63-68)."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w")):
+        _check_input(t, n)
+    bits = _WORD_BITS.get(x.dtype)
+    if bits is None:
+        raise RuntimeError(f'"logic_layer_cuda_eval_kernel" not implemented for \'{x.dtype}\'')
+    if x.dim() != 2 or w.dim() != 1 or w.dtype != torch.uint8:
+        raise RuntimeError(f"expected x [in,W] and w [out] uint8, got {tuple(x.shape)}, {tuple(w.shape)} {w.dtype}")
+    out_dim = w.shape[0]
+    _check_index(a, "a", out_dim)
+    _check_index(b, "b", out_dim)
+    dev = _same_device(x, a, b, w)
+    in_dim, words = x.shape
+    y = torch.empty((out_dim, words), dtype=x.dtype, device=dev)
+    with torch.cuda.device(dev):
+        st = _lib.load().dl_logic_eval(_p(x), _p(a), _p(b), _p(w), _p(y), in_dim, out_dim, words, bits, _stream(dev))
+    if st:
+        _raise(st, "logic_layer_cuda_eval")
+    return y
+
+
+def tensor_packbits_cuda(t, bit_count):
+    """bool [F,B] -> (int{bit_count} [F, ceil(B/bit_count)], pad_len)   (difflogic.cpp:69-74)."""
+    _check_input(t, "t")
+    if bit_count not in _BITS_TO_DTYPE:
+        raise ValueError("`bit_count` has to be in { 8, 16, 32, 64 }")
+    if t.dtype != torch.bool or t.dim() != 2:
+        raise RuntimeError(f"expected t to be a 2-D bool tensor, got {t.dtype} with {t.dim()} dims")
+    features, batch = t.shape
+    words = -(-batch // bit_count)
+    out = torch.empty((features, words), dtype=_BITS_TO_DTYPE[bit_count], device=t.device)
+    pad = ctypes.c_int64(0)
+    with torch.cuda.device(t.device):
+        st = _lib.load().dl_tensor_packbits(_p(t), _p(out), features, batch, bit_count, ctypes.byref(pad),
+                                            _stream(t.device))
+    if st:
+        _raise(st, "tensor_packbits_cuda")
+    return out, int(pad.value)
+
+
+def groupbitsum(b, pad_len, k):
+    """int words [out,W] -> int32 [W*bits - pad_len, k]   (difflogic.cpp:75-83)."""
+    _check_input(b, "b")
+    bits = _WORD_BITS.get(b.dtype)
+    if bits is None or b.dim() != 2:
+        raise RuntimeError(f'"groupbitsum_kernel" not implemented for \'{b.dtype}\' with {b.dim()} dims')
+    if k <= 0 or b.shape[0] % k != 0:
+        raise ValueError(f"in_dim ({b.shape[0]}) has to be divisible by k ({k}) but it is not")
+    in_dim, words = b.shape
+    batch = words * bits - int(pad_len)
+    if pad_len < 0 or batch < 0:
+        raise RuntimeError(f"pad_len ({pad_len}) has to be in [0, {words * bits}]")
+    out = torch.empty((batch, k), dtype=torch.int32, device=b.device)
+    with torch.cuda.device(b.device):
+        st = _lib.load().dl_groupbitsum(_p(b), _p(out), in_dim, words, bits, int(pad_len), int(k), _stream(b.device))
+    if st:
+        _raise(st, "groupbitsum")
+    return out

@@ -1,0 +1,103 @@
+/* difflogic_hip.h -- C ABI of libdifflogic_hip.so: the LogicLayer kernel family for AMD
+ * MI355X (gfx950), hand-written HIP.
+ *
+ * Conventions
+ * -----------
+ * - Every pointer is a DEVICE pointer on the current HIP device unless stated otherwise.
+ *   The library never allocates, frees or synchronises: the caller owns all buffers
+ *   (inputs are read-only, outputs are fully overwritten) and orders work through the
+ *   `stream` argument (a hipStream_t passed as void*; NULL = the null stream).
+ * - All matrices are feature-major and batch-contiguous: element (row f, column r) of an
+ *   [F, R] matrix lives at f*R + r.
+ * - Index tables `a`, `b` hold values in [0, in_dim); `start`/`idx` are the CSR reverse
+ *   index the reference builds at difflogic/difflogic.py:60-69.  The kernels trust them.
+ * - Every function returns a dl_status (0 = success).  Nothing here calls exit().
+ * - Functions are re-entrant; there is no global state.
+ *
+ * Each entry point replaces one function of the reference's extension module
+ * `difflogic_cuda` (difflogic/cuda/difflogic.cpp:45-84); the comment above each declaration
+ * names it.
+ */
+#ifndef DIFFLOGIC_HIP_H
+#define DIFFLOGIC_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum dl_status {
+    DL_OK = 0,
+    DL_ERR_INVALID_ARGUMENT = 1, /* null pointer, negative size, misaligned buffer            */
+    DL_ERR_BIT_COUNT = 2,        /* bit_count not in {8, 16, 32, 64}                          */
+    DL_ERR_NOT_DIVISIBLE = 3,    /* groupbitsum: in_dim not divisible by k                    */
+    DL_ERR_DTYPE = 4,            /* dtype not one of dl_dtype                                 */
+    DL_ERR_LAUNCH = 5,           /* the HIP runtime refused the launch (see hipGetLastError)  */
+    DL_ERR_TOO_LARGE = 6         /* a size exceeds what the entry point supports              */
+} dl_status;
+
+typedef enum dl_dtype { DL_F16 = 0, DL_F32 = 1, DL_F64 = 2 } dl_dtype;
+
+/* Library version (major*10000 + minor*100 + patch) and a static message per status. */
+int dl_version(void);
+const char *dl_status_string(int status);
+
+/* ---- training mode -------------------------------------------------------------------- */
+
+/* Replaces `forward` = logic_layer_cuda_forward (difflogic/cuda/difflogic.cpp:46-51,
+ * difflogic/cuda/difflogic_kernel.cu:259-297).
+ *   x [in_dim, batch], w [out_dim, 16], y [out_dim, batch] of `dtype`; a, b [out_dim] int64.
+ *   y[n,r] = sum_i w[n,i] * f_i(x[a[n],r], x[b[n],r]),  f_i = real-valued gate i. */
+int dl_logic_forward(const void *x, const int64_t *a, const int64_t *b, const void *w, void *y,
+                     int64_t in_dim, int64_t out_dim, int64_t batch, int dtype, void *stream);
+
+/* Replaces `backward_w` = logic_layer_cuda_backward_w (difflogic.cpp:52-56,
+ * difflogic_kernel.cu:300-364), including the host-side sum + 16-way stack.
+ *   grad_w[n,i] = sum_r grad_y[n,r] * f_i(x[a[n],r], x[b[n],r]);  grad_w [out_dim, 16].
+ * Deterministic: fixed-order in-wave and LDS reductions, no atomics. */
+int dl_logic_backward_w(const void *x, const int64_t *a, const int64_t *b, const void *grad_y,
+                        void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch, int dtype,
+                        void *stream);
+
+/* Replaces `backward_x` = logic_layer_cuda_backward_x (difflogic.cpp:57-62,
+ * difflogic_kernel.cu:367-410).
+ *   grad_x[c,r] = scale * sum over neurons n reading input c of
+ *                 grad_y[n,r] * d y[n,r] / d x[c,r];          grad_x [in_dim, batch].
+ *   start [in_dim+1], idx [2*out_dim] int64: the reverse index.  A neuron with
+ *   a[n] == b[n] contributes d/da + d/db (autograd semantics of the python implementation).
+ *   `scale` folds the reference's GradFactor (difflogic/functional.py:130-138); pass 1.0 for
+ *   the reference's backward_x. */
+int dl_logic_backward_x(const void *x, const int64_t *a, const int64_t *b, const void *w,
+                        const void *grad_y, const int64_t *start, const int64_t *idx, void *grad_x,
+                        int64_t in_dim, int64_t out_dim, int64_t batch, double scale, int dtype,
+                        void *stream);
+
+/* ---- packed inference mode ------------------------------------------------------------ */
+
+/* Replaces `eval` = logic_layer_cuda_eval (difflogic.cpp:63-68, difflogic_kernel.cu:503-541).
+ *   x [in_dim, words], y [out_dim, words] of signed integers of `bit_count` bits;
+ *   w [out_dim] uint8 gate ids (4-bit truth tables, difflogic_kernel.cu:418-435).
+ *   y[n,c] = gate_{w[n]}(x[a[n],c], x[b[n],c]) bitwise. */
+int dl_logic_eval(const void *x, const int64_t *a, const int64_t *b, const uint8_t *w, void *y,
+                  int64_t in_dim, int64_t out_dim, int64_t words, int bit_count, void *stream);
+
+/* Replaces `tensor_packbits_cuda` (difflogic.cpp:69-74, difflogic_kernel.cu:583-625).
+ *   t [features, batch] bool bytes -> out [features, ceil(batch/bit_count)] words;
+ *   bit i of word c = sample bit_count*c + i, tail bits zero.
+ *   *pad_len (HOST pointer, may be NULL) receives (bit_count - batch % bit_count) % bit_count. */
+int dl_tensor_packbits(const uint8_t *t, void *out, int64_t features, int64_t batch, int bit_count,
+                       int64_t *pad_len, void *stream);
+
+/* Replaces `groupbitsum` (difflogic.cpp:75-83, difflogic_kernel.cu:666-700), including the
+ * final transpose.
+ *   b [in_dim, words] words -> out [words*bit_count - pad_len, k] int32 (sample-major):
+ *   out[s, c] = number of set sample-s bits over neurons c*in_dim/k ... (c+1)*in_dim/k - 1. */
+int dl_groupbitsum(const void *b, int32_t *out, int64_t in_dim, int64_t words, int bit_count,
+                   int64_t pad_len, int64_t k, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DIFFLOGIC_HIP_H */

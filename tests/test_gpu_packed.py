@@ -1,0 +1,179 @@
+"""Parity of the packed-inference HIP kernels (through the C ABI and the Python API) with the
+CPU oracle.  Bit-exact: every comparison is equality."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import interp
+from oracle import packed_oracle as po
+from tests.helpers import build_model, random_layers
+
+pytestmark = pytest.mark.gpu
+
+NP_WORD = {8: np.int8, 16: np.int16, 32: np.int32, 64: np.int64}
+
+
+@pytest.fixture(scope="module")
+def ext():
+    import difflogic_amd
+    return difflogic_amd.difflogic_cuda
+
+
+def _dev(a):
+    return torch.as_tensor(np.ascontiguousarray(a)).cuda()
+
+
+@pytest.mark.parametrize("bits", [8, 16, 32, 64])
+@pytest.mark.parametrize("F,B", [(1, 1), (3, 7), (5, 64), (5, 65), (7, 1000), (4, 1024), (9, 4112), (2, 70000),
+                                 (784, 256)])
+def test_packbits(ext, bits, F, B):
+    rng = np.random.default_rng(F * 131 + B + bits)
+    t = rng.random((F, B)) < 0.3
+    want, pad = po.packbits(t, bits)
+    got, got_pad = ext.tensor_packbits_cuda(_dev(t), bits)
+    assert got_pad == pad and got.dtype == torch.as_tensor(want).dtype and tuple(got.shape) == want.shape
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
+def test_packbits_nonzero_bytes_count_as_true(ext):
+    raw = torch.tensor([[0, 1, 2, 128, 255, 0, 7, 0] * 4], dtype=torch.uint8).cuda()
+    got, _ = ext.tensor_packbits_cuda(raw.view(torch.bool), 32)
+    want, _ = po.packbits(raw.cpu().numpy() != 0, 32)
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("bits", [8, 16, 32, 64])
+@pytest.mark.parametrize("W", [1, 2, 3, 5, 64, 127, 128, 129, 300])
+def test_eval_layer_random(ext, bits, W):
+    rng = np.random.default_rng(W * 7 + bits)
+    in_dim, out_dim = 37, 203
+    x = rng.integers(np.iinfo(NP_WORD[bits]).min, np.iinfo(NP_WORD[bits]).max, (in_dim, W), dtype=NP_WORD[bits],
+                     endpoint=True)
+    (a, b, op), = random_layers(rng, in_dim, [out_dim])
+    want = po.eval_layer(x, a, b, op)
+    got = ext.eval(_dev(x), _dev(a), _dev(b), _dev(op))
+    assert got.dtype == torch.as_tensor(want).dtype
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
+def test_eval_every_gate_on_every_input_pair(ext):
+    t = np.array([[0, 0, 1, 1], [0, 1, 0, 1]], dtype=bool)
+    x, _ = po.packbits(t, 64)
+    ops = np.arange(16, dtype=np.uint8)
+    got = ext.eval(_dev(x), _dev(np.zeros(16, np.int64)), _dev(np.ones(16, np.int64)), _dev(ops)).cpu().numpy()
+    assert np.array_equal(got, po.eval_layer(x, np.zeros(16, int), np.ones(16, int), ops))
+    bits = po.unpackbits(got, 4)
+    for i in range(16):
+        assert bits[i].astype(int).tolist() == [int(c) for c in format(i, "04b")]
+
+
+def test_eval_unaligned_views(ext):
+    # a row length that is a multiple of 8 but not 16 bytes, and an odd int8 row length
+    rng = np.random.default_rng(5)
+    for bits, W in ((64, 3), (8, 13), (16, 5), (32, 3)):
+        x = rng.integers(-100, 100, (9, W)).astype(NP_WORD[bits])
+        (a, b, op), = random_layers(rng, 9, [40])
+        got = ext.eval(_dev(x), _dev(a), _dev(b), _dev(op)).cpu().numpy()
+        assert np.array_equal(got, po.eval_layer(x, a, b, op))
+
+
+@pytest.mark.parametrize("bits,in_dim,W,k,pad", [
+    (64, 30, 1, 3, 0), (64, 30, 3, 5, 17), (64, 640, 70, 10, 63), (64, 130, 129, 2, 1), (64, 7, 5, 7, 0),
+    (64, 51, 2, 1, 5), (32, 64, 6, 4, 3), (32, 64, 5, 4, 3), (16, 40, 12, 5, 0), (16, 40, 7, 5, 9),
+    (8, 24, 16, 3, 2), (8, 24, 9, 3, 7), (64, 40000, 2, 2, 11), (64, 70000, 1, 1, 0),
+])
+def test_groupbitsum(ext, bits, in_dim, W, k, pad):
+    rng = np.random.default_rng(in_dim + W + k)
+    x = rng.integers(np.iinfo(NP_WORD[bits]).min, np.iinfo(NP_WORD[bits]).max, (in_dim, W), dtype=NP_WORD[bits],
+                     endpoint=True)
+    want = po.groupbitsum(x, pad, k)
+    got = ext.groupbitsum(_dev(x), pad, k)
+    assert got.dtype == torch.int32 and tuple(got.shape) == want.shape
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
+def test_groupbitsum_saturated_counts(ext):
+    # all bits set: every count equals the class size, for sizes around the counter-plane limits
+    for per_class in (15, 16, 17, 4095 * 4, 4096 * 4, 4096 * 4 + 1):
+        x = torch.full((per_class * 2, 3), -1, dtype=torch.int64).cuda()
+        got = ext.groupbitsum(x, 5, 2)
+        assert got.shape == (3 * 64 - 5, 2) and bool((got == per_class).all())
+
+
+def test_errors(ext):
+    x = torch.zeros(6, 2, dtype=torch.int64).cuda()
+    with pytest.raises(ValueError):
+        ext.groupbitsum(x, 0, 4)
+    with pytest.raises(ValueError):
+        ext.tensor_packbits_cuda(torch.zeros(2, 8, dtype=torch.bool).cuda(), 12)
+    with pytest.raises(RuntimeError):
+        ext.tensor_packbits_cuda(torch.zeros(2, 8, dtype=torch.bool), 8)            # CPU tensor
+    with pytest.raises(RuntimeError):
+        ext.groupbitsum(torch.zeros(6, 4, dtype=torch.int64).cuda()[:, ::2], 0, 3)  # not contiguous
+    with pytest.raises(RuntimeError):
+        ext.eval(x, torch.zeros(3, dtype=torch.int64).cuda(), torch.zeros(4, dtype=torch.int64).cuda(),
+                 torch.zeros(3, dtype=torch.uint8).cuda())                          # a/b/w lengths differ
+    # empty batch
+    out, pad = ext.tensor_packbits_cuda(torch.zeros(3, 0, dtype=torch.bool).cuda(), 64)
+    assert out.shape == (3, 0) and pad == 0
+    assert ext.groupbitsum(out, 0, 3).shape == (0, 3)
+
+
+def test_compiled_fixtures_through_the_api(golden_dir):
+    """The reference's own CompiledLogicNet outputs, reproduced by PackBitsTensor -> LogicLayer
+    (eval) -> GroupSum on the GPU."""
+    import difflogic_amd as dl
+    comp = np.load(os.path.join(golden_dir, "compiled.npz"))
+    for name in (str(c) for c in comp["cases"]):
+        F, k, bits, batch, L = (int(v) for v in comp[name + "_meta"])
+        layers = [(comp[f"{name}_a{i}"], comp[f"{name}_b{i}"], comp[f"{name}_op{i}"]) for i in range(L)]
+        model = build_model(F, layers, k).eval()
+        x = torch.as_tensor(comp[name + "_x"])
+        for bc in (bits, 64):
+            with torch.no_grad():
+                got = model(dl.PackBitsTensor(x.cuda(), bit_count=bc))
+            assert got.dtype == torch.int32
+            assert np.array_equal(got.cpu().numpy(), comp[name + "_y"]), (name, bc)
+
+
+@pytest.mark.parametrize("F,widths,k,B", [(784, [8000] * 6, 10, 4096 + 37), (100, [1000, 3000, 2000], 5, 777),
+                                          (9216, [25600, 25600], 10, 1024)])
+def test_net_against_c_interpreter(F, widths, k, B):
+    import difflogic_amd as dl
+    rng = np.random.default_rng(F + B)
+    layers = random_layers(rng, F, widths)
+    x = rng.random((B, F)) < 0.2
+    want = interp.net_eval(x, layers, k, threads=8)
+    model = build_model(F, layers, k).eval()
+    with torch.no_grad():
+        got = model(dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=64))
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
+def test_packed_equals_float_eval():
+    """On {0,1} inputs the float eval path (one-hot gates) times tau equals the packed counts."""
+    import difflogic_amd as dl
+    rng = np.random.default_rng(11)
+    layers = random_layers(rng, 50, [200, 200, 120])
+    x = rng.random((300, 50)) < 0.4
+    model = build_model(50, layers, 4, tau=7.0).eval()
+    with torch.no_grad():
+        packed = model(dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=32))
+        flt = model(torch.as_tensor(x).float().cuda())
+    assert np.array_equal(packed.cpu().numpy(), np.rint(flt.cpu().numpy() * 7.0).astype(np.int32))
+    assert np.array_equal(packed.cpu().numpy(), po.net_eval_bitwise(x, layers, 4))
+
+
+def test_pack_tensor_repr_and_modes():
+    import difflogic_amd as dl
+    t = torch.tensor([[1, 0], [0, 0], [1, 1]], dtype=torch.bool)          # [B=3, F=2]
+    p = dl.PackBitsTensor(t.cuda(), bit_count=8)
+    assert p.pad_len == 5 and p.t.shape == (2, 1) and p.flatten() is p
+    assert repr(p) == "10100000\n00100000"
+    layer = dl.LogicLayer(2, 4)
+    with pytest.raises(AssertionError):
+        layer(p)                                                          # training mode
+    with pytest.raises(NotImplementedError):
+        dl.PackBitsTensor(t, device="cpu")

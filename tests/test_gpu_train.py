@@ -1,0 +1,206 @@
+"""Parity of the training-mode HIP kernels with the float oracle (the python implementation
+restated on CPU).
+
+Tolerance: fp32 results must satisfy |got - want| <= 1e-5 * max|want| + 1e-5 * |want|
+(1e-5 relative, with the tensor's scale as the floor for entries that cancel to ~0).  The
+oracle value is computed in fp32 like the reference's python implementation; an fp64 oracle
+run bounds both."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import float_oracle as fo
+from tests.helpers import build_model, random_layers
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-5
+
+
+def close(got, want, rtol=RTOL):
+    got, want = got.detach().double().cpu(), want.detach().double().cpu()
+    scale = want.abs().max().item() if want.numel() else 0.0
+    err = (got - want).abs()
+    ok = bool((err <= rtol * scale + rtol * want.abs()).all())
+    return ok, float(err.max()) / (scale + 1e-300) if want.numel() else 0.0
+
+
+@pytest.fixture(scope="module")
+def ext():
+    import difflogic_amd
+    return difflogic_amd.difflogic_cuda
+
+
+def _case(seed, in_dim, out_dim, batch, dtype=torch.float32, equal_pairs=True):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.rand(in_dim, batch, generator=g, dtype=dtype)
+    a = torch.randint(0, in_dim, (out_dim,), generator=g)
+    b = torch.randint(0, in_dim, (out_dim,), generator=g)
+    if equal_pairs and out_dim > 3:
+        b[1] = a[1]
+        b[out_dim // 2] = a[out_dim // 2]
+    w = torch.softmax(torch.randn(out_dim, 16, generator=g, dtype=dtype), -1)
+    gy = torch.randn(out_dim, batch, generator=g, dtype=dtype)
+    return x, a, b, w, gy
+
+
+def _csr(a, b, in_dim):
+    from difflogic_amd.functional import build_reverse_index
+    return build_reverse_index(a, b, in_dim)
+
+
+SHAPES = [(5, 9, 1), (12, 30, 7), (20, 40, 64), (33, 100, 256), (64, 130, 260), (50, 77, 513), (16, 40, 2048),
+          (8, 6, 5000)]
+
+
+@pytest.mark.parametrize("in_dim,out_dim,batch", SHAPES)
+def test_forward_fp32(ext, in_dim, out_dim, batch):
+    x, a, b, w, _ = _case(batch, in_dim, out_dim, batch)
+    want = fo.ext_forward(x, a, b, w)
+    got = ext.forward(x.cuda(), a.cuda(), b.cuda(), w.cuda())
+    ok, err = close(got, want)
+    assert ok, err
+    want64 = fo.ext_forward(x.double(), a, b, w.double())
+    assert close(got, want64)[0]
+
+
+@pytest.mark.parametrize("in_dim,out_dim,batch", SHAPES)
+def test_backward_w_fp32(ext, in_dim, out_dim, batch):
+    x, a, b, w, gy = _case(batch + 1, in_dim, out_dim, batch)
+    want = fo.ext_backward_w(x, a, b, gy)
+    got = ext.backward_w(x.cuda(), a.cuda(), b.cuda(), gy.cuda())
+    assert got.shape == (out_dim, 16)
+    # the batch sum of B products carries ~sqrt(B) * eps of rounding in either implementation:
+    # compare both fp32 results with the fp64 value
+    want64 = fo.ext_backward_w(x.double(), a, b, gy.double())
+    ok, err = close(got, want64)
+    assert ok, (err, close(want, want64)[1])
+    assert bool((got[:, 0] == 0).all())
+
+
+@pytest.mark.parametrize("in_dim,out_dim,batch", SHAPES)
+def test_backward_x_fp32(ext, in_dim, out_dim, batch):
+    x, a, b, w, gy = _case(batch + 2, in_dim, out_dim, batch)
+    start, idx = _csr(a, b, in_dim)
+    want64 = fo.ext_backward_x(x.double(), a, b, w.double(), gy.double())
+    got = ext.backward_x(x.cuda(), a.cuda(), b.cuda(), w.cuda(), gy.cuda(), start.cuda(), idx.cuda())
+    ok, err = close(got, want64)
+    assert ok, err
+    got2 = ext.backward_x(x.cuda(), a.cuda(), b.cuda(), w.cuda(), gy.cuda(), start.cuda(), idx.cuda(), 2.5)
+    assert close(got2, want64 * 2.5)[0]
+
+
+def test_backward_x_unused_inputs_get_zero(ext):
+    x, a, b, w, gy = _case(0, 10, 12, 64, equal_pairs=False)
+    a = a.clamp(max=4)
+    b = b.clamp(max=4)
+    start, idx = _csr(a, b, 10)
+    got = ext.backward_x(x.cuda(), a.cuda(), b.cuda(), w.cuda(), gy.cuda(), start.cuda(), idx.cuda())
+    assert bool((got[5:] == 0).all())
+    assert close(got, fo.ext_backward_x(x.double(), a, b, w.double(), gy.double()))[0]
+
+
+@pytest.mark.parametrize("dtype,rtol", [(torch.float64, 1e-12), (torch.float16, 4e-3)])
+def test_other_dtypes(ext, dtype, rtol):
+    in_dim, out_dim, batch = 24, 50, 264
+    x, a, b, w, gy = _case(3, in_dim, out_dim, batch, torch.float64)
+    start, idx = _csr(a, b, in_dim)
+    xq, wq, gq = x.to(dtype), w.to(dtype), gy.to(dtype)
+    xr, wr, gr = xq.double(), wq.double(), gq.double()       # the oracle sees the rounded inputs
+    y = ext.forward(xq.cuda(), a.cuda(), b.cuda(), wq.cuda())
+    assert y.dtype == dtype and close(y, fo.ext_forward(xr, a, b, wr), rtol)[0]
+    gw = ext.backward_w(xq.cuda(), a.cuda(), b.cuda(), gq.cuda())
+    assert gw.dtype == dtype and close(gw, fo.ext_backward_w(xr, a, b, gr), rtol)[0]
+    gx = ext.backward_x(xq.cuda(), a.cuda(), b.cuda(), wq.cuda(), gq.cuda(), start.cuda(), idx.cuda())
+    assert gx.dtype == dtype and close(gx, fo.ext_backward_x(xr, a, b, wr, gr), rtol)[0]
+
+
+def test_backward_is_deterministic(ext):
+    x, a, b, w, gy = _case(9, 100, 3000, 512)
+    start, idx = _csr(a, b, 100)
+    dev = [t.cuda() for t in (x, a, b, w, gy, start, idx)]
+    w1 = ext.backward_w(dev[0], dev[1], dev[2], dev[4])
+    x1 = ext.backward_x(*dev)
+    for _ in range(3):
+        assert torch.equal(w1, ext.backward_w(dev[0], dev[1], dev[2], dev[4]))
+        assert torch.equal(x1, ext.backward_x(*dev))
+
+
+def test_one_hot_binary_forward_is_exact(ext):
+    rng = np.random.default_rng(4)
+    x = torch.as_tensor((rng.random((40, 300)) < 0.5).astype(np.float32))
+    (a, b, op), = random_layers(rng, 40, [160])
+    w = torch.nn.functional.one_hot(torch.as_tensor(op).long(), 16).float()
+    got = ext.forward(x.cuda(), torch.as_tensor(a).cuda(), torch.as_tensor(b).cuda(), w.cuda())
+    want = fo.ext_forward(x, torch.as_tensor(a), torch.as_tensor(b), w)
+    assert torch.equal(got.cpu(), want)
+
+
+def test_input_checks(ext):
+    x, a, b, w, gy = _case(0, 8, 10, 16)
+    with pytest.raises(RuntimeError):
+        ext.forward(x, a, b, w)                                     # CPU tensors
+    with pytest.raises(RuntimeError):
+        ext.forward(x.cuda().t().contiguous().t(), a.cuda(), b.cuda(), w.cuda())   # not contiguous
+    with pytest.raises(RuntimeError):
+        ext.forward(x.cuda().int(), a.cuda(), b.cuda(), w.cuda())   # dtype
+    with pytest.raises(RuntimeError):
+        ext.forward(x.cuda(), a.cuda()[:5], b.cuda(), w.cuda())     # table length
+
+
+@pytest.mark.parametrize("conn,grad_factor,batch", [("random", 1.0, 128), ("unique", 1.0, 100), ("random", 2.0, 36)])
+def test_train_step_matches_python_implementation(conn, grad_factor, batch):
+    """Flatten -> 4 x LogicLayer -> GroupSum -> CrossEntropy: loss and every gradient against
+    the CPU python implementation with the same wiring and logits."""
+    import difflogic_amd as dl
+    torch.manual_seed(0)
+    F, widths, k, tau = 60, [400, 400, 400, 300], 10, 10.0
+    mods, d = [torch.nn.Flatten()], F
+    for wd in widths:
+        mods.append(dl.LogicLayer(d, wd, grad_factor=grad_factor, connections=conn))
+        d = wd
+    model = torch.nn.Sequential(*mods, dl.GroupSum(k, tau)).train()
+    layers = [m for m in model if isinstance(m, dl.LogicLayer)]
+    x = (torch.rand(batch, F) < 0.2).float()
+    labels = torch.randint(0, k, (batch,))
+
+    logits = [l.weights.detach().cpu().clone().requires_grad_(True) for l in layers]
+    oracle = fo.PythonNet([(l.indices[0].cpu(), l.indices[1].cpu(), lg) for l, lg in zip(layers, logits)], k, tau,
+                          grad_factor)
+    xo = x.clone().requires_grad_(True)
+    want_out = oracle(xo, training=True)
+    want_loss = torch.nn.functional.cross_entropy(want_out, labels)
+    want_loss.backward()
+
+    xg = x.cuda().requires_grad_(True)
+    got_out = model(xg)
+    got_loss = torch.nn.functional.cross_entropy(got_out, labels.cuda())
+    got_loss.backward()
+
+    assert close(got_out, want_out)[0]
+    assert abs(got_loss.item() - want_loss.item()) <= RTOL * abs(want_loss.item())
+    for l, lg in zip(layers, logits):
+        ok, err = close(l.weights.grad, lg.grad, 2e-5)
+        assert ok, err
+    ok, err = close(xg.grad, xo.grad, 2e-5)
+    assert ok, err
+
+
+def test_eval_mode_and_state_dict_round_trip():
+    import difflogic_amd as dl
+    torch.manual_seed(1)
+    m1 = torch.nn.Sequential(torch.nn.Flatten(), dl.LogicLayer(30, 64), dl.LogicLayer(64, 40), dl.GroupSum(4, 2.0))
+    assert list(m1.state_dict().keys()) == ["1.weights", "2.weights"]
+    torch.manual_seed(2)
+    m2 = torch.nn.Sequential(torch.nn.Flatten(), dl.LogicLayer(30, 64), dl.LogicLayer(64, 40), dl.GroupSum(4, 2.0))
+    m2.load_state_dict(m1.state_dict())
+    for l1, l2 in ((m1[1], m2[1]), (m1[2], m2[2])):
+        l2.set_connections(*l1.indices)
+    x = (torch.rand(17, 30) < 0.5).float().cuda()
+    m1.eval(), m2.eval()
+    with torch.no_grad():
+        y1, y2 = m1(x), m2(x)
+    assert torch.equal(y1, y2)
+    layers = [(l.indices[0].cpu(), l.indices[1].cpu(), l.weights.detach().cpu()) for l in (m1[1], m1[2])]
+    want = fo.PythonNet(layers, 4, 2.0)(x.cpu(), training=False)
+    assert torch.equal(y1.cpu(), want)
