@@ -1,0 +1,317 @@
+#!/usr/bin/env python3
+"""Benchmark of the LogicLayer kernel path on one MI355X.
+
+Headline workload (the one BASELINE.json's metric is quoted on): bit-packed inference of the
+discretised net 784 -> 6 x 64000 -> GroupSum(k=10) on 2^20 synthetic samples.  One step is
+one pass of the whole path over the batch, starting from a bool [B, 784] tensor resident in
+HBM: PackBitsTensor (transpose + pack, 64-bit words) -> six LogicLayer.eval launches ->
+GroupSum bit counts [B, 10] int32.
+
+Prints ONE JSON line.  `roofline` describes the dominant kernel (the per-layer gate
+evaluation): algorithmic bytes per launch = 8*W*(in+out) + 17*out, divided by the launch
+duration measured with events on the launch stream inside the timed region.  `cpu_baseline`
+times the CPU oracle (single thread, like the reference's generated C) on a bounded sample.
+`extra.train` reports the fp32 forward+backward path (784 -> 6 x 64000, B = 512).
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch-log2", type=int, default=20)
+    ap.add_argument("--width", type=int, default=64000)
+    ap.add_argument("--layers", type=int, default=6)
+    ap.add_argument("--features", type=int, default=784)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-train", action="store_true")
+    ap.add_argument("--cpu-sample-log2", type=int, default=17)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run 4 plain device copies of 1 GiB (for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE)")
+    return ap.parse_args()
+
+
+def eval_layer_bytes(in_dim, out_dim, words):
+    return 8 * words * (in_dim + out_dim) + 17 * out_dim
+
+
+def packed_bench(args, torch, dl):
+    F, width, L, k = args.features, args.width, args.layers, 10
+    B = 1 << args.batch_log2
+    W = B // 64
+    torch.manual_seed(0)
+    mods, d = [torch.nn.Flatten()], F
+    for _ in range(L):
+        mods.append(dl.LogicLayer(d, width, connections="random"))
+        d = width
+    model = torch.nn.Sequential(*mods, dl.GroupSum(k, 30.0)).eval()
+    g = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.rand(B, F, device="cuda", generator=g) < 0.2
+
+    ext = dl.difflogic_cuda
+    real_eval = ext.eval
+    launches = []          # (in_dim, out_dim, start_event, end_event)
+    record = {"on": False}
+
+    def timed_eval(xw, a, b, w):
+        if not record["on"]:
+            return real_eval(xw, a, b, w)
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        y = real_eval(xw, a, b, w)
+        e.record()
+        launches.append((xw.shape[0], w.shape[0], s, e))
+        return y
+
+    ext.eval = timed_eval
+
+    def step():
+        with torch.no_grad():
+            return model(dl.PackBitsTensor(x, bit_count=64))
+
+    try:
+        for _ in range(args.warmup):
+            out = step()
+        torch.cuda.synchronize()
+        record["on"] = True
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            out = step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    finally:
+        ext.eval = real_eval
+        record["on"] = False
+
+    ms_per_step = elapsed / args.steps * 1e3
+    # dominant kernel: the square (width -> width) gate-evaluation launches
+    sq = [(i, o, s.elapsed_time(e)) for i, o, s, e in launches if i == o]
+    if not sq:
+        sq = [(i, o, s.elapsed_time(e)) for i, o, s, e in launches]
+    alg = sum(eval_layer_bytes(i, o, W) for i, o, _ in sq) / len(sq)
+    avg_ms = sum(t for _, _, t in sq) / len(sq)
+    achieved = alg / (avg_ms * 1e-3) / 1e9
+    first = [s.elapsed_time(e) for i, o, s, e in launches if i != o]
+    total_alg = sum(eval_layer_bytes(i, o, W) for i, o, *_ in launches) / args.steps + 8 * W * width + 4 * k * B
+    roofline = {
+        "bound": "hbm", "kernel": "eval_kernel<u32x4> %d->%d" % (sq[0][0], sq[0][1]),
+        "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+        "traffic": load_traffic(), "algorithmic_bytes_per_launch": int(alg), "avg_launch_ms": round(avg_ms, 4),
+        "launches_timed": len(sq),
+    }
+    info = {
+        "first_layer_avg_ms": round(sum(first) / len(first), 4) if first else None,
+        "path_algorithmic_GB_per_step": round(total_alg / 1e9, 2),
+        "path_GBps_algorithmic": round(total_alg / (ms_per_step * 1e-3) / 1e9, 1),
+        "checksum": int(out.sum().item()),
+    }
+    return B * args.steps / elapsed, ms_per_step, roofline, info, model, x
+
+
+def load_traffic():
+    """HBM bytes per launch of the dominant kernel from the committed rocprofv3 --pmc summary
+    (profiles/eval_kernel_traffic.json), or None when it has not been measured."""
+    p = os.path.join(ROOT, "profiles", "eval_kernel_traffic.json")
+    if os.path.exists(p):
+        with open(p) as f:
+            return json.load(f).get("hbm_bytes_per_launch")
+    return None
+
+
+def cpu_baseline(args, model, x, dl):
+    """The oracle's table-driven C interpreter (same per-word arithmetic as the C the reference
+    generates), one thread, on the first 2^cpu_sample_log2 samples of the batch."""
+    import numpy as np
+
+    from oracle import interp
+    layers = [(m.indices[0].cpu().numpy(), m.indices[1].cpu().numpy(),
+               m.weights.argmax(-1).to("cpu").numpy().astype(np.uint8)) for m in model if isinstance(m, dl.LogicLayer)]
+    n = min(1 << args.cpu_sample_log2, x.shape[0])
+    xs = x[:n].cpu().numpy()
+    interp.net_eval(xs[:64], layers, 10)            # load the library, touch the tables
+    t0 = time.perf_counter()
+    want = interp.net_eval(xs, layers, 10, threads=1)
+    dt = time.perf_counter() - t0
+    with __import__("torch").no_grad():
+        got = model(dl.PackBitsTensor(x[:n], bit_count=64)).cpu().numpy()
+    return {"value": round(n / dt, 1), "unit": "samples/s", "cores": 1, "kind": "port",
+            "sample": "first %d of %d samples, same net; oracle/c/packed_interp.c, 1 thread, %.1f s" % (n, x.shape[0], dt),
+            "gpu_matches_cpu_on_sample": bool((got == want).all())}
+
+
+def train_bench(args, torch, dl):
+    """fp32 forward + backward of 784 -> 6 x 64000 -> GroupSum(10, tau 30), B = 512, 'unique'
+    connections, grad_factor 1: per-kernel event timings against the algorithmic bytes
+    fwd 4B(in+out)+80 out, backward_w 4B(in+out)+64 out, backward_x 4B(2 in+out)+64 out."""
+    F, width, L, k, B = 784, 64000, 6, 10, 512
+    torch.manual_seed(0)
+    mods, d = [torch.nn.Flatten()], F
+    for _ in range(L):
+        mods.append(dl.LogicLayer(d, width, connections="unique"))
+        d = width
+    model = torch.nn.Sequential(*mods, dl.GroupSum(k, 30.0)).train()
+    g = torch.Generator(device="cuda").manual_seed(2)
+    x = (torch.rand(B, F, device="cuda", generator=g) < 0.2).float()
+    labels = torch.randint(0, k, (B,), device="cuda", generator=g)
+    loss_fn = torch.nn.CrossEntropyLoss()
+
+    ext = dl.difflogic_cuda
+    real = {n: getattr(ext, n) for n in ("forward", "backward_w", "backward_x")}
+    rec = {n: [] for n in real}
+    on = {"v": False}
+
+    def wrap(name):
+        def f(*a, **kw):
+            if not on["v"]:
+                return real[name](*a, **kw)
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            r = real[name](*a, **kw)
+            e.record()
+            rec[name].append((a[0].shape[0], r.shape[0] if name != "backward_x" else a[4].shape[0], s, e))
+            return r
+        return f
+
+    for n in real:
+        setattr(ext, n, wrap(n))
+
+    def step():
+        model.zero_grad(set_to_none=True)
+        loss = loss_fn(model(x), labels)
+        loss.backward()
+        return loss
+
+    steps, warmup = max(5, args.steps), max(3, args.warmup)
+    try:
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        on["v"] = True
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            loss = step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    finally:
+        for n in real:
+            setattr(ext, n, real[n])
+
+    def alg(name, i, o):
+        if name == "forward":
+            return 4 * B * (i + o) + 80 * o
+        if name == "backward_w":
+            return 4 * B * (i + o) + 64 * o
+        return 4 * B * (2 * i + o) + 64 * o
+
+    kernels = {}
+    tot_bytes = tot_ms = 0.0
+    for name, items in rec.items():
+        by = sum(alg(name, i, o) for i, o, _, _ in items)
+        ms = sum(s.elapsed_time(e) for _, _, s, e in items)
+        tot_bytes += by
+        tot_ms += ms
+        kernels[name] = {"GBps": round(by / (ms * 1e-3) / 1e9, 1), "frac_hbm": round(by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                         "ms_per_step": round(ms / steps, 4)}
+    neuron_samples = L * width * B
+    return {
+        "workload": "fp32 fwd+bwd 784->6x64000->GroupSum(10,tau=30), B=512, connections=unique, CrossEntropy",
+        "neuron_samples_per_s": round(neuron_samples * steps / elapsed, 1),
+        "neuron_samples_per_s_kernels_only": round(neuron_samples * steps / (tot_ms * 1e-3), 1),
+        "ms_per_step": round(elapsed / steps * 1e3, 4),
+        "kernel_GBps_algorithmic": round(tot_bytes / (tot_ms * 1e-3) / 1e9, 1),
+        "kernel_frac_hbm": round(tot_bytes / (tot_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "kernels": kernels, "loss": round(loss.item(), 6), "dtype": "f32",
+    }
+
+
+def train_cpu_baseline(torch):
+    """Full training step (forward, CrossEntropy, backward, Adam lr 0.01) of the python
+    implementation restated in oracle/float_oracle.py: 784 -> 4 x 8000 -> GroupSum(10, tau 10),
+    B = 128, 'random' connections; median of 5 steps after 2 warm-ups, 1 thread."""
+    from oracle import connections as oc
+    from oracle import float_oracle as fo
+    threads = torch.get_num_threads()
+    torch.set_num_threads(1)
+    try:
+        torch.manual_seed(0)
+        layers, d = [], 784
+        for _ in range(4):
+            lg = torch.randn(8000, 16, requires_grad=True)
+            a, b = oc.random_connections(d, 8000)
+            layers.append((a, b, lg))
+            d = 8000
+        net = fo.PythonNet(layers, 10, 10.0)
+        opt = torch.optim.Adam([l[2] for l in layers], lr=0.01)
+        x = (torch.rand(128, 784) < 0.2).float()
+        y = torch.randint(0, 10, (128,))
+        times = []
+        for i in range(7):
+            t0 = time.perf_counter()
+            loss = torch.nn.functional.cross_entropy(net(x), y)
+            opt.zero_grad()
+            loss.backward()
+            opt.step()
+            times.append(time.perf_counter() - t0)
+        med = statistics.median(times[2:])
+    finally:
+        torch.set_num_threads(threads)
+    return {"value": round(4 * 8000 * 128 / med, 1), "unit": "neuron-samples/s", "cores": 1, "kind": "port",
+            "sample": "784->4x8000 B=128 full step (fwd+CE+bwd+Adam), median of 5, %.3f s/step" % med}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (the path shards along the batch without "
+              "communication; see DESIGN.md); --gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    import difflogic_amd as dl
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    value, ms, roofline, info, model, x = packed_bench(args, torch, dl)
+    result = {
+        "metric": "packed-eval samples/s (784->6x64k)", "value": round(value, 1), "unit": "samples/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int64", "data": "synthetic",
+        "config": {"workload": "packed inference %d->%dx%d->GroupSum(10), batch 2^%d, int64 words, bool input "
+                               "resident in HBM; step = pack + %d eval layers + groupbitsum"
+                               % (args.features, args.layers, args.width, args.batch_log2, args.layers),
+                   "connections": "random", "seed": 0},
+        "roofline": roofline,
+    }
+    result["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(args, model, x, dl)
+    extra = dict(info)
+    del model, x
+    torch.cuda.empty_cache()
+    if not args.no_train:
+        extra["train"] = train_bench(args, torch, dl)
+        if not args.no_cpu_baseline:
+            extra["train"]["cpu_baseline"] = train_cpu_baseline(torch)
+    result["extra"] = extra
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

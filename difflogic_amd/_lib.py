@@ -27,6 +27,7 @@ SIGNATURES = {
     "dl_logic_backward_x": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _dbl, _int, _vp],
     "dl_logic_eval": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "dl_tensor_packbits": [_vp, _vp, _i64, _i64, _int, ctypes.POINTER(_i64), _vp],
+    "dl_tensor_packbits_batch_major": [_vp, _vp, _i64, _i64, _int, ctypes.POINTER(_i64), _vp],
     "dl_groupbitsum": [_vp, _vp, _i64, _i64, _int, _i64, _i64, _vp],
 }
 _RESTYPES = {"dl_status_string": ctypes.c_char_p}
@@ -42,7 +43,7 @@ def load():
     if not os.path.exists(LIB_PATH):
         raise ImportError(
             f"{LIB_PATH} is missing: the HIP kernel library has not been built. "
-            "Run `python -m difflogic_amd.build` (needs hipcc); there is no fallback implementation.")
+            "Run `python difflogic_amd/build.py` (needs hipcc); there is no fallback implementation.")
     lib = ctypes.CDLL(LIB_PATH)
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)          # AttributeError if the symbol is not exported

@@ -1,6 +1,6 @@
 """Builds libdifflogic_hip.so (the C-ABI kernel library) in-tree with hipcc for gfx950.
 
-    python -m difflogic_amd.build
+    python difflogic_amd/build.py
 """
 import os
 import shutil

@@ -155,6 +155,86 @@ __global__ __launch_bounds__(DL_BLOCK) void packbits_generic_kernel(const uint8_
     }
 }
 
+// Batch-major input: bool [batch, features] -> packed [features, row bytes] in one pass, i.e.
+// the transpose and the packing fused.  A workgroup owns 64*BPL features x 16 word columns
+// (1024 samples).  Each wave reads sample rows with lanes along the features (BPL bool bytes
+// per lane, coalesced), folds 8 samples into one register whose byte k carries feature k's 8
+// bits, assembles 64-sample words per feature, and parks them in LDS; the workgroup then writes
+// 128 contiguous bytes per feature row.
+template <int BPL> struct BoolLoad;
+template <> struct BoolLoad<4> {
+    static __device__ __forceinline__ uint32_t flags(const uint8_t *p) {
+        const uint32_t v = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(p));
+        return ((((v & 0x7f7f7f7fu) + 0x7f7f7f7fu) | v) >> 7) & 0x01010101u;   // 1 per non-zero byte
+    }
+};
+template <> struct BoolLoad<1> {
+    static __device__ __forceinline__ uint32_t flags(const uint8_t *p) { return (uint32_t) (*p != 0); }
+};
+
+template <int BPL>
+__global__ __launch_bounds__(DL_BLOCK) void packbits_batch_major_kernel(const uint8_t *__restrict__ x,
+                                                                        uint8_t *__restrict__ out, int64_t batch,
+                                                                        int64_t features, int64_t out_row_bytes) {
+    constexpr int FW = DL_WAVE * BPL;   // features per workgroup
+    constexpr int WC = 16;              // 64-sample word columns per workgroup
+    __shared__ uint64_t tile[FW][WC + 1];
+
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t f0 = (int64_t) blockIdx.y * FW;
+    const int64_t w0 = (int64_t) blockIdx.x * WC;
+    const int64_t fl = f0 + (int64_t) lane * BPL;
+    const bool feat_live = fl < features;           // features % BPL == 0
+
+#pragma unroll 1
+    for (int q = 0; q < WC / 4; ++q) {
+        const int wc = wave * (WC / 4) + q;
+        const int64_t s0 = (w0 + wc) * 64;
+        uint32_t oct[8];                            // oct[j]: byte k = feature k, samples 8j .. 8j+7
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            uint32_t acc = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int64_t s = s0 + 8 * j + i;
+                uint32_t n = 0;
+                if (feat_live && s < batch) n = BoolLoad<BPL>::flags(x + s * features + fl);
+                acc |= n << i;
+            }
+            oct[j] = acc;
+        }
+#pragma unroll
+        for (int k = 0; k < BPL; ++k) {
+            uint32_t lo = 0, hi = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                lo |= ((oct[j] >> (8 * k)) & 0xffu) << (8 * j);
+                hi |= ((oct[4 + j] >> (8 * k)) & 0xffu) << (8 * j);
+            }
+            tile[lane * BPL + k][wc] = ((uint64_t) hi << 32) | lo;
+        }
+    }
+    __syncthreads();
+
+    // 16 consecutive threads write the 16 words (128 bytes) of one feature row.
+    const int wi = (int) (threadIdx.x & 15u);
+    const int64_t byte0 = (w0 + wi) * 8;
+    const bool whole_words = (out_row_bytes & 7) == 0;
+    for (int r = (int) (threadIdx.x >> 4); r < FW; r += DL_BLOCK / 16) {
+        const int64_t f = f0 + r;
+        if (f >= features || byte0 >= out_row_bytes) continue;
+        const uint64_t v = tile[r][wi];
+        uint8_t *dst = out + f * out_row_bytes + byte0;
+        if (whole_words) {
+            *reinterpret_cast<uint64_t *>(dst) = v;
+        } else {
+            const int nb = (int) ((out_row_bytes - byte0 < 8) ? (out_row_bytes - byte0) : 8);
+            for (int t = 0; t < nb; ++t) dst[t] = (uint8_t) (v >> (8 * t));
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 // Vertical bit count (GroupSum on packed words).  For each class (a contiguous block of
 // per_class neuron rows) and each sample bit, the number of rows with that bit set.
@@ -324,6 +404,33 @@ extern "C" int dl_tensor_packbits(const uint8_t *t, void *out, int64_t features,
         if (gx > 65535) gx = 65535;
         hipLaunchKernelGGL(packbits_generic_kernel, dim3((unsigned) gx, gy), dim3(DL_BLOCK), 0, s, t,
                            (uint8_t *) out, features, batch, out_row_bytes);
+    }
+    return dl_launch_status();
+}
+
+extern "C" int dl_tensor_packbits_batch_major(const uint8_t *x, void *out, int64_t batch, int64_t features,
+                                              int bit_count, int64_t *pad_len, void *stream) {
+    if (!valid_bit_count(bit_count)) return DL_ERR_BIT_COUNT;
+    if (features < 0 || batch < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (pad_len) *pad_len = (bit_count - batch % bit_count) % bit_count;
+    if (features == 0 || batch == 0) return DL_OK;
+    if (!x || !out) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    const int64_t words = dl_ceil_div(batch, bit_count);
+    const int64_t out_row_bytes = words * (bit_count / 8);
+    if (out_row_bytes % 8 == 0 && !dl_aligned(out, 8)) return DL_ERR_INVALID_ARGUMENT;
+    const int64_t gx = dl_ceil_div(dl_ceil_div(batch, 64), 16);
+    if (gx > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    if (features % 4 == 0 && dl_aligned(x, 4)) {
+        const int64_t gy = dl_ceil_div(features, 256);
+        if (gy > 65535) return DL_ERR_TOO_LARGE;
+        hipLaunchKernelGGL(packbits_batch_major_kernel<4>, dim3((unsigned) gx, (unsigned) gy), dim3(DL_BLOCK), 0, s, x,
+                           (uint8_t *) out, batch, features, out_row_bytes);
+    } else {
+        const int64_t gy = dl_ceil_div(features, 64);
+        if (gy > 65535) return DL_ERR_TOO_LARGE;
+        hipLaunchKernelGGL(packbits_batch_major_kernel<1>, dim3((unsigned) gx, (unsigned) gy), dim3(DL_BLOCK), 0, s, x,
+                           (uint8_t *) out, batch, features, out_row_bytes);
     }
     return dl_launch_status();
 }

@@ -181,6 +181,27 @@ def tensor_packbits_cuda(t, bit_count):
     return out, int(pad.value)
 
 
+def tensor_packbits_batch_major(x, bit_count):
+    """bool [B,F] (sample-major, as the user holds it) -> (int{bit_count} [F, ceil(B/bit_count)],
+    pad_len): the transpose and tensor_packbits_cuda of difflogic/packbitstensor.py:15-16 in
+    one kernel.  Not part of the reference's extension; PackBitsTensor uses it."""
+    _check_input(x, "x")
+    if bit_count not in _BITS_TO_DTYPE:
+        raise ValueError("`bit_count` has to be in { 8, 16, 32, 64 }")
+    if x.dtype != torch.bool or x.dim() != 2:
+        raise RuntimeError(f"expected x to be a 2-D bool tensor, got {x.dtype} with {x.dim()} dims")
+    batch, features = x.shape
+    words = -(-batch // bit_count)
+    out = torch.empty((features, words), dtype=_BITS_TO_DTYPE[bit_count], device=x.device)
+    pad = ctypes.c_int64(0)
+    with torch.cuda.device(x.device):
+        st = _lib.load().dl_tensor_packbits_batch_major(_p(x), _p(out), batch, features, bit_count, ctypes.byref(pad),
+                                                        _stream(x.device))
+    if st:
+        _raise(st, "tensor_packbits_batch_major")
+    return out, int(pad.value)
+
+
 def groupbitsum(b, pad_len, k):
     """int words [out,W] -> int32 [W*bits - pad_len, k]   (difflogic.cpp:75-83)."""
     _check_input(b, "b")

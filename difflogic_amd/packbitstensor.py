@@ -15,8 +15,12 @@ class PackBitsTensor:
         self.bit_count = bit_count
         self.device = device
         if device == "cuda":
-            t = t.to(device).T.contiguous()
-            self.t, self.pad_len = difflogic_cuda.tensor_packbits_cuda(t, self.bit_count)
+            t = t.to(device)
+            if t.dtype == torch.bool and t.is_contiguous():
+                # transpose + pack in one kernel
+                self.t, self.pad_len = difflogic_cuda.tensor_packbits_batch_major(t, self.bit_count)
+            else:
+                self.t, self.pad_len = difflogic_cuda.tensor_packbits_cuda(t.T.contiguous(), self.bit_count)
         else:
             raise NotImplementedError(device)
 

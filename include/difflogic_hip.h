@@ -90,6 +90,13 @@ int dl_logic_eval(const void *x, const int64_t *a, const int64_t *b, const uint8
 int dl_tensor_packbits(const uint8_t *t, void *out, int64_t features, int64_t batch, int bit_count,
                        int64_t *pad_len, void *stream);
 
+/* Fuses the two steps of the reference's PackBitsTensor constructor
+ * (difflogic/packbitstensor.py:15-16: `t.T.contiguous()` followed by tensor_packbits_cuda):
+ *   x [batch, features] bool bytes, SAMPLE-major -> out [features, ceil(batch/bit_count)] words,
+ *   same bit order and padding as dl_tensor_packbits. */
+int dl_tensor_packbits_batch_major(const uint8_t *x, void *out, int64_t batch, int64_t features,
+                                   int bit_count, int64_t *pad_len, void *stream);
+
 /* Replaces `groupbitsum` (difflogic.cpp:75-83, difflogic_kernel.cu:666-700), including the
  * final transpose.
  *   b [in_dim, words] words -> out [words*bit_count - pad_len, k] int32 (sample-major):

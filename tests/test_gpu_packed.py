@@ -45,6 +45,28 @@ def test_packbits_nonzero_bytes_count_as_true(ext):
 
 
 @pytest.mark.parametrize("bits", [8, 16, 32, 64])
+@pytest.mark.parametrize("B,F", [(1, 1), (7, 3), (64, 8), (65, 12), (1000, 7), (1024, 256), (4112, 260), (70000, 2),
+                                 (3000, 784), (130, 1028)])
+def test_packbits_batch_major(ext, bits, B, F):
+    rng = np.random.default_rng(F * 131 + B + bits)
+    x = rng.random((B, F)) < 0.3
+    want, pad = po.packbits(x.T, bits)
+    got, got_pad = ext.tensor_packbits_batch_major(_dev(x), bits)
+    assert got_pad == pad and got.dtype == torch.as_tensor(want).dtype and tuple(got.shape) == want.shape
+    assert np.array_equal(got.cpu().numpy(), want)
+    # and it agrees with the two-step path of the reference
+    two, _ = ext.tensor_packbits_cuda(_dev(x).T.contiguous(), bits)
+    assert torch.equal(got, two)
+
+
+def test_packbits_batch_major_nonzero_bytes(ext):
+    raw = torch.tensor([[0, 1, 2, 128], [255, 0, 7, 0], [3, 3, 0, 0]], dtype=torch.uint8).cuda()
+    got, _ = ext.tensor_packbits_batch_major(raw.view(torch.bool), 8)
+    want, _ = po.packbits((raw.cpu().numpy() != 0).T, 8)
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("bits", [8, 16, 32, 64])
 @pytest.mark.parametrize("W", [1, 2, 3, 5, 64, 127, 128, 129, 300])
 def test_eval_layer_random(ext, bits, W):
     rng = np.random.default_rng(W * 7 + bits)

@@ -1,0 +1,109 @@
+"""Host logic of the Python API on CPU: constructor semantics, wiring initialisers against the
+reference's fixtures, the reverse index, the eager implementation, state_dict format."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import difflogic_amd as dl
+from difflogic_amd import functional as F
+from oracle import connections as oc
+from oracle import float_oracle as fo
+
+
+def test_constructor_defaults_and_rng_order():
+    torch.manual_seed(0)
+    layer = dl.LogicLayer(20, 16, device="cpu")
+    assert layer.implementation == "python" and layer.connections == "random"
+    assert layer.num_neurons == 16 and layer.num_weights == 16 and layer.grad_factor == 1.0
+    assert layer.weights.shape == (16, 16) and list(layer.state_dict()) == ["weights"]
+    assert repr(layer) == "LogicLayer(20, 16, train)"
+    torch.manual_seed(0)
+    w = torch.randn(16, 16)                                  # logits first, then the wiring
+    a, b = oc.random_connections(20, 16)
+    assert torch.equal(layer.weights.detach(), w)
+    assert torch.equal(layer.indices[0], a) and torch.equal(layer.indices[1], b)
+    with pytest.raises(AssertionError):
+        dl.LogicLayer(100, 10, device="cpu")                 # fewer than in/2 neurons
+    with pytest.raises(AssertionError):
+        dl.LogicLayer(10, 10, device="cpu", connections="dense")
+    with pytest.raises(AssertionError):
+        dl.LogicLayer(10, 10, device="cpu", implementation="fast")
+    assert repr(dl.GroupSum(10, 30.0)) == "GroupSum(k=10, tau=30.0)"
+
+
+def test_wiring_matches_reference_fixtures(golden_dir):
+    conn = np.load(os.path.join(golden_dir, "connections.npz"))
+    for key in (str(c) for c in conn["cases"]):
+        kind, in_dim, out_dim, seed = key.split("_")
+        in_dim, out_dim, seed = int(in_dim), int(out_dim), int(seed)
+        torch.manual_seed(seed)
+        if kind == "unique":
+            a, b = F.get_unique_connections(in_dim, out_dim, "cpu")
+        else:
+            layer = dl.LogicLayer(in_dim, out_dim, device="cpu", connections="random")
+            a, b = layer.indices
+        assert np.array_equal(a.numpy(), conn[key + "_a"]) and np.array_equal(b.numpy(), conn[key + "_b"]), key
+
+
+def test_reverse_index_matches_loop_definition():
+    g = torch.Generator().manual_seed(0)
+    a = torch.randint(0, 13, (200,), generator=g)
+    b = torch.randint(0, 13, (200,), generator=g)
+    b[5] = a[5]
+    start, idx = F.build_reverse_index(a, b, 13)
+    s2, i2 = oc.reverse_index(a.numpy(), b.numpy(), 13)
+    assert np.array_equal(start.numpy(), s2) and np.array_equal(idx.numpy(), i2)
+    layer = dl.LogicLayer(13, 200, device="cpu", implementation="python")
+    layer.set_connections(a, b)
+    assert torch.equal(layer.indices[0], a)
+    with pytest.raises(ValueError):
+        layer.set_connections(a, b + 100)
+    with pytest.raises(ValueError):
+        layer.set_connections(a[:5], b[:5])
+
+
+def test_eager_implementation_matches_oracle_and_autograd():
+    torch.manual_seed(3)
+    layer = dl.LogicLayer(12, 30, device="cpu", grad_factor=1.5).double()
+    x = torch.rand(9, 12, dtype=torch.float64, requires_grad=True)
+    y = layer(x)
+    w = torch.softmax(layer.weights, -1)
+    want = fo.layer_forward_sequential(x, layer.indices[0], layer.indices[1], w)
+    assert torch.allclose(y, want, atol=1e-14)
+    gy = torch.randn_like(y)
+    gx, = torch.autograd.grad(y, x, gy, retain_graph=True)
+    gx_want, = torch.autograd.grad(want, x, gy)
+    assert torch.allclose(gx, 1.5 * gx_want, atol=1e-13)
+    layer.eval()
+    xb = (torch.rand(9, 12) < 0.5).double()
+    hard = layer(xb)
+    assert set(hard.unique().tolist()) <= {0.0, 1.0}
+    for i in range(16):
+        a, b = torch.rand(4, dtype=torch.float64), torch.rand(4, dtype=torch.float64)
+        from oracle.gates import real_gate
+        assert torch.allclose(F.bin_op(a, b, i), real_gate(a, b, i), atol=1e-15)
+
+
+def test_group_sum_and_grad_factor():
+    gs = dl.GroupSum(3, 2.0, device="cpu")
+    x = torch.arange(12.).reshape(1, 12)
+    assert torch.equal(gs(x), torch.tensor([[6., 22., 38.]]) / 2)
+    with pytest.raises(AssertionError):
+        gs(torch.zeros(1, 10))
+    t = torch.ones(3, requires_grad=True)
+    F.GradFactor.apply(t, 4.0).sum().backward()
+    assert torch.equal(t.grad, torch.full((3,), 4.0))
+
+
+def test_packbits_tensor_is_gpu_only():
+    with pytest.raises(NotImplementedError):
+        dl.PackBitsTensor(torch.zeros(4, 3, dtype=torch.bool), device="cpu")
+    layer = dl.LogicLayer(3, 4, device="cpu").eval()
+
+    class Fake(dl.PackBitsTensor):
+        def __init__(self):
+            pass
+    with pytest.raises(AssertionError):
+        layer(Fake())                                        # packed inference needs device='cuda'
