@@ -29,6 +29,7 @@ SIGNATURES = {
     "dl_tensor_packbits": [_vp, _vp, _i64, _i64, _int, ctypes.POINTER(_i64), _vp],
     "dl_tensor_packbits_batch_major": [_vp, _vp, _i64, _i64, _int, ctypes.POINTER(_i64), _vp],
     "dl_groupbitsum": [_vp, _vp, _i64, _i64, _int, _i64, _i64, _vp],
+    "dl_logic_eval_groupbitsum": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _i64, _i64, _vp],
 }
 _RESTYPES = {"dl_status_string": ctypes.c_char_p}
 

@@ -253,8 +253,15 @@ __device__ __forceinline__ void csa(uint64_t &carry, uint64_t &sum, uint64_t a, 
     sum = u ^ c;
 }
 
-template <int NPH>
+//
+// FUSED: the counted rows are not read but computed on the fly as the gate layer
+// y[n] = gate_{op[n]}(x[a[n]], x[b[n]]) over the rows of `bits` (= the layer's input), so the
+// last layer's output never exists in memory.
+template <int NPH, bool FUSED>
 __global__ __launch_bounds__(DL_BLOCK) void groupbitsum_kernel(const uint64_t *__restrict__ bits,
+                                                               const int64_t *__restrict__ ga,
+                                                               const int64_t *__restrict__ gb,
+                                                               const uint8_t *__restrict__ gop,
                                                                int32_t *__restrict__ out, int64_t words,
                                                                int64_t per_class, int64_t k, int64_t batch) {
     constexpr int NP = NPH + 4;
@@ -280,13 +287,36 @@ __global__ __launch_bounds__(DL_BLOCK) void groupbitsum_kernel(const uint64_t *_
     for (int p = 0; p < NPH; ++p) high[p] = 0;
 
     const uint64_t *row = bits + (cls * per_class + r_begin) * words + (live ? col : 0);
+    const uint64_t *xcol = bits + (live ? col : 0);
     for (int64_t r = r_begin; r < r_end; r += 16) {
         uint64_t v[16];
+        if (!FUSED) {
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            v[j] = (live && r + j < r_end) ? __builtin_nontemporal_load(row + (int64_t) j * words) : 0;
+            for (int j = 0; j < 16; ++j) {
+                v[j] = (live && r + j < r_end) ? __builtin_nontemporal_load(row + (int64_t) j * words) : 0;
+            }
+            row += 16 * words;
+        } else {
+            uint64_t va[16], vb[16];
+            uint32_t op[16];
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int64_t n = cls * per_class + ((r + j < r_end) ? r + j : r_end - 1);
+                const int64_t ia = ga[n], ib = gb[n];
+                op[j] = gop[n];
+                va[j] = live ? xcol[ia * words] : 0;
+                vb[j] = live ? xcol[ib * words] : 0;
+            }
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const GateMasks m = gate_masks(op[j]);
+                const uint64_t m00 = ((uint64_t) m.m00 << 32) | m.m00, m01 = ((uint64_t) m.m01 << 32) | m.m01;
+                const uint64_t m10 = ((uint64_t) m.m10 << 32) | m.m10, m11 = ((uint64_t) m.m11 << 32) | m.m11;
+                const uint64_t hi = (vb[j] & m11) | (~vb[j] & m10), lo = (vb[j] & m01) | (~vb[j] & m00);
+                const uint64_t y = (va[j] & hi) | (~va[j] & lo);
+                v[j] = (live && r + j < r_end) ? y : 0;
+            }
         }
-        row += 16 * words;
         uint64_t t2a, t2b, t4a, t4b, t8a, t8b, t16;
         csa(t2a, ones, ones, v[0], v[1]);
         csa(t2b, ones, ones, v[2], v[3]);
@@ -360,6 +390,22 @@ __global__ __launch_bounds__(DL_BLOCK) void groupbitsum_generic_kernel(const uin
             out[s * k + cls] = acc;
         }
     }
+}
+
+template <bool FUSED>
+void launch_groupbitsum(const uint64_t *bits, const int64_t *a, const int64_t *b, const uint8_t *op, int32_t *out,
+                        int64_t words64, int64_t per_class, int64_t k, int64_t batch, dim3 grid, hipStream_t s) {
+    const int64_t chunk = (per_class + 3) / 4;      // rows one wave counts
+    // NPH planes above weight 8 hold counts up to 16 * 2^NPH - 1.
+    if (chunk < (16LL << 8))
+        hipLaunchKernelGGL((groupbitsum_kernel<8, FUSED>), grid, dim3(DL_BLOCK), 0, s, bits, a, b, op, out, words64,
+                           per_class, k, batch);
+    else if (chunk < (16LL << 14))
+        hipLaunchKernelGGL((groupbitsum_kernel<14, FUSED>), grid, dim3(DL_BLOCK), 0, s, bits, a, b, op, out, words64,
+                           per_class, k, batch);
+    else
+        hipLaunchKernelGGL((groupbitsum_kernel<27, FUSED>), grid, dim3(DL_BLOCK), 0, s, bits, a, b, op, out, words64,
+                           per_class, k, batch);
 }
 
 bool valid_bit_count(int bit_count) { return bit_count == 8 || bit_count == 16 || bit_count == 32 || bit_count == 64; }
@@ -454,15 +500,8 @@ extern "C" int dl_groupbitsum(const void *b, int32_t *out, int64_t in_dim, int64
         const int64_t gx = dl_ceil_div(words64, DL_WAVE);
         if (gx > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
         const dim3 grid((unsigned) gx, (unsigned) k);
-        const int64_t chunk = (per_class + 3) / 4;      // rows one wave counts
-        const uint64_t *bw = (const uint64_t *) b;
-        // NPH planes above weight 8 hold counts up to 16 * 2^NPH - 1.
-        if (chunk < (16LL << 8))
-            hipLaunchKernelGGL(groupbitsum_kernel<8>, grid, dim3(DL_BLOCK), 0, s, bw, out, words64, per_class, k, batch);
-        else if (chunk < (16LL << 14))
-            hipLaunchKernelGGL(groupbitsum_kernel<14>, grid, dim3(DL_BLOCK), 0, s, bw, out, words64, per_class, k, batch);
-        else
-            hipLaunchKernelGGL(groupbitsum_kernel<27>, grid, dim3(DL_BLOCK), 0, s, bw, out, words64, per_class, k, batch);
+        launch_groupbitsum<false>((const uint64_t *) b, nullptr, nullptr, nullptr, out, words64, per_class, k, batch,
+                                  grid, s);
     } else {
         int64_t gx = dl_ceil_div(batch, DL_BLOCK);
         if (gx > 0x7fffffffLL) gx = 0x7fffffffLL;
@@ -470,5 +509,27 @@ extern "C" int dl_groupbitsum(const void *b, int32_t *out, int64_t in_dim, int64
         hipLaunchKernelGGL(groupbitsum_generic_kernel, dim3((unsigned) gx, gy), dim3(DL_BLOCK), 0, s,
                            (const uint8_t *) b, out, row_bytes, per_class, k, batch);
     }
+    return dl_launch_status();
+}
+
+extern "C" int dl_logic_eval_groupbitsum(const void *x, const int64_t *a, const int64_t *b, const uint8_t *w,
+                                         int32_t *out, int64_t in_dim, int64_t out_dim, int64_t words, int bit_count,
+                                         int64_t pad_len, int64_t k, void *stream) {
+    if (!valid_bit_count(bit_count)) return DL_ERR_BIT_COUNT;
+    if (in_dim < 0 || out_dim < 0 || words < 0 || k <= 0 || pad_len < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim % k != 0) return DL_ERR_NOT_DIVISIBLE;
+    const int64_t batch = words * bit_count - pad_len;
+    if (batch < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (batch == 0) return DL_OK;
+    if (!out) return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim > 0 && (!x || !a || !b || !w || in_dim == 0)) return DL_ERR_INVALID_ARGUMENT;
+    const int64_t per_class = out_dim / k;
+    const int64_t row_bytes = words * (bit_count / 8);
+    if (row_bytes % 8 != 0 || !dl_aligned(x, 8) || k > 65535 || per_class > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    const int64_t words64 = row_bytes / 8;
+    const int64_t gx = dl_ceil_div(words64, DL_WAVE);
+    if (gx > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    launch_groupbitsum<true>((const uint64_t *) x, a, b, w, out, words64, per_class, k, batch,
+                             dim3((unsigned) gx, (unsigned) k), (hipStream_t) stream);
     return dl_launch_status();
 }

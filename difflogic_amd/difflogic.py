@@ -103,14 +103,15 @@ class LogicLayer(torch.nn.Module):
             return LogicLayerCudaFunction.apply(x, a, b, w, *tail).transpose(0, 1)
 
     def forward_cuda_eval(self, x: PackBitsTensor):
-        """Packed inference.  Rebinds ``x.t`` and returns ``x`` (in place on the wrapper)."""
+        """Packed inference.  Updates ``x`` in place (as the reference rebinds ``x.t``) and
+        returns it.  The evaluation is deferred until ``x.t`` is read, the next layer is applied
+        or GroupSum consumes it; GroupSum then runs fused with this layer."""
         assert not self.training
         assert isinstance(x, PackBitsTensor)
         assert x.t.shape[0] == self.in_dim, (x.t.shape, self.in_dim)
         a, b = self.indices
         w = self.weights.argmax(-1).to(torch.uint8)
-        x.t = difflogic_cuda.eval(x.t, a, b, w)
-        return x
+        return x.defer_layer(a, b, w)
 
     def extra_repr(self):
         return "{}, {}, {}".format(self.in_dim, self.out_dim, "train" if self.training else "eval")

@@ -220,3 +220,35 @@ def groupbitsum(b, pad_len, k):
     if st:
         _raise(st, "groupbitsum")
     return out
+
+
+def eval_groupbitsum(x, a, b, w, pad_len, k):
+    """groupbitsum(eval(x, a, b, w), pad_len, k) without materialising the layer's output.
+    Not part of the reference's extension; the lazy PackBitsTensor uses it for the last layer.
+    Falls back to the two separate kernels where the fused one does not apply."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w")):
+        _check_input(t, n)
+    bits = _WORD_BITS.get(x.dtype)
+    if bits is None:
+        raise RuntimeError(f'"logic_layer_cuda_eval_kernel" not implemented for \'{x.dtype}\'')
+    if x.dim() != 2 or w.dim() != 1 or w.dtype != torch.uint8:
+        raise RuntimeError(f"expected x [in,W] and w [out] uint8, got {tuple(x.shape)}, {tuple(w.shape)} {w.dtype}")
+    out_dim = w.shape[0]
+    _check_index(a, "a", out_dim)
+    _check_index(b, "b", out_dim)
+    if k <= 0 or out_dim % k != 0:
+        raise ValueError(f"in_dim ({out_dim}) has to be divisible by k ({k}) but it is not")
+    dev = _same_device(x, a, b, w)
+    in_dim, words = x.shape
+    batch = words * bits - int(pad_len)
+    if pad_len < 0 or batch < 0:
+        raise RuntimeError(f"pad_len ({pad_len}) has to be in [0, {words * bits}]")
+    out = torch.empty((batch, k), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        st = _lib.load().dl_logic_eval_groupbitsum(_p(x), _p(a), _p(b), _p(w), _p(out), in_dim, out_dim, words, bits,
+                                                   int(pad_len), int(k), _stream(dev))
+    if st == _lib.DL_ERR_TOO_LARGE:
+        return groupbitsum(eval(x, a, b, w), pad_len, k)
+    if st:
+        _raise(st, "logic_layer_cuda_eval_groupbitsum")
+    return out

@@ -104,6 +104,17 @@ int dl_tensor_packbits_batch_major(const uint8_t *x, void *out, int64_t batch, i
 int dl_groupbitsum(const void *b, int32_t *out, int64_t in_dim, int64_t words, int bit_count,
                    int64_t pad_len, int64_t k, void *stream);
 
+/* Fuses the last LogicLayer's `eval` with `groupbitsum` (the sequence
+ * difflogic/difflogic.py:147 then difflogic/packbitstensor.py:22): the layer's output words are
+ * counted as they are produced and never written.
+ *   x [in_dim, words] words; a, b [out_dim]; w [out_dim] uint8 gate ids; k classes
+ *   -> out [words*bit_count - pad_len, k] int32, identical to dl_groupbitsum(dl_logic_eval(x)).
+ * Needs rows that are a whole number of 64-bit words (words*bit_count % 64 == 0) and k <= 65535;
+ * otherwise returns DL_ERR_TOO_LARGE and the caller uses the two separate entry points. */
+int dl_logic_eval_groupbitsum(const void *x, const int64_t *a, const int64_t *b, const uint8_t *w,
+                              int32_t *out, int64_t in_dim, int64_t out_dim, int64_t words,
+                              int bit_count, int64_t pad_len, int64_t k, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

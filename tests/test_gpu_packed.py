@@ -199,3 +199,47 @@ def test_pack_tensor_repr_and_modes():
         layer(p)                                                          # training mode
     with pytest.raises(NotImplementedError):
         dl.PackBitsTensor(t, device="cpu")
+
+
+@pytest.mark.parametrize("bits,in_dim,out_dim,W,k,pad", [
+    (64, 30, 60, 1, 3, 0), (64, 50, 640, 70, 10, 63), (64, 33, 130, 129, 2, 1), (32, 20, 64, 6, 4, 3),
+    (16, 20, 40, 12, 5, 0), (8, 12, 24, 16, 3, 2), (8, 12, 24, 9, 3, 7), (64, 100, 40000, 2, 2, 11),
+    (64, 64, 70000, 1, 1, 0), (32, 20, 64, 5, 4, 3),
+])
+def test_fused_eval_groupbitsum(ext, bits, in_dim, out_dim, W, k, pad):
+    rng = np.random.default_rng(in_dim + W + k + out_dim)
+    x = rng.integers(np.iinfo(NP_WORD[bits]).min, np.iinfo(NP_WORD[bits]).max, (in_dim, W), dtype=NP_WORD[bits],
+                     endpoint=True)
+    (a, b, op), = random_layers(rng, in_dim, [out_dim])
+    want = po.groupbitsum(po.eval_layer(x, a, b, op), pad, k)
+    got = ext.eval_groupbitsum(_dev(x), _dev(a), _dev(b), _dev(op), pad, k)
+    assert got.dtype == torch.int32 and tuple(got.shape) == want.shape
+    assert np.array_equal(got.cpu().numpy(), want)
+    two_step = ext.groupbitsum(ext.eval(_dev(x), _dev(a), _dev(b), _dev(op)), pad, k)
+    assert torch.equal(got, two_step)
+
+
+def test_lazy_pack_tensor_keeps_t_current():
+    """``.t`` read between layers and after the last layer equals the eager per-layer result."""
+    import difflogic_amd as dl
+    rng = np.random.default_rng(21)
+    layers = random_layers(rng, 20, [64, 64, 33])
+    x = rng.random((200, 20)) < 0.5
+    model = build_model(20, layers, 3).eval()
+    p = dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=64)
+    t = p.t.cpu().numpy()
+    for layer, (a, b, op) in zip([m for m in model if isinstance(m, dl.LogicLayer)], layers):
+        with torch.no_grad():
+            p = layer(p)
+        t = po.eval_layer(t, a, b, op)
+        assert np.array_equal(p.t.cpu().numpy(), t)
+    assert np.array_equal(p.group_sum(3).cpu().numpy(), po.groupbitsum(t, p.pad_len, 3))
+    with pytest.raises(ValueError):
+        p.group_sum(7)
+    # deferred last layer + group_sum (fused) and a user assigning .t
+    p2 = dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=64)
+    with torch.no_grad():
+        got = model(p2)
+    assert np.array_equal(got.cpu().numpy(), po.groupbitsum(t, p.pad_len, 3))
+    p2.t = torch.zeros_like(p2.t)
+    assert int(p2.group_sum(3).sum()) == 0
