@@ -226,14 +226,38 @@ def train_bench(args, torch, dl):
         kernels[name] = {"GBps": round(by / (ms * 1e-3) / 1e9, 1), "frac_hbm": round(by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                          "ms_per_step": round(ms / steps, 4)}
     neuron_samples = L * width * B
+    eager_loss = loss.item()
+    # Drop every reference to the eager autograd graph before capturing: gradient-accumulation
+    # nodes kept alive by `loss` belong to the default stream and would be replayed into the
+    # capture stream's backward.
+    del loss
+    model.zero_grad(set_to_none=True)
+    import gc
+    gc.collect()
+    torch.cuda.synchronize()
+    # the same step replayed as one HIP graph (removes the host launch overhead)
+    from difflogic_amd.graphs import GraphedTrainStep
+    graphed = GraphedTrainStep(model, loss_fn, x, labels)
+    for _ in range(warmup):
+        graphed.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        gl = graphed.step()
+    torch.cuda.synchronize()
+    g_elapsed = time.perf_counter() - t0
     return {
+        "graphed_neuron_samples_per_s": round(neuron_samples * steps / g_elapsed, 1),
+        "graphed_ms_per_step": round(g_elapsed / steps * 1e3, 4),
+        "graphed_GBps_algorithmic": round(tot_bytes / steps / (g_elapsed / steps) / 1e9, 1),
+        "graphed_loss": round(gl.item(), 6),
         "workload": "fp32 fwd+bwd 784->6x64000->GroupSum(10,tau=30), B=512, connections=unique, CrossEntropy",
         "neuron_samples_per_s": round(neuron_samples * steps / elapsed, 1),
         "neuron_samples_per_s_kernels_only": round(neuron_samples * steps / (tot_ms * 1e-3), 1),
         "ms_per_step": round(elapsed / steps * 1e3, 4),
         "kernel_GBps_algorithmic": round(tot_bytes / (tot_ms * 1e-3) / 1e9, 1),
         "kernel_frac_hbm": round(tot_bytes / (tot_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-        "kernels": kernels, "loss": round(loss.item(), 6), "dtype": "f32",
+        "kernels": kernels, "loss": round(eager_loss, 6), "dtype": "f32",
     }
 
 

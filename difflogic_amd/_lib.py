@@ -25,13 +25,16 @@ SIGNATURES = {
     "dl_logic_forward": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "dl_logic_backward_w": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "dl_logic_backward_x": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _dbl, _int, _vp],
+    "dl_group_sum_workspace_bytes": [_i64, _i64, _i64, _int],
+    "dl_group_sum_forward": [_vp, _vp, _vp, _i64, _i64, _i64, _dbl, _int, _vp],
+    "dl_group_sum_backward": [_vp, _vp, _i64, _i64, _i64, _dbl, _int, _vp],
     "dl_logic_eval": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "dl_tensor_packbits": [_vp, _vp, _i64, _i64, _int, ctypes.POINTER(_i64), _vp],
     "dl_tensor_packbits_batch_major": [_vp, _vp, _i64, _i64, _int, ctypes.POINTER(_i64), _vp],
     "dl_groupbitsum": [_vp, _vp, _i64, _i64, _int, _i64, _i64, _vp],
     "dl_logic_eval_groupbitsum": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _i64, _i64, _vp],
 }
-_RESTYPES = {"dl_status_string": ctypes.c_char_p}
+_RESTYPES = {"dl_status_string": ctypes.c_char_p, "dl_group_sum_workspace_bytes": ctypes.c_int64}
 
 _lib = None
 

@@ -354,6 +354,155 @@ int backward_x_t(const void *x, const int64_t *a, const int64_t *b, const void *
     return dl_launch_status();
 }
 
+// ------------------------------------------------------------------------------------------
+// GroupSum on the feature-major layout.
+//   forward : y[r, c] = (1/tau) * sum_{n in class c} x[n, r]       x [out, B] -> y [B, k]
+//   backward: gx[n, r] = g[r, class(n)] / tau                      g [B, k]   -> gx [out, B]
+// Forward is two passes with a fixed summation order: pass 1 sums SPLIT-th parts of every
+// class block over the rows (lanes along the batch, the workgroup's four waves interleave
+// rows and combine through LDS) into partial[s, c, r]; pass 2 adds the partials in order.
+// ------------------------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ __launch_bounds__(DL_BLOCK) void group_sum_partial_kernel(const T *__restrict__ x,
+                                                                     typename Acc<T>::type *__restrict__ partial,
+                                                                     int64_t per_class, int64_t ncols, int64_t k,
+                                                                     int64_t rows_per_split) {
+    typedef typename Acc<T>::type C;
+    typedef Pack<T, VEC> P;
+    __shared__ C lds[4][DL_WAVE * VEC];
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t col = (int64_t) blockIdx.x * DL_WAVE + lane;
+    const int64_t cls = blockIdx.y, split = blockIdx.z;
+    int64_t r0 = split * rows_per_split, r1 = r0 + rows_per_split;
+    if (r1 > per_class) r1 = per_class;
+    C acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = (C) 0;
+    if (col < ncols) {
+        const P *xv = reinterpret_cast<const P *>(x) + (cls * per_class) * ncols + col;
+        int64_t r = r0 + wave;
+        for (; r + 12 < r1; r += 16) {      // four independent row loads in flight per wave
+            const P v0 = xv[r * ncols], v1 = xv[(r + 4) * ncols], v2 = xv[(r + 8) * ncols], v3 = xv[(r + 12) * ncols];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] += (up<T>(v0.v[e]) + up<T>(v1.v[e])) + (up<T>(v2.v[e]) + up<T>(v3.v[e]));
+        }
+        for (; r < r1; r += 4) {
+            const P v = xv[r * ncols];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] += up<T>(v.v[e]);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) lds[wave][lane * VEC + e] = acc[e];
+    __syncthreads();
+    if (wave == 0 && col < ncols) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const int i = lane * VEC + e;
+            const C sum = (lds[0][i] + lds[1][i]) + (lds[2][i] + lds[3][i]);
+            partial[((int64_t) split * k + cls) * (ncols * VEC) + col * VEC + e] = sum;
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(DL_BLOCK) void group_sum_finish_kernel(const typename Acc<T>::type *__restrict__ partial,
+                                                                    T *__restrict__ y, int64_t batch, int64_t k,
+                                                                    int splits, typename Acc<T>::type inv_tau) {
+    typedef typename Acc<T>::type C;
+    const int64_t i = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x;     // i = r * k + c
+    if (i >= batch * k) return;
+    const int64_t r = i / k, c = i - r * k;
+    C sum = (C) 0;
+    for (int s = 0; s < splits; ++s) sum += partial[((int64_t) s * k + c) * batch + r];
+    y[i] = down<T, C>(sum * inv_tau);
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(DL_BLOCK) void group_sum_backward_kernel(const T *__restrict__ g, T *__restrict__ gx,
+                                                                      int64_t out_dim, int64_t per_class,
+                                                                      int64_t ncols, int64_t k,
+                                                                      typename Acc<T>::type inv_tau) {
+    typedef typename Acc<T>::type C;
+    typedef Pack<T, VEC> P;
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t col = (int64_t) blockIdx.x * DL_WAVE + lane;
+    if (col >= ncols) return;
+    constexpr int ROWS = 16;                                              // rows per wave
+    const int64_t n0 = ((int64_t) blockIdx.y * 4 + wave) * ROWS;
+    P *ov = reinterpret_cast<P *>(gx);
+    int64_t cached_cls = -1;
+    P val;
+    for (int64_t n = n0; n < n0 + ROWS && n < out_dim; ++n) {
+        const int64_t cls = n / per_class;
+        if (cls != cached_cls) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) val.v[e] = down<T, C>(up<T>(g[(col * VEC + e) * k + cls]) * inv_tau);
+            cached_cls = cls;
+        }
+        ov[n * ncols + col] = val;
+    }
+}
+
+template <typename T>
+int group_sum_forward_t(const void *x, void *y, void *workspace, int64_t out_dim, int64_t batch, int64_t k, int splits,
+                        double tau, hipStream_t s) {
+    typedef typename Acc<T>::type C;
+    constexpr int V = Vec16<T>::n;
+    const int64_t per_class = out_dim / k;
+    const int64_t rows_per_split = dl_ceil_div(per_class, splits);
+    const bool vec = batch % V == 0 && dl_aligned(x, 16);
+    const int64_t ncols = vec ? batch / V : batch;
+    const int64_t gx = dl_ceil_div(ncols, DL_WAVE);
+    if (gx > 0x7fffffffLL || k > 65535) return DL_ERR_TOO_LARGE;
+    const dim3 grid((unsigned) gx, (unsigned) k, (unsigned) splits);
+    if (vec)
+        hipLaunchKernelGGL((group_sum_partial_kernel<T, V>), grid, dim3(DL_BLOCK), 0, s, (const T *) x, (C *) workspace,
+                           per_class, ncols, k, rows_per_split);
+    else
+        hipLaunchKernelGGL((group_sum_partial_kernel<T, 1>), grid, dim3(DL_BLOCK), 0, s, (const T *) x, (C *) workspace,
+                           per_class, ncols, k, rows_per_split);
+    int st = dl_launch_status();
+    if (st != DL_OK) return st;
+    const int64_t blocks = dl_ceil_div(batch * k, DL_BLOCK);
+    if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    hipLaunchKernelGGL((group_sum_finish_kernel<T>), dim3((unsigned) blocks), dim3(DL_BLOCK), 0, s, (const C *) workspace,
+                       (T *) y, batch, k, splits, (C) (1.0 / tau));
+    return dl_launch_status();
+}
+
+template <typename T>
+int group_sum_backward_t(const void *g, void *gx, int64_t out_dim, int64_t batch, int64_t k, double tau, hipStream_t s) {
+    typedef typename Acc<T>::type C;
+    constexpr int V = Vec16<T>::n;
+    const bool vec = batch % V == 0 && dl_aligned(gx, 16);
+    const int64_t ncols = vec ? batch / V : batch;
+    const int64_t gxd = dl_ceil_div(ncols, DL_WAVE), gyd = dl_ceil_div(out_dim, 64);
+    if (gxd > 0x7fffffffLL || gyd > 65535) return DL_ERR_TOO_LARGE;
+    const dim3 grid((unsigned) gxd, (unsigned) gyd);
+    if (vec)
+        hipLaunchKernelGGL((group_sum_backward_kernel<T, V>), grid, dim3(DL_BLOCK), 0, s, (const T *) g, (T *) gx, out_dim,
+                           out_dim / k, ncols, k, (C) (1.0 / tau));
+    else
+        hipLaunchKernelGGL((group_sum_backward_kernel<T, 1>), grid, dim3(DL_BLOCK), 0, s, (const T *) g, (T *) gx, out_dim,
+                           out_dim / k, ncols, k, (C) (1.0 / tau));
+    return dl_launch_status();
+}
+
+// Number of row splits per class: enough workgroups to fill the chip, at least 64 rows each.
+int group_sum_splits(int64_t out_dim, int64_t batch, int64_t k) {
+    const int64_t per_class = out_dim / k;
+    const int64_t col_tiles = dl_ceil_div(batch, 4 * DL_WAVE);
+    int64_t want = dl_ceil_div(2048, col_tiles * k);
+    const int64_t max_by_rows = per_class / 64 > 0 ? per_class / 64 : 1;
+    if (want > max_by_rows) want = max_by_rows;
+    if (want < 1) want = 1;
+    if (want > 1024) want = 1024;
+    return (int) want;
+}
+
 }  // namespace
 
 extern "C" int dl_logic_forward(const void *x, const int64_t *a, const int64_t *b, const void *w, void *y,
@@ -400,6 +549,43 @@ extern "C" int dl_logic_backward_x(const void *x, const int64_t *a, const int64_
     case DL_F16: return backward_x_t<__half>(x, a, b, w, grad_y, start, idx, grad_x, in_dim, batch, scale, s);
     case DL_F32: return backward_x_t<float>(x, a, b, w, grad_y, start, idx, grad_x, in_dim, batch, scale, s);
     default: return backward_x_t<double>(x, a, b, w, grad_y, start, idx, grad_x, in_dim, batch, scale, s);
+    }
+}
+
+extern "C" int64_t dl_group_sum_workspace_bytes(int64_t out_dim, int64_t batch, int64_t k, int dtype) {
+    if (out_dim < 0 || batch < 0 || k <= 0 || out_dim % k != 0) return 0;
+    const int64_t elem = dtype == DL_F64 ? 8 : 4;
+    return (int64_t) group_sum_splits(out_dim, batch, k) * k * batch * elem;
+}
+
+extern "C" int dl_group_sum_forward(const void *x, void *y, void *workspace, int64_t out_dim, int64_t batch, int64_t k,
+                                    double tau, int dtype, void *stream) {
+    if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
+    if (out_dim < 0 || batch < 0 || k <= 0 || tau == 0.0) return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim % k != 0) return DL_ERR_NOT_DIVISIBLE;
+    if (batch == 0) return DL_OK;
+    if (!y || !workspace || (out_dim > 0 && !x)) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    const int splits = group_sum_splits(out_dim, batch, k);
+    switch (dtype) {
+    case DL_F16: return group_sum_forward_t<__half>(x, y, workspace, out_dim, batch, k, splits, tau, s);
+    case DL_F32: return group_sum_forward_t<float>(x, y, workspace, out_dim, batch, k, splits, tau, s);
+    default: return group_sum_forward_t<double>(x, y, workspace, out_dim, batch, k, splits, tau, s);
+    }
+}
+
+extern "C" int dl_group_sum_backward(const void *grad_y, void *grad_x, int64_t out_dim, int64_t batch, int64_t k,
+                                     double tau, int dtype, void *stream) {
+    if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
+    if (out_dim < 0 || batch < 0 || k <= 0 || tau == 0.0) return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim % k != 0) return DL_ERR_NOT_DIVISIBLE;
+    if (batch == 0 || out_dim == 0) return DL_OK;
+    if (!grad_y || !grad_x) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    switch (dtype) {
+    case DL_F16: return group_sum_backward_t<__half>(grad_y, grad_x, out_dim, batch, k, tau, s);
+    case DL_F32: return group_sum_backward_t<float>(grad_y, grad_x, out_dim, batch, k, tau, s);
+    default: return group_sum_backward_t<double>(grad_y, grad_x, out_dim, batch, k, tau, s);
     }
 }
 

@@ -141,6 +141,10 @@ class GroupSum(torch.nn.Module):
         if isinstance(x, PackBitsTensor):
             return x.group_sum(self.k)
         assert x.shape[-1] % self.k == 0, (x.shape, self.k)
+        if (x.is_cuda and x.dim() == 2 and x.dtype in (torch.float16, torch.float32, torch.float64)
+                and x.numel() > 0 and x.stride(0) == 1 and x.stride(1) == x.shape[0]):
+            # the transposed view a 'cuda' LogicLayer returns: sum on the feature-major storage
+            return GroupSumCudaFunction.apply(x.transpose(0, 1), self.k, float(self.tau))
         return x.reshape(*x.shape[:-1], self.k, x.shape[-1] // self.k).sum(-1) / self.tau
 
     def extra_repr(self):
@@ -169,3 +173,17 @@ class LogicLayerCudaFunction(torch.autograd.Function):
         if ctx.needs_input_grad[3]:
             grad_w = difflogic_cuda.backward_w(x, a, b, grad_y)
         return grad_x, None, None, grad_w, None, None, None
+
+
+class GroupSumCudaFunction(torch.autograd.Function):
+    """GroupSum on a feature-major [out, B] activation: -> [B, k].  The gradient comes back
+    feature-major too, so the layer below needs no transposing copy of it."""
+
+    @staticmethod
+    def forward(ctx, x, k, tau):
+        ctx.out_dim, ctx.tau = x.shape[0], tau
+        return difflogic_cuda.group_sum_forward(x, k, tau)
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        return difflogic_cuda.group_sum_backward(grad_y.contiguous(), ctx.out_dim, ctx.tau), None, None

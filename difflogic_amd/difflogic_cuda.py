@@ -252,3 +252,40 @@ def eval_groupbitsum(x, a, b, w, pad_len, k):
     if st:
         _raise(st, "logic_layer_cuda_eval_groupbitsum")
     return out
+
+
+def group_sum_forward(x, k, tau):
+    """Feature-major GroupSum: x [out,B] -> [B,k] = per-class sums over neurons / tau
+    (difflogic/difflogic.py:195-196 on the layout the layer kernels produce)."""
+    _check_input(x, "x")
+    code = _float_code(x, "group_sum_forward")
+    if x.dim() != 2:
+        raise RuntimeError(f"expected x [out,B], got {tuple(x.shape)}")
+    out_dim, batch = x.shape
+    if k <= 0 or out_dim % k != 0:
+        raise ValueError(f"in_dim ({out_dim}) has to be divisible by k ({k}) but it is not")
+    lib = _lib.load()
+    y = torch.empty((batch, k), dtype=x.dtype, device=x.device)
+    ws = torch.empty(max(1, lib.dl_group_sum_workspace_bytes(out_dim, batch, k, code)), dtype=torch.uint8,
+                     device=x.device)
+    with torch.cuda.device(x.device):
+        st = lib.dl_group_sum_forward(_p(x), _p(y), _p(ws), out_dim, batch, int(k), float(tau), code, _stream(x.device))
+    if st:
+        _raise(st, "group_sum_forward")
+    return y
+
+
+def group_sum_backward(grad_y, out_dim, tau):
+    """grad_y [B,k] -> grad_x [out,B]: every neuron of class c receives grad_y[:, c] / tau."""
+    _check_input(grad_y, "grad_y")
+    code = _float_code(grad_y, "group_sum_backward")
+    batch, k = grad_y.shape
+    if k <= 0 or out_dim % k != 0:
+        raise ValueError(f"in_dim ({out_dim}) has to be divisible by k ({k}) but it is not")
+    grad_x = torch.empty((out_dim, batch), dtype=grad_y.dtype, device=grad_y.device)
+    with torch.cuda.device(grad_y.device):
+        st = _lib.load().dl_group_sum_backward(_p(grad_y), _p(grad_x), out_dim, batch, int(k), float(tau), code,
+                                               _stream(grad_y.device))
+    if st:
+        _raise(st, "group_sum_backward")
+    return grad_x

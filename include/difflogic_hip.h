@@ -74,6 +74,20 @@ int dl_logic_backward_x(const void *x, const int64_t *a, const int64_t *b, const
                         int64_t in_dim, int64_t out_dim, int64_t batch, double scale, int dtype,
                         void *stream);
 
+/* ---- GroupSum on the feature-major layout (training mode) ------------------------------- */
+
+/* Replaces the float branch of GroupSum.forward (difflogic/difflogic.py:195-196) for the
+ * [out_dim, batch] layout the layer kernels produce, and its autograd backward:
+ *   forward : y[r, c] = (1/tau) * sum over the out_dim/k neurons of class c of x[n, r];
+ *             x [out_dim, batch] -> y [batch, k].  Deterministic (fixed summation order).
+ *             `workspace` is scratch of dl_group_sum_workspace_bytes(...) bytes.
+ *   backward: grad_x[n, r] = grad_y[r, class(n)] / tau;  grad_y [batch, k] -> grad_x [out_dim, batch]. */
+int64_t dl_group_sum_workspace_bytes(int64_t out_dim, int64_t batch, int64_t k, int dtype);
+int dl_group_sum_forward(const void *x, void *y, void *workspace, int64_t out_dim, int64_t batch,
+                         int64_t k, double tau, int dtype, void *stream);
+int dl_group_sum_backward(const void *grad_y, void *grad_x, int64_t out_dim, int64_t batch, int64_t k,
+                          double tau, int dtype, void *stream);
+
 /* ---- packed inference mode ------------------------------------------------------------ */
 
 /* Replaces `eval` = logic_layer_cuda_eval (difflogic.cpp:63-68, difflogic_kernel.cu:503-541).

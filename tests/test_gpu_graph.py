@@ -1,0 +1,75 @@
+"""A HIP-graph replay of the training step must reproduce the eager step on every replay,
+with eager work and synchronisations between replays."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _model(dl, seed):
+    torch.manual_seed(seed)
+    mods, d = [torch.nn.Flatten()], 60
+    for w in (400, 400, 300):
+        mods.append(dl.LogicLayer(d, w, grad_factor=1.5))
+        d = w
+    return torch.nn.Sequential(*mods, dl.GroupSum(10, 10.0)).train()
+
+
+def test_graphed_step_equals_eager_on_every_replay():
+    import difflogic_amd as dl
+    from difflogic_amd.graphs import GraphedTrainStep
+    model = _model(dl, 0)
+    loss_fn = torch.nn.CrossEntropyLoss()
+    g = torch.Generator(device="cuda").manual_seed(0)
+    xs = [(torch.rand(64, 60, device="cuda", generator=g) < 0.3).float() for _ in range(4)]
+    ys = [torch.randint(0, 10, (64,), device="cuda", generator=g) for _ in range(4)]
+
+    import copy
+    eager = copy.deepcopy(model)                      # same logits and wiring, its own .grad tensors
+    graphed = GraphedTrainStep(model, loss_fn, xs[0], ys[0])
+    for rep in range(6):
+        x, y = xs[rep % 4], ys[rep % 4]
+        loss_g = graphed.step(x, y)
+        torch.cuda.synchronize()
+        # eager work between the replays
+        eager.zero_grad(set_to_none=True)
+        loss_e = loss_fn(eager(x), y)
+        loss_e.backward()
+        torch.cuda.synchronize()
+        assert torch.equal(loss_g, loss_e.detach()), rep
+        for pg, pe in zip(model.parameters(), eager.parameters()):
+            assert pg.grad is not None and torch.equal(pg.grad, pe.grad), rep
+
+
+def test_graphed_step_with_optimizer_tracks_eager_training():
+    import copy
+
+    import difflogic_amd as dl
+    from difflogic_amd.graphs import GraphedTrainStep
+    model = _model(dl, 1)
+    eager = copy.deepcopy(model)
+    loss_fn = torch.nn.CrossEntropyLoss()
+    g = torch.Generator(device="cuda").manual_seed(1)
+    x = (torch.rand(32, 60, device="cuda", generator=g) < 0.3).float()
+    y = torch.randint(0, 10, (32,), device="cuda", generator=g)
+    opt_g = torch.optim.Adam(model.parameters(), lr=0.01, capturable=True)
+    opt_e = torch.optim.Adam(eager.parameters(), lr=0.01, capturable=True)
+    # the constructor's warm-up steps train the model too: keep the eager copy in step
+    graphed = GraphedTrainStep(model, loss_fn, x, y, optimizer=opt_g, warmup=2)
+    for _ in range(3):                                # 2 warm-ups + the captured (not executed) step is not run
+        pass
+    losses_g, losses_e = [], []
+    for _ in range(2):
+        opt_e.zero_grad(set_to_none=True)
+        loss_fn(eager(x), y).backward()
+        opt_e.step()
+    for rep in range(5):
+        losses_g.append(graphed.step().item())
+        opt_e.zero_grad(set_to_none=True)
+        le = loss_fn(eager(x), y)
+        le.backward()
+        opt_e.step()
+        losses_e.append(le.item())
+        torch.cuda.synchronize()
+    assert losses_g == losses_e, (losses_g, losses_e)
+    assert losses_g[-1] < losses_g[0]

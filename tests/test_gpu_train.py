@@ -204,3 +204,38 @@ def test_eval_mode_and_state_dict_round_trip():
     layers = [(l.indices[0].cpu(), l.indices[1].cpu(), l.weights.detach().cpu()) for l in (m1[1], m1[2])]
     want = fo.PythonNet(layers, 4, 2.0)(x.cpu(), training=False)
     assert torch.equal(y1.cpu(), want)
+
+
+@pytest.mark.parametrize("out_dim,batch,k", [(30, 1, 3), (640, 100, 10), (64000, 512, 10), (8000, 128, 10), (77, 260, 7),
+                                             (1200, 2048, 2), (40, 5000, 1)])
+def test_group_sum_feature_major(ext, out_dim, batch, k):
+    g = torch.Generator().manual_seed(out_dim + batch)
+    x = torch.rand(out_dim, batch, generator=g)
+    tau = 3.5
+    want = fo.group_sum(x.double().t(), k, tau)
+    got = ext.group_sum_forward(x.cuda(), k, tau)
+    assert got.shape == (batch, k)
+    ok, err = close(got, want)
+    assert ok, err
+    assert torch.equal(got, ext.group_sum_forward(x.cuda(), k, tau))           # deterministic
+    gy = torch.randn(batch, k, generator=g)
+    gx = ext.group_sum_backward(gy.cuda(), out_dim, tau)
+    want_gx = (gy.double() / tau).t().repeat_interleave(out_dim // k, dim=0)
+    assert gx.shape == (out_dim, batch) and close(gx, want_gx)[0]
+
+
+def test_group_sum_module_uses_feature_major_path_and_matches_torch():
+    import difflogic_amd as dl
+    gs = dl.GroupSum(10, 30.0)
+    y_fm = torch.rand(640, 96, device="cuda", requires_grad=True)
+    out = gs(y_fm.transpose(0, 1))
+    ref = y_fm.detach().t().reshape(96, 10, 64).sum(-1) / 30.0
+    assert close(out, ref)[0]
+    out.square().sum().backward()
+    want = (2 * ref / 30.0).t().repeat_interleave(64, dim=0)
+    assert close(y_fm.grad, want)[0]
+    # a plain [B, out] tensor still takes the generic path
+    z = torch.rand(96, 640, device="cuda")
+    assert close(gs(z), z.reshape(96, 10, 64).sum(-1) / 30.0)[0]
+    with pytest.raises(ValueError):
+        dl.difflogic_cuda.group_sum_forward(torch.rand(7, 4, device="cuda"), 2, 1.0)
