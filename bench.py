@@ -4,12 +4,13 @@
 Headline workload (the one BASELINE.json's metric is quoted on): bit-packed inference of the
 discretised net 784 -> 6 x 64000 -> GroupSum(k=10) on 2^20 synthetic samples.  One step is
 one pass of the whole path over the batch, starting from a bool [B, 784] tensor resident in
-HBM: PackBitsTensor (transpose + pack, 64-bit words) -> six LogicLayer.eval launches ->
-GroupSum bit counts [B, 10] int32.
+HBM: PackBitsTensor (transpose + pack, 64-bit words) -> six LogicLayers (evaluated in fused
+groups) -> GroupSum bit counts [B, 10] int32.
 
-Prints ONE JSON line.  `roofline` describes the dominant kernel (the per-layer gate
-evaluation): algorithmic bytes per launch = 8*W*(in+out) + 17*out, divided by the launch
-duration measured with events on the launch stream inside the timed region.  `cpu_baseline`
+Prints ONE JSON line.  `roofline` describes the dominant launch (the one that takes the most
+time per step): its algorithmic bytes (per layer 8*W*(in+out) + 17*out, summed over the layers a
+fused launch replaces) divided by the launch duration measured with events on the launch stream
+inside the timed region.  `cpu_baseline`
 times the CPU oracle (single thread, like the reference's generated C) on a bounded sample.
 `extra.train` reports the fp32 forward+backward path (784 -> 6 x 64000, B = 512).
 """
@@ -62,21 +63,42 @@ def packed_bench(args, torch, dl):
     x = torch.rand(B, F, device="cuda", generator=g) < 0.2
 
     ext = dl.difflogic_cuda
-    real_eval = ext.eval
-    launches = []          # (in_dim, out_dim, start_event, end_event)
+    names = ("tensor_packbits_batch_major", "eval", "eval_fused", "eval_fused_groupbitsum", "groupbitsum")
+    real = {n: getattr(ext, n) for n in names}
+    launches = []          # (kernel label, algorithmic bytes, start_event, end_event)
     record = {"on": False}
 
-    def timed_eval(xw, a, b, w):
-        if not record["on"]:
-            return real_eval(xw, a, b, w)
-        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        s.record()
-        y = real_eval(xw, a, b, w)
-        e.record()
-        launches.append((xw.shape[0], w.shape[0], s, e))
-        return y
+    def describe(name, a):
+        """(label, algorithmic bytes): per layer 8*W*(in+out) + 17*out, the count 8*W*out + 4*k*B, the
+        packing B*F + F*W*8; a fused launch is charged the sum over the layers it replaces."""
+        if name == "tensor_packbits_batch_major":
+            return "packbits_batch_major %dx%d" % tuple(a[0].shape), B * F + 8 * W * F
+        if name == "groupbitsum":
+            return "groupbitsum %d" % a[0].shape[0], 8 * W * a[0].shape[0] + 4 * k * B
+        if name == "eval":
+            return "eval %d->%d" % (a[0].shape[0], a[3].shape[0]), eval_layer_bytes(a[0].shape[0], a[3].shape[0], W)
+        dims = [a[0].shape[0]] + [l[2].shape[0] for l in a[1]]
+        by = sum(eval_layer_bytes(i, o, W) for i, o in zip(dims[:-1], dims[1:]))
+        label = "eval_fused x%d %s" % (len(a[1]), "->".join(str(d) for d in dims))
+        if name == "eval_fused_groupbitsum":
+            by += 8 * W * dims[-1] + 4 * k * B
+            label += " +groupbitsum"
+        return label, by
 
-    ext.eval = timed_eval
+    def timed(name):
+        def wrapper(*a, **kw):
+            if not record["on"]:
+                return real[name](*a, **kw)
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            y = real[name](*a, **kw)
+            e.record()
+            launches.append(describe(name, a) + (s, e))
+            return y
+        return wrapper
+
+    for n in names:
+        setattr(ext, n, timed(n))
 
     def step():
         with torch.no_grad():
@@ -93,27 +115,33 @@ def packed_bench(args, torch, dl):
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
     finally:
-        ext.eval = real_eval
+        for n in names:
+            setattr(ext, n, real[n])
         record["on"] = False
 
     ms_per_step = elapsed / args.steps * 1e3
-    # dominant kernel: the square (width -> width) gate-evaluation launches
-    sq = [(i, o, s.elapsed_time(e)) for i, o, s, e in launches if i == o]
-    if not sq:
-        sq = [(i, o, s.elapsed_time(e)) for i, o, s, e in launches]
-    alg = sum(eval_layer_bytes(i, o, W) for i, o, _ in sq) / len(sq)
-    avg_ms = sum(t for _, _, t in sq) / len(sq)
+    per_kernel = {}
+    for label, by, s, e in launches:
+        d = per_kernel.setdefault(label, {"n": 0, "ms": 0.0, "bytes": by})
+        d["n"] += 1
+        d["ms"] += s.elapsed_time(e)
+    # dominant kernel = the launch kind that takes the most time in a step
+    dom = max(per_kernel, key=lambda kk: per_kernel[kk]["ms"])
+    avg_ms = per_kernel[dom]["ms"] / per_kernel[dom]["n"]
+    alg = per_kernel[dom]["bytes"]
     achieved = alg / (avg_ms * 1e-3) / 1e9
-    first = [s.elapsed_time(e) for i, o, s, e in launches if i != o]
-    total_alg = sum(eval_layer_bytes(i, o, W) for i, o, *_ in launches) / args.steps + 8 * W * width + 4 * k * B
+    total_alg = sum(v["bytes"] * v["n"] for v in per_kernel.values()) / args.steps
     roofline = {
-        "bound": "hbm", "kernel": "eval_kernel<u32x4> %d->%d" % (sq[0][0], sq[0][1]),
+        "bound": "hbm", "kernel": dom,
         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-        "traffic": load_traffic(), "algorithmic_bytes_per_launch": int(alg), "avg_launch_ms": round(avg_ms, 4),
-        "launches_timed": len(sq),
+        "traffic": load_traffic(dom), "algorithmic_bytes_per_launch": int(alg), "avg_launch_ms": round(avg_ms, 4),
+        "launches_timed": per_kernel[dom]["n"],
     }
     info = {
-        "first_layer_avg_ms": round(sum(first) / len(first), 4) if first else None,
+        "kernels": {kk: {"avg_ms": round(v["ms"] / v["n"], 4), "launches_per_step": v["n"] / args.steps,
+                         "algorithmic_GB": round(v["bytes"] / 1e9, 3),
+                         "GBps_algorithmic": round(v["bytes"] / (v["ms"] / v["n"] * 1e-3) / 1e9, 1)}
+                    for kk, v in per_kernel.items()},
         "path_algorithmic_GB_per_step": round(total_alg / 1e9, 2),
         "path_GBps_algorithmic": round(total_alg / (ms_per_step * 1e-3) / 1e9, 1),
         "checksum": int(out.sum().item()),
@@ -121,13 +149,16 @@ def packed_bench(args, torch, dl):
     return B * args.steps / elapsed, ms_per_step, roofline, info, model, x
 
 
-def load_traffic():
-    """HBM bytes per launch of the dominant kernel from the committed rocprofv3 --pmc summary
-    (profiles/eval_kernel_traffic.json), or None when it has not been measured."""
-    p = os.path.join(ROOT, "profiles", "eval_kernel_traffic.json")
+def load_traffic(kernel_label):
+    """HBM-side bytes per launch of the dominant kernel from the committed rocprofv3 --pmc summary
+    (profiles/packed_kernel_traffic.json, keyed by the launch label), or None when that launch
+    has not been measured."""
+    p = os.path.join(ROOT, "profiles", "packed_kernel_traffic.json")
     if os.path.exists(p):
         with open(p) as f:
-            return json.load(f).get("hbm_bytes_per_launch")
+            entry = json.load(f).get(kernel_label)
+        if entry:
+            return entry.get("hbm_bytes_per_launch")
     return None
 
 
@@ -320,7 +351,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int64", "data": "synthetic",
         "config": {"workload": "packed inference %d->%dx%d->GroupSum(10), batch 2^%d, int64 words, bool input "
-                               "resident in HBM; step = pack + %d eval layers + groupbitsum"
+                               "resident in HBM; step = pack + %d gate layers + groupbitsum"
                                % (args.features, args.layers, args.width, args.batch_log2, args.layers),
                    "connections": "random", "seed": 0},
         "roofline": roofline,

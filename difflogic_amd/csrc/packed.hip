@@ -28,6 +28,9 @@ __device__ __forceinline__ GateMasks gate_masks(uint32_t op) {
 template <typename V> struct Splat;
 template <> struct Splat<dl_u32x4> { static __device__ __forceinline__ dl_u32x4 of(uint32_t v) { return dl_u32x4{v, v, v, v}; } };
 template <> struct Splat<dl_u32x2> { static __device__ __forceinline__ dl_u32x2 of(uint32_t v) { return dl_u32x2{v, v}; } };
+template <> struct Splat<uint64_t> {
+    static __device__ __forceinline__ uint64_t of(uint32_t v) { return ((uint64_t) v << 32) | v; }
+};
 template <> struct Splat<uint32_t> { static __device__ __forceinline__ uint32_t of(uint32_t v) { return v; } };
 template <> struct Splat<uint16_t> { static __device__ __forceinline__ uint16_t of(uint32_t v) { return (uint16_t) v; } };
 template <> struct Splat<uint8_t> { static __device__ __forceinline__ uint8_t of(uint32_t v) { return (uint8_t) v; } };
@@ -81,6 +84,116 @@ __global__ __launch_bounds__(DL_BLOCK) void eval_kernel(const V *__restrict__ x,
                         const V r = gate_apply<V>(va[j], vb[j], gate_masks(op[j]));
                         __builtin_nontemporal_store(r, &y[(n0 + j) * ncols + col]);
                     }
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Fused evaluation of D consecutive layers.  Output neuron n of the group's last layer is a
+// depth-D binary tree of gates over 2^D rows of the group's input.  A small kernel flattens the
+// D wiring tables into per-neuron composites (2^D int32 row ids + the 2^D - 1 gate ids packed
+// 4 bits each), and the evaluation kernel gathers the leaves and folds the tree in registers:
+// the D - 1 intermediate activations never exist in memory.  Bit-identical to D calls of the
+// single-layer kernel.
+//
+// Packing of the gate ids follows the fold order: for a subtree of depth d at bit offset `off`
+// the left child's subtree sits at off, the right child's at off + 4*(2^(d-1) - 1), and the
+// subtree's own gate at off + 4*(2^d - 2).  Leaves are in left-to-right order (`a` before `b`).
+// ------------------------------------------------------------------------------------------
+#define DL_MAX_FUSE_DEPTH 4
+
+struct TreeTables {
+    const int64_t *a[DL_MAX_FUSE_DEPTH];   // [0] = first (lowest) layer of the group
+    const int64_t *b[DL_MAX_FUSE_DEPTH];
+    const uint8_t *w[DL_MAX_FUSE_DEPTH];
+};
+
+template <int D>
+__global__ __launch_bounds__(DL_BLOCK) void compose_tree_kernel(TreeTables t, int32_t *__restrict__ leaves,
+                                                                uint64_t *__restrict__ gates, int64_t out_dim) {
+    const int64_t n = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x;
+    if (n >= out_dim) return;
+    int64_t nodes[1 << D];
+    nodes[0] = n;
+    uint64_t packed = 0;
+#pragma unroll
+    for (int r = 0; r < D; ++r) {                  // r = distance from the root; layer index D-1-r
+        const int layer = D - 1 - r;
+        int64_t next[1 << D];
+#pragma unroll
+        for (int i = 0; i < (1 << r); ++i) {
+            const int64_t node = nodes[i];
+            next[2 * i] = t.a[layer][node];
+            next[2 * i + 1] = t.b[layer][node];
+            int off = 0, d = D;                    // bit slot of node (r, i)
+#pragma unroll
+            for (int kbit = r - 1; kbit >= 0; --kbit) {
+                off += ((i >> kbit) & 1) * ((1 << (d - 1)) - 1);
+                d -= 1;
+            }
+            const int slot = off + 2 * ((1 << (d - 1)) - 1);
+            packed |= (uint64_t) (t.w[layer][node] & 15u) << (4 * slot);
+        }
+#pragma unroll
+        for (int i = 0; i < (2 << r); ++i) nodes[i] = next[i];
+    }
+#pragma unroll
+    for (int i = 0; i < (1 << D); ++i) leaves[n * (1 << D) + i] = (int32_t) nodes[i];
+    gates[n] = packed;
+}
+
+template <typename V, int D> struct TreeFold {
+    static __device__ __forceinline__ V run(const V *leaf, uint64_t gates) {
+        constexpr int half = 1 << (D - 1);
+        const V l = TreeFold<V, D - 1>::run(leaf, gates);
+        const V r = TreeFold<V, D - 1>::run(leaf + half, gates >> (4 * (half - 1)));
+        return gate_apply<V>(l, r, gate_masks((uint32_t) (gates >> (4 * (2 * half - 2))) & 15u));
+    }
+};
+template <typename V> struct TreeFold<V, 0> {
+    static __device__ __forceinline__ V run(const V *leaf, uint64_t) { return leaf[0]; }
+};
+
+// Same tiling and dispatch order as eval_kernel; one wave = NPW output neurons x 64 vectors.
+template <typename V, int D, int NPW, int ITERS>
+__global__ __launch_bounds__(DL_BLOCK) void eval_tree_kernel(const V *__restrict__ x,
+                                                             const int32_t *__restrict__ leaves,
+                                                             const uint64_t *__restrict__ gates, V *__restrict__ y,
+                                                             int64_t out_dim, int64_t ncols) {
+    constexpr int G = 1 << D;
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t n_first = ((int64_t) blockIdx.x * 4 + wave) * (NPW * ITERS);
+
+    for (int64_t ct = blockIdx.y; ct * DL_WAVE < ncols; ct += gridDim.y) {
+        const int64_t col = ct * DL_WAVE + lane;
+        const bool live = col < ncols;
+#pragma unroll 1
+        for (int it = 0; it < ITERS; ++it) {
+            const int64_t n0 = n_first + (int64_t) it * NPW;
+            if (n0 >= out_dim) break;
+            int32_t id[NPW][G];
+            uint64_t gt[NPW];
+#pragma unroll
+            for (int j = 0; j < NPW; ++j) {
+                const int64_t n = (n0 + j < out_dim) ? n0 + j : out_dim - 1;
+                gt[j] = gates[n];
+#pragma unroll
+                for (int g = 0; g < G; ++g) id[j][g] = leaves[n * G + g];
+            }
+            if (live) {
+                V v[NPW][G];
+#pragma unroll
+                for (int j = 0; j < NPW; ++j) {
+#pragma unroll
+                    for (int g = 0; g < G; ++g) v[j][g] = x[(int64_t) id[j][g] * ncols + col];
+                }
+#pragma unroll
+                for (int j = 0; j < NPW; ++j) {
+                    if (n0 + j < out_dim)
+                        __builtin_nontemporal_store(TreeFold<V, D>::run(v[j], gt[j]), &y[(n0 + j) * ncols + col]);
                 }
             }
         }
@@ -254,17 +367,17 @@ __device__ __forceinline__ void csa(uint64_t &carry, uint64_t &sum, uint64_t a, 
 }
 
 //
-// FUSED: the counted rows are not read but computed on the fly as the gate layer
-// y[n] = gate_{op[n]}(x[a[n]], x[b[n]]) over the rows of `bits` (= the layer's input), so the
-// last layer's output never exists in memory.
-template <int NPH, bool FUSED>
+// TREE > 0: the counted rows are not read but computed on the fly as the last TREE layers of the
+// net over the rows of `bits` (= the input of those layers), from the composites that
+// compose_tree_kernel writes; the output of the last layer never exists in memory.
+template <int NPH, int TREE>
 __global__ __launch_bounds__(DL_BLOCK) void groupbitsum_kernel(const uint64_t *__restrict__ bits,
-                                                               const int64_t *__restrict__ ga,
-                                                               const int64_t *__restrict__ gb,
-                                                               const uint8_t *__restrict__ gop,
+                                                               const int32_t *__restrict__ leaves,
+                                                               const uint64_t *__restrict__ gates,
                                                                int32_t *__restrict__ out, int64_t words,
                                                                int64_t per_class, int64_t k, int64_t batch) {
     constexpr int NP = NPH + 4;
+    constexpr int G = 1 << TREE;
     __shared__ uint64_t planes_lds[4][NP][DL_WAVE];
     __shared__ int32_t tile[DL_WAVE][DL_WAVE + 1];   // [column][sample], padded against bank conflicts
 
@@ -290,31 +403,30 @@ __global__ __launch_bounds__(DL_BLOCK) void groupbitsum_kernel(const uint64_t *_
     const uint64_t *xcol = bits + (live ? col : 0);
     for (int64_t r = r_begin; r < r_end; r += 16) {
         uint64_t v[16];
-        if (!FUSED) {
+        if (TREE == 0) {
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
                 v[j] = (live && r + j < r_end) ? __builtin_nontemporal_load(row + (int64_t) j * words) : 0;
             }
             row += 16 * words;
         } else {
-            uint64_t va[16], vb[16];
-            uint32_t op[16];
+            constexpr int SUB = (TREE == 1) ? 16 : 8;        // neurons whose leaves are in flight together
 #pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                const int64_t n = cls * per_class + ((r + j < r_end) ? r + j : r_end - 1);
-                const int64_t ia = ga[n], ib = gb[n];
-                op[j] = gop[n];
-                va[j] = live ? xcol[ia * words] : 0;
-                vb[j] = live ? xcol[ib * words] : 0;
-            }
+            for (int h = 0; h < 16; h += SUB) {
+                uint64_t leaf[SUB][G];
+                uint64_t gt[SUB];
 #pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                const GateMasks m = gate_masks(op[j]);
-                const uint64_t m00 = ((uint64_t) m.m00 << 32) | m.m00, m01 = ((uint64_t) m.m01 << 32) | m.m01;
-                const uint64_t m10 = ((uint64_t) m.m10 << 32) | m.m10, m11 = ((uint64_t) m.m11 << 32) | m.m11;
-                const uint64_t hi = (vb[j] & m11) | (~vb[j] & m10), lo = (vb[j] & m01) | (~vb[j] & m00);
-                const uint64_t y = (va[j] & hi) | (~va[j] & lo);
-                v[j] = (live && r + j < r_end) ? y : 0;
+                for (int j = 0; j < SUB; ++j) {
+                    const int64_t n = cls * per_class + ((r + h + j < r_end) ? r + h + j : r_end - 1);
+                    gt[j] = gates[n];
+#pragma unroll
+                    for (int g = 0; g < G; ++g) leaf[j][g] = live ? xcol[(int64_t) leaves[n * G + g] * words] : 0;
+                }
+#pragma unroll
+                for (int j = 0; j < SUB; ++j) {
+                    const uint64_t y = TreeFold<uint64_t, TREE>::run(leaf[j], gt[j]);
+                    v[h + j] = (live && r + h + j < r_end) ? y : 0;
+                }
             }
         }
         uint64_t t2a, t2b, t4a, t4b, t8a, t8b, t16;
@@ -392,20 +504,75 @@ __global__ __launch_bounds__(DL_BLOCK) void groupbitsum_generic_kernel(const uin
     }
 }
 
-template <bool FUSED>
-void launch_groupbitsum(const uint64_t *bits, const int64_t *a, const int64_t *b, const uint8_t *op, int32_t *out,
+template <int TREE>
+void launch_groupbitsum(const uint64_t *bits, const int32_t *leaves, const uint64_t *gates, int32_t *out,
                         int64_t words64, int64_t per_class, int64_t k, int64_t batch, dim3 grid, hipStream_t s) {
     const int64_t chunk = (per_class + 3) / 4;      // rows one wave counts
     // NPH planes above weight 8 hold counts up to 16 * 2^NPH - 1.
     if (chunk < (16LL << 8))
-        hipLaunchKernelGGL((groupbitsum_kernel<8, FUSED>), grid, dim3(DL_BLOCK), 0, s, bits, a, b, op, out, words64,
+        hipLaunchKernelGGL((groupbitsum_kernel<8, TREE>), grid, dim3(DL_BLOCK), 0, s, bits, leaves, gates, out, words64,
                            per_class, k, batch);
     else if (chunk < (16LL << 14))
-        hipLaunchKernelGGL((groupbitsum_kernel<14, FUSED>), grid, dim3(DL_BLOCK), 0, s, bits, a, b, op, out, words64,
+        hipLaunchKernelGGL((groupbitsum_kernel<14, TREE>), grid, dim3(DL_BLOCK), 0, s, bits, leaves, gates, out, words64,
                            per_class, k, batch);
     else
-        hipLaunchKernelGGL((groupbitsum_kernel<27, FUSED>), grid, dim3(DL_BLOCK), 0, s, bits, a, b, op, out, words64,
+        hipLaunchKernelGGL((groupbitsum_kernel<27, TREE>), grid, dim3(DL_BLOCK), 0, s, bits, leaves, gates, out, words64,
                            per_class, k, batch);
+}
+
+// Validates the description of a fused group and launches the composite builder.
+// dims = {in_dim, width of layer 0, ..., width of layer depth-1} (host array).
+int compose_tree(int depth, const int64_t *const *a, const int64_t *const *b, const uint8_t *const *w,
+                 const int64_t *dims, void *workspace, int32_t **leaves, uint64_t **gates, hipStream_t s) {
+    if (depth < 1 || depth > DL_MAX_FUSE_DEPTH || !a || !b || !w || !dims || !workspace) return DL_ERR_INVALID_ARGUMENT;
+    TreeTables t;
+    for (int l = 0; l < depth; ++l) {
+        if (!a[l] || !b[l] || !w[l] || dims[l] <= 0 || dims[l + 1] <= 0) return DL_ERR_INVALID_ARGUMENT;
+        if (dims[l] > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+        t.a[l] = a[l];
+        t.b[l] = b[l];
+        t.w[l] = w[l];
+    }
+    for (int l = depth; l < DL_MAX_FUSE_DEPTH; ++l) t.a[l] = t.b[l] = nullptr, t.w[l] = nullptr;
+    if (!dl_aligned(workspace, 8)) return DL_ERR_INVALID_ARGUMENT;
+    const int64_t out_dim = dims[depth];
+    *gates = (uint64_t *) workspace;
+    *leaves = (int32_t *) ((uint64_t *) workspace + out_dim);
+    const int64_t blocks = dl_ceil_div(out_dim, DL_BLOCK);
+    if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    const dim3 grid((unsigned) blocks), block(DL_BLOCK);
+    switch (depth) {
+    case 1: hipLaunchKernelGGL(compose_tree_kernel<1>, grid, block, 0, s, t, *leaves, *gates, out_dim); break;
+    case 2: hipLaunchKernelGGL(compose_tree_kernel<2>, grid, block, 0, s, t, *leaves, *gates, out_dim); break;
+    case 3: hipLaunchKernelGGL(compose_tree_kernel<3>, grid, block, 0, s, t, *leaves, *gates, out_dim); break;
+    default: hipLaunchKernelGGL(compose_tree_kernel<4>, grid, block, 0, s, t, *leaves, *gates, out_dim); break;
+    }
+    return dl_launch_status();
+}
+
+template <typename V>
+int launch_eval_tree(int depth, const void *x, const int32_t *leaves, const uint64_t *gates, void *y, int64_t out_dim,
+                     int64_t row_bytes, hipStream_t s) {
+    const int64_t ncols = row_bytes / (int64_t) sizeof(V);
+    int64_t ctiles = dl_ceil_div(ncols, DL_WAVE);
+    if (ctiles > 65535) ctiles = 65535;
+    const V *xv = (const V *) x;
+    V *yv = (V *) y;
+#define DL_TREE_LAUNCH(D, NPW, ITERS)                                                                                 \
+    {                                                                                                                  \
+        const int64_t ntiles = dl_ceil_div(out_dim, 4 * NPW * ITERS);                                                  \
+        if (ntiles > 0x7fffffffLL) return DL_ERR_TOO_LARGE;                                                            \
+        hipLaunchKernelGGL((eval_tree_kernel<V, D, NPW, ITERS>), dim3((unsigned) ntiles, (unsigned) ctiles),           \
+                           dim3(DL_BLOCK), 0, s, xv, leaves, gates, yv, out_dim, ncols);                               \
+    }
+    switch (depth) {
+    case 1: DL_TREE_LAUNCH(1, 4, 4) break;
+    case 2: DL_TREE_LAUNCH(2, 2, 4) break;
+    case 3: DL_TREE_LAUNCH(3, 2, 4) break;
+    default: DL_TREE_LAUNCH(4, 1, 8) break;
+    }
+#undef DL_TREE_LAUNCH
+    return dl_launch_status();
 }
 
 bool valid_bit_count(int bit_count) { return bit_count == 8 || bit_count == 16 || bit_count == 32 || bit_count == 64; }
@@ -500,8 +667,7 @@ extern "C" int dl_groupbitsum(const void *b, int32_t *out, int64_t in_dim, int64
         const int64_t gx = dl_ceil_div(words64, DL_WAVE);
         if (gx > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
         const dim3 grid((unsigned) gx, (unsigned) k);
-        launch_groupbitsum<false>((const uint64_t *) b, nullptr, nullptr, nullptr, out, words64, per_class, k, batch,
-                                  grid, s);
+        launch_groupbitsum<0>((const uint64_t *) b, nullptr, nullptr, out, words64, per_class, k, batch, grid, s);
     } else {
         int64_t gx = dl_ceil_div(batch, DL_BLOCK);
         if (gx > 0x7fffffffLL) gx = 0x7fffffffLL;
@@ -512,24 +678,58 @@ extern "C" int dl_groupbitsum(const void *b, int32_t *out, int64_t in_dim, int64
     return dl_launch_status();
 }
 
-extern "C" int dl_logic_eval_groupbitsum(const void *x, const int64_t *a, const int64_t *b, const uint8_t *w,
-                                         int32_t *out, int64_t in_dim, int64_t out_dim, int64_t words, int bit_count,
-                                         int64_t pad_len, int64_t k, void *stream) {
+extern "C" int64_t dl_logic_eval_fused_workspace_bytes(int depth, int64_t out_dim) {
+    if (depth < 1 || depth > DL_MAX_FUSE_DEPTH || out_dim < 0) return 0;
+    return out_dim * (8 + 4 * (int64_t) (1 << depth));
+}
+
+extern "C" int dl_logic_eval_fused(const void *x, int depth, const int64_t *const *a, const int64_t *const *b,
+                                   const uint8_t *const *w, const int64_t *dims, void *y, int64_t words, int bit_count,
+                                   void *workspace, void *stream) {
     if (!valid_bit_count(bit_count)) return DL_ERR_BIT_COUNT;
-    if (in_dim < 0 || out_dim < 0 || words < 0 || k <= 0 || pad_len < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (depth < 1 || depth > DL_MAX_FUSE_DEPTH || !dims || words < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (words == 0) return DL_OK;
+    if (!x || !y) return DL_ERR_INVALID_ARGUMENT;
+    const int64_t row_bytes = words * (bit_count / 8);
+    const uintptr_t mis = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) | (uintptr_t) row_bytes;
+    if (mis % 8 != 0) return DL_ERR_TOO_LARGE;       // rows are not whole 64-bit words: use dl_logic_eval per layer
+    hipStream_t s = (hipStream_t) stream;
+    int32_t *leaves;
+    uint64_t *gates;
+    const int st = compose_tree(depth, a, b, w, dims, workspace, &leaves, &gates, s);
+    if (st != DL_OK) return st;
+    if (mis % 16 == 0) return launch_eval_tree<dl_u32x4>(depth, x, leaves, gates, y, dims[depth], row_bytes, s);
+    return launch_eval_tree<dl_u32x2>(depth, x, leaves, gates, y, dims[depth], row_bytes, s);
+}
+
+extern "C" int dl_logic_eval_fused_groupbitsum(const void *x, int depth, const int64_t *const *a,
+                                               const int64_t *const *b, const uint8_t *const *w, const int64_t *dims,
+                                               int32_t *out, int64_t words, int bit_count, int64_t pad_len, int64_t k,
+                                               void *workspace, void *stream) {
+    if (!valid_bit_count(bit_count)) return DL_ERR_BIT_COUNT;
+    if (depth < 1 || depth > 2 || !dims || words < 0 || k <= 0 || pad_len < 0) return DL_ERR_INVALID_ARGUMENT;
+    const int64_t out_dim = dims[depth];
+    if (out_dim <= 0) return DL_ERR_INVALID_ARGUMENT;
     if (out_dim % k != 0) return DL_ERR_NOT_DIVISIBLE;
     const int64_t batch = words * bit_count - pad_len;
     if (batch < 0) return DL_ERR_INVALID_ARGUMENT;
     if (batch == 0) return DL_OK;
-    if (!out) return DL_ERR_INVALID_ARGUMENT;
-    if (out_dim > 0 && (!x || !a || !b || !w || in_dim == 0)) return DL_ERR_INVALID_ARGUMENT;
+    if (!out || !x) return DL_ERR_INVALID_ARGUMENT;
     const int64_t per_class = out_dim / k;
     const int64_t row_bytes = words * (bit_count / 8);
     if (row_bytes % 8 != 0 || !dl_aligned(x, 8) || k > 65535 || per_class > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     const int64_t words64 = row_bytes / 8;
     const int64_t gx = dl_ceil_div(words64, DL_WAVE);
     if (gx > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
-    launch_groupbitsum<true>((const uint64_t *) x, a, b, w, out, words64, per_class, k, batch,
-                             dim3((unsigned) gx, (unsigned) k), (hipStream_t) stream);
+    hipStream_t s = (hipStream_t) stream;
+    int32_t *leaves;
+    uint64_t *gates;
+    const int st = compose_tree(depth, a, b, w, dims, workspace, &leaves, &gates, s);
+    if (st != DL_OK) return st;
+    const dim3 grid((unsigned) gx, (unsigned) k);
+    if (depth == 1)
+        launch_groupbitsum<1>((const uint64_t *) x, leaves, gates, out, words64, per_class, k, batch, grid, s);
+    else
+        launch_groupbitsum<2>((const uint64_t *) x, leaves, gates, out, words64, per_class, k, batch, grid, s);
     return dl_launch_status();
 }

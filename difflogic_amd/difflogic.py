@@ -104,11 +104,11 @@ class LogicLayer(torch.nn.Module):
 
     def forward_cuda_eval(self, x: PackBitsTensor):
         """Packed inference.  Updates ``x`` in place (as the reference rebinds ``x.t``) and
-        returns it.  The evaluation is deferred until ``x.t`` is read, the next layer is applied
-        or GroupSum consumes it; GroupSum then runs fused with this layer."""
+        returns it.  The evaluation is deferred until ``x.t`` is read or GroupSum consumes it;
+        deferred layers run in fused groups (PackBitsTensor.plan_groups)."""
         assert not self.training
         assert isinstance(x, PackBitsTensor)
-        assert x.t.shape[0] == self.in_dim, (x.t.shape, self.in_dim)
+        assert x.features == self.in_dim, (x.features, self.in_dim)
         a, b = self.indices
         w = self.weights.argmax(-1).to(torch.uint8)
         return x.defer_layer(a, b, w)

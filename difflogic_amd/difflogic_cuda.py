@@ -222,35 +222,90 @@ def groupbitsum(b, pad_len, k):
     return out
 
 
-def eval_groupbitsum(x, a, b, w, pad_len, k):
-    """groupbitsum(eval(x, a, b, w), pad_len, k) without materialising the layer's output.
-    Not part of the reference's extension; the lazy PackBitsTensor uses it for the last layer.
-    Falls back to the two separate kernels where the fused one does not apply."""
-    for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w")):
-        _check_input(t, n)
+MAX_FUSE_DEPTH = 4          # layers dl_logic_eval_fused can fold into one kernel
+MAX_FUSE_DEPTH_COUNT = 2    # layers dl_logic_eval_fused_groupbitsum can fold
+
+
+def _fused_args(x, layers):
+    """Validates a group of consecutive layers [(a, b, w), ...] applied to x and builds the host
+    arrays of device pointers the C ABI takes."""
+    _check_input(x, "x")
     bits = _WORD_BITS.get(x.dtype)
     if bits is None:
         raise RuntimeError(f'"logic_layer_cuda_eval_kernel" not implemented for \'{x.dtype}\'')
-    if x.dim() != 2 or w.dim() != 1 or w.dtype != torch.uint8:
-        raise RuntimeError(f"expected x [in,W] and w [out] uint8, got {tuple(x.shape)}, {tuple(w.shape)} {w.dtype}")
-    out_dim = w.shape[0]
-    _check_index(a, "a", out_dim)
-    _check_index(b, "b", out_dim)
+    if x.dim() != 2 or not layers:
+        raise RuntimeError(f"expected x [in,W] and at least one layer, got {tuple(x.shape)}, {len(layers)} layers")
+    dims = [x.shape[0]]
+    tensors = [x]
+    for a, b, w in layers:
+        _check_input(w, "w")
+        if w.dim() != 1 or w.dtype != torch.uint8:
+            raise RuntimeError(f"expected w [out] uint8, got {tuple(w.shape)} {w.dtype}")
+        _check_index(a, "a", w.shape[0])
+        _check_index(b, "b", w.shape[0])
+        dims.append(w.shape[0])
+        tensors += [a, b, w]
+    dev = _same_device(*tensors)
+    depth = len(layers)
+    ptrs = lambda i: (ctypes.c_void_p * depth)(*[l[i].data_ptr() for l in layers])  # noqa: E731
+    return dev, bits, depth, ptrs(0), ptrs(1), ptrs(2), (ctypes.c_int64 * (depth + 1))(*dims), dims
+
+
+def _fused_workspace(depth, out_dim, dev):
+    n = _lib.load().dl_logic_eval_fused_workspace_bytes(depth, out_dim)
+    return torch.empty(max(1, -(-n // 8)), dtype=torch.int64, device=dev)
+
+
+def eval_fused(x, layers):
+    """``eval`` applied once per layer of ``layers`` = [(a, b, w), ...] (at most MAX_FUSE_DEPTH),
+    in one kernel that never writes the intermediate activations.  Not part of the reference's
+    extension.  Falls back to one ``eval`` per layer where the fused kernel does not apply."""
+    dev, bits, depth, pa, pb, pw, pdims, dims = _fused_args(x, layers)
+    if depth > MAX_FUSE_DEPTH:
+        raise RuntimeError(f"at most {MAX_FUSE_DEPTH} layers can be fused, got {depth}")
+    words = x.shape[1]
+    if depth == 1 or 0 in dims or words == 0:
+        st = _lib.DL_ERR_TOO_LARGE
+    else:
+        y = torch.empty((dims[-1], words), dtype=x.dtype, device=dev)
+        ws = _fused_workspace(depth, dims[-1], dev)
+        with torch.cuda.device(dev):
+            st = _lib.load().dl_logic_eval_fused(_p(x), depth, pa, pb, pw, pdims, _p(y), words, bits, _p(ws),
+                                                 _stream(dev))
+    if st == _lib.DL_ERR_TOO_LARGE:
+        for a, b, w in layers:
+            x = eval(x, a, b, w)
+        return x
+    if st:
+        _raise(st, "logic_layer_cuda_eval_fused")
+    return y
+
+
+def eval_fused_groupbitsum(x, layers, pad_len, k):
+    """groupbitsum(eval(... eval(x, layer 0) ..., last layer), pad_len, k) for the net's last
+    one or two layers without materialising their output.  Not part of the reference's
+    extension.  Falls back to the separate kernels where the fused one does not apply."""
+    dev, bits, depth, pa, pb, pw, pdims, dims = _fused_args(x, layers)
+    if depth > MAX_FUSE_DEPTH_COUNT:
+        raise RuntimeError(f"at most {MAX_FUSE_DEPTH_COUNT} layers can be fused with the count, got {depth}")
+    out_dim, words = dims[-1], x.shape[1]
     if k <= 0 or out_dim % k != 0:
         raise ValueError(f"in_dim ({out_dim}) has to be divisible by k ({k}) but it is not")
-    dev = _same_device(x, a, b, w)
-    in_dim, words = x.shape
     batch = words * bits - int(pad_len)
     if pad_len < 0 or batch < 0:
         raise RuntimeError(f"pad_len ({pad_len}) has to be in [0, {words * bits}]")
-    out = torch.empty((batch, k), dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
-        st = _lib.load().dl_logic_eval_groupbitsum(_p(x), _p(a), _p(b), _p(w), _p(out), in_dim, out_dim, words, bits,
-                                                   int(pad_len), int(k), _stream(dev))
+    if 0 in dims:
+        st = _lib.DL_ERR_TOO_LARGE
+    else:
+        out = torch.empty((batch, k), dtype=torch.int32, device=dev)
+        ws = _fused_workspace(depth, out_dim, dev)
+        with torch.cuda.device(dev):
+            st = _lib.load().dl_logic_eval_fused_groupbitsum(_p(x), depth, pa, pb, pw, pdims, _p(out), words, bits,
+                                                             int(pad_len), int(k), _p(ws), _stream(dev))
     if st == _lib.DL_ERR_TOO_LARGE:
-        return groupbitsum(eval(x, a, b, w), pad_len, k)
+        return groupbitsum(eval_fused(x, layers), pad_len, k)
     if st:
-        _raise(st, "logic_layer_cuda_eval_groupbitsum")
+        _raise(st, "logic_layer_cuda_eval_fused_groupbitsum")
     return out
 
 

@@ -5,22 +5,63 @@ import torch
 
 from . import difflogic_cuda
 
+# Inputs with at most this many rows stay resident in the L2 caches while a 1 KB column tile of
+# all neurons is swept, so gathers from them are cheap and deeper fusion pays off.
+_L2_RESIDENT_ROWS = 2048
+
+
+def plan_groups(dims, count_at_end):
+    """Splits consecutive layers into fused groups.
+
+    ``dims`` = [in_dim, width_1, ..., width_L].  Returns a list of group sizes summing to L; when
+    ``count_at_end`` the last group is the one fused with the bit count.  Chosen by dynamic
+    programming over a traffic model in units of one activation row: a group of depth D gathers
+    2^D rows per output neuron (from L2 when its input has few rows, through the memory fabric
+    otherwise) and writes one row per output neuron unless it ends in the count."""
+    n = len(dims) - 1
+    if n == 0:
+        return []
+
+    def cost(first, depth, last):
+        rows_in, out = dims[first], dims[first + depth]
+        gathers = (1 << depth) * out
+        written = 0 if (last and count_at_end) else out
+        if rows_in <= _L2_RESIDENT_ROWS:
+            t = max(gathers / 27.0, written / 5.6)
+        else:
+            t = max((gathers + written) / 7.9, (rows_in + written) / 5.0)
+        if last and count_at_end:
+            t *= 1.25                 # the vertical counters share the kernel
+        return t
+
+    best = [(0.0, [])] + [None] * n    # best[i] = (cost, groups) for the first i layers
+    for i in range(1, n + 1):
+        for depth in range(1, min(i, difflogic_cuda.MAX_FUSE_DEPTH) + 1):
+            last = i == n
+            if last and count_at_end and depth > difflogic_cuda.MAX_FUSE_DEPTH_COUNT:
+                continue
+            prev = best[i - depth]
+            c = prev[0] + cost(i - depth, depth, last)
+            if best[i] is None or c < best[i][0]:
+                best[i] = (c, prev[1] + [depth])
+    return best[n][1]
+
 
 class PackBitsTensor:
     """``.t`` is int{bit_count} [features, ceil(B / bit_count)]; bit i of word c of a row is
     sample ``bit_count*c + i``; ``.pad_len`` samples at the end of the last word are padding.
 
-    The most recent LogicLayer applied to the object is held back (``defer_layer``) until
-    ``.t`` is read or ``group_sum`` is called, so that a layer followed directly by GroupSum
-    runs as one fused kernel and its output words are never written to memory.  Reading
-    ``.t`` always returns the up-to-date words, as in the reference."""
+    Layers applied to the object are held back (``defer_layer``) until ``.t`` is read or
+    ``group_sum`` is called; consecutive layers are then evaluated in fused groups (and the last
+    group together with the bit count), so most intermediate activations never reach memory.
+    Reading ``.t`` always returns the up-to-date words, as in the reference."""
 
     def __init__(self, t: torch.BoolTensor, bit_count=32, device="cuda"):
         assert len(t.shape) == 2, t.shape
         self.bit_count = bit_count
         self.device = device
         self._t = None
-        self._pending = None          # (a, b, w) of a layer applied to _t but not yet evaluated
+        self._pending = []            # [(a, b, w)] applied to _t but not yet evaluated
         if device == "cuda":
             t = t.to(device)
             if t.dtype == torch.bool and t.is_contiguous():
@@ -32,33 +73,46 @@ class PackBitsTensor:
             raise NotImplementedError(device)
 
     @property
+    def features(self):
+        """Number of rows ``.t`` has (after the deferred layers)."""
+        return self._pending[-1][2].shape[0] if self._pending else self._t.shape[0]
+
+    def _dims(self):
+        return [self._t.shape[0]] + [w.shape[0] for _, _, w in self._pending]
+
+    def _run_groups(self, groups):
+        pos = 0
+        for depth in groups:
+            self._t = difflogic_cuda.eval_fused(self._t, self._pending[pos:pos + depth])
+            pos += depth
+        self._pending = self._pending[pos:]
+
+    @property
     def t(self):
-        if self._pending is not None:
-            a, b, w = self._pending
-            self._pending = None
-            self._t = difflogic_cuda.eval(self._t, a, b, w)
+        if self._pending:
+            self._run_groups(plan_groups(self._dims(), count_at_end=False))
         return self._t
 
     @t.setter
     def t(self, value):
-        self._pending = None
+        self._pending = []
         self._t = value
 
     def defer_layer(self, a, b, w):
-        """Applies the gate layer (a, b, w) lazily: evaluates any earlier deferred layer now and
-        holds this one back."""
-        self._t = self.t
-        self._pending = (a, b, w)
+        """Applies the gate layer (a, b, w) lazily."""
+        self._pending.append((a, b, w))
         return self
 
     def group_sum(self, k):
         assert self.device == "cuda", self.device
-        if self._pending is not None:
-            a, b, w = self._pending
-            if w.shape[0] % k != 0:
-                raise ValueError(f"in_dim ({w.shape[0]}) has to be divisible by k ({k}) but it is not")
-            return difflogic_cuda.eval_groupbitsum(self._t, a, b, w, self.pad_len, k)
-        return difflogic_cuda.groupbitsum(self.t, self.pad_len, k)
+        if self._pending:
+            if self.features % k != 0:
+                raise ValueError(f"in_dim ({self.features}) has to be divisible by k ({k}) but it is not")
+            groups = plan_groups(self._dims(), count_at_end=True)
+            self._run_groups(groups[:-1])
+            # the last group stays pending: the object's state does not change by counting
+            return difflogic_cuda.eval_fused_groupbitsum(self._t, self._pending, self.pad_len, k)
+        return difflogic_cuda.groupbitsum(self._t, self.pad_len, k)
 
     def flatten(self, start_dim=0, end_dim=-1, **kwargs):
         """Returns the object itself; the arguments are ignored."""

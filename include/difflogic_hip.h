@@ -118,16 +118,30 @@ int dl_tensor_packbits_batch_major(const uint8_t *x, void *out, int64_t batch, i
 int dl_groupbitsum(const void *b, int32_t *out, int64_t in_dim, int64_t words, int bit_count,
                    int64_t pad_len, int64_t k, void *stream);
 
-/* Fuses the last LogicLayer's `eval` with `groupbitsum` (the sequence
- * difflogic/difflogic.py:147 then difflogic/packbitstensor.py:22): the layer's output words are
- * counted as they are produced and never written.
- *   x [in_dim, words] words; a, b [out_dim]; w [out_dim] uint8 gate ids; k classes
- *   -> out [words*bit_count - pad_len, k] int32, identical to dl_groupbitsum(dl_logic_eval(x)).
- * Needs rows that are a whole number of 64-bit words (words*bit_count % 64 == 0) and k <= 65535;
- * otherwise returns DL_ERR_TOO_LARGE and the caller uses the two separate entry points. */
-int dl_logic_eval_groupbitsum(const void *x, const int64_t *a, const int64_t *b, const uint8_t *w,
-                              int32_t *out, int64_t in_dim, int64_t out_dim, int64_t words,
-                              int bit_count, int64_t pad_len, int64_t k, void *stream);
+/* Fused evaluation of `depth` (1..4) consecutive layers: same result as `depth` calls of
+ * dl_logic_eval (the loop difflogic/difflogic.py:147 runs once per layer), but the intermediate
+ * activations are never written: every output neuron is evaluated as a depth-`depth` tree of gates
+ * over 2^depth gathered rows of x.  No counterpart in the reference.
+ *   a, b, w   HOST arrays of `depth` DEVICE pointers, [0] = the group's first layer
+ *   dims      HOST array {in_dim, width of layer 0, ..., width of layer depth-1}
+ *   x [in_dim, words] -> y [dims[depth], words]
+ *   workspace DEVICE scratch of dl_logic_eval_fused_workspace_bytes(depth, dims[depth]) bytes,
+ *             8-byte aligned (holds the flattened per-neuron wiring; rebuilt by every call).
+ * Rows must be whole 64-bit words (words*bit_count % 64 == 0, 8-byte aligned buffers); otherwise
+ * DL_ERR_TOO_LARGE is returned and the caller evaluates layer by layer. */
+int64_t dl_logic_eval_fused_workspace_bytes(int depth, int64_t out_dim);
+int dl_logic_eval_fused(const void *x, int depth, const int64_t *const *a, const int64_t *const *b,
+                        const uint8_t *const *w, const int64_t *dims, void *y, int64_t words,
+                        int bit_count, void *workspace, void *stream);
+
+/* The net's last `depth` (1 or 2) layers fused with `groupbitsum` (the sequence
+ * difflogic/difflogic.py:147 then difflogic/packbitstensor.py:22): the last layer's output words
+ * are counted as they are produced and never written.  Arguments as dl_logic_eval_fused, result
+ * as dl_groupbitsum: out [words*bit_count - pad_len, k] int32.  Also needs k <= 65535. */
+int dl_logic_eval_fused_groupbitsum(const void *x, int depth, const int64_t *const *a,
+                                    const int64_t *const *b, const uint8_t *const *w,
+                                    const int64_t *dims, int32_t *out, int64_t words, int bit_count,
+                                    int64_t pad_len, int64_t k, void *workspace, void *stream);
 
 #ifdef __cplusplus
 }

@@ -201,22 +201,65 @@ def test_pack_tensor_repr_and_modes():
         dl.PackBitsTensor(t, device="cpu")
 
 
-@pytest.mark.parametrize("bits,in_dim,out_dim,W,k,pad", [
-    (64, 30, 60, 1, 3, 0), (64, 50, 640, 70, 10, 63), (64, 33, 130, 129, 2, 1), (32, 20, 64, 6, 4, 3),
-    (16, 20, 40, 12, 5, 0), (8, 12, 24, 16, 3, 2), (8, 12, 24, 9, 3, 7), (64, 100, 40000, 2, 2, 11),
-    (64, 64, 70000, 1, 1, 0), (32, 20, 64, 5, 4, 3),
+def _chain(rng, in_dim, widths):
+    layers = random_layers(rng, in_dim, widths)
+    return layers, [tuple(_dev(t) for t in l) for l in layers]
+
+
+@pytest.mark.parametrize("bits,in_dim,widths,W", [
+    (64, 30, [60], 3), (64, 30, [60, 50], 1), (64, 50, [64, 70, 40], 70), (64, 33, [130, 90, 100, 77], 129),
+    (32, 20, [64, 64], 6), (32, 20, [64, 64, 64], 5), (16, 20, [40, 30], 12), (8, 12, [24, 24, 24, 24], 16),
+    (8, 12, [24, 30], 9), (64, 784, [4000, 4000, 4000, 4000], 40), (64, 3000, [3000, 3000], 64),
 ])
-def test_fused_eval_groupbitsum(ext, bits, in_dim, out_dim, W, k, pad):
-    rng = np.random.default_rng(in_dim + W + k + out_dim)
+def test_eval_fused_equals_layer_by_layer(ext, bits, in_dim, widths, W):
+    rng = np.random.default_rng(in_dim + W + len(widths))
     x = rng.integers(np.iinfo(NP_WORD[bits]).min, np.iinfo(NP_WORD[bits]).max, (in_dim, W), dtype=NP_WORD[bits],
                      endpoint=True)
-    (a, b, op), = random_layers(rng, in_dim, [out_dim])
-    want = po.groupbitsum(po.eval_layer(x, a, b, op), pad, k)
-    got = ext.eval_groupbitsum(_dev(x), _dev(a), _dev(b), _dev(op), pad, k)
+    layers, dev_layers = _chain(rng, in_dim, widths)
+    want = x
+    for a, b, op in layers:
+        want = po.eval_layer(want, a, b, op)
+    got = ext.eval_fused(_dev(x), dev_layers)
+    assert got.dtype == torch.as_tensor(want).dtype and tuple(got.shape) == want.shape
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
+def test_eval_fused_every_gate_combination(ext):
+    # depth 2 over the four input pairs: 16^3 gate triples, one output neuron each
+    t = np.array([[0, 0, 1, 1], [0, 1, 0, 1]], dtype=bool)
+    x, _ = po.packbits(t, 64)
+    g1, g2, g3 = np.meshgrid(np.arange(16), np.arange(16), np.arange(16), indexing="ij")
+    l1 = (np.zeros(256, np.int64), np.ones(256, np.int64), np.arange(256) // 16 % 16)          # 256 first-layer gates
+    l1 = (np.zeros(32, np.int64), np.ones(32, np.int64), (np.arange(32) % 16).astype(np.uint8))
+    a2 = g1.reshape(-1).astype(np.int64)
+    b2 = (16 + g2.reshape(-1)).astype(np.int64)
+    l2 = (a2, b2, g3.reshape(-1).astype(np.uint8))
+    want = po.eval_layer(po.eval_layer(x, *l1), *l2)
+    got = ext.eval_fused(_dev(x), [tuple(_dev(v) for v in l1), tuple(_dev(v) for v in l2)])
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("bits,in_dim,widths,W,k,pad", [
+    (64, 30, [60], 1, 3, 0), (64, 50, [640], 70, 10, 63), (64, 33, [130], 129, 2, 1), (32, 20, [64], 6, 4, 3),
+    (16, 20, [40], 12, 5, 0), (8, 12, [24], 16, 3, 2), (8, 12, [24], 9, 3, 7), (64, 100, [40000], 2, 2, 11),
+    (64, 64, [70000], 1, 1, 0), (32, 20, [64], 5, 4, 3),
+    (64, 30, [60, 90], 1, 3, 0), (64, 50, [100, 640], 70, 10, 63), (64, 33, [66, 130], 129, 2, 1),
+    (32, 20, [40, 64], 6, 4, 3), (8, 12, [24, 24], 9, 3, 7), (64, 100, [200, 40000], 2, 2, 11),
+    (64, 784, [8000, 8000], 33, 10, 5),
+])
+def test_fused_eval_groupbitsum(ext, bits, in_dim, widths, W, k, pad):
+    rng = np.random.default_rng(in_dim + W + k + widths[-1])
+    x = rng.integers(np.iinfo(NP_WORD[bits]).min, np.iinfo(NP_WORD[bits]).max, (in_dim, W), dtype=NP_WORD[bits],
+                     endpoint=True)
+    layers, dev_layers = _chain(rng, in_dim, widths)
+    y = x
+    for a, b, op in layers:
+        y = po.eval_layer(y, a, b, op)
+    want = po.groupbitsum(y, pad, k)
+    got = ext.eval_fused_groupbitsum(_dev(x), dev_layers, pad, k)
     assert got.dtype == torch.int32 and tuple(got.shape) == want.shape
     assert np.array_equal(got.cpu().numpy(), want)
-    two_step = ext.groupbitsum(ext.eval(_dev(x), _dev(a), _dev(b), _dev(op)), pad, k)
-    assert torch.equal(got, two_step)
+    assert torch.equal(got, ext.groupbitsum(ext.eval_fused(_dev(x), dev_layers), pad, k))
 
 
 def test_lazy_pack_tensor_keeps_t_current():

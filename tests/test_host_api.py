@@ -107,3 +107,17 @@ def test_packbits_tensor_is_gpu_only():
             pass
     with pytest.raises(AssertionError):
         layer(Fake())                                        # packed inference needs device='cuda'
+
+
+def test_group_planner():
+    from difflogic_amd.packbitstensor import plan_groups
+    for dims, count in [([784] + [64000] * 6, True), ([784] + [8000] * 6, False), ([9216] + [256000] * 4, True),
+                        ([100, 200], True), ([100, 200, 300, 400, 500, 600, 700, 800, 900], True), ([5, 5], False)]:
+        groups = plan_groups(dims, count)
+        assert sum(groups) == len(dims) - 1 and all(1 <= g <= 4 for g in groups)
+        if count:
+            assert groups[-1] <= 2
+    assert plan_groups([7], True) == []
+    # a wide net over few inputs: deep first group (its gathers hit in L2), pairs afterwards
+    assert plan_groups([784] + [64000] * 6, True) == [4, 2]
+    assert plan_groups([64000] * 5, False) == [2, 2]
