@@ -352,41 +352,53 @@ __global__ __launch_bounds__(DL_BLOCK) void packbits_batch_major_kernel(const ui
 // Vertical bit count (GroupSum on packed words).  For each class (a contiguous block of
 // per_class neuron rows) and each sample bit, the number of rows with that bit set.
 //
-// Lanes run along 64-bit word columns (coalesced row reads); each wave takes a quarter of the
-// class's rows and keeps bit-sliced counters: 16 rows at a time are compressed by a
-// carry-save-adder tree into planes of weight 1, 2, 4, 8 and a carry of weight 16 that is
-// rippled into NPH higher planes.  The four waves' planes are exchanged through LDS, each
-// wave expands 16 of the 64 sample bits to integers, and the [column][sample] tile is written
-// out with lanes along samples.
-// ------------------------------------------------------------------------------------------
-
-__device__ __forceinline__ void csa(uint64_t &carry, uint64_t &sum, uint64_t a, uint64_t b, uint64_t c) {
-    const uint64_t u = a ^ b;
-    carry = (a & b) | (u & c);
-    sum = u ^ c;
-}
-
+// Lanes run along vectors V of the rows (16 bytes = 128 samples per lane where the row length
+// allows it, else 8 bytes); each wave takes a quarter of the class's rows and keeps bit-sliced
+// counters per lane: 16 rows at a time are compressed by a carry-save-adder tree into planes of
+// weight 1, 2, 4, 8 and a carry of weight 16 that is rippled into NPH higher planes.  The four
+// waves' planes are exchanged through LDS and each wave expands a quarter of every lane's sample
+// bits to integers and stores them.
 //
 // TREE > 0: the counted rows are not read but computed on the fly as the last TREE layers of the
 // net over the rows of `bits` (= the input of those layers), from the composites that
 // compose_tree_kernel writes; the output of the last layer never exists in memory.
-template <int NPH, int TREE>
-__global__ __launch_bounds__(DL_BLOCK) void groupbitsum_kernel(const uint64_t *__restrict__ bits,
+// ------------------------------------------------------------------------------------------
+
+template <typename V> __device__ __forceinline__ void csa(V &carry, V &sum, V a, V b, V c) {
+    const V u = a ^ b;
+    carry = (a & b) | (u & c);
+    sum = u ^ c;
+}
+
+template <typename V> struct Words;        // access to the 32-bit components of a vector
+template <> struct Words<uint64_t> {
+    static constexpr int n = 2;
+    static __device__ __forceinline__ uint32_t get(uint64_t v, int c) { return (uint32_t) (v >> (32 * c)); }
+    static __device__ __forceinline__ uint64_t zero() { return 0; }
+};
+template <> struct Words<dl_u32x4> {
+    static constexpr int n = 4;
+    static __device__ __forceinline__ uint32_t get(dl_u32x4 v, int c) { return v[c]; }
+    static __device__ __forceinline__ dl_u32x4 zero() { return dl_u32x4{0, 0, 0, 0}; }
+};
+
+template <typename V, int NPH, int TREE>
+__global__ __launch_bounds__(DL_BLOCK) void groupbitsum_kernel(const V *__restrict__ bits,
                                                                const int32_t *__restrict__ leaves,
                                                                const uint64_t *__restrict__ gates,
-                                                               int32_t *__restrict__ out, int64_t words,
+                                                               int32_t *__restrict__ out, int64_t ncols,
                                                                int64_t per_class, int64_t k, int64_t batch) {
     constexpr int NP = NPH + 4;
     constexpr int G = 1 << TREE;
-    __shared__ uint64_t planes_lds[4][NP][DL_WAVE];
-    __shared__ int32_t tile[DL_WAVE][DL_WAVE + 1];   // [column][sample], padded against bank conflicts
+    constexpr int NC = Words<V>::n;              // 32-bit components per lane
+    constexpr int BITS = 8 * NC;                 // sample bits of a lane that one wave expands
+    __shared__ uint32_t planes_lds[4][NP][NC][DL_WAVE];
 
     const int wave = dl_wave_in_block();
     const int lane = dl_lane();
     const int64_t cls = blockIdx.y;
-    const int64_t c0 = (int64_t) blockIdx.x * DL_WAVE;
-    const int64_t col = c0 + lane;
-    const bool live = col < words;
+    const int64_t col = (int64_t) blockIdx.x * DL_WAVE + lane;
+    const bool live = col < ncols;
 
     const int64_t chunk = (per_class + 3) / 4;
     int64_t r_begin = (int64_t) wave * chunk;
@@ -394,96 +406,96 @@ __global__ __launch_bounds__(DL_BLOCK) void groupbitsum_kernel(const uint64_t *_
     int64_t r_end = r_begin + chunk;
     if (r_end > per_class) r_end = per_class;
 
-    uint64_t ones = 0, twos = 0, fours = 0, eights = 0;
-    uint64_t high[NPH];
+    V ones = Words<V>::zero(), twos = ones, fours = ones, eights = ones;
+    V high[NPH];
 #pragma unroll
-    for (int p = 0; p < NPH; ++p) high[p] = 0;
+    for (int p = 0; p < NPH; ++p) high[p] = Words<V>::zero();
 
-    const uint64_t *row = bits + (cls * per_class + r_begin) * words + (live ? col : 0);
-    const uint64_t *xcol = bits + (live ? col : 0);
-    for (int64_t r = r_begin; r < r_end; r += 16) {
-        uint64_t v[16];
+    const V *row = bits + (cls * per_class + r_begin) * ncols + (live ? col : 0);
+    const V *xcol = bits + (live ? col : 0);
+
+    // Four rows at a time: fetch (or compute) them, compress them to one vector of weight 4.
+    auto quad = [&](int64_t q0) -> V {
+        V v[4];
         if (TREE == 0) {
 #pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                v[j] = (live && r + j < r_end) ? __builtin_nontemporal_load(row + (int64_t) j * words) : 0;
-            }
-            row += 16 * words;
+            for (int j = 0; j < 4; ++j)
+                v[j] = (live && q0 + j < r_end) ? __builtin_nontemporal_load(row + (q0 - r_begin + j) * ncols)
+                                                : Words<V>::zero();
         } else {
-            constexpr int SUB = (TREE == 1) ? 16 : 8;        // neurons whose leaves are in flight together
+            V leaf[4][G];
+            uint64_t gt[4];
 #pragma unroll
-            for (int h = 0; h < 16; h += SUB) {
-                uint64_t leaf[SUB][G];
-                uint64_t gt[SUB];
+            for (int j = 0; j < 4; ++j) {
+                const int64_t n = cls * per_class + ((q0 + j < r_end) ? q0 + j : r_end - 1);
+                gt[j] = gates[n];
 #pragma unroll
-                for (int j = 0; j < SUB; ++j) {
-                    const int64_t n = cls * per_class + ((r + h + j < r_end) ? r + h + j : r_end - 1);
-                    gt[j] = gates[n];
+                for (int g = 0; g < G; ++g)
+                    leaf[j][g] = live ? xcol[(int64_t) leaves[n * G + g] * ncols] : Words<V>::zero();
+            }
 #pragma unroll
-                    for (int g = 0; g < G; ++g) leaf[j][g] = live ? xcol[(int64_t) leaves[n * G + g] * words] : 0;
-                }
-#pragma unroll
-                for (int j = 0; j < SUB; ++j) {
-                    const uint64_t y = TreeFold<uint64_t, TREE>::run(leaf[j], gt[j]);
-                    v[h + j] = (live && r + h + j < r_end) ? y : 0;
-                }
+            for (int j = 0; j < 4; ++j) {
+                const V y = TreeFold<V, TREE>::run(leaf[j], gt[j]);
+                v[j] = (live && q0 + j < r_end) ? y : Words<V>::zero();
             }
         }
-        uint64_t t2a, t2b, t4a, t4b, t8a, t8b, t16;
+        V t2a, t2b, t4;
         csa(t2a, ones, ones, v[0], v[1]);
         csa(t2b, ones, ones, v[2], v[3]);
-        csa(t4a, twos, twos, t2a, t2b);
-        csa(t2a, ones, ones, v[4], v[5]);
-        csa(t2b, ones, ones, v[6], v[7]);
-        csa(t4b, twos, twos, t2a, t2b);
-        csa(t8a, fours, fours, t4a, t4b);
-        csa(t2a, ones, ones, v[8], v[9]);
-        csa(t2b, ones, ones, v[10], v[11]);
-        csa(t4a, twos, twos, t2a, t2b);
-        csa(t2a, ones, ones, v[12], v[13]);
-        csa(t2b, ones, ones, v[14], v[15]);
-        csa(t4b, twos, twos, t2a, t2b);
-        csa(t8b, fours, fours, t4a, t4b);
+        csa(t4, twos, twos, t2a, t2b);
+        return t4;
+    };
+    for (int64_t r = r_begin; r < r_end; r += 16) {
+        V t8a, t8b, t16;
+        {
+            const V t4a = quad(r), t4b = quad(r + 4);
+            csa(t8a, fours, fours, t4a, t4b);
+        }
+        {
+            const V t4a = quad(r + 8), t4b = quad(r + 12);
+            csa(t8b, fours, fours, t4a, t4b);
+        }
         csa(t16, eights, eights, t8a, t8b);
 #pragma unroll
         for (int p = 0; p < NPH; ++p) {
-            const uint64_t old = high[p];
+            const V old = high[p];
             high[p] = old ^ t16;
             t16 = old & t16;
         }
     }
 
-    planes_lds[wave][0][lane] = ones;
-    planes_lds[wave][1][lane] = twos;
-    planes_lds[wave][2][lane] = fours;
-    planes_lds[wave][3][lane] = eights;
 #pragma unroll
-    for (int p = 0; p < NPH; ++p) planes_lds[wave][4 + p][lane] = high[p];
+    for (int c = 0; c < NC; ++c) {
+        planes_lds[wave][0][c][lane] = Words<V>::get(ones, c);
+        planes_lds[wave][1][c][lane] = Words<V>::get(twos, c);
+        planes_lds[wave][2][c][lane] = Words<V>::get(fours, c);
+        planes_lds[wave][3][c][lane] = Words<V>::get(eights, c);
+#pragma unroll
+        for (int p = 0; p < NPH; ++p) planes_lds[wave][4 + p][c][lane] = Words<V>::get(high[p], c);
+    }
     __syncthreads();
 
-    // This wave expands sample bits [16*wave, 16*wave + 16) of every column.
-    int32_t cnt[16];
+    // This wave expands bits [BITS*wave, BITS*wave + BITS) of every lane's 32*NC sample bits
+    // (kept rolled: this phase must not set the kernel's register budget, the main loop does).
+    int32_t cnt[BITS];
 #pragma unroll
-    for (int s = 0; s < 16; ++s) cnt[s] = 0;
-    const int shift = 16 * wave;
+    for (int s = 0; s < BITS; ++s) cnt[s] = 0;
+    const int first_bit = BITS * wave;
+    const int comp = first_bit >> 5, shift = first_bit & 31;
+#pragma unroll 1
     for (int q = 0; q < 4; ++q) {
-#pragma unroll
+#pragma unroll 1
         for (int p = 0; p < NP; ++p) {
-            const uint32_t slice = (uint32_t) (planes_lds[q][p][lane] >> shift) & 0xffffu;
+            const uint32_t slice = planes_lds[q][p][comp][lane] >> shift;
 #pragma unroll
-            for (int s = 0; s < 16; ++s) cnt[s] += (int32_t) (((slice >> s) & 1u) << p);
+            for (int s = 0; s < BITS; ++s) cnt[s] += (int32_t) (((slice >> s) & 1u) << p);
         }
     }
+    if (live) {
+        const int64_t sample0 = col * (32 * NC) + first_bit;
 #pragma unroll
-    for (int s = 0; s < 16; ++s) tile[lane][shift + s] = cnt[s];
-    __syncthreads();
-
-    // Lanes along samples: thread t writes sample (t % 64) of columns t/64, t/64 + 4, ...
-    const int s = lane;
-    for (int cc = wave; cc < DL_WAVE; cc += 4) {
-        const int64_t c = c0 + cc;
-        const int64_t sample = c * 64 + s;
-        if (c < words && sample < batch) out[sample * k + cls] = tile[cc][s];
+        for (int s = 0; s < BITS; ++s)
+            if (sample0 + s < batch) out[(sample0 + s) * k + cls] = cnt[s];
     }
 }
 
@@ -504,20 +516,33 @@ __global__ __launch_bounds__(DL_BLOCK) void groupbitsum_generic_kernel(const uin
     }
 }
 
-template <int TREE>
-void launch_groupbitsum(const uint64_t *bits, const int32_t *leaves, const uint64_t *gates, int32_t *out,
-                        int64_t words64, int64_t per_class, int64_t k, int64_t batch, dim3 grid, hipStream_t s) {
+template <typename V, int TREE>
+void launch_groupbitsum_v(const void *bits, const int32_t *leaves, const uint64_t *gates, int32_t *out, int64_t row_bytes,
+                          int64_t per_class, int64_t k, int64_t batch, hipStream_t s) {
+    const int64_t ncols = row_bytes / (int64_t) sizeof(V);
+    const dim3 grid((unsigned) dl_ceil_div(ncols, DL_WAVE), (unsigned) k);
     const int64_t chunk = (per_class + 3) / 4;      // rows one wave counts
+    const V *b = (const V *) bits;
     // NPH planes above weight 8 hold counts up to 16 * 2^NPH - 1.
     if (chunk < (16LL << 8))
-        hipLaunchKernelGGL((groupbitsum_kernel<8, TREE>), grid, dim3(DL_BLOCK), 0, s, bits, leaves, gates, out, words64,
+        hipLaunchKernelGGL((groupbitsum_kernel<V, 8, TREE>), grid, dim3(DL_BLOCK), 0, s, b, leaves, gates, out, ncols,
                            per_class, k, batch);
     else if (chunk < (16LL << 14))
-        hipLaunchKernelGGL((groupbitsum_kernel<14, TREE>), grid, dim3(DL_BLOCK), 0, s, bits, leaves, gates, out, words64,
+        hipLaunchKernelGGL((groupbitsum_kernel<V, 14, TREE>), grid, dim3(DL_BLOCK), 0, s, b, leaves, gates, out, ncols,
                            per_class, k, batch);
     else
-        hipLaunchKernelGGL((groupbitsum_kernel<27, TREE>), grid, dim3(DL_BLOCK), 0, s, bits, leaves, gates, out, words64,
+        hipLaunchKernelGGL((groupbitsum_kernel<V, 27, TREE>), grid, dim3(DL_BLOCK), 0, s, b, leaves, gates, out, ncols,
                            per_class, k, batch);
+}
+
+// Rows of whole 64-bit words, 8-byte aligned: 16-byte lanes where rows and base allow it.
+template <int TREE>
+void launch_groupbitsum(const void *bits, const int32_t *leaves, const uint64_t *gates, int32_t *out, int64_t row_bytes,
+                        int64_t per_class, int64_t k, int64_t batch, hipStream_t s) {
+    if (row_bytes % 16 == 0 && dl_aligned(bits, 16))
+        launch_groupbitsum_v<dl_u32x4, TREE>(bits, leaves, gates, out, row_bytes, per_class, k, batch, s);
+    else
+        launch_groupbitsum_v<uint64_t, TREE>(bits, leaves, gates, out, row_bytes, per_class, k, batch, s);
 }
 
 // Validates the description of a fused group and launches the composite builder.
@@ -663,11 +688,8 @@ extern "C" int dl_groupbitsum(const void *b, int32_t *out, int64_t in_dim, int64
     if (per_class > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
 
     if (row_bytes % 8 == 0 && dl_aligned(b, 8) && k <= 65535) {
-        const int64_t words64 = row_bytes / 8;
-        const int64_t gx = dl_ceil_div(words64, DL_WAVE);
-        if (gx > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
-        const dim3 grid((unsigned) gx, (unsigned) k);
-        launch_groupbitsum<0>((const uint64_t *) b, nullptr, nullptr, out, words64, per_class, k, batch, grid, s);
+        if (dl_ceil_div(row_bytes / 8, DL_WAVE) > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+        launch_groupbitsum<0>(b, nullptr, nullptr, out, row_bytes, per_class, k, batch, s);
     } else {
         int64_t gx = dl_ceil_div(batch, DL_BLOCK);
         if (gx > 0x7fffffffLL) gx = 0x7fffffffLL;
@@ -718,18 +740,15 @@ extern "C" int dl_logic_eval_fused_groupbitsum(const void *x, int depth, const i
     const int64_t per_class = out_dim / k;
     const int64_t row_bytes = words * (bit_count / 8);
     if (row_bytes % 8 != 0 || !dl_aligned(x, 8) || k > 65535 || per_class > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
-    const int64_t words64 = row_bytes / 8;
-    const int64_t gx = dl_ceil_div(words64, DL_WAVE);
-    if (gx > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    if (dl_ceil_div(row_bytes / 8, DL_WAVE) > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     hipStream_t s = (hipStream_t) stream;
     int32_t *leaves;
     uint64_t *gates;
     const int st = compose_tree(depth, a, b, w, dims, workspace, &leaves, &gates, s);
     if (st != DL_OK) return st;
-    const dim3 grid((unsigned) gx, (unsigned) k);
     if (depth == 1)
-        launch_groupbitsum<1>((const uint64_t *) x, leaves, gates, out, words64, per_class, k, batch, grid, s);
+        launch_groupbitsum<1>(x, leaves, gates, out, row_bytes, per_class, k, batch, s);
     else
-        launch_groupbitsum<2>((const uint64_t *) x, leaves, gates, out, words64, per_class, k, batch, grid, s);
+        launch_groupbitsum<2>(x, leaves, gates, out, row_bytes, per_class, k, batch, s);
     return dl_launch_status();
 }
