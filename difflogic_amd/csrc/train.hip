@@ -406,17 +406,25 @@ __global__ __launch_bounds__(DL_BLOCK) void group_sum_partial_kernel(const T *__
     }
 }
 
+// One wave per 64 consecutive samples of one class; the four waves of a workgroup take
+// interleaved splits and are added in wave order, so the summation order is fixed.
 template <typename T>
 __global__ __launch_bounds__(DL_BLOCK) void group_sum_finish_kernel(const typename Acc<T>::type *__restrict__ partial,
                                                                     T *__restrict__ y, int64_t batch, int64_t k,
                                                                     int splits, typename Acc<T>::type inv_tau) {
     typedef typename Acc<T>::type C;
-    const int64_t i = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x;     // i = r * k + c
-    if (i >= batch * k) return;
-    const int64_t r = i / k, c = i - r * k;
+    __shared__ C lds[4][DL_WAVE];
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t r = (int64_t) blockIdx.x * DL_WAVE + lane;
+    const int64_t c = blockIdx.y;
     C sum = (C) 0;
-    for (int s = 0; s < splits; ++s) sum += partial[((int64_t) s * k + c) * batch + r];
-    y[i] = down<T, C>(sum * inv_tau);
+    if (r < batch)
+        for (int s = wave; s < splits; s += 4) sum += partial[((int64_t) s * k + c) * batch + r];
+    lds[wave][lane] = sum;
+    __syncthreads();
+    if (wave == 0 && r < batch)
+        y[r * k + c] = down<T, C>(((lds[0][lane] + lds[1][lane]) + (lds[2][lane] + lds[3][lane])) * inv_tau);
 }
 
 template <typename T, int VEC>
@@ -466,10 +474,10 @@ int group_sum_forward_t(const void *x, void *y, void *workspace, int64_t out_dim
                            per_class, ncols, k, rows_per_split);
     int st = dl_launch_status();
     if (st != DL_OK) return st;
-    const int64_t blocks = dl_ceil_div(batch * k, DL_BLOCK);
+    const int64_t blocks = dl_ceil_div(batch, DL_WAVE);
     if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
-    hipLaunchKernelGGL((group_sum_finish_kernel<T>), dim3((unsigned) blocks), dim3(DL_BLOCK), 0, s, (const C *) workspace,
-                       (T *) y, batch, k, splits, (C) (1.0 / tau));
+    hipLaunchKernelGGL((group_sum_finish_kernel<T>), dim3((unsigned) blocks, (unsigned) k), dim3(DL_BLOCK), 0, s,
+                       (const C *) workspace, (T *) y, batch, k, splits, (C) (1.0 / tau));
     return dl_launch_status();
 }
 
@@ -495,7 +503,7 @@ int group_sum_backward_t(const void *g, void *gx, int64_t out_dim, int64_t batch
 int group_sum_splits(int64_t out_dim, int64_t batch, int64_t k) {
     const int64_t per_class = out_dim / k;
     const int64_t col_tiles = dl_ceil_div(batch, 4 * DL_WAVE);
-    int64_t want = dl_ceil_div(2048, col_tiles * k);
+    int64_t want = dl_ceil_div(1024, col_tiles * k);
     const int64_t max_by_rows = per_class / 64 > 0 ? per_class / 64 : 1;
     if (want > max_by_rows) want = max_by_rows;
     if (want < 1) want = 1;
