@@ -382,16 +382,55 @@ template <> struct Words<dl_u32x4> {
     static __device__ __forceinline__ dl_u32x4 zero() { return dl_u32x4{0, 0, 0, 0}; }
 };
 
-template <typename V, int NPH, int TREE>
-__global__ __launch_bounds__(DL_BLOCK) void groupbitsum_kernel(const V *__restrict__ bits,
-                                                               const int32_t *__restrict__ leaves,
-                                                               const uint64_t *__restrict__ gates,
-                                                               int32_t *__restrict__ out, int64_t ncols,
-                                                               int64_t per_class, int64_t k, int64_t batch) {
+// Expands bit-sliced counters to integers and stores them: planes[q][p][c][lane] is component c
+// of plane p (weight 2^p) of partial counter q for the lane's vector; the workgroup's wave w
+// handles bits [BITS*w, BITS*w + BITS) of the lane's 32*NC sample bits, summing the NQ partials.
+// (Kept rolled: this phase must not set the kernel's register budget.)
+template <typename V, int NP, int NQ>
+__device__ __forceinline__ void expand_counts(const uint32_t (*planes)[NP][Words<V>::n][DL_WAVE], int wave, int lane,
+                                              int64_t col, bool live, int64_t cls, int64_t k, int64_t batch,
+                                              int32_t *__restrict__ out) {
+    constexpr int NC = Words<V>::n;
+    constexpr int BITS = 8 * NC;
+    int32_t cnt[BITS];
+#pragma unroll
+    for (int s = 0; s < BITS; ++s) cnt[s] = 0;
+    const int first_bit = BITS * wave;
+    const int comp = first_bit >> 5, shift = first_bit & 31;
+#pragma unroll 1
+    for (int q = 0; q < NQ; ++q) {
+#pragma unroll 1
+        for (int p = 0; p < NP; ++p) {
+            const uint32_t slice = planes[q][p][comp][lane] >> shift;
+#pragma unroll
+            for (int s = 0; s < BITS; ++s) cnt[s] += (int32_t) (((slice >> s) & 1u) << p);
+        }
+    }
+    if (live) {
+        const int64_t sample0 = col * (32 * NC) + first_bit;
+#pragma unroll
+        for (int s = 0; s < BITS; ++s)
+            if (sample0 + s < batch) out[(sample0 + s) * k + cls] = cnt[s];
+    }
+}
+
+// Four vectors -> one vector of weight 4, through the running planes of weight 1 and 2.
+template <typename V> __device__ __forceinline__ V csa_quad(V &ones, V &twos, const V *v) {
+    V t2a, t2b, t4;
+    csa(t2a, ones, ones, v[0], v[1]);
+    csa(t2b, ones, ones, v[2], v[3]);
+    csa(t4, twos, twos, t2a, t2b);
+    return t4;
+}
+
+// Single pass over stored rows: blockIdx.x = column tile, blockIdx.y = class; every row is read
+// exactly once, so the dispatch order does not matter for cache reuse.
+template <typename V, int NPH>
+__global__ __launch_bounds__(DL_BLOCK) void groupbitsum_kernel(const V *__restrict__ bits, int32_t *__restrict__ out,
+                                                               int64_t ncols, int64_t per_class, int64_t k,
+                                                               int64_t batch) {
     constexpr int NP = NPH + 4;
-    constexpr int G = 1 << TREE;
-    constexpr int NC = Words<V>::n;              // 32-bit components per lane
-    constexpr int BITS = 8 * NC;                 // sample bits of a lane that one wave expands
+    constexpr int NC = Words<V>::n;
     __shared__ uint32_t planes_lds[4][NP][NC][DL_WAVE];
 
     const int wave = dl_wave_in_block();
@@ -412,38 +451,13 @@ __global__ __launch_bounds__(DL_BLOCK) void groupbitsum_kernel(const V *__restri
     for (int p = 0; p < NPH; ++p) high[p] = Words<V>::zero();
 
     const V *row = bits + (cls * per_class + r_begin) * ncols + (live ? col : 0);
-    const V *xcol = bits + (live ? col : 0);
-
-    // Four rows at a time: fetch (or compute) them, compress them to one vector of weight 4.
     auto quad = [&](int64_t q0) -> V {
         V v[4];
-        if (TREE == 0) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                v[j] = (live && q0 + j < r_end) ? __builtin_nontemporal_load(row + (q0 - r_begin + j) * ncols)
-                                                : Words<V>::zero();
-        } else {
-            V leaf[4][G];
-            uint64_t gt[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int64_t n = cls * per_class + ((q0 + j < r_end) ? q0 + j : r_end - 1);
-                gt[j] = gates[n];
-#pragma unroll
-                for (int g = 0; g < G; ++g)
-                    leaf[j][g] = live ? xcol[(int64_t) leaves[n * G + g] * ncols] : Words<V>::zero();
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const V y = TreeFold<V, TREE>::run(leaf[j], gt[j]);
-                v[j] = (live && q0 + j < r_end) ? y : Words<V>::zero();
-            }
-        }
-        V t2a, t2b, t4;
-        csa(t2a, ones, ones, v[0], v[1]);
-        csa(t2b, ones, ones, v[2], v[3]);
-        csa(t4, twos, twos, t2a, t2b);
-        return t4;
+        for (int j = 0; j < 4; ++j)
+            v[j] = (live && q0 + j < r_end) ? __builtin_nontemporal_load(row + (q0 - r_begin + j) * ncols)
+                                            : Words<V>::zero();
+        return csa_quad(ones, twos, v);
     };
     for (int64_t r = r_begin; r < r_end; r += 16) {
         V t8a, t8b, t16;
@@ -474,29 +488,161 @@ __global__ __launch_bounds__(DL_BLOCK) void groupbitsum_kernel(const V *__restri
         for (int p = 0; p < NPH; ++p) planes_lds[wave][4 + p][c][lane] = Words<V>::get(high[p], c);
     }
     __syncthreads();
+    expand_counts<V, NP, 4>(planes_lds, wave, lane, col, live, cls, k, batch, out);
+}
 
-    // This wave expands bits [BITS*wave, BITS*wave + BITS) of every lane's 32*NC sample bits
-    // (kept rolled: this phase must not set the kernel's register budget, the main loop does).
-    int32_t cnt[BITS];
+// ------------------------------------------------------------------------------------------
+// Count fused with the net's last TREE layers, in two passes so that the gathers keep their
+// cache reuse.  A gathered input row is used by several neurons of every class; the reuse only
+// hits the Infinity Cache if the chip works on few 1 KB column tiles at a time, i.e. if the
+// dispatch is column-tile-major like eval_tree_kernel's, with all classes of a tile together.
+//   pass 1: blockIdx.x = chunk of COUNT_ROWS neurons of one class, blockIdx.y = column tile.
+//           The workgroup computes its neurons' output vectors (never stored), counts them
+//           bit-sliced (32 per wave -> 6 planes, four waves added -> 8 planes) and writes the
+//           planes: 8 vectors per lane per 128 neurons instead of 128 output vectors.
+//   pass 2: blockIdx.x = column tile, blockIdx.y = class: adds the chunks' planes bit-sliced,
+//           expands them to integers and stores the counts.
+// ------------------------------------------------------------------------------------------
+#define DL_COUNT_ROWS 128     // neurons per workgroup in pass 1 (32 per wave)
+#define DL_COUNT_PLANES 8     // planes a workgroup writes: counts 0 .. 128
+
+// a + b for bit-sliced numbers: a has NA planes, b NB <= NA planes; result NA + 1 planes in a.
+template <typename V, int NA, int NB> __device__ __forceinline__ void sliced_add(V *a, const V *b) {
+    V carry = Words<V>::zero();
 #pragma unroll
-    for (int s = 0; s < BITS; ++s) cnt[s] = 0;
-    const int first_bit = BITS * wave;
-    const int comp = first_bit >> 5, shift = first_bit & 31;
-#pragma unroll 1
-    for (int q = 0; q < 4; ++q) {
-#pragma unroll 1
-        for (int p = 0; p < NP; ++p) {
-            const uint32_t slice = planes_lds[q][p][comp][lane] >> shift;
-#pragma unroll
-            for (int s = 0; s < BITS; ++s) cnt[s] += (int32_t) (((slice >> s) & 1u) << p);
+    for (int p = 0; p < NA; ++p) {
+        if (p < NB) {
+            V c2, sum;
+            csa(c2, sum, a[p], b[p], carry);
+            a[p] = sum;
+            carry = c2;
+        } else {
+            const V old = a[p];
+            a[p] = old ^ carry;
+            carry = old & carry;
         }
     }
-    if (live) {
-        const int64_t sample0 = col * (32 * NC) + first_bit;
+    a[NA] = carry;
+}
+
+template <typename V, int TREE>
+__global__ __launch_bounds__(DL_BLOCK) void count_partial_kernel(const V *__restrict__ x,
+                                                                 const int32_t *__restrict__ leaves,
+                                                                 const uint64_t *__restrict__ gates,
+                                                                 V *__restrict__ partial, int64_t ncols,
+                                                                 int64_t per_class, int64_t chunks_per_class) {
+    constexpr int G = 1 << TREE;
+    __shared__ V lds[3][6][DL_WAVE];
+
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t chunk = blockIdx.x;
+    const int64_t cls = chunk / chunks_per_class;
+    const int64_t r_begin = (chunk - cls * chunks_per_class) * DL_COUNT_ROWS + (int64_t) wave * (DL_COUNT_ROWS / 4);
+    int64_t r_end = r_begin + DL_COUNT_ROWS / 4;
+    if (r_end > per_class) r_end = per_class;
+    const int64_t col = (int64_t) blockIdx.y * DL_WAVE + lane;
+    const bool live = col < ncols;
+    const V *xcol = x + (live ? col : 0);
+
+    V n[8];                                  // this wave's count: planes of weight 1 .. 32 (+2 spare)
 #pragma unroll
-        for (int s = 0; s < BITS; ++s)
-            if (sample0 + s < batch) out[(sample0 + s) * k + cls] = cnt[s];
+    for (int p = 0; p < 8; ++p) n[p] = Words<V>::zero();
+    auto quad = [&](int64_t q0) -> V {
+        V v[4];
+        V leaf[4][G];
+        uint64_t gt[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int64_t r = q0 + j;
+            if (r >= per_class) r = per_class - 1;
+            const int64_t nn = cls * per_class + r;
+            gt[j] = gates[nn];
+#pragma unroll
+            for (int g = 0; g < G; ++g)
+                leaf[j][g] = live ? xcol[(int64_t) leaves[nn * G + g] * ncols] : Words<V>::zero();
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const V y = TreeFold<V, TREE>::run(leaf[j], gt[j]);
+            v[j] = (live && q0 + j < r_end) ? y : Words<V>::zero();
+        }
+        return csa_quad(n[0], n[1], v);
+    };
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {            // two blocks of 16 neurons
+        const int64_t r = r_begin + 16 * h;
+        V t8a, t8b, t16;
+        {
+            const V t4a = quad(r), t4b = quad(r + 4);
+            csa(t8a, n[2], n[2], t4a, t4b);
+        }
+        {
+            const V t4a = quad(r + 8), t4b = quad(r + 12);
+            csa(t8b, n[2], n[2], t4a, t4b);
+        }
+        csa(t16, n[3], n[3], t8a, t8b);
+        const V old = n[4];                  // weight 16, then 32
+        n[4] = old ^ t16;
+        n[5] = n[5] | (old & t16);
     }
+
+    // waves 1..3 park their six planes; wave 0 adds them: (w0 + w1) + (w2 + w3)
+    if (wave != 0) {
+#pragma unroll
+        for (int p = 0; p < 6; ++p) lds[wave - 1][p][lane] = n[p];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    V m[8], t[8];
+#pragma unroll
+    for (int p = 0; p < 6; ++p) t[p] = lds[0][p][lane];
+    sliced_add<V, 6, 6>(n, t);               // n: 7 planes
+#pragma unroll
+    for (int p = 0; p < 6; ++p) {
+        m[p] = lds[1][p][lane];
+        t[p] = lds[2][p][lane];
+    }
+    m[6] = m[7] = Words<V>::zero();
+    sliced_add<V, 6, 6>(m, t);               // m: 7 planes
+    sliced_add<V, 7, 7>(n, m);               // n: 8 planes
+    if (live) {
+        V *dst = partial + (((int64_t) blockIdx.y * gridDim.x + chunk) * DL_COUNT_PLANES) * DL_WAVE + lane;
+#pragma unroll
+        for (int p = 0; p < DL_COUNT_PLANES; ++p) __builtin_nontemporal_store(n[p], dst + (int64_t) p * DL_WAVE);
+    }
+}
+
+template <typename V, int NP>
+__global__ __launch_bounds__(DL_BLOCK) void count_finish_kernel(const V *__restrict__ partial, int32_t *__restrict__ out,
+                                                                int64_t ncols, int64_t chunks_per_class, int64_t k,
+                                                                int64_t batch) {
+    constexpr int NC = Words<V>::n;
+    __shared__ uint32_t planes_lds[4][NP][NC][DL_WAVE];
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t tile = blockIdx.x, cls = blockIdx.y;
+    const int64_t col = tile * DL_WAVE + lane;
+    const bool live = col < ncols;
+
+    V acc[NP + 1];
+#pragma unroll
+    for (int p = 0; p <= NP; ++p) acc[p] = Words<V>::zero();
+    const V *src = partial + ((tile * (k * chunks_per_class) + cls * chunks_per_class) * DL_COUNT_PLANES) * DL_WAVE + lane;
+    for (int64_t c = wave; c < chunks_per_class; c += 4) {
+        V part[DL_COUNT_PLANES];
+#pragma unroll
+        for (int p = 0; p < DL_COUNT_PLANES; ++p)
+            part[p] = live ? __builtin_nontemporal_load(src + (c * DL_COUNT_PLANES + p) * DL_WAVE) : Words<V>::zero();
+        sliced_add<V, NP, DL_COUNT_PLANES>(acc, part);      // the carry out of plane NP-1 is zero by construction
+    }
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+#pragma unroll
+        for (int p = 0; p < NP; ++p) planes_lds[wave][p][c][lane] = Words<V>::get(acc[p], c);
+    }
+    __syncthreads();
+    expand_counts<V, NP, 4>(planes_lds, wave, lane, col, live, cls, k, batch, out);
 }
 
 // Any word width / row length: one thread per (sample, class), like the reference, but with
@@ -516,33 +662,72 @@ __global__ __launch_bounds__(DL_BLOCK) void groupbitsum_generic_kernel(const uin
     }
 }
 
-template <typename V, int TREE>
-void launch_groupbitsum_v(const void *bits, const int32_t *leaves, const uint64_t *gates, int32_t *out, int64_t row_bytes,
-                          int64_t per_class, int64_t k, int64_t batch, hipStream_t s) {
+template <typename V>
+void launch_groupbitsum_v(const void *bits, int32_t *out, int64_t row_bytes, int64_t per_class, int64_t k,
+                          int64_t batch, hipStream_t s) {
     const int64_t ncols = row_bytes / (int64_t) sizeof(V);
     const dim3 grid((unsigned) dl_ceil_div(ncols, DL_WAVE), (unsigned) k);
     const int64_t chunk = (per_class + 3) / 4;      // rows one wave counts
     const V *b = (const V *) bits;
     // NPH planes above weight 8 hold counts up to 16 * 2^NPH - 1.
     if (chunk < (16LL << 8))
-        hipLaunchKernelGGL((groupbitsum_kernel<V, 8, TREE>), grid, dim3(DL_BLOCK), 0, s, b, leaves, gates, out, ncols,
-                           per_class, k, batch);
+        hipLaunchKernelGGL((groupbitsum_kernel<V, 8>), grid, dim3(DL_BLOCK), 0, s, b, out, ncols, per_class, k, batch);
     else if (chunk < (16LL << 14))
-        hipLaunchKernelGGL((groupbitsum_kernel<V, 14, TREE>), grid, dim3(DL_BLOCK), 0, s, b, leaves, gates, out, ncols,
-                           per_class, k, batch);
+        hipLaunchKernelGGL((groupbitsum_kernel<V, 14>), grid, dim3(DL_BLOCK), 0, s, b, out, ncols, per_class, k, batch);
     else
-        hipLaunchKernelGGL((groupbitsum_kernel<V, 27, TREE>), grid, dim3(DL_BLOCK), 0, s, b, leaves, gates, out, ncols,
-                           per_class, k, batch);
+        hipLaunchKernelGGL((groupbitsum_kernel<V, 27>), grid, dim3(DL_BLOCK), 0, s, b, out, ncols, per_class, k, batch);
 }
 
 // Rows of whole 64-bit words, 8-byte aligned: 16-byte lanes where rows and base allow it.
-template <int TREE>
-void launch_groupbitsum(const void *bits, const int32_t *leaves, const uint64_t *gates, int32_t *out, int64_t row_bytes,
-                        int64_t per_class, int64_t k, int64_t batch, hipStream_t s) {
+void launch_groupbitsum(const void *bits, int32_t *out, int64_t row_bytes, int64_t per_class, int64_t k, int64_t batch,
+                        hipStream_t s) {
     if (row_bytes % 16 == 0 && dl_aligned(bits, 16))
-        launch_groupbitsum_v<dl_u32x4, TREE>(bits, leaves, gates, out, row_bytes, per_class, k, batch, s);
+        launch_groupbitsum_v<dl_u32x4>(bits, out, row_bytes, per_class, k, batch, s);
     else
-        launch_groupbitsum_v<uint64_t, TREE>(bits, leaves, gates, out, row_bytes, per_class, k, batch, s);
+        launch_groupbitsum_v<uint64_t>(bits, out, row_bytes, per_class, k, batch, s);
+}
+
+// Scratch of the two-pass fused count: DL_COUNT_PLANES row vectors per chunk per column tile.
+int64_t count_scratch_bytes(int64_t out_dim, int64_t k, int64_t row_bytes) {
+    const int64_t chunks = k * dl_ceil_div(out_dim / k, DL_COUNT_ROWS);
+    const int64_t vec = row_bytes % 16 == 0 ? 16 : 8;
+    const int64_t tiles = dl_ceil_div(row_bytes / vec, DL_WAVE);
+    return tiles * chunks * DL_COUNT_PLANES * DL_WAVE * vec;
+}
+
+template <typename V, int TREE>
+int launch_count_fused_v(const void *x, const int32_t *leaves, const uint64_t *gates, void *scratch, int32_t *out,
+                         int64_t row_bytes, int64_t per_class, int64_t k, int64_t batch, hipStream_t s) {
+    const int64_t ncols = row_bytes / (int64_t) sizeof(V);
+    const int64_t tiles = dl_ceil_div(ncols, DL_WAVE);
+    const int64_t chunks_per_class = dl_ceil_div(per_class, DL_COUNT_ROWS);
+    if (k * chunks_per_class > 0x7fffffffLL || tiles > 65535) return DL_ERR_TOO_LARGE;
+    hipLaunchKernelGGL((count_partial_kernel<V, TREE>), dim3((unsigned) (k * chunks_per_class), (unsigned) tiles),
+                       dim3(DL_BLOCK), 0, s, (const V *) x, leaves, gates, (V *) scratch, ncols, per_class,
+                       chunks_per_class);
+    int st = dl_launch_status();
+    if (st != DL_OK) return st;
+    const dim3 grid((unsigned) tiles, (unsigned) k);
+    // planes needed for counts up to per_class (pass 1 rounds a class up to whole chunks of 128)
+    const int64_t top = chunks_per_class * DL_COUNT_ROWS;
+    if (top < (1LL << 13))
+        hipLaunchKernelGGL((count_finish_kernel<V, 13>), grid, dim3(DL_BLOCK), 0, s, (const V *) scratch, out, ncols,
+                           chunks_per_class, k, batch);
+    else if (top < (1LL << 18))
+        hipLaunchKernelGGL((count_finish_kernel<V, 18>), grid, dim3(DL_BLOCK), 0, s, (const V *) scratch, out, ncols,
+                           chunks_per_class, k, batch);
+    else
+        hipLaunchKernelGGL((count_finish_kernel<V, 31>), grid, dim3(DL_BLOCK), 0, s, (const V *) scratch, out, ncols,
+                           chunks_per_class, k, batch);
+    return dl_launch_status();
+}
+
+template <int TREE>
+int launch_count_fused(const void *x, const int32_t *leaves, const uint64_t *gates, void *scratch, int32_t *out,
+                       int64_t row_bytes, int64_t per_class, int64_t k, int64_t batch, hipStream_t s) {
+    if (row_bytes % 16 == 0 && dl_aligned(x, 16) && dl_aligned(scratch, 16))
+        return launch_count_fused_v<dl_u32x4, TREE>(x, leaves, gates, scratch, out, row_bytes, per_class, k, batch, s);
+    return launch_count_fused_v<uint64_t, TREE>(x, leaves, gates, scratch, out, row_bytes, per_class, k, batch, s);
 }
 
 // Validates the description of a fused group and launches the composite builder.
@@ -689,7 +874,7 @@ extern "C" int dl_groupbitsum(const void *b, int32_t *out, int64_t in_dim, int64
 
     if (row_bytes % 8 == 0 && dl_aligned(b, 8) && k <= 65535) {
         if (dl_ceil_div(row_bytes / 8, DL_WAVE) > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
-        launch_groupbitsum<0>(b, nullptr, nullptr, out, row_bytes, per_class, k, batch, s);
+        launch_groupbitsum(b, out, row_bytes, per_class, k, batch, s);
     } else {
         int64_t gx = dl_ceil_div(batch, DL_BLOCK);
         if (gx > 0x7fffffffLL) gx = 0x7fffffffLL;
@@ -746,9 +931,20 @@ extern "C" int dl_logic_eval_fused_groupbitsum(const void *x, int depth, const i
     uint64_t *gates;
     const int st = compose_tree(depth, a, b, w, dims, workspace, &leaves, &gates, s);
     if (st != DL_OK) return st;
+    // scratch for the partial counters follows the flattened wiring in the workspace
+    const int64_t tables = dl_logic_eval_fused_workspace_bytes(depth, out_dim);
+    void *scratch = (char *) workspace + ((tables + 15) / 16) * 16;
     if (depth == 1)
-        launch_groupbitsum<1>(x, leaves, gates, out, row_bytes, per_class, k, batch, s);
-    else
-        launch_groupbitsum<2>(x, leaves, gates, out, row_bytes, per_class, k, batch, s);
-    return dl_launch_status();
+        return launch_count_fused<1>(x, leaves, gates, scratch, out, row_bytes, per_class, k, batch, s);
+    return launch_count_fused<2>(x, leaves, gates, scratch, out, row_bytes, per_class, k, batch, s);
+}
+
+extern "C" int64_t dl_logic_eval_fused_groupbitsum_workspace_bytes(int depth, int64_t out_dim, int64_t words,
+                                                                    int bit_count, int64_t k) {
+    if (depth < 1 || depth > 2 || out_dim < 0 || words < 0 || k <= 0 || !valid_bit_count(bit_count)) return 0;
+    if (out_dim % k != 0) return 0;
+    const int64_t row_bytes = words * (bit_count / 8);
+    if (row_bytes % 8 != 0) return 0;
+    const int64_t tables = dl_logic_eval_fused_workspace_bytes(depth, out_dim);
+    return ((tables + 15) / 16) * 16 + count_scratch_bytes(out_dim, k, row_bytes);
 }

@@ -298,7 +298,8 @@ def eval_fused_groupbitsum(x, layers, pad_len, k):
         st = _lib.DL_ERR_TOO_LARGE
     else:
         out = torch.empty((batch, k), dtype=torch.int32, device=dev)
-        ws = _fused_workspace(depth, out_dim, dev)
+        nbytes = _lib.load().dl_logic_eval_fused_groupbitsum_workspace_bytes(depth, out_dim, words, bits, int(k))
+        ws = torch.empty(max(2, -(-nbytes // 8)), dtype=torch.int64, device=dev)
         with torch.cuda.device(dev):
             st = _lib.load().dl_logic_eval_fused_groupbitsum(_p(x), depth, pa, pb, pw, pdims, _p(out), words, bits,
                                                              int(pad_len), int(k), _p(ws), _stream(dev))

@@ -137,7 +137,12 @@ int dl_logic_eval_fused(const void *x, int depth, const int64_t *const *a, const
 /* The net's last `depth` (1 or 2) layers fused with `groupbitsum` (the sequence
  * difflogic/difflogic.py:147 then difflogic/packbitstensor.py:22): the last layer's output words
  * are counted as they are produced and never written.  Arguments as dl_logic_eval_fused, result
- * as dl_groupbitsum: out [words*bit_count - pad_len, k] int32.  Also needs k <= 65535. */
+ * as dl_groupbitsum: out [words*bit_count - pad_len, k] int32.  Also needs k <= 65535.
+ *   workspace DEVICE scratch of dl_logic_eval_fused_groupbitsum_workspace_bytes(...) bytes,
+ *             16-byte aligned: the flattened wiring plus the bit-sliced partial counters that the
+ *             first of the two passes hands to the second. */
+int64_t dl_logic_eval_fused_groupbitsum_workspace_bytes(int depth, int64_t out_dim, int64_t words,
+                                                        int bit_count, int64_t k);
 int dl_logic_eval_fused_groupbitsum(const void *x, int depth, const int64_t *const *a,
                                     const int64_t *const *b, const uint8_t *const *w,
                                     const int64_t *dims, int32_t *out, int64_t words, int bit_count,
