@@ -185,8 +185,10 @@ def cpu_baseline(args, model, x, dl):
 
 def train_bench(args, torch, dl):
     """fp32 forward + backward of 784 -> 6 x 64000 -> GroupSum(10, tau 30), B = 512, 'unique'
-    connections, grad_factor 1: per-kernel event timings against the algorithmic bytes
-    fwd 4B(in+out)+80 out, backward_w 4B(in+out)+64 out, backward_x 4B(2 in+out)+64 out."""
+    connections, grad_factor 1, CrossEntropy.  Reports the whole step (eager and replayed as one
+    HIP graph) and each layer kernel timed alone (back-to-back launches on a 64000 -> 64000 layer)
+    against its algorithmic bytes: forward 4B(in+out)+80 out, backward_w 4B(in+out)+64 out,
+    backward_x 4B(2 in+out)+64 out."""
     F, width, L, k, B = 784, 64000, 6, 10, 512
     torch.manual_seed(0)
     mods, d = [torch.nn.Flatten()], F
@@ -198,26 +200,7 @@ def train_bench(args, torch, dl):
     x = (torch.rand(B, F, device="cuda", generator=g) < 0.2).float()
     labels = torch.randint(0, k, (B,), device="cuda", generator=g)
     loss_fn = torch.nn.CrossEntropyLoss()
-
-    ext = dl.difflogic_cuda
-    real = {n: getattr(ext, n) for n in ("forward", "backward_w", "backward_x")}
-    rec = {n: [] for n in real}
-    on = {"v": False}
-
-    def wrap(name):
-        def f(*a, **kw):
-            if not on["v"]:
-                return real[name](*a, **kw)
-            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            s.record()
-            r = real[name](*a, **kw)
-            e.record()
-            rec[name].append((a[0].shape[0], r.shape[0] if name != "backward_x" else a[4].shape[0], s, e))
-            return r
-        return f
-
-    for n in real:
-        setattr(ext, n, wrap(n))
+    steps, warmup = max(5, args.steps), max(3, args.warmup)
 
     def step():
         model.zero_grad(set_to_none=True)
@@ -225,39 +208,45 @@ def train_bench(args, torch, dl):
         loss.backward()
         return loss
 
-    steps, warmup = max(5, args.steps), max(3, args.warmup)
-    try:
-        for _ in range(warmup):
-            step()
-        torch.cuda.synchronize()
-        on["v"] = True
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            loss = step()
-        torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
-    finally:
-        for n in real:
-            setattr(ext, n, real[n])
-
-    def alg(name, i, o):
-        if name == "forward":
-            return 4 * B * (i + o) + 80 * o
-        if name == "backward_w":
-            return 4 * B * (i + o) + 64 * o
-        return 4 * B * (2 * i + o) + 64 * o
-
-    kernels = {}
-    tot_bytes = tot_ms = 0.0
-    for name, items in rec.items():
-        by = sum(alg(name, i, o) for i, o, _, _ in items)
-        ms = sum(s.elapsed_time(e) for _, _, s, e in items)
-        tot_bytes += by
-        tot_ms += ms
-        kernels[name] = {"GBps": round(by / (ms * 1e-3) / 1e9, 1), "frac_hbm": round(by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                         "ms_per_step": round(ms / steps, 4)}
-    neuron_samples = L * width * B
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loss = step()
+    torch.cuda.synchronize()
+    eager = (time.perf_counter() - t0) / steps
     eager_loss = loss.item()
+
+    # each layer kernel alone, 20 launches back to back on one square layer
+    ext = dl.difflogic_cuda
+    layer = model[2]
+    a, b = layer.indices
+    xs = torch.rand(width, B, device="cuda", generator=g)
+    gy = torch.randn(width, B, device="cuda", generator=g)
+    logits = layer.weights.detach()
+    _, probs = ext.forward_logits(xs, a, b, logits)
+    start, idx = layer.given_x_indices_of_y_start, layer.given_x_indices_of_y
+    calls = {
+        "forward_logits": (lambda: ext.forward_logits(xs, a, b, logits), 4 * B * 2 * width + 80 * width),
+        "backward_logits": (lambda: ext.backward_logits(xs, a, b, gy, probs), 4 * B * 2 * width + 64 * width),
+        "backward_x": (lambda: ext.backward_x(xs, a, b, probs, gy, start, idx), 4 * B * 3 * width + 64 * width),
+    }
+    kernels = {}
+    for name, (fn, by) in calls.items():
+        for _ in range(3):
+            fn()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(20):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        us = s.elapsed_time(e) / 20 * 1e3
+        kernels[name] = {"us_per_launch": round(us, 2), "GBps_algorithmic": round(by / (us * 1e-6) / 1e9, 1),
+                         "frac_hbm": round(by / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+    del xs, gy
+
     # Drop every reference to the eager autograd graph before capturing: gradient-accumulation
     # nodes kept alive by `loss` belong to the default stream and would be replayed into the
     # capture stream's backward.
@@ -266,7 +255,6 @@ def train_bench(args, torch, dl):
     import gc
     gc.collect()
     torch.cuda.synchronize()
-    # the same step replayed as one HIP graph (removes the host launch overhead)
     from difflogic_amd.graphs import GraphedTrainStep
     graphed = GraphedTrainStep(model, loss_fn, x, labels)
     for _ in range(warmup):
@@ -276,19 +264,21 @@ def train_bench(args, torch, dl):
     for _ in range(steps):
         gl = graphed.step()
     torch.cuda.synchronize()
-    g_elapsed = time.perf_counter() - t0
+    replay = (time.perf_counter() - t0) / steps
+
+    dims = [F] + [width] * L
+    alg = sum(4 * B * (i + o) + 80 * o + 4 * B * (i + o) + 64 * o for i, o in zip(dims[:-1], dims[1:]))
+    alg += sum(4 * B * (2 * i + o) + 64 * o for i, o in zip(dims[1:-1], dims[2:]))     # no backward_x for layer 1
+    neuron_samples = L * width * B
     return {
-        "graphed_neuron_samples_per_s": round(neuron_samples * steps / g_elapsed, 1),
-        "graphed_ms_per_step": round(g_elapsed / steps * 1e3, 4),
-        "graphed_GBps_algorithmic": round(tot_bytes / steps / (g_elapsed / steps) / 1e9, 1),
-        "graphed_loss": round(gl.item(), 6),
         "workload": "fp32 fwd+bwd 784->6x64000->GroupSum(10,tau=30), B=512, connections=unique, CrossEntropy",
-        "neuron_samples_per_s": round(neuron_samples * steps / elapsed, 1),
-        "neuron_samples_per_s_kernels_only": round(neuron_samples * steps / (tot_ms * 1e-3), 1),
-        "ms_per_step": round(elapsed / steps * 1e3, 4),
-        "kernel_GBps_algorithmic": round(tot_bytes / (tot_ms * 1e-3) / 1e9, 1),
-        "kernel_frac_hbm": round(tot_bytes / (tot_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-        "kernels": kernels, "loss": round(eager_loss, 6), "dtype": "f32",
+        "dtype": "f32", "algorithmic_GB_per_step": round(alg / 1e9, 3),
+        "graph_replay": {"neuron_samples_per_s": round(neuron_samples / replay, 1), "ms_per_step": round(replay * 1e3, 4),
+                         "GBps_algorithmic": round(alg / replay / 1e9, 1),
+                         "frac_hbm": round(alg / replay / 1e9 / HBM_PEAK_GBS, 4), "loss": round(gl.item(), 6)},
+        "eager": {"neuron_samples_per_s": round(neuron_samples / eager, 1), "ms_per_step": round(eager * 1e3, 4),
+                  "loss": round(eager_loss, 6)},
+        "kernels_alone_64000x64000": kernels,
     }
 
 

@@ -28,11 +28,7 @@ template <> __device__ __forceinline__ __half down<__half, float>(float v) { ret
 // The four corner values of neuron n's gate mixture.
 template <typename C> struct Corners { C p00, p01, p10, p11; };
 
-template <typename T> __device__ __forceinline__ Corners<typename Acc<T>::type> corners(const T *__restrict__ w, int64_t n) {
-    typedef typename Acc<T>::type C;
-    C g[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) g[i] = up<T>(w[n * 16 + i]);
+template <typename C> __device__ __forceinline__ Corners<C> corners_of(const C (&g)[16]) {
     Corners<C> c;
     c.p00 = ((g[8] + g[9]) + (g[10] + g[11])) + ((g[12] + g[13]) + (g[14] + g[15]));
     c.p01 = ((g[4] + g[5]) + (g[6] + g[7])) + ((g[12] + g[13]) + (g[14] + g[15]));
@@ -41,13 +37,106 @@ template <typename T> __device__ __forceinline__ Corners<typename Acc<T>::type> 
     return c;
 }
 
+template <typename T> __device__ __forceinline__ Corners<typename Acc<T>::type> corners(const T *__restrict__ w, int64_t n) {
+    typedef typename Acc<T>::type C;
+    C g[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) g[i] = up<T>(w[n * 16 + i]);
+    return corners_of<C>(g);
+}
+
+// ------------------------------------------------------------------------------------------
+// Wave-wide sums with a fixed association order (deterministic).
+// ------------------------------------------------------------------------------------------
+template <int CTRL> __device__ __forceinline__ float dpp_f32(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]  : lane ^ 1
+    v += dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]  : lane ^ 2
+    v += dpp_f32<0x141>(v);  // row_half_mirror      : the other quad of the 8-lane half row
+    v += dpp_f32<0x140>(v);  // row_mirror           : the other half of the 16-lane row
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+    for (int m = 1; m < DL_WAVE; m <<= 1) v += __shfl_xor(v, m, DL_WAVE);
+    return v;
+}
+
+// Sum over each aligned group of 16 lanes, result in every lane of the group.
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_f32<0xB1>(v);
+    v += dpp_f32<0x4E>(v);
+    v += dpp_f32<0x141>(v);
+    v += dpp_f32<0x140>(v);
+    return v;
+}
+
+__device__ __forceinline__ double row16_sum(double v) {
+#pragma unroll
+    for (int m = 1; m < 16; m <<= 1) v += __shfl_xor(v, m, DL_WAVE);
+    return v;
+}
+
+__device__ __forceinline__ float dl_exp(float v) { return expf(v); }
+__device__ __forceinline__ double dl_exp(double v) { return exp(v); }
+
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_f32<0xB1>(v));
+    v = fmaxf(v, dpp_f32<0x4E>(v));
+    v = fmaxf(v, dpp_f32<0x141>(v));
+    v = fmaxf(v, dpp_f32<0x140>(v));
+    return v;
+}
+
+__device__ __forceinline__ double row16_max(double v) {
+#pragma unroll
+    for (int m = 1; m < 16; m <<= 1) v = fmax(v, __shfl_xor(v, m, DL_WAVE));
+    return v;
+}
+
+__device__ __forceinline__ float lane_value(float v, int i) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), i));
+}
+
+__device__ __forceinline__ double lane_value(double v, int i) {
+    const uint64_t u = __builtin_bit_cast(uint64_t, v);
+    const uint32_t lo = (uint32_t) __builtin_amdgcn_readlane((int) (uint32_t) u, i);
+    const uint32_t hi = (uint32_t) __builtin_amdgcn_readlane((int) (uint32_t) (u >> 32), i);
+    return __builtin_bit_cast(double, ((uint64_t) hi << 32) | lo);
+}
+
+// softmax over neuron n's 16 gate logits, exp(l - max) / sum.  Lane i of every 16-lane row works
+// on gate i & 15 (one exp and one division per lane, row-wide max and sum by DPP); the 16
+// probabilities are then broadcast as wave-uniform values g[0..15], and `mine` is lane's own.
+template <typename T> __device__ __forceinline__ void softmax16(const T *__restrict__ logits, int64_t n, int lane,
+                                                                typename Acc<T>::type (&g)[16],
+                                                                typename Acc<T>::type &mine) {
+    typedef typename Acc<T>::type C;
+    const C l = up<T>(logits[n * 16 + (lane & 15)]);
+    const C e = dl_exp(l - row16_max(l));
+    mine = e / row16_sum(e);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) g[i] = lane_value(mine, i);
+}
+
 // ------------------------------------------------------------------------------------------
 // forward: one wave = NPW neurons x 64 vectors of the batch.
 // ------------------------------------------------------------------------------------------
-template <typename T, int VEC, int NPW>
+// LOGITS: `w` holds the raw gate logits; the kernel applies the softmax itself and (column tile 0
+// only) stores the probabilities to `probs` for the backward pass.
+template <typename T, int VEC, int NPW, bool LOGITS>
 __global__ __launch_bounds__(DL_BLOCK) void forward_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
                                                            const int64_t *__restrict__ b, const T *__restrict__ w,
-                                                           T *__restrict__ y, int64_t out_dim, int64_t ncols) {
+                                                           T *__restrict__ y, T *__restrict__ probs, int64_t out_dim,
+                                                           int64_t ncols) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
     const int wave = dl_wave_in_block();
@@ -62,7 +151,15 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_kernel(const T *__restrict__
         const int64_t n = (n0 + j < out_dim) ? n0 + j : out_dim - 1;
         ia[j] = a[n];
         ib[j] = b[n];
-        const Corners<C> c = corners<T>(w, n);
+        Corners<C> c;
+        if (LOGITS) {
+            C g[16], mine;
+            softmax16<T>(w, n, lane, g, mine);
+            c = corners_of<C>(g);
+            if (blockIdx.y == 0 && n0 + j < out_dim && lane < 16) probs[n * 16 + lane] = down<T, C>(mine);
+        } else {
+            c = corners<T>(w, n);
+        }
         p00[j] = c.p00;
         p10[j] = c.p10;
         d0[j] = c.p01 - c.p00;
@@ -95,42 +192,19 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_kernel(const T *__restrict__
 }
 
 // ------------------------------------------------------------------------------------------
-// Wave-wide sums with a fixed association order (deterministic).
-// ------------------------------------------------------------------------------------------
-template <int CTRL> __device__ __forceinline__ float dpp_f32(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
-}
-
-__device__ __forceinline__ float wave_sum(float v) {
-    v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]  : lane ^ 1
-    v += dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]  : lane ^ 2
-    v += dpp_f32<0x141>(v);  // row_half_mirror      : the other quad of the 8-lane half row
-    v += dpp_f32<0x140>(v);  // row_mirror           : the other half of the 16-lane row
-    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
-    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
-    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
-    const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
-    return (r0 + r1) + (r2 + r3);
-}
-
-__device__ __forceinline__ double wave_sum(double v) {
-#pragma unroll
-    for (int m = 1; m < DL_WAVE; m <<= 1) v += __shfl_xor(v, m, DL_WAVE);
-    return v;
-}
-
-// ------------------------------------------------------------------------------------------
 // backward_w: per neuron, the four corner-weighted batch sums
 //     S_st = sum_r g[r] * a^s (1-a)^(1-s) * b^t (1-b)^(1-t)
 // and grad_w[n, i] = sum of the S_st at which gate i is true.
 // WPN = waves that share one neuron's batch (1: a wave owns NPW neurons; 4: the workgroup's
 // four waves split the batch of NPW neurons and combine through LDS in wave order).
 // ------------------------------------------------------------------------------------------
+// probs != nullptr: chain the softmax backward, gw[n,i] = p_i * (g_i - sum_j p_j g_j), i.e. the
+// gradient with respect to the logits that `probs` (forward_kernel's LOGITS output) came from.
 template <typename T, int VEC, int NPW, int WPN>
 __global__ __launch_bounds__(DL_BLOCK) void backward_w_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
                                                               const int64_t *__restrict__ b,
-                                                              const T *__restrict__ gy, T *__restrict__ gw,
-                                                              int64_t out_dim, int64_t ncols) {
+                                                              const T *__restrict__ gy, const T *__restrict__ probs,
+                                                              T *__restrict__ gw, int64_t out_dim, int64_t ncols) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
     __shared__ C partial[4][NPW][4];
@@ -210,18 +284,21 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_w_kernel(const T *__restric
     }
 
     // lane i < 16 holds gate i: add the corners whose truth-table bit is set.
-    if (lane < 16) {
 #pragma unroll
-        for (int j = 0; j < NPW; ++j) {
-            if (n0 + j < out_dim) {
-                C r = (C) 0;
-                if (lane & 8) r += s00[j];
-                if (lane & 4) r += s01[j];
-                if (lane & 2) r += s10[j];
-                if (lane & 1) r += s11[j];
-                gw[(n0 + j) * 16 + lane] = down<T, C>(r);
-            }
+    for (int j = 0; j < NPW; ++j) {
+        const bool valid = lane < 16 && n0 + j < out_dim;
+        C r = (C) 0;
+        if (lane & 8) r += s00[j];
+        if (lane & 4) r += s01[j];
+        if (lane & 2) r += s10[j];
+        if (lane & 1) r += s11[j];
+        if (probs != nullptr) {
+            const C p = valid ? up<T>(probs[(n0 + j) * 16 + lane]) : (C) 0;
+            C dot = p * r;                           // summed over the 16-lane row, all lanes take part
+            dot = row16_sum(dot);
+            r = p * (r - dot);
         }
+        if (valid) gw[(n0 + j) * 16 + lane] = down<T, C>(r);
     }
 }
 
@@ -292,26 +369,27 @@ unsigned col_tiles(int64_t ncols) {
     return (unsigned) (t > 65535 ? 65535 : t);
 }
 
-template <typename T>
-int forward_t(const void *x, const int64_t *a, const int64_t *b, const void *w, void *y, int64_t out_dim,
+template <typename T, bool LOGITS>
+int forward_t(const void *x, const int64_t *a, const int64_t *b, const void *w, void *y, void *probs, int64_t out_dim,
               int64_t batch, hipStream_t s) {
     constexpr int NPW = 4;
     const int64_t blocks = dl_ceil_div(out_dim, 4 * NPW);
     if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     constexpr int V = Vec16<T>::n;
     if (batch % V == 0 && dl_aligned(x, 16) && dl_aligned(y, 16)) {
-        hipLaunchKernelGGL((forward_kernel<T, V, NPW>), dim3((unsigned) blocks, col_tiles(batch / V)), dim3(DL_BLOCK), 0, s,
-                           (const T *) x, a, b, (const T *) w, (T *) y, out_dim, batch / V);
+        hipLaunchKernelGGL((forward_kernel<T, V, NPW, LOGITS>), dim3((unsigned) blocks, col_tiles(batch / V)),
+                           dim3(DL_BLOCK), 0, s, (const T *) x, a, b, (const T *) w, (T *) y, (T *) probs, out_dim,
+                           batch / V);
     } else {
-        hipLaunchKernelGGL((forward_kernel<T, 1, NPW>), dim3((unsigned) blocks, col_tiles(batch)), dim3(DL_BLOCK), 0, s,
-                           (const T *) x, a, b, (const T *) w, (T *) y, out_dim, batch);
+        hipLaunchKernelGGL((forward_kernel<T, 1, NPW, LOGITS>), dim3((unsigned) blocks, col_tiles(batch)), dim3(DL_BLOCK),
+                           0, s, (const T *) x, a, b, (const T *) w, (T *) y, (T *) probs, out_dim, batch);
     }
     return dl_launch_status();
 }
 
 template <typename T>
-int backward_w_t(const void *x, const int64_t *a, const int64_t *b, const void *gy, void *gw, int64_t out_dim,
-                 int64_t batch, hipStream_t s) {
+int backward_w_t(const void *x, const int64_t *a, const int64_t *b, const void *gy, const void *probs, void *gw,
+                 int64_t out_dim, int64_t batch, hipStream_t s) {
     constexpr int NPW = 2;
     constexpr int V = Vec16<T>::n;
     const bool vec = batch % V == 0 && dl_aligned(x, 16) && dl_aligned(gy, 16);
@@ -321,16 +399,16 @@ int backward_w_t(const void *x, const int64_t *a, const int64_t *b, const void *
     const int64_t blocks = split ? dl_ceil_div(out_dim, NPW) : dl_ceil_div(out_dim, 4 * NPW);
     if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     const dim3 grid((unsigned) blocks), block(DL_BLOCK);
-    const T *xp = (const T *) x, *gp = (const T *) gy;
+    const T *xp = (const T *) x, *gp = (const T *) gy, *pp = (const T *) probs;
     T *wp = (T *) gw;
     if (vec && split)
-        hipLaunchKernelGGL((backward_w_kernel<T, V, NPW, 4>), grid, block, 0, s, xp, a, b, gp, wp, out_dim, ncols);
+        hipLaunchKernelGGL((backward_w_kernel<T, V, NPW, 4>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols);
     else if (vec)
-        hipLaunchKernelGGL((backward_w_kernel<T, V, NPW, 1>), grid, block, 0, s, xp, a, b, gp, wp, out_dim, ncols);
+        hipLaunchKernelGGL((backward_w_kernel<T, V, NPW, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols);
     else if (split)
-        hipLaunchKernelGGL((backward_w_kernel<T, 1, NPW, 4>), grid, block, 0, s, xp, a, b, gp, wp, out_dim, ncols);
+        hipLaunchKernelGGL((backward_w_kernel<T, 1, NPW, 4>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols);
     else
-        hipLaunchKernelGGL((backward_w_kernel<T, 1, NPW, 1>), grid, block, 0, s, xp, a, b, gp, wp, out_dim, ncols);
+        hipLaunchKernelGGL((backward_w_kernel<T, 1, NPW, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols);
     return dl_launch_status();
 }
 
@@ -521,9 +599,24 @@ extern "C" int dl_logic_forward(const void *x, const int64_t *a, const int64_t *
     if (!x || !a || !b || !w || !y || in_dim == 0) return DL_ERR_INVALID_ARGUMENT;
     hipStream_t s = (hipStream_t) stream;
     switch (dtype) {
-    case DL_F16: return forward_t<__half>(x, a, b, w, y, out_dim, batch, s);
-    case DL_F32: return forward_t<float>(x, a, b, w, y, out_dim, batch, s);
-    default: return forward_t<double>(x, a, b, w, y, out_dim, batch, s);
+    case DL_F16: return forward_t<__half, false>(x, a, b, w, y, nullptr, out_dim, batch, s);
+    case DL_F32: return forward_t<float, false>(x, a, b, w, y, nullptr, out_dim, batch, s);
+    default: return forward_t<double, false>(x, a, b, w, y, nullptr, out_dim, batch, s);
+    }
+}
+
+extern "C" int dl_logic_forward_logits(const void *x, const int64_t *a, const int64_t *b, const void *logits, void *y,
+                                       void *probs, int64_t in_dim, int64_t out_dim, int64_t batch, int dtype,
+                                       void *stream) {
+    if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
+    if (in_dim < 0 || out_dim < 0 || batch <= 0) return DL_ERR_INVALID_ARGUMENT;   // probs are written by column tile 0
+    if (out_dim == 0) return DL_OK;
+    if (!x || !a || !b || !logits || !y || !probs || in_dim == 0) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    switch (dtype) {
+    case DL_F16: return forward_t<__half, true>(x, a, b, logits, y, probs, out_dim, batch, s);
+    case DL_F32: return forward_t<float, true>(x, a, b, logits, y, probs, out_dim, batch, s);
+    default: return forward_t<double, true>(x, a, b, logits, y, probs, out_dim, batch, s);
     }
 }
 
@@ -537,9 +630,25 @@ extern "C" int dl_logic_backward_w(const void *x, const int64_t *a, const int64_
     if (batch > 0 && (!x || !grad_y)) return DL_ERR_INVALID_ARGUMENT;
     hipStream_t s = (hipStream_t) stream;
     switch (dtype) {
-    case DL_F16: return backward_w_t<__half>(x, a, b, grad_y, grad_w, out_dim, batch, s);
-    case DL_F32: return backward_w_t<float>(x, a, b, grad_y, grad_w, out_dim, batch, s);
-    default: return backward_w_t<double>(x, a, b, grad_y, grad_w, out_dim, batch, s);
+    case DL_F16: return backward_w_t<__half>(x, a, b, grad_y, nullptr, grad_w, out_dim, batch, s);
+    case DL_F32: return backward_w_t<float>(x, a, b, grad_y, nullptr, grad_w, out_dim, batch, s);
+    default: return backward_w_t<double>(x, a, b, grad_y, nullptr, grad_w, out_dim, batch, s);
+    }
+}
+
+extern "C" int dl_logic_backward_logits(const void *x, const int64_t *a, const int64_t *b, const void *grad_y,
+                                        const void *probs, void *grad_logits, int64_t in_dim, int64_t out_dim,
+                                        int64_t batch, int dtype, void *stream) {
+    if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
+    if (in_dim < 0 || out_dim < 0 || batch < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim == 0) return DL_OK;
+    if (!a || !b || !probs || !grad_logits || in_dim == 0) return DL_ERR_INVALID_ARGUMENT;
+    if (batch > 0 && (!x || !grad_y)) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    switch (dtype) {
+    case DL_F16: return backward_w_t<__half>(x, a, b, grad_y, probs, grad_logits, out_dim, batch, s);
+    case DL_F32: return backward_w_t<float>(x, a, b, grad_y, probs, grad_logits, out_dim, batch, s);
+    default: return backward_w_t<double>(x, a, b, grad_y, probs, grad_logits, out_dim, batch, s);
     }
 }
 

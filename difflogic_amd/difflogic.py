@@ -96,6 +96,9 @@ class LogicLayer(torch.nn.Module):
         a, b = self.indices
         tail = (self.given_x_indices_of_y_start, self.given_x_indices_of_y, float(self.grad_factor))
         if self.training:
+            if self.weights.dtype == x.dtype and x.shape[1] > 0:
+                # softmax and its backward run inside the layer kernels
+                return LogicLayerLogitsFunction.apply(x, a, b, self.weights, *tail).transpose(0, 1)
             w = torch.nn.functional.softmax(self.weights, dim=-1).to(x.dtype)
             return LogicLayerCudaFunction.apply(x, a, b, w, *tail).transpose(0, 1)
         w = torch.nn.functional.one_hot(self.weights.argmax(-1), 16).to(x.dtype)
@@ -173,6 +176,30 @@ class LogicLayerCudaFunction(torch.autograd.Function):
         if ctx.needs_input_grad[3]:
             grad_w = difflogic_cuda.backward_w(x, a, b, grad_y)
         return grad_x, None, None, grad_w, None, None, None
+
+
+class LogicLayerLogitsFunction(torch.autograd.Function):
+    """LogicLayerCudaFunction on the raw gate logits: ``forward(x, a, b, softmax(logits))`` and
+    its gradients, with the softmax and the softmax backward inside the layer kernels."""
+
+    @staticmethod
+    def forward(ctx, x, a, b, logits, given_x_indices_of_y_start, given_x_indices_of_y, grad_factor=1.0):
+        y, probs = difflogic_cuda.forward_logits(x, a, b, logits.detach().contiguous())
+        ctx.save_for_backward(x, a, b, probs, given_x_indices_of_y_start, given_x_indices_of_y)
+        ctx.grad_factor = grad_factor
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        x, a, b, probs, given_x_indices_of_y_start, given_x_indices_of_y = ctx.saved_tensors
+        grad_y = grad_y.contiguous()
+        grad_logits = grad_x = None
+        if ctx.needs_input_grad[0]:
+            grad_x = difflogic_cuda.backward_x(x, a, b, probs, grad_y, given_x_indices_of_y_start,
+                                               given_x_indices_of_y, ctx.grad_factor)
+        if ctx.needs_input_grad[3]:
+            grad_logits = difflogic_cuda.backward_logits(x, a, b, grad_y, probs)
+        return grad_x, None, None, grad_logits, None, None, None
 
 
 class GroupSumCudaFunction(torch.autograd.Function):

@@ -140,6 +140,55 @@ def backward_x(x, a, b, w, grad_y, given_x_indices_of_y_start, given_x_indices_o
     return grad_x
 
 
+def forward_logits(x, a, b, logits):
+    """``forward(x, a, b, softmax(logits, -1))`` with the softmax computed inside the kernel.
+    Returns (y [out,B], probs [out,16]); ``probs`` feeds backward_x / backward_logits.  Not part of
+    the reference's extension (difflogic/difflogic.py:123-126 runs the softmax in torch)."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (logits, "logits")):
+        _check_input(t, n)
+    code = _float_code(x, "logic_layer_cuda_forward")
+    if x.dim() != 2 or logits.dim() != 2 or logits.shape[1] != 16 or logits.dtype != x.dtype or x.shape[1] == 0:
+        raise RuntimeError(f"expected x [in,B>0] and logits [out,16] of one dtype, got {tuple(x.shape)} {x.dtype}, "
+                           f"{tuple(logits.shape)} {logits.dtype}")
+    out_dim = logits.shape[0]
+    _check_index(a, "a", out_dim)
+    _check_index(b, "b", out_dim)
+    dev = _same_device(x, a, b, logits)
+    in_dim, batch = x.shape
+    y = torch.empty((out_dim, batch), dtype=x.dtype, device=dev)
+    probs = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
+    with torch.cuda.device(dev):
+        st = _lib.load().dl_logic_forward_logits(_p(x), _p(a), _p(b), _p(logits), _p(y), _p(probs), in_dim, out_dim,
+                                                 batch, code, _stream(dev))
+    if st:
+        _raise(st, "logic_layer_cuda_forward_logits")
+    return y, probs
+
+
+def backward_logits(x, a, b, grad_y, probs):
+    """Gradient with respect to the gate logits: backward_w chained with the softmax backward,
+    ``p * (g - (p * g).sum(-1, keepdim=True))`` with ``g = backward_w(x, a, b, grad_y)``."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (grad_y, "grad_y"), (probs, "probs")):
+        _check_input(t, n)
+    code = _float_code(x, "logic_layer_cuda_backward_w")
+    if (x.dim() != 2 or grad_y.dim() != 2 or grad_y.shape[1] != x.shape[1] or grad_y.dtype != x.dtype
+            or probs.shape != (grad_y.shape[0], 16) or probs.dtype != x.dtype):
+        raise RuntimeError(f"expected x [in,B], grad_y [out,B], probs [out,16] of one dtype, got {tuple(x.shape)}, "
+                           f"{tuple(grad_y.shape)}, {tuple(probs.shape)}")
+    out_dim = grad_y.shape[0]
+    _check_index(a, "a", out_dim)
+    _check_index(b, "b", out_dim)
+    dev = _same_device(x, a, b, grad_y, probs)
+    in_dim, batch = x.shape
+    grad_logits = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
+    with torch.cuda.device(dev):
+        st = _lib.load().dl_logic_backward_logits(_p(x), _p(a), _p(b), _p(grad_y), _p(probs), _p(grad_logits), in_dim,
+                                                  out_dim, batch, code, _stream(dev))
+    if st:
+        _raise(st, "logic_layer_cuda_backward_logits")
+    return grad_logits
+
+
 def eval(x, a, b, w):  # noqa: A001  (the reference's name)
     """x [in,W] int words, w [out] uint8 gate ids -> y [out,W]   (difflogic.cpp:63-68)."""
     for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w")):

@@ -61,6 +61,20 @@ int dl_logic_backward_w(const void *x, const int64_t *a, const int64_t *b, const
                         void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch, int dtype,
                         void *stream);
 
+/* forward / backward_w with the softmax over the 16 gate logits folded in, i.e. the pair
+ * `softmax(weights)` + `forward` of difflogic/difflogic.py:123-126 and `backward_w` + the softmax
+ * backward that autograd chains after it.  No counterpart in the reference's extension.
+ *   dl_logic_forward_logits : logits [out_dim,16] -> y [out_dim,batch] and probs [out_dim,16]
+ *                             (= softmax(logits), kept for the backward pass; batch >= 1)
+ *   dl_logic_backward_logits: grad_logits[n,i] = p_i * (g_i - sum_j p_j g_j) with
+ *                             g = dl_logic_backward_w(x, a, b, grad_y), p = probs. */
+int dl_logic_forward_logits(const void *x, const int64_t *a, const int64_t *b, const void *logits,
+                            void *y, void *probs, int64_t in_dim, int64_t out_dim, int64_t batch,
+                            int dtype, void *stream);
+int dl_logic_backward_logits(const void *x, const int64_t *a, const int64_t *b, const void *grad_y,
+                             const void *probs, void *grad_logits, int64_t in_dim, int64_t out_dim,
+                             int64_t batch, int dtype, void *stream);
+
 /* Replaces `backward_x` = logic_layer_cuda_backward_x (difflogic.cpp:57-62,
  * difflogic_kernel.cu:367-410).
  *   grad_x[c,r] = scale * sum over neurons n reading input c of

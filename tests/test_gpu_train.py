@@ -239,3 +239,28 @@ def test_group_sum_module_uses_feature_major_path_and_matches_torch():
     assert close(gs(z), z.reshape(96, 10, 64).sum(-1) / 30.0)[0]
     with pytest.raises(ValueError):
         dl.difflogic_cuda.group_sum_forward(torch.rand(7, 4, device="cuda"), 2, 1.0)
+
+
+@pytest.mark.parametrize("dtype,rtol", [(torch.float32, 1e-5), (torch.float64, 1e-12)])
+@pytest.mark.parametrize("in_dim,out_dim,batch", [(12, 30, 7), (33, 100, 256), (50, 77, 513), (16, 40, 2048)])
+def test_logits_entry_points(ext, dtype, rtol, in_dim, out_dim, batch):
+    """forward_logits / backward_logits = softmax + forward / backward_w + softmax backward."""
+    g = torch.Generator().manual_seed(batch)
+    x = torch.rand(in_dim, batch, generator=g, dtype=torch.float64)
+    a = torch.randint(0, in_dim, (out_dim,), generator=g)
+    b = torch.randint(0, in_dim, (out_dim,), generator=g)
+    logits = (3 * torch.randn(out_dim, 16, generator=g, dtype=torch.float64)).requires_grad_(True)
+    gy = torch.randn(out_dim, batch, generator=g, dtype=torch.float64)
+    xq, lq, gq = x.to(dtype), logits.detach().to(dtype), gy.to(dtype)
+    want_p = torch.softmax(lq.double(), -1)
+    want_y = fo.ext_forward(xq.double(), a, b, want_p)
+    y, probs = ext.forward_logits(xq.cuda(), a.cuda(), b.cuda(), lq.cuda())
+    assert y.dtype == dtype and probs.shape == (out_dim, 16)
+    assert close(probs, want_p, rtol)[0] and close(y, want_y, rtol)[0]
+    lw = lq.double().clone().requires_grad_(True)
+    yy = fo.layer_forward_sequential(xq.double().t(), a, b, torch.softmax(lw, -1))
+    want_g, = torch.autograd.grad(yy, lw, gq.double().t())
+    got_g = ext.backward_logits(xq.cuda(), a.cuda(), b.cuda(), gq.cuda(), probs)
+    ok, err = close(got_g, want_g, 2 * rtol)
+    assert ok, err
+    assert torch.equal(got_g, ext.backward_logits(xq.cuda(), a.cuda(), b.cuda(), gq.cuda(), probs))
