@@ -63,7 +63,8 @@ def packed_bench(args, torch, dl):
     x = torch.rand(B, F, device="cuda", generator=g) < 0.2
 
     ext = dl.difflogic_cuda
-    names = ("tensor_packbits_batch_major", "eval", "eval_fused", "eval_fused_groupbitsum", "groupbitsum")
+    names = ("tensor_packbits_batch_major", "eval", "eval_fused", "eval_chained", "eval_fused_groupbitsum",
+             "groupbitsum")
     real = {n: getattr(ext, n) for n in names}
     launches = []          # (kernel label, algorithmic bytes, start_event, end_event)
     record = {"on": False}
@@ -79,7 +80,8 @@ def packed_bench(args, torch, dl):
             return "eval %d->%d" % (a[0].shape[0], a[3].shape[0]), eval_layer_bytes(a[0].shape[0], a[3].shape[0], W)
         dims = [a[0].shape[0]] + [l[2].shape[0] for l in a[1]]
         by = sum(eval_layer_bytes(i, o, W) for i, o in zip(dims[:-1], dims[1:]))
-        label = "eval_fused x%d %s" % (len(a[1]), "->".join(str(d) for d in dims))
+        label = "%s x%d %s" % (name if name != "eval_fused_groupbitsum" else "eval_fused", len(a[1]),
+                               "->".join(str(d) for d in dims))
         if name == "eval_fused_groupbitsum":
             by += 8 * W * dims[-1] + 4 * k * B
             label += " +groupbitsum"

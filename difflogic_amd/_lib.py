@@ -36,11 +36,16 @@ SIGNATURES = {
     "dl_groupbitsum": [_vp, _vp, _i64, _i64, _int, _i64, _i64, _vp],
     "dl_logic_eval_fused_workspace_bytes": [_int, _i64],
     "dl_logic_eval_fused": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _vp, _vp],
+    "dl_eval_schedule_chunk": [],
+    "dl_eval_schedule_capacity": [_i64, _int],
+    "dl_eval_schedule_build": [_vp, _vp, _i64, _i64, _int, _vp, _vp, _vp],
+    "dl_logic_eval_chained": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _int, _vp, _vp],
     "dl_logic_eval_fused_groupbitsum_workspace_bytes": [_int, _i64, _i64, _int, _i64],
     "dl_logic_eval_fused_groupbitsum": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _i64, _vp, _vp],
 }
 _RESTYPES = {"dl_status_string": ctypes.c_char_p, "dl_group_sum_workspace_bytes": ctypes.c_int64,
              "dl_logic_eval_fused_workspace_bytes": ctypes.c_int64,
+             "dl_eval_schedule_capacity": ctypes.c_int64, "dl_eval_schedule_build": ctypes.c_int64,
              "dl_logic_eval_fused_groupbitsum_workspace_bytes": ctypes.c_int64}
 
 _lib = None

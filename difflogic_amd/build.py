@@ -12,7 +12,7 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB_NAME = "libdifflogic_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ("packed.hip", "train.hip")
+SOURCES = ("packed.hip", "train.hip", "schedule.cpp")
 
 HIPCC_FLAGS = (
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared", "-fvisibility=default",

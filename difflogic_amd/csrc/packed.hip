@@ -200,6 +200,95 @@ __global__ __launch_bounds__(DL_BLOCK) void eval_tree_kernel(const V *__restrict
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// Chained variant of eval_tree_kernel.  The group's top layer is walked along the trails of an
+// evaluation schedule (schedule.cpp): consecutive top-layer neurons share one input, whose value
+// (a depth-DS subtree over 2^DS gathered rows; DS = 0: the input row itself) stays in registers,
+// so a neuron costs 2^DS gathers instead of 2^(DS+1).  One wave = CHUNK consecutive steps x 64
+// vectors; the first vertex of a chunk is evaluated again (CHUNK + 1 subtrees per chunk).
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t swap_gate_inputs(uint32_t op) {   // f'(a, b) = f(b, a)
+    return (op & 9u) | ((op & 4u) >> 1) | ((op & 2u) << 1);
+}
+
+template <typename V, int DS> struct Subtree {
+    int32_t leaf[1 << DS];
+    uint64_t gates;
+    __device__ __forceinline__ void locate(int32_t vertex, const int32_t *__restrict__ sub_leaves,
+                                           const uint64_t *__restrict__ sub_gates) {
+        gates = sub_gates[vertex];
+#pragma unroll
+        for (int g = 0; g < (1 << DS); ++g) leaf[g] = sub_leaves[(int64_t) vertex * (1 << DS) + g];
+    }
+    __device__ __forceinline__ void gather(const V *__restrict__ xcol, int64_t ncols, V *v) const {
+#pragma unroll
+        for (int g = 0; g < (1 << DS); ++g) v[g] = xcol[(int64_t) leaf[g] * ncols];
+    }
+};
+template <typename V> struct Subtree<V, 0> {
+    int32_t leaf[1];
+    uint64_t gates;
+    __device__ __forceinline__ void locate(int32_t vertex, const int32_t *, const uint64_t *) {
+        leaf[0] = vertex;
+        gates = 0;
+    }
+    __device__ __forceinline__ void gather(const V *__restrict__ xcol, int64_t ncols, V *v) const {
+        v[0] = xcol[(int64_t) leaf[0] * ncols];
+    }
+};
+
+template <typename V, int DS, int CHUNK, int ITERS>
+__global__ __launch_bounds__(DL_BLOCK) void eval_chain_kernel(const V *__restrict__ x,
+                                                              const int32_t *__restrict__ sub_leaves,
+                                                              const uint64_t *__restrict__ sub_gates,
+                                                              const int32_t *__restrict__ verts,
+                                                              const int32_t *__restrict__ neuron,
+                                                              const uint8_t *__restrict__ flip,
+                                                              const uint8_t *__restrict__ w_top, V *__restrict__ y,
+                                                              int64_t nchunks, int64_t ncols) {
+    constexpr int G = 1 << DS;
+    static_assert(CHUNK % 2 == 0, "steps are processed in pairs");
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t c_first = ((int64_t) blockIdx.x * 4 + wave) * ITERS;
+
+    for (int64_t ct = blockIdx.y; ct * DL_WAVE < ncols; ct += gridDim.y) {
+        const int64_t col = ct * DL_WAVE + lane;
+        if (col >= ncols) continue;
+        const V *xcol = x + col;
+        V *ycol = y + col;
+#pragma unroll 1
+        for (int it = 0; it < ITERS; ++it) {
+            const int64_t c = c_first + it;
+            if (c >= nchunks) break;
+            const int64_t s0 = c * CHUNK;
+            Subtree<V, DS> first;
+            first.locate(verts[s0], sub_leaves, sub_gates);
+            V leaves0[G];
+            first.gather(xcol, ncols, leaves0);
+            V prev = TreeFold<V, DS>::run(leaves0, first.gates);
+#pragma unroll
+            for (int j = 0; j < CHUNK; j += 2) {
+                Subtree<V, DS> ta, tb;
+                ta.locate(verts[s0 + j + 1], sub_leaves, sub_gates);
+                tb.locate(verts[s0 + j + 2], sub_leaves, sub_gates);
+                const int32_t na = neuron[s0 + j], nb = neuron[s0 + j + 1];
+                uint32_t oa = w_top[na >= 0 ? na : 0], ob = w_top[nb >= 0 ? nb : 0];
+                if (flip[s0 + j]) oa = swap_gate_inputs(oa);
+                if (flip[s0 + j + 1]) ob = swap_gate_inputs(ob);
+                V la[G], lb[G];
+                ta.gather(xcol, ncols, la);
+                tb.gather(xcol, ncols, lb);
+                const V va = TreeFold<V, DS>::run(la, ta.gates);
+                const V vb = TreeFold<V, DS>::run(lb, tb.gates);
+                if (na >= 0) __builtin_nontemporal_store(gate_apply<V>(prev, va, gate_masks(oa)), ycol + (int64_t) na * ncols);
+                if (nb >= 0) __builtin_nontemporal_store(gate_apply<V>(va, vb, gate_masks(ob)), ycol + (int64_t) nb * ncols);
+                prev = vb;
+            }
+        }
+    }
+}
+
 template <typename V, int NPW, int ITERS>
 int launch_eval(const void *x, const int64_t *a, const int64_t *b, const uint8_t *w, void *y, int64_t out_dim,
                 int64_t row_bytes, hipStream_t stream) {
@@ -947,4 +1036,61 @@ extern "C" int64_t dl_logic_eval_fused_groupbitsum_workspace_bytes(int depth, in
     if (row_bytes % 8 != 0) return 0;
     const int64_t tables = dl_logic_eval_fused_workspace_bytes(depth, out_dim);
     return ((tables + 15) / 16) * 16 + count_scratch_bytes(out_dim, k, row_bytes);
+}
+
+#define DL_EVAL_SCHEDULE_CHUNK 8
+
+extern "C" int dl_eval_schedule_chunk(void) { return DL_EVAL_SCHEDULE_CHUNK; }
+
+template <typename V>
+int launch_eval_chain(int sub_depth, const void *x, const int32_t *sub_leaves, const uint64_t *sub_gates,
+                      const int32_t *verts, const int32_t *neuron, const uint8_t *flip, const uint8_t *w_top, void *y,
+                      int64_t nchunks, int64_t row_bytes, hipStream_t s) {
+    const int64_t ncols = row_bytes / (int64_t) sizeof(V);
+    int64_t ctiles = dl_ceil_div(ncols, DL_WAVE);
+    if (ctiles > 65535) ctiles = 65535;
+#define DL_CHAIN_LAUNCH(DS, ITERS)                                                                                     \
+    {                                                                                                                  \
+        const int64_t gx = dl_ceil_div(nchunks, 4 * ITERS);                                                            \
+        if (gx > 0x7fffffffLL) return DL_ERR_TOO_LARGE;                                                                \
+        hipLaunchKernelGGL((eval_chain_kernel<V, DS, DL_EVAL_SCHEDULE_CHUNK, ITERS>),                                  \
+                           dim3((unsigned) gx, (unsigned) ctiles), dim3(DL_BLOCK), 0, s, (const V *) x, sub_leaves,    \
+                           sub_gates, verts, neuron, flip, w_top, (V *) y, nchunks, ncols);                            \
+    }
+    switch (sub_depth) {
+    case 0: DL_CHAIN_LAUNCH(0, 2) break;
+    case 1: DL_CHAIN_LAUNCH(1, 2) break;
+    case 2: DL_CHAIN_LAUNCH(2, 1) break;
+    default: DL_CHAIN_LAUNCH(3, 1) break;
+    }
+#undef DL_CHAIN_LAUNCH
+    return dl_launch_status();
+}
+
+extern "C" int dl_logic_eval_chained(const void *x, int depth, const int64_t *const *a, const int64_t *const *b,
+                                     const uint8_t *const *w, const int64_t *dims, const int32_t *verts,
+                                     const int32_t *neuron, const uint8_t *flip, int64_t steps, void *y, int64_t words,
+                                     int bit_count, void *workspace, void *stream) {
+    if (!valid_bit_count(bit_count)) return DL_ERR_BIT_COUNT;
+    if (depth < 1 || depth > DL_MAX_FUSE_DEPTH || !dims || !w || words < 0 || steps < 0 ||
+        steps % DL_EVAL_SCHEDULE_CHUNK != 0)
+        return DL_ERR_INVALID_ARGUMENT;
+    if (words == 0 || dims[depth] == 0) return DL_OK;
+    if (!x || !y || !verts || !neuron || !flip || !w[depth - 1] || steps < dims[depth]) return DL_ERR_INVALID_ARGUMENT;
+    const int64_t row_bytes = words * (bit_count / 8);
+    const uintptr_t mis = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) | (uintptr_t) row_bytes;
+    if (mis % 8 != 0) return DL_ERR_TOO_LARGE;       // rows are not whole 64-bit words: use dl_logic_eval per layer
+    hipStream_t s = (hipStream_t) stream;
+    int32_t *sub_leaves = nullptr;
+    uint64_t *sub_gates = nullptr;
+    if (depth > 1) {                                 // flatten the layers below the top one, per vertex
+        const int st = compose_tree(depth - 1, a, b, w, dims, workspace, &sub_leaves, &sub_gates, s);
+        if (st != DL_OK) return st;
+    }
+    const int64_t nchunks = steps / DL_EVAL_SCHEDULE_CHUNK;
+    if (mis % 16 == 0)
+        return launch_eval_chain<dl_u32x4>(depth - 1, x, sub_leaves, sub_gates, verts, neuron, flip, w[depth - 1], y,
+                                           nchunks, row_bytes, s);
+    return launch_eval_chain<dl_u32x2>(depth - 1, x, sub_leaves, sub_gates, verts, neuron, flip, w[depth - 1], y, nchunks,
+                                       row_bytes, s);
 }

@@ -330,6 +330,79 @@ def eval_fused(x, layers):
     return y
 
 
+class EvalSchedule:
+    """Device-resident evaluation schedule of one layer's wiring (see eval_chained): the order in
+    which dl_logic_eval_chained walks the layer's neurons so that consecutive ones share an
+    input.  Built on the host from (a, b); depends on nothing else."""
+
+    def __init__(self, a, b, in_dim):
+        import numpy as np
+        lib = _lib.load()
+        a_h = np.ascontiguousarray(a.detach().cpu().numpy(), dtype=np.int64)
+        b_h = np.ascontiguousarray(b.detach().cpu().numpy(), dtype=np.int64)
+        out_dim = a_h.shape[0]
+        chunk = lib.dl_eval_schedule_chunk()
+        cap = lib.dl_eval_schedule_capacity(out_dim, chunk)
+        verts = np.empty(cap + 1, dtype=np.int32)
+        neuron = np.empty(cap, dtype=np.int32)
+        flip = np.empty(cap, dtype=np.uint8)
+        steps = lib.dl_eval_schedule_build(a_h.ctypes.data, b_h.ctypes.data, int(in_dim), out_dim, chunk,
+                                           verts.ctypes.data, neuron.ctypes.data, flip.ctypes.data)
+        if steps < 0:
+            _raise(-steps, "eval_schedule_build")
+        self.in_dim, self.out_dim, self.steps, self.chunk = int(in_dim), out_dim, int(steps), chunk
+        self.verts = torch.from_numpy(verts[:steps + 1].copy()).to(a.device)
+        self.neuron = torch.from_numpy(neuron[:steps].copy()).to(a.device)
+        self.flip = torch.from_numpy(flip[:steps].copy()).to(a.device)
+        self._wiring = (a, b)        # keeps the tensors (and their addresses) alive while cached
+
+
+_SCHEDULES = {}                      # (ptr a, ptr b, versions, in_dim) -> EvalSchedule, most recent last
+_SCHEDULES_MAX = 64
+
+
+def schedule_for(a, b, in_dim):
+    """The cached EvalSchedule of the wiring (a, b), rebuilt when the tensors are replaced or
+    modified in place."""
+    key = (a.data_ptr(), b.data_ptr(), a._version, b._version, int(in_dim), a.shape[0])
+    sched = _SCHEDULES.pop(key, None)
+    if sched is None:
+        sched = EvalSchedule(a, b, in_dim)
+        while len(_SCHEDULES) >= _SCHEDULES_MAX:
+            _SCHEDULES.pop(next(iter(_SCHEDULES)))
+    _SCHEDULES[key] = sched
+    return sched
+
+
+def eval_chained(x, layers, schedule=None):
+    """Same result as ``eval_fused(x, layers)``; the group's top layer is walked along
+    ``schedule`` (default: the cached schedule of its wiring), which halves the rows gathered per
+    neuron.  Not part of the reference's extension.  Falls back to eval_fused where it does not
+    apply."""
+    dev, bits, depth, pa, pb, pw, pdims, dims = _fused_args(x, layers)
+    if depth > MAX_FUSE_DEPTH:
+        raise RuntimeError(f"at most {MAX_FUSE_DEPTH} layers can be fused, got {depth}")
+    words = x.shape[1]
+    if 0 in dims or words == 0:
+        return eval_fused(x, layers)
+    if schedule is None:
+        schedule = schedule_for(layers[-1][0], layers[-1][1], dims[-2])
+    if schedule.in_dim != dims[-2] or schedule.out_dim != dims[-1]:
+        raise RuntimeError(f"schedule is for a {schedule.in_dim}->{schedule.out_dim} layer, the group ends in "
+                           f"{dims[-2]}->{dims[-1]}")
+    y = torch.empty((dims[-1], words), dtype=x.dtype, device=dev)
+    ws = _fused_workspace(depth - 1, dims[-2], dev) if depth > 1 else None
+    with torch.cuda.device(dev):
+        st = _lib.load().dl_logic_eval_chained(_p(x), depth, pa, pb, pw, pdims, _p(schedule.verts), _p(schedule.neuron),
+                                               _p(schedule.flip), schedule.steps, _p(y), words, bits,
+                                               _p(ws) if ws is not None else None, _stream(dev))
+    if st == _lib.DL_ERR_TOO_LARGE:
+        return eval_fused(x, layers)
+    if st:
+        _raise(st, "logic_layer_cuda_eval_chained")
+    return y
+
+
 def eval_fused_groupbitsum(x, layers, pad_len, k):
     """groupbitsum(eval(... eval(x, layer 0) ..., last layer), pad_len, k) for the net's last
     one or two layers without materialising their output.  Not part of the reference's

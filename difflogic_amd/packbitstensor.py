@@ -10,28 +10,37 @@ from . import difflogic_cuda
 _L2_RESIDENT_ROWS = 2048
 
 
+def _chained(depth):
+    """Groups of two or more layers run along the top layer's evaluation schedule."""
+    return depth >= 2
+
+
 def plan_groups(dims, count_at_end):
     """Splits consecutive layers into fused groups.
 
     ``dims`` = [in_dim, width_1, ..., width_L].  Returns a list of group sizes summing to L; when
     ``count_at_end`` the last group is the one fused with the bit count.  Chosen by dynamic
-    programming over a traffic model in units of one activation row: a group of depth D gathers
-    2^D rows per output neuron (from L2 when its input has few rows, through the memory fabric
-    otherwise) and writes one row per output neuron unless it ends in the count."""
+    programming over a traffic model: a group of depth D gathers 2^D rows per output neuron,
+    2^(D-1) when it runs chained, from L2 when its input has few rows and through the memory fabric
+    otherwise, and writes one row per output neuron unless it ends in the count."""
     n = len(dims) - 1
     if n == 0:
         return []
 
     def cost(first, depth, last):
+        # milliseconds per 64000 rows of 16384 words, fitted to launches measured on MI355X
         rows_in, out = dims[first], dims[first + depth]
+        counted = last and count_at_end
         gathers = (1 << depth) * out
-        written = 0 if (last and count_at_end) else out
-        if rows_in <= _L2_RESIDENT_ROWS:
-            t = max(gathers / 27.0, written / 5.6)
-        else:
-            t = max((gathers + written) / 7.9, (rows_in + written) / 5.0)
-        if last and count_at_end:
-            t *= 1.25                 # the vertical counters share the kernel
+        if _chained(depth) and not counted:
+            gathers = gathers * 9 / 16             # half, plus one extra subtree per chunk of 8
+        written = 0 if counted else out
+        if rows_in <= _L2_RESIDENT_ROWS:           # gathers hit in L2; writes stream to HBM
+            t = max(1.5 * written, 0.3 * gathers + 0.5 * out)
+        else:                                      # L2 <-> fabric traffic, with the HBM copy rate as floor
+            t = max(1.1 * (gathers + written), 1.68 * (rows_in + written))
+        if counted:
+            t += 0.2 * out                         # second pass over the partial counters
         return t
 
     best = [(0.0, [])] + [None] * n    # best[i] = (cost, groups) for the first i layers
@@ -83,7 +92,8 @@ class PackBitsTensor:
     def _run_groups(self, groups):
         pos = 0
         for depth in groups:
-            self._t = difflogic_cuda.eval_fused(self._t, self._pending[pos:pos + depth])
+            run = difflogic_cuda.eval_chained if _chained(depth) else difflogic_cuda.eval_fused
+            self._t = run(self._t, self._pending[pos:pos + depth])
             pos += depth
         self._pending = self._pending[pos:]
 

@@ -148,6 +148,29 @@ int dl_logic_eval_fused(const void *x, int depth, const int64_t *const *a, const
                         const uint8_t *const *w, const int64_t *dims, void *y, int64_t words,
                         int bit_count, void *workspace, void *stream);
 
+/* Same result as dl_logic_eval_fused, computed along an evaluation schedule of the group's top
+ * layer: its neurons are ordered so that consecutive ones share an input, whose value (a subtree
+ * of depth-1 layers over 2^(depth-1) gathered rows) stays in registers; a neuron then costs
+ * 2^(depth-1) gathers instead of 2^depth.  No counterpart in the reference.  The schedule
+ * depends only on the top layer's wiring; build it once per layer.
+ *   dl_eval_schedule_chunk()      steps one wave walks at a time (the step count is a multiple)
+ *   dl_eval_schedule_capacity()   upper bound of steps for out_dim neurons
+ *   dl_eval_schedule_build()      HOST pointers in and out.  a, b [out_dim] (the top layer's wiring)
+ *                                 are validated against in_dim.  Writes verts [steps + 1],
+ *                                 neuron [steps] (-1 = no output at this step), flip [steps];
+ *                                 returns the number of steps, or a negated dl_status.
+ *   dl_logic_eval_chained()       as dl_logic_eval_fused plus the DEVICE schedule arrays; workspace
+ *                                 of dl_logic_eval_fused_workspace_bytes(depth-1, dims[depth-1])
+ *                                 bytes (none needed for depth 1). */
+int dl_eval_schedule_chunk(void);
+int64_t dl_eval_schedule_capacity(int64_t out_dim, int chunk);
+int64_t dl_eval_schedule_build(const int64_t *a, const int64_t *b, int64_t in_dim, int64_t out_dim,
+                               int chunk, int32_t *verts, int32_t *neuron, uint8_t *flip);
+int dl_logic_eval_chained(const void *x, int depth, const int64_t *const *a, const int64_t *const *b,
+                          const uint8_t *const *w, const int64_t *dims, const int32_t *verts,
+                          const int32_t *neuron, const uint8_t *flip, int64_t steps, void *y,
+                          int64_t words, int bit_count, void *workspace, void *stream);
+
 /* The net's last `depth` (1 or 2) layers fused with `groupbitsum` (the sequence
  * difflogic/difflogic.py:147 then difflogic/packbitstensor.py:22): the last layer's output words
  * are counted as they are produced and never written.  Arguments as dl_logic_eval_fused, result

@@ -286,3 +286,64 @@ def test_lazy_pack_tensor_keeps_t_current():
     assert np.array_equal(got.cpu().numpy(), po.groupbitsum(t, p.pad_len, 3))
     p2.t = torch.zeros_like(p2.t)
     assert int(p2.group_sum(3).sum()) == 0
+
+
+@pytest.mark.parametrize("bits,in_dim,widths,W,kind", [
+    (64, 64, [64], 130, "random"), (64, 100, [100, 100], 3, "random"), (64, 30, [200, 200, 200], 64, "random"),
+    (32, 50, [60, 70], 7, "unique"), (8, 7, [20, 20], 16, "any"), (64, 5, [3, 3], 5, "self"),
+    (64, 784, [6000, 6000, 6000, 6000], 64, "random"), (64, 3000, [3000, 3000], 128, "random"),
+    (64, 40, [80, 80, 80, 80], 9, "any"), (64, 500, [64000], 16, "random"),
+])
+def test_eval_chained_equals_eval_fused(ext, bits, in_dim, widths, W, kind):
+    from oracle import connections as oc
+    rng = np.random.default_rng(in_dim + len(widths) + W)
+    torch.manual_seed(in_dim)
+    layers, d = [], in_dim
+    for o in widths:
+        if kind == "random":
+            a, b = (t.numpy() for t in oc.random_connections(d, o))
+        elif kind == "unique":
+            a, b = (t.numpy() for t in oc.unique_connections(d, o))
+        elif kind == "self":
+            a, b = np.array([1, 1, 2]), np.array([1, 1, 2])
+        else:
+            a, b = rng.integers(0, d, o), rng.integers(0, d, o)
+        layers.append((a.astype(np.int64), b.astype(np.int64), rng.integers(0, 16, o).astype(np.uint8)))
+        d = o
+    x = rng.integers(np.iinfo(NP_WORD[bits]).min, np.iinfo(NP_WORD[bits]).max, (in_dim, W), dtype=NP_WORD[bits],
+                     endpoint=True)
+    want = x
+    for a, b, op in layers:
+        want = po.eval_layer(want, a, b, op)
+    dev_layers = [tuple(_dev(t) for t in l) for l in layers]
+    got = ext.eval_chained(_dev(x), dev_layers)
+    assert got.dtype == torch.as_tensor(want).dtype and np.array_equal(got.cpu().numpy(), want)
+    sched = ext.schedule_for(dev_layers[-1][0], dev_layers[-1][1], (in_dim if len(widths) == 1 else widths[-2]))
+    assert sched.steps % sched.chunk == 0 and sched.steps >= widths[-1]
+    assert ext.schedule_for(dev_layers[-1][0], dev_layers[-1][1], sched.in_dim) is sched         # cached
+
+
+def test_eval_schedule_rejects_bad_wiring(ext):
+    with pytest.raises(RuntimeError):
+        ext.EvalSchedule(torch.tensor([0, 5]).cuda(), torch.tensor([1, 1]).cuda(), 3)
+
+
+def test_schedule_follows_in_place_wiring_changes():
+    import difflogic_amd as dl
+    rng = np.random.default_rng(8)
+    F = 300
+    layers = random_layers(rng, F, [600, 600, 600])
+    x = rng.random((130, F)) < 0.5
+    model = build_model(F, layers, 10).eval()
+    with torch.no_grad():
+        got = model(dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=64)).cpu().numpy()
+    assert np.array_equal(got, interp.net_eval(x, layers, 10, threads=4))
+    layers2 = random_layers(rng, F, [600, 600, 600])
+    for m, (a, b, op) in zip([model[1], model[2], model[3]], layers2):
+        m.indices[0].copy_(torch.as_tensor(a))              # in place: same storage, new version
+        m.indices[1].copy_(torch.as_tensor(b))
+        with torch.no_grad():
+            m.weights.copy_(torch.nn.functional.one_hot(torch.as_tensor(op).long(), 16).float())
+    with torch.no_grad():
+        got2 = model(dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=64)).cpu().numpy()
+    assert np.array_equal(got2, interp.net_eval(x, layers2, 10, threads=4))

