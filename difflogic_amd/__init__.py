@@ -1,7 +1,7 @@
 """difflogic's LogicLayer kernel family for AMD MI355X (gfx950).
 
 Same Python API as the reference package (difflogic/__init__.py:1-3): ``LogicLayer``,
-``GroupSum`` and ``PackBitsTensor``; ``difflogic_amd.difflogic_cuda`` stands in for the
+``GroupSum``, ``PackBitsTensor`` and ``CompiledLogicNet``; ``difflogic_amd.difflogic_cuda`` stands in for the
 reference's extension module of that name.  Importing the package loads
 libdifflogic_hip.so; it raises ImportError if the library has not been built.
 """
@@ -12,5 +12,6 @@ _lib.load()
 from . import difflogic_cuda  # noqa: E402
 from .difflogic import GroupSum, LogicLayer  # noqa: E402
 from .packbitstensor import PackBitsTensor  # noqa: E402
+from .compiled_model import CompiledLogicNet  # noqa: E402
 
-__all__ = ["LogicLayer", "GroupSum", "PackBitsTensor", "difflogic_cuda"]
+__all__ = ["LogicLayer", "GroupSum", "PackBitsTensor", "CompiledLogicNet", "difflogic_cuda"]
