@@ -113,8 +113,16 @@ class LogicLayer(torch.nn.Module):
         assert isinstance(x, PackBitsTensor)
         assert x.features == self.in_dim, (x.features, self.in_dim)
         a, b = self.indices
-        w = self.weights.argmax(-1).to(torch.uint8)
-        return x.defer_layer(a, b, w)
+        return x.defer_layer(a, b, self._gate_ids())
+
+    def _gate_ids(self):
+        """uint8 [out_dim] argmax gate per neuron, recomputed only when ``weights`` changed."""
+        key = (self.weights.data_ptr(), self.weights._version)
+        cached = getattr(self, "_gate_ids_cache", None)
+        if cached is None or cached[0] != key:
+            cached = (key, self.weights.detach().argmax(-1).to(torch.uint8))
+            self._gate_ids_cache = cached
+        return cached[1]
 
     def extra_repr(self):
         return "{}, {}, {}".format(self.in_dim, self.out_dim, "train" if self.training else "eval")
