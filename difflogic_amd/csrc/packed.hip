@@ -437,6 +437,67 @@ __global__ __launch_bounds__(DL_BLOCK) void packbits_batch_major_kernel(const ui
     }
 }
 
+// Variant for narrow inputs (features % 16 == 0, staging + result tile within 64 KB of LDS): the 64 sample rows of one
+// word column are one contiguous block of the input, which the workgroup copies into LDS with
+// fully coalesced 16-byte loads (no partial cache lines however the rows fall), then every
+// thread folds one group of four features from LDS exactly as above.  WC word columns per
+// workgroup, so that a feature row is written in runs of 8 * WC bytes.
+template <int WC>
+__global__ __launch_bounds__(DL_BLOCK) void packbits_batch_major_lds_kernel(const uint8_t *__restrict__ x,
+                                                                            uint8_t *__restrict__ out, int64_t batch,
+                                                                            int64_t features,
+                                                                            int64_t out_row_bytes) {
+    extern __shared__ __align__(16) uint8_t lds_raw[];
+    dl_u32x4 *stage = reinterpret_cast<dl_u32x4 *>(lds_raw);                        // 64 * features bytes
+    uint64_t *words = reinterpret_cast<uint64_t *>(lds_raw + 64 * features);         // [features][WC]
+    const int64_t w0 = (int64_t) blockIdx.x * WC;
+    const int groups = (int) (features / 4);                                         // dword columns
+    const int chunks = (int) (4 * features);                                         // 16-byte chunks per word column
+
+    for (int wc = 0; wc < WC; ++wc) {
+        const int64_t s0 = (w0 + wc) * 64;
+        if (s0 >= batch) break;                                                      // uniform
+        const int64_t valid = (batch - s0 < 64 ? batch - s0 : 64) * features / 16;   // chunks holding real samples
+        const dl_u32x4 *src = reinterpret_cast<const dl_u32x4 *>(x + s0 * features);
+        __syncthreads();                                                             // previous column's readers are done
+        for (int i = threadIdx.x; i < chunks; i += DL_BLOCK)
+            stage[i] = i < valid ? __builtin_nontemporal_load(src + i) : dl_u32x4{0, 0, 0, 0};
+        __syncthreads();
+        const uint32_t *flags = reinterpret_cast<const uint32_t *>(lds_raw);
+        for (int g = threadIdx.x; g < groups; g += DL_BLOCK) {
+            uint32_t oct[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                uint32_t acc = 0;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint32_t v = flags[(8 * j + i) * groups + g];
+                    acc |= (((((v & 0x7f7f7f7fu) + 0x7f7f7f7fu) | v) >> 7) & 0x01010101u) << i;
+                }
+                oct[j] = acc;
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                uint32_t lo = 0, hi = 0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    lo |= ((oct[j] >> (8 * k)) & 0xffu) << (8 * j);
+                    hi |= ((oct[4 + j] >> (8 * k)) & 0xffu) << (8 * j);
+                }
+                words[(4 * g + k) * WC + wc] = ((uint64_t) hi << 32) | lo;
+            }
+        }
+    }
+    __syncthreads();
+    // WC consecutive threads write the WC words of one feature row (out_row_bytes % 8 == 0 here)
+    const int64_t total_words = out_row_bytes / 8;
+    for (int i = threadIdx.x; i < (int) features * WC; i += DL_BLOCK) {
+        const int f = i / WC, wc = i - f * WC;
+        if (w0 + wc < total_words)
+            *reinterpret_cast<uint64_t *>(out + (int64_t) f * out_row_bytes + (w0 + wc) * 8) = words[f * WC + wc];
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 // Vertical bit count (GroupSum on packed words).  For each class (a contiguous block of
 // per_class neuron rows) and each sample bit, the number of rows with that bit set.
@@ -933,7 +994,15 @@ extern "C" int dl_tensor_packbits_batch_major(const uint8_t *x, void *out, int64
     if (out_row_bytes % 8 == 0 && !dl_aligned(out, 8)) return DL_ERR_INVALID_ARGUMENT;
     const int64_t gx = dl_ceil_div(dl_ceil_div(batch, 64), 16);
     if (gx > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
-    if (features % 4 == 0 && dl_aligned(x, 4)) {
+    constexpr int WC = 2;
+    const bool fits_lds = 64 * features + features * WC * 8 <= 65536;      // default dynamic LDS limit
+    if (features % 16 == 0 && fits_lds && dl_aligned(x, 16) && out_row_bytes % 8 == 0) {
+        const int64_t blocks = dl_ceil_div(dl_ceil_div(batch, 64), WC);
+        if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+        const size_t lds = (size_t) (64 * features + features * WC * 8);
+        hipLaunchKernelGGL(packbits_batch_major_lds_kernel<WC>, dim3((unsigned) blocks), dim3(DL_BLOCK), lds, s, x,
+                           (uint8_t *) out, batch, features, out_row_bytes);
+    } else if (features % 4 == 0 && dl_aligned(x, 4)) {
         const int64_t gy = dl_ceil_div(features, 256);
         if (gy > 65535) return DL_ERR_TOO_LARGE;
         hipLaunchKernelGGL(packbits_batch_major_kernel<4>, dim3((unsigned) gx, (unsigned) gy), dim3(DL_BLOCK), 0, s, x,
