@@ -188,7 +188,8 @@ def cpu_baseline(args, model, x, dl):
 def train_bench(args, torch, dl):
     """fp32 forward + backward of 784 -> 6 x 64000 -> GroupSum(10, tau 30), B = 512, 'unique'
     connections, grad_factor 1, CrossEntropy.  Reports the whole step (eager and replayed as one
-    HIP graph) and each layer kernel timed alone (back-to-back launches on a 64000 -> 64000 layer)
+    HIP graph) and each layer kernel timed alone (back-to-back launches on a 64000 -> 64000 layer,
+    forward and backward_w in their chained form, as the layer runs them)
     against its algorithmic bytes: forward 4B(in+out)+80 out, backward_w 4B(in+out)+64 out,
     backward_x 4B(2 in+out)+64 out."""
     F, width, L, k, B = 784, 64000, 6, 10, 512
@@ -229,9 +230,10 @@ def train_bench(args, torch, dl):
     logits = layer.weights.detach()
     _, probs = ext.forward_logits(xs, a, b, logits)
     start, idx = layer.given_x_indices_of_y_start, layer.given_x_indices_of_y
+    sched = layer._train_schedule()
     calls = {
-        "forward_logits": (lambda: ext.forward_logits(xs, a, b, logits), 4 * B * 2 * width + 80 * width),
-        "backward_logits": (lambda: ext.backward_logits(xs, a, b, gy, probs), 4 * B * 2 * width + 64 * width),
+        "forward_logits": (lambda: ext.forward_logits(xs, a, b, logits, sched), 4 * B * 2 * width + 80 * width),
+        "backward_logits": (lambda: ext.backward_logits(xs, a, b, gy, probs, sched), 4 * B * 2 * width + 64 * width),
         "backward_x": (lambda: ext.backward_x(xs, a, b, probs, gy, start, idx), 4 * B * 3 * width + 64 * width),
     }
     kernels = {}

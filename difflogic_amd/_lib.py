@@ -26,6 +26,8 @@ SIGNATURES = {
     "dl_logic_backward_w": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "dl_logic_forward_logits": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "dl_logic_backward_logits": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
+    "dl_logic_forward_chained": [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
+    "dl_logic_backward_w_chained": [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "dl_logic_backward_x": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _dbl, _int, _vp],
     "dl_group_sum_workspace_bytes": [_i64, _i64, _i64, _int],
     "dl_group_sum_forward": [_vp, _vp, _vp, _i64, _i64, _i64, _dbl, _int, _vp],

@@ -16,6 +16,9 @@ SOURCES = ("packed.hip", "train.hip", "schedule.cpp")
 
 HIPCC_FLAGS = (
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared", "-fvisibility=default",
+    # no automatic mul+add fusion: kernels that state the same arithmetic give the same bits
+    # (the chained and unchained training kernels are checked for equality); fma is written out
+    "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 )
 

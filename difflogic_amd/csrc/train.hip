@@ -25,6 +25,16 @@ template <> __device__ __forceinline__ float up<__half>(__half v) { return __hal
 template <typename T, typename C> __device__ __forceinline__ T down(C v) { return (T) v; }
 template <> __device__ __forceinline__ __half down<__half, float>(float v) { return __float2half(v); }
 
+__device__ __forceinline__ float dl_fma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double dl_fma(double a, double b, double c) { return __builtin_fma(a, b, c); }
+
+// y = lerp(lerp(P00, P01, b), lerp(P10, P11, b), a), three fused multiply-adds.
+template <typename C> __device__ __forceinline__ C mix(C av, C bv, C p00, C p10, C d0, C d1) {
+    const C lo = dl_fma(bv, d0, p00);
+    const C hi = dl_fma(bv, d1, p10);
+    return dl_fma(av, hi - lo, lo);
+}
+
 // The four corner values of neuron n's gate mixture.
 template <typename C> struct Corners { C p00, p01, p10, p11; };
 
@@ -180,15 +190,35 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_kernel(const T *__restrict__
                 P r;
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
-                    const C av = up<T>(va[j].v[e]), bv = up<T>(vb[j].v[e]);
-                    const C lo = p00[j] + bv * d0[j];
-                    const C hi = p10[j] + bv * d1[j];
-                    r.v[e] = down<T, C>(lo + av * (hi - lo));
+                    r.v[e] = down<T, C>(mix<C>(up<T>(va[j].v[e]), up<T>(vb[j].v[e]), p00[j], p10[j], d0[j], d1[j]));
                 }
                 yv[(n0 + j) * ncols + col] = r;
             }
         }
     }
+}
+
+// Lane i < 16 holds gate i: its gradient is the sum of the corner sums at which gate i is true.
+// probs != nullptr chains the softmax backward, p_i * (g_i - sum_j p_j g_j).  Called by whole
+// waves (the 16-lane row sum needs every lane).
+template <typename T>
+__device__ __forceinline__ void store_grad_w(int lane, bool neuron_valid, int64_t n, typename Acc<T>::type s00,
+                                             typename Acc<T>::type s01, typename Acc<T>::type s10,
+                                             typename Acc<T>::type s11, const T *__restrict__ probs,
+                                             T *__restrict__ gw) {
+    typedef typename Acc<T>::type C;
+    const bool valid = lane < 16 && neuron_valid;
+    C r = (C) 0;
+    if (lane & 8) r += s00;
+    if (lane & 4) r += s01;
+    if (lane & 2) r += s10;
+    if (lane & 1) r += s11;
+    if (probs != nullptr) {
+        const C p = valid ? up<T>(probs[n * 16 + lane]) : (C) 0;
+        const C dot = row16_sum(p * r);
+        r = p * (r - dot);
+    }
+    if (valid) gw[n * 16 + lane] = down<T, C>(r);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -283,23 +313,9 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_w_kernel(const T *__restric
         }
     }
 
-    // lane i < 16 holds gate i: add the corners whose truth-table bit is set.
 #pragma unroll
-    for (int j = 0; j < NPW; ++j) {
-        const bool valid = lane < 16 && n0 + j < out_dim;
-        C r = (C) 0;
-        if (lane & 8) r += s00[j];
-        if (lane & 4) r += s01[j];
-        if (lane & 2) r += s10[j];
-        if (lane & 1) r += s11[j];
-        if (probs != nullptr) {
-            const C p = valid ? up<T>(probs[(n0 + j) * 16 + lane]) : (C) 0;
-            C dot = p * r;                           // summed over the 16-lane row, all lanes take part
-            dot = row16_sum(dot);
-            r = p * (r - dot);
-        }
-        if (valid) gw[(n0 + j) * 16 + lane] = down<T, C>(r);
-    }
+    for (int j = 0; j < NPW; ++j)
+        store_grad_w<T>(lane, n0 + j < out_dim, n0 + j, s00[j], s01[j], s10[j], s11[j], probs, gw);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -359,6 +375,145 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_x_kernel(const T *__restric
 #pragma unroll
         for (int q = 0; q < VEC; ++q) r.v[q] = down<T, C>(acc[q] * scale);
         ov[c * ncols + col] = r;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Chained forward / backward_w.  The layer's neurons are walked along the trails of an
+// evaluation schedule (schedule.cpp): step s brings in input row verts[s + 1] and evaluates
+// neuron[s] from (verts[s], verts[s + 1]); flip[s] tells which of the two is the neuron's `a`
+// input.  The shared row stays in registers, so a neuron costs one gathered row instead of two.
+// Arithmetic and summation order per element are those of the unchained kernels: the fp32 and
+// fp64 results are bit-identical (fp16 outputs can differ in the last bit, where the compiler
+// folds the final conversion into a fused multiply-add in one kernel and not in the other).
+// ------------------------------------------------------------------------------------------
+template <typename T, bool LOGITS>
+__device__ __forceinline__ void neuron_corners(const T *__restrict__ w, int64_t n, int lane, bool store_probs,
+                                               T *__restrict__ probs, typename Acc<T>::type &p00,
+                                               typename Acc<T>::type &p10, typename Acc<T>::type &d0,
+                                               typename Acc<T>::type &d1) {
+    typedef typename Acc<T>::type C;
+    Corners<C> c;
+    if (LOGITS) {
+        C g[16], mine;
+        softmax16<T>(w, n, lane, g, mine);
+        c = corners_of<C>(g);
+        if (store_probs && lane < 16) probs[n * 16 + lane] = down<T, C>(mine);
+    } else {
+        c = corners<T>(w, n);
+    }
+    p00 = c.p00;
+    p10 = c.p10;
+    d0 = c.p01 - c.p00;
+    d1 = c.p11 - c.p10;
+}
+
+template <typename T, int VEC, int CHUNK, bool LOGITS>
+__global__ __launch_bounds__(DL_BLOCK) void forward_chain_kernel(const T *__restrict__ x,
+                                                                 const int32_t *__restrict__ verts,
+                                                                 const int32_t *__restrict__ neuron,
+                                                                 const uint8_t *__restrict__ flip,
+                                                                 const T *__restrict__ w, T *__restrict__ y,
+                                                                 T *__restrict__ probs, int64_t nchunks, int64_t ncols) {
+    typedef typename Acc<T>::type C;
+    typedef Pack<T, VEC> P;
+    static_assert(CHUNK % 2 == 0, "steps are processed in pairs");
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t c = (int64_t) blockIdx.x * 4 + wave;
+    if (c >= nchunks) return;
+    const int64_t s0 = c * CHUNK;
+    const P *xv = reinterpret_cast<const P *>(x);
+    P *yv = reinterpret_cast<P *>(y);
+
+    for (int64_t ct = blockIdx.y; ct * DL_WAVE < ncols; ct += gridDim.y) {
+        const int64_t col = ct * DL_WAVE + lane;
+        const bool live = col < ncols;
+        const int64_t cl = live ? col : 0;
+        P prev = xv[(int64_t) verts[s0] * ncols + cl];
+#pragma unroll
+        for (int j = 0; j < CHUNK; j += 2) {
+            const int32_t v1 = verts[s0 + j + 1], v2 = verts[s0 + j + 2];
+            const int32_t n1 = neuron[s0 + j], n2 = neuron[s0 + j + 1];
+            const bool f1 = flip[s0 + j] != 0, f2 = flip[s0 + j + 1] != 0;
+            const P x1 = xv[(int64_t) v1 * ncols + cl], x2 = xv[(int64_t) v2 * ncols + cl];
+            C p00a, p10a, d0a, d1a, p00b, p10b, d0b, d1b;
+            neuron_corners<T, LOGITS>(w, n1 >= 0 ? n1 : 0, lane, n1 >= 0 && ct == 0, probs, p00a, p10a, d0a, d1a);
+            neuron_corners<T, LOGITS>(w, n2 >= 0 ? n2 : 0, lane, n2 >= 0 && ct == 0, probs, p00b, p10b, d0b, d1b);
+            P r1, r2;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const C u0 = up<T>(prev.v[e]), u1 = up<T>(x1.v[e]), u2 = up<T>(x2.v[e]);
+                r1.v[e] = down<T, C>(mix<C>(f1 ? u1 : u0, f1 ? u0 : u1, p00a, p10a, d0a, d1a));
+                r2.v[e] = down<T, C>(mix<C>(f2 ? u2 : u1, f2 ? u1 : u2, p00b, p10b, d0b, d1b));
+            }
+            if (live && n1 >= 0) yv[(int64_t) n1 * ncols + col] = r1;
+            if (live && n2 >= 0) yv[(int64_t) n2 * ncols + col] = r2;
+            prev = x2;
+        }
+    }
+}
+
+// One wave owns CHUNK steps and the whole batch: lane l holds vectors l, l + 64, ... (CPL of them).
+template <typename T, int VEC, int CPL, int CHUNK>
+__global__ __launch_bounds__(DL_BLOCK) void backward_w_chain_kernel(const T *__restrict__ x,
+                                                                    const int32_t *__restrict__ verts,
+                                                                    const int32_t *__restrict__ neuron,
+                                                                    const uint8_t *__restrict__ flip,
+                                                                    const T *__restrict__ gy,
+                                                                    const T *__restrict__ probs, T *__restrict__ gw,
+                                                                    int64_t nchunks, int64_t ncols) {
+    typedef typename Acc<T>::type C;
+    typedef Pack<T, VEC> P;
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t c = (int64_t) blockIdx.x * 4 + wave;
+    if (c >= nchunks) return;
+    const int64_t s0 = c * CHUNK;
+    const P *xv = reinterpret_cast<const P *>(x);
+    const P *gv = reinterpret_cast<const P *>(gy);
+    P zero;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) zero.v[e] = down<T, C>((C) 0);
+
+    auto load_row = [&](const P *base, int64_t row, P *dst) {
+#pragma unroll
+        for (int q = 0; q < CPL; ++q) {
+            const int64_t col = lane + q * DL_WAVE;
+            dst[q] = col < ncols ? base[row * ncols + col] : zero;
+        }
+    };
+    P prev[CPL];
+    load_row(xv, verts[s0], prev);
+#pragma unroll 1
+    for (int j = 0; j < CHUNK; ++j) {
+        const int32_t n = neuron[s0 + j];
+        const bool f = flip[s0 + j] != 0;
+        P cur[CPL], g[CPL];
+        load_row(xv, verts[s0 + j + 1], cur);
+        load_row(gv, n >= 0 ? n : 0, g);
+        C s00 = (C) 0, s01 = (C) 0, s10 = (C) 0, s11 = (C) 0;
+#pragma unroll
+        for (int q = 0; q < CPL; ++q) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const C u0 = up<T>(prev[q].v[e]), u1 = up<T>(cur[q].v[e]), gg = up<T>(g[q].v[e]);
+                const C av = f ? u1 : u0, bv = f ? u0 : u1;
+                const C ga = gg * av, gna = gg - ga;
+                const C t11 = ga * bv, t01 = gna * bv;
+                s11 += t11;
+                s10 += ga - t11;
+                s01 += t01;
+                s00 += gna - t01;
+            }
+        }
+        s00 = wave_sum(s00);
+        s01 = wave_sum(s01);
+        s10 = wave_sum(s10);
+        s11 = wave_sum(s11);
+        store_grad_w<T>(lane, n >= 0, n >= 0 ? n : 0, s00, s01, s10, s11, probs, gw);
+#pragma unroll
+        for (int q = 0; q < CPL; ++q) prev[q] = cur[q];
     }
 }
 
@@ -589,7 +744,85 @@ int group_sum_splits(int64_t out_dim, int64_t batch, int64_t k) {
     return (int) want;
 }
 
+#define DL_TRAIN_CHUNK 8     // must equal the chunk the schedule was built with (dl_eval_schedule_chunk)
+
+template <typename T, bool LOGITS>
+int forward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, const uint8_t *flip, int64_t steps,
+                    const void *w, void *y, void *probs, int64_t batch, hipStream_t s) {
+    constexpr int V = Vec16<T>::n;
+    if (batch % V != 0 || !dl_aligned(x, 16) || !dl_aligned(y, 16)) return DL_ERR_TOO_LARGE;
+    const int64_t nchunks = steps / DL_TRAIN_CHUNK, ncols = batch / V;
+    const int64_t blocks = dl_ceil_div(nchunks, 4);
+    if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    hipLaunchKernelGGL((forward_chain_kernel<T, V, DL_TRAIN_CHUNK, LOGITS>), dim3((unsigned) blocks, col_tiles(ncols)),
+                       dim3(DL_BLOCK), 0, s, (const T *) x, verts, neuron, flip, (const T *) w, (T *) y, (T *) probs,
+                       nchunks, ncols);
+    return dl_launch_status();
+}
+
+template <typename T>
+int backward_w_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, const uint8_t *flip, int64_t steps,
+                       const void *gy, const void *probs, void *gw, int64_t batch, hipStream_t s) {
+    constexpr int V = Vec16<T>::n;
+    if (batch % V != 0 || !dl_aligned(x, 16) || !dl_aligned(gy, 16)) return DL_ERR_TOO_LARGE;
+    const int64_t nchunks = steps / DL_TRAIN_CHUNK, ncols = batch / V;
+    const int64_t blocks = dl_ceil_div(nchunks, 4);
+    if (blocks > 0x7fffffffLL || ncols > 4 * DL_WAVE) return DL_ERR_TOO_LARGE;   // a lane holds at most 4 vectors of a row
+    const dim3 grid((unsigned) blocks), block(DL_BLOCK);
+    const T *xp = (const T *) x, *gp = (const T *) gy, *pp = (const T *) probs;
+    if (ncols <= DL_WAVE)
+        hipLaunchKernelGGL((backward_w_chain_kernel<T, V, 1, DL_TRAIN_CHUNK>), grid, block, 0, s, xp, verts, neuron, flip,
+                           gp, pp, (T *) gw, nchunks, ncols);
+    else if (ncols <= 2 * DL_WAVE)
+        hipLaunchKernelGGL((backward_w_chain_kernel<T, V, 2, DL_TRAIN_CHUNK>), grid, block, 0, s, xp, verts, neuron, flip,
+                           gp, pp, (T *) gw, nchunks, ncols);
+    else
+        hipLaunchKernelGGL((backward_w_chain_kernel<T, V, 4, DL_TRAIN_CHUNK>), grid, block, 0, s, xp, verts, neuron, flip,
+                           gp, pp, (T *) gw, nchunks, ncols);
+    return dl_launch_status();
+}
+
 }  // namespace
+
+extern "C" int dl_logic_forward_chained(const void *x, const int32_t *verts, const int32_t *neuron, const uint8_t *flip,
+                                        int64_t steps, const void *w, void *y, void *probs, int64_t in_dim,
+                                        int64_t out_dim, int64_t batch, int dtype, void *stream) {
+    if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
+    if (in_dim < 0 || out_dim < 0 || batch <= 0 || steps < out_dim || steps % DL_TRAIN_CHUNK != 0)
+        return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim == 0) return DL_OK;
+    if (!x || !verts || !neuron || !flip || !w || !y || in_dim == 0) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    if (probs) {
+        switch (dtype) {
+        case DL_F16: return forward_chain_t<__half, true>(x, verts, neuron, flip, steps, w, y, probs, batch, s);
+        case DL_F32: return forward_chain_t<float, true>(x, verts, neuron, flip, steps, w, y, probs, batch, s);
+        default: return forward_chain_t<double, true>(x, verts, neuron, flip, steps, w, y, probs, batch, s);
+        }
+    }
+    switch (dtype) {
+    case DL_F16: return forward_chain_t<__half, false>(x, verts, neuron, flip, steps, w, y, nullptr, batch, s);
+    case DL_F32: return forward_chain_t<float, false>(x, verts, neuron, flip, steps, w, y, nullptr, batch, s);
+    default: return forward_chain_t<double, false>(x, verts, neuron, flip, steps, w, y, nullptr, batch, s);
+    }
+}
+
+extern "C" int dl_logic_backward_w_chained(const void *x, const int32_t *verts, const int32_t *neuron,
+                                           const uint8_t *flip, int64_t steps, const void *grad_y, const void *probs,
+                                           void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch, int dtype,
+                                           void *stream) {
+    if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
+    if (in_dim < 0 || out_dim < 0 || batch <= 0 || steps < out_dim || steps % DL_TRAIN_CHUNK != 0)
+        return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim == 0) return DL_OK;
+    if (!x || !verts || !neuron || !flip || !grad_y || !grad_w || in_dim == 0) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    switch (dtype) {
+    case DL_F16: return backward_w_chain_t<__half>(x, verts, neuron, flip, steps, grad_y, probs, grad_w, batch, s);
+    case DL_F32: return backward_w_chain_t<float>(x, verts, neuron, flip, steps, grad_y, probs, grad_w, batch, s);
+    default: return backward_w_chain_t<double>(x, verts, neuron, flip, steps, grad_y, probs, grad_w, batch, s);
+    }
+}
 
 extern "C" int dl_logic_forward(const void *x, const int64_t *a, const int64_t *b, const void *w, void *y,
                                 int64_t in_dim, int64_t out_dim, int64_t batch, int dtype, void *stream) {

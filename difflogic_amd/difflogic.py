@@ -98,7 +98,8 @@ class LogicLayer(torch.nn.Module):
         if self.training:
             if self.weights.dtype == x.dtype and x.shape[1] > 0:
                 # softmax and its backward run inside the layer kernels
-                return LogicLayerLogitsFunction.apply(x, a, b, self.weights, *tail).transpose(0, 1)
+                return LogicLayerLogitsFunction.apply(x, a, b, self.weights, *tail,
+                                                      self._train_schedule()).transpose(0, 1)
             w = torch.nn.functional.softmax(self.weights, dim=-1).to(x.dtype)
             return LogicLayerCudaFunction.apply(x, a, b, w, *tail).transpose(0, 1)
         w = torch.nn.functional.one_hot(self.weights.argmax(-1), 16).to(x.dtype)
@@ -114,6 +115,19 @@ class LogicLayer(torch.nn.Module):
         assert x.features == self.in_dim, (x.features, self.in_dim)
         a, b = self.indices
         return x.defer_layer(a, b, self._gate_ids())
+
+    # Below this many inputs a 1 KB column tile of the whole input stays in the L2 caches and the
+    # second gather of a row hits there; above it the chained kernels halve the gathered rows.
+    _CHAIN_MIN_IN_DIM = 4096
+    # Narrower layers are latency-bound; a wave walking 8 neurons in sequence only lengthens that.
+    _CHAIN_MIN_OUT_DIM = 32768
+
+    def _train_schedule(self):
+        """Evaluation schedule of this layer's wiring for the chained forward / backward_w
+        kernels (cached per wiring), or None where chaining does not pay."""
+        if self.in_dim < self._CHAIN_MIN_IN_DIM or self.out_dim < self._CHAIN_MIN_OUT_DIM:
+            return None
+        return difflogic_cuda.schedule_for(self.indices[0], self.indices[1], self.in_dim)
 
     def _gate_ids(self):
         """uint8 [out_dim] argmax gate per neuron, recomputed only when ``weights`` changed."""
@@ -191,10 +205,12 @@ class LogicLayerLogitsFunction(torch.autograd.Function):
     its gradients, with the softmax and the softmax backward inside the layer kernels."""
 
     @staticmethod
-    def forward(ctx, x, a, b, logits, given_x_indices_of_y_start, given_x_indices_of_y, grad_factor=1.0):
-        y, probs = difflogic_cuda.forward_logits(x, a, b, logits.detach().contiguous())
+    def forward(ctx, x, a, b, logits, given_x_indices_of_y_start, given_x_indices_of_y, grad_factor=1.0,
+                schedule=None):
+        y, probs = difflogic_cuda.forward_logits(x, a, b, logits.detach().contiguous(), schedule)
         ctx.save_for_backward(x, a, b, probs, given_x_indices_of_y_start, given_x_indices_of_y)
         ctx.grad_factor = grad_factor
+        ctx.schedule = schedule
         return y
 
     @staticmethod
@@ -206,8 +222,8 @@ class LogicLayerLogitsFunction(torch.autograd.Function):
             grad_x = difflogic_cuda.backward_x(x, a, b, probs, grad_y, given_x_indices_of_y_start,
                                                given_x_indices_of_y, ctx.grad_factor)
         if ctx.needs_input_grad[3]:
-            grad_logits = difflogic_cuda.backward_logits(x, a, b, grad_y, probs)
-        return grad_x, None, None, grad_logits, None, None, None
+            grad_logits = difflogic_cuda.backward_logits(x, a, b, grad_y, probs, ctx.schedule)
+        return grad_x, None, None, grad_logits, None, None, None, None
 
 
 class GroupSumCudaFunction(torch.autograd.Function):

@@ -140,10 +140,12 @@ def backward_x(x, a, b, w, grad_y, given_x_indices_of_y_start, given_x_indices_o
     return grad_x
 
 
-def forward_logits(x, a, b, logits):
+def forward_logits(x, a, b, logits, schedule=None):
     """``forward(x, a, b, softmax(logits, -1))`` with the softmax computed inside the kernel.
     Returns (y [out,B], probs [out,16]); ``probs`` feeds backward_x / backward_logits.  Not part of
-    the reference's extension (difflogic/difflogic.py:123-126 runs the softmax in torch)."""
+    the reference's extension (difflogic/difflogic.py:123-126 runs the softmax in torch).
+    ``schedule`` (an EvalSchedule of (a, b)) selects the chained kernel: same result, one
+    gathered input row per neuron instead of two."""
     for t, n in ((x, "x"), (a, "a"), (b, "b"), (logits, "logits")):
         _check_input(t, n)
     code = _float_code(x, "logic_layer_cuda_forward")
@@ -157,17 +159,32 @@ def forward_logits(x, a, b, logits):
     in_dim, batch = x.shape
     y = torch.empty((out_dim, batch), dtype=x.dtype, device=dev)
     probs = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
+    lib = _lib.load()
     with torch.cuda.device(dev):
-        st = _lib.load().dl_logic_forward_logits(_p(x), _p(a), _p(b), _p(logits), _p(y), _p(probs), in_dim, out_dim,
-                                                 batch, code, _stream(dev))
+        st = _lib.DL_ERR_TOO_LARGE
+        if schedule is not None and out_dim > 0:
+            _check_schedule(schedule, in_dim, out_dim, dev)
+            st = lib.dl_logic_forward_chained(_p(x), _p(schedule.verts), _p(schedule.neuron), _p(schedule.flip),
+                                              schedule.steps, _p(logits), _p(y), _p(probs), in_dim, out_dim, batch, code,
+                                              _stream(dev))
+        if st == _lib.DL_ERR_TOO_LARGE:
+            st = lib.dl_logic_forward_logits(_p(x), _p(a), _p(b), _p(logits), _p(y), _p(probs), in_dim, out_dim, batch,
+                                             code, _stream(dev))
     if st:
         _raise(st, "logic_layer_cuda_forward_logits")
     return y, probs
 
 
-def backward_logits(x, a, b, grad_y, probs):
+def _check_schedule(schedule, in_dim, out_dim, dev):
+    if schedule.in_dim != in_dim or schedule.out_dim != out_dim or schedule.verts.device != dev:
+        raise RuntimeError(f"schedule is for a {schedule.in_dim}->{schedule.out_dim} layer on {schedule.verts.device}, "
+                           f"the call is for {in_dim}->{out_dim} on {dev}")
+
+
+def backward_logits(x, a, b, grad_y, probs, schedule=None):
     """Gradient with respect to the gate logits: backward_w chained with the softmax backward,
-    ``p * (g - (p * g).sum(-1, keepdim=True))`` with ``g = backward_w(x, a, b, grad_y)``."""
+    ``p * (g - (p * g).sum(-1, keepdim=True))`` with ``g = backward_w(x, a, b, grad_y)``.
+    ``schedule`` selects the chained kernel (bit-identical result)."""
     for t, n in ((x, "x"), (a, "a"), (b, "b"), (grad_y, "grad_y"), (probs, "probs")):
         _check_input(t, n)
     code = _float_code(x, "logic_layer_cuda_backward_w")
@@ -181,9 +198,17 @@ def backward_logits(x, a, b, grad_y, probs):
     dev = _same_device(x, a, b, grad_y, probs)
     in_dim, batch = x.shape
     grad_logits = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
+    lib = _lib.load()
     with torch.cuda.device(dev):
-        st = _lib.load().dl_logic_backward_logits(_p(x), _p(a), _p(b), _p(grad_y), _p(probs), _p(grad_logits), in_dim,
-                                                  out_dim, batch, code, _stream(dev))
+        st = _lib.DL_ERR_TOO_LARGE
+        if schedule is not None and out_dim > 0 and batch > 0:
+            _check_schedule(schedule, in_dim, out_dim, dev)
+            st = lib.dl_logic_backward_w_chained(_p(x), _p(schedule.verts), _p(schedule.neuron), _p(schedule.flip),
+                                                 schedule.steps, _p(grad_y), _p(probs), _p(grad_logits), in_dim, out_dim,
+                                                 batch, code, _stream(dev))
+        if st == _lib.DL_ERR_TOO_LARGE:
+            st = lib.dl_logic_backward_logits(_p(x), _p(a), _p(b), _p(grad_y), _p(probs), _p(grad_logits), in_dim,
+                                              out_dim, batch, code, _stream(dev))
     if st:
         _raise(st, "logic_layer_cuda_backward_logits")
     return grad_logits

@@ -75,6 +75,27 @@ int dl_logic_backward_logits(const void *x, const int64_t *a, const int64_t *b, 
                              const void *probs, void *grad_logits, int64_t in_dim, int64_t out_dim,
                              int64_t batch, int dtype, void *stream);
 
+/* forward / backward_w walked along an evaluation schedule of the layer's wiring (built with
+ * dl_eval_schedule_build, declared below): consecutive neurons share an input row, which stays in
+ * registers, so a neuron costs one gathered row instead of two.  Results are bit-identical to
+ * dl_logic_forward(_logits) / dl_logic_backward_w(_logits) in fp32 and fp64 (fp16 outputs can
+ * differ in the last bit).  No counterpart in the reference.
+ *   verts [steps+1], neuron [steps], flip [steps]: DEVICE copies of the schedule.
+ *   probs: forward  - NULL: `w` holds probabilities; else `w` holds logits and probs receives
+ *                     softmax(w) (as dl_logic_forward_logits);
+ *          backward - NULL: plain grad_w; else the softmax backward is chained
+ *                     (as dl_logic_backward_logits).
+ * Return DL_ERR_TOO_LARGE where the chained kernels do not apply (batch not a multiple of 16
+ * bytes of elements, unaligned buffers; backward: rows longer than 256 vectors of 16 bytes);
+ * the caller then uses the unchained entry points. */
+int dl_logic_forward_chained(const void *x, const int32_t *verts, const int32_t *neuron,
+                             const uint8_t *flip, int64_t steps, const void *w, void *y, void *probs,
+                             int64_t in_dim, int64_t out_dim, int64_t batch, int dtype, void *stream);
+int dl_logic_backward_w_chained(const void *x, const int32_t *verts, const int32_t *neuron,
+                                const uint8_t *flip, int64_t steps, const void *grad_y,
+                                const void *probs, void *grad_w, int64_t in_dim, int64_t out_dim,
+                                int64_t batch, int dtype, void *stream);
+
 /* Replaces `backward_x` = logic_layer_cuda_backward_x (difflogic.cpp:57-62,
  * difflogic_kernel.cu:367-410).
  *   grad_x[c,r] = scale * sum over neurons n reading input c of

@@ -264,3 +264,54 @@ def test_logits_entry_points(ext, dtype, rtol, in_dim, out_dim, batch):
     ok, err = close(got_g, want_g, 2 * rtol)
     assert ok, err
     assert torch.equal(got_g, ext.backward_logits(xq.cuda(), a.cuda(), b.cuda(), gq.cuda(), probs))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16])
+@pytest.mark.parametrize("in_dim,out_dim,batch,kind", [(64, 64, 256, "random"), (100, 300, 512, "random"),
+                                                       (50, 60, 1024, "unique"), (30, 47, 260, "any"),
+                                                       (5, 3, 64, "self"), (40, 90, 4096, "any"), (20, 40, 6, "any")])
+def test_chained_training_kernels_are_bit_identical(ext, dtype, in_dim, out_dim, batch, kind):
+    from oracle import connections as oc
+    g = torch.Generator().manual_seed(in_dim + batch)
+    torch.manual_seed(in_dim)
+    if kind == "random":
+        a, b = oc.random_connections(in_dim, out_dim)
+    elif kind == "unique":
+        a, b = oc.unique_connections(in_dim, out_dim)
+    elif kind == "self":
+        a, b = torch.tensor([1, 1, 2]), torch.tensor([1, 1, 2])
+    else:
+        a, b = torch.randint(0, in_dim, (out_dim,), generator=g), torch.randint(0, in_dim, (out_dim,), generator=g)
+    x = torch.rand(in_dim, batch, generator=g).to(dtype).cuda()
+    logits = torch.randn(out_dim, 16, generator=g).to(dtype).cuda()
+    gy = torch.randn(out_dim, batch, generator=g).to(dtype).cuda()
+    a, b = a.cuda(), b.cuda()
+    sched = ext.schedule_for(a, b, in_dim)
+    y0, p0 = ext.forward_logits(x, a, b, logits)
+    y1, p1 = ext.forward_logits(x, a, b, logits, sched)
+    g0 = ext.backward_logits(x, a, b, gy, p0)
+    g1 = ext.backward_logits(x, a, b, gy, p0, sched)
+    if dtype == torch.float16:
+        # the fp32 arithmetic is the same, but the compiler may round the final fp32 -> fp16
+        # conversion in one step (fused multiply-add with fp16 result) in one kernel and in two in
+        # the other: rare last-bit differences are allowed
+        for u, v in ((y0, y1), (p0, p1), (g0, g1)):
+            diff = (u.float() - v.float()).abs()
+            assert float((diff > 0).float().mean()) < 0.01
+            assert bool((diff <= 2.0 ** -10 * u.float().abs().clamp(min=2.0 ** -14)).all())
+    else:
+        assert torch.equal(y0, y1) and torch.equal(p0, p1) and torch.equal(g0, g1)
+
+
+def test_layer_uses_schedule_for_wide_inputs():
+    import difflogic_amd as dl
+    torch.manual_seed(0)
+    wide, narrow = dl.LogicLayer(5000, 40000), dl.LogicLayer(100, 40000)
+    assert wide._train_schedule() is not None and narrow._train_schedule() is None
+    assert dl.LogicLayer(5000, 5000)._train_schedule() is None
+    x = torch.rand(64, 5000, device="cuda", requires_grad=True)
+    y = wide(x)
+    y.square().sum().backward()
+    ref = fo.layer_forward_sequential(x.detach().cpu().double(), wide.indices[0].cpu(), wide.indices[1].cpu(),
+                                      torch.softmax(wide.weights.detach().cpu().double(), -1))
+    assert close(y, ref)[0]
