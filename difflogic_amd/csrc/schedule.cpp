@@ -90,3 +90,47 @@ extern "C" int64_t dl_eval_schedule_build(const int64_t *a, const int64_t *b, in
     }
     return steps;
 }
+
+// Destinations for dl_logic_backward_chained.  Position p of the schedule (vertex verts[p]) takes
+// part in neuron[p - 1] and neuron[p]; if either exists the kernel produces one partial grad_x
+// row there.  A vertex with exactly one such position is written straight to grad_x
+// (dst[p] = vertex).  Every other vertex becomes a fix-up entry: its positions are numbered into
+// consecutive overflow rows (dst[p] = in_dim + row), summed after the pass; a vertex at no
+// position at all gets an entry with no rows (zero gradient).
+extern "C" int64_t dl_backward_schedule_build(const int32_t *verts, const int32_t *neuron, int64_t steps,
+                                              int64_t in_dim, int32_t *dst, int32_t *fix_vertex, int32_t *fix_start,
+                                              int64_t *n_fix) {
+    if (!verts || !neuron || !dst || !fix_vertex || !fix_start || !n_fix || steps < 0 || in_dim <= 0)
+        return -DL_ERR_INVALID_ARGUMENT;
+    if (in_dim > 0x3fffffffLL || steps > 0x3fffffffLL) return -DL_ERR_TOO_LARGE;
+    auto produces = [&](int64_t p) { return (p > 0 && neuron[p - 1] >= 0) || (p < steps && neuron[p] >= 0); };
+    std::vector<int32_t> count((size_t) in_dim, 0);
+    for (int64_t p = 0; p <= steps; ++p) {
+        if (verts[p] < 0 || verts[p] >= in_dim) return -DL_ERR_INVALID_ARGUMENT;
+        if (produces(p)) ++count[(size_t) verts[p]];
+    }
+    // fix-up entries in vertex order; next_row[v] = the vertex's next free overflow row
+    std::vector<int32_t> next_row((size_t) in_dim, -1);
+    int64_t entries = 0, rows = 0;
+    for (int64_t v = 0; v < in_dim; ++v) {
+        if (count[(size_t) v] == 1) continue;
+        fix_vertex[entries] = (int32_t) v;
+        fix_start[entries] = (int32_t) rows;
+        next_row[(size_t) v] = (int32_t) rows;
+        rows += count[(size_t) v];
+        ++entries;
+    }
+    fix_start[entries] = (int32_t) rows;
+    if (in_dim + rows > 0x7fffffffLL) return -DL_ERR_TOO_LARGE;
+    for (int64_t p = 0; p <= steps; ++p) {
+        const int32_t v = verts[p];
+        if (!produces(p))
+            dst[p] = -1;
+        else if (count[(size_t) v] == 1)
+            dst[p] = v;
+        else
+            dst[p] = (int32_t) (in_dim + next_row[(size_t) v]++);
+    }
+    *n_fix = entries;
+    return rows;
+}

@@ -517,6 +517,156 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_w_chain_kernel(const T *__r
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// Chained backward: grad_w AND grad_x of a layer in one pass along the schedule.  Step s reads
+// input row verts[s + 1] and grad_y row neuron[s] (the other input row is still in registers),
+// which is all that backward_w and both directions of backward_x need for that neuron:
+//     to a:  g * ((P10 - P00) + b * dd)      to b:  g * ((P01 - P00) + a * dd)
+//     dd = (P11 - P10) - (P01 - P00)
+// A vertex in the middle of a trail collects the share of the neuron before it (kept in
+// `carry`) and of the neuron after it and is written once: position p of the schedule goes to
+// row dst[p] (-1: nothing to write; >= in_dim: row dst[p] - in_dim of `overflow`, for vertices
+// that occur at several positions and are summed afterwards by backward_fix_kernel).  A chunk
+// owns positions [s0, s0 + CHUNK); it recomputes the last neuron of the chunk before it to get
+// the carry into its first position, so chunks do not exchange partial rows.
+// ------------------------------------------------------------------------------------------
+template <typename T, int VEC, int CPL, int CHUNK>
+__global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
+    const T *__restrict__ x, const int32_t *__restrict__ verts, const int32_t *__restrict__ neuron,
+    const uint8_t *__restrict__ flip, const int32_t *__restrict__ dst, const T *__restrict__ w,
+    const T *__restrict__ gy, const T *__restrict__ probs, T *__restrict__ gw, T *__restrict__ gx,
+    T *__restrict__ overflow, int64_t steps, int64_t in_dim, int64_t ncols, typename Acc<T>::type scale) {
+    typedef typename Acc<T>::type C;
+    typedef Pack<T, VEC> P;
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t s0 = ((int64_t) blockIdx.x * 4 + wave) * CHUNK;
+    if (s0 >= steps) return;
+    const int64_t s1 = s0 + CHUNK < steps ? s0 + CHUNK : steps;
+    const P *xv = reinterpret_cast<const P *>(x);
+    const P *gv = reinterpret_cast<const P *>(gy);
+    P zero;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) zero.v[e] = down<T, C>((C) 0);
+
+    auto load_row = [&](const P *base, int64_t row, bool valid, P *out) {
+#pragma unroll
+        for (int q = 0; q < CPL; ++q) {
+            const int64_t col = lane + q * DL_WAVE;
+            out[q] = (valid && col < ncols) ? base[row * ncols + col] : zero;
+        }
+    };
+    auto store_row = [&](int32_t row, const C (&val)[CPL][VEC]) {
+        if (row < 0) return;
+        P *base = row < in_dim ? reinterpret_cast<P *>(gx) + (int64_t) row * ncols
+                               : reinterpret_cast<P *>(overflow) + ((int64_t) row - in_dim) * ncols;
+#pragma unroll
+        for (int q = 0; q < CPL; ++q) {
+            const int64_t col = lane + q * DL_WAVE;
+            P r;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) r.v[e] = down<T, C>(val[q][e] * scale);
+            if (col < ncols) base[col] = r;
+        }
+    };
+
+    P prev[CPL];
+    C carry[CPL][VEC];
+    load_row(xv, verts[s0], true, prev);
+#pragma unroll
+    for (int q = 0; q < CPL; ++q)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) carry[q][e] = (C) 0;
+    if (s0 > 0 && neuron[s0 - 1] >= 0) {             // share of the neuron that ends at this chunk's first vertex
+        const int32_t n = neuron[s0 - 1];
+        const bool f = flip[s0 - 1] != 0;
+        P before[CPL], g[CPL];
+        load_row(xv, verts[s0 - 1], true, before);
+        load_row(gv, n, true, g);
+        const Corners<C> k = corners<T>(w, n);
+        const C d0 = k.p01 - k.p00, dd = (k.p11 - k.p10) - d0, da = k.p10 - k.p00;
+        const C kv = f ? da : d0;
+#pragma unroll
+        for (int q = 0; q < CPL; ++q)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) carry[q][e] = up<T>(g[q].v[e]) * dl_fma(up<T>(before[q].v[e]), dd, kv);
+    }
+#pragma unroll 1
+    for (int64_t s = s0; s < s1; ++s) {
+        const int32_t n = neuron[s];
+        const bool valid = n >= 0;
+        const int64_t nn = valid ? n : 0;
+        const bool f = flip[s] != 0;
+        P cur[CPL], g[CPL];
+        load_row(xv, verts[s + 1], true, cur);
+        load_row(gv, nn, valid, g);                  // zero gradient for a step without a neuron
+        const Corners<C> k = corners<T>(w, nn);
+        const C d0 = k.p01 - k.p00, dd = (k.p11 - k.p10) - d0, da = k.p10 - k.p00;
+        const C ku = f ? d0 : da, kv = f ? da : d0;
+        C s00 = (C) 0, s01 = (C) 0, s10 = (C) 0, s11 = (C) 0;
+        C out[CPL][VEC];
+#pragma unroll
+        for (int q = 0; q < CPL; ++q) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const C u0 = up<T>(prev[q].v[e]), u1 = up<T>(cur[q].v[e]), gg = up<T>(g[q].v[e]);
+                const C av = f ? u1 : u0, bv = f ? u0 : u1;
+                const C ga = gg * av, gna = gg - ga;
+                const C t11 = ga * bv, t01 = gna * bv;
+                s11 += t11;
+                s10 += ga - t11;
+                s01 += t01;
+                s00 += gna - t01;
+                out[q][e] = carry[q][e] + gg * dl_fma(u1, dd, ku);
+                carry[q][e] = gg * dl_fma(u0, dd, kv);
+            }
+        }
+        store_row(dst[s], out);
+        s00 = wave_sum(s00);
+        s01 = wave_sum(s01);
+        s10 = wave_sum(s10);
+        s11 = wave_sum(s11);
+        store_grad_w<T>(lane, valid, nn, s00, s01, s10, s11, probs, gw);
+#pragma unroll
+        for (int q = 0; q < CPL; ++q) prev[q] = cur[q];
+    }
+    if (s1 == steps) store_row(dst[steps], carry);   // the schedule's last position
+}
+
+// grad_x rows of the vertices that backward_chain_kernel could not finish in one write: vertex
+// fix_vertex[i] is the sum, in slot order, of overflow rows [fix_start[i], fix_start[i + 1])
+// (no rows: the input feeds no neuron and its gradient is zero).
+template <typename T, int VEC>
+__global__ __launch_bounds__(DL_BLOCK) void backward_fix_kernel(const T *__restrict__ overflow,
+                                                                const int32_t *__restrict__ fix_vertex,
+                                                                const int32_t *__restrict__ fix_start,
+                                                                T *__restrict__ gx, int64_t n_fix, int64_t ncols) {
+    typedef typename Acc<T>::type C;
+    typedef Pack<T, VEC> P;
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t i = (int64_t) blockIdx.x * 4 + wave;
+    if (i >= n_fix) return;
+    const int64_t v = fix_vertex[i];
+    const int32_t r0 = fix_start[i], r1 = fix_start[i + 1];
+    const P *ov = reinterpret_cast<const P *>(overflow);
+    P *out = reinterpret_cast<P *>(gx);
+    for (int64_t col = (int64_t) blockIdx.y * DL_WAVE + lane; col < ncols; col += (int64_t) gridDim.y * DL_WAVE) {
+        C acc[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = (C) 0;
+        for (int32_t r = r0; r < r1; ++r) {
+            const P part = ov[(int64_t) r * ncols + col];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] += up<T>(part.v[e]);
+        }
+        P res;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) res.v[e] = down<T, C>(acc[e]);
+        out[v * ncols + col] = res;
+    }
+}
+
 template <typename T> struct Vec16 { static constexpr int n = 16 / (int) sizeof(T); };
 
 unsigned col_tiles(int64_t ncols) {
@@ -782,7 +932,65 @@ int backward_w_chain_t(const void *x, const int32_t *verts, const int32_t *neuro
     return dl_launch_status();
 }
 
+#define DL_BACKWARD_CHUNK 16   // steps per wave of backward_chain_kernel (any value: chunks recompute their carry-in)
+
+template <typename T>
+int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, const uint8_t *flip, const int32_t *dst,
+                     int64_t steps, const void *w, const void *gy, bool softmax_backward, const int32_t *fix_vertex,
+                     const int32_t *fix_start, int64_t n_fix, void *gw, void *gx, void *overflow, int64_t in_dim,
+                     int64_t batch, double scale, hipStream_t s) {
+    typedef typename Acc<T>::type C;
+    constexpr int V = Vec16<T>::n;
+    if (batch % V != 0 || !dl_aligned(x, 16) || !dl_aligned(gy, 16) || !dl_aligned(gx, 16) || !dl_aligned(overflow, 16))
+        return DL_ERR_TOO_LARGE;
+    const int64_t ncols = batch / V;
+    const int64_t blocks = dl_ceil_div(dl_ceil_div(steps, DL_BACKWARD_CHUNK), 4), fix_blocks = dl_ceil_div(n_fix, 4);
+    if (blocks > 0x7fffffffLL || fix_blocks > 0x7fffffffLL || ncols > 4 * DL_WAVE) return DL_ERR_TOO_LARGE;
+    const dim3 grid((unsigned) blocks), block(DL_BLOCK);
+    const T *xp = (const T *) x, *wp = (const T *) w, *gp = (const T *) gy, *pp = softmax_backward ? wp : nullptr;
+#define DL_LAUNCH_BACKWARD_CHAIN(CPL)                                                                                   \
+    hipLaunchKernelGGL((backward_chain_kernel<T, V, CPL, DL_BACKWARD_CHUNK>), grid, block, 0, s, xp, verts, neuron, flip, \
+                       dst, wp, gp, pp, (T *) gw, (T *) gx, (T *) overflow, steps, in_dim, ncols, (C) scale)
+    if (ncols <= DL_WAVE)
+        DL_LAUNCH_BACKWARD_CHAIN(1);
+    else if (ncols <= 2 * DL_WAVE)
+        DL_LAUNCH_BACKWARD_CHAIN(2);
+    else
+        DL_LAUNCH_BACKWARD_CHAIN(4);
+#undef DL_LAUNCH_BACKWARD_CHAIN
+    int st = dl_launch_status();
+    if (st != DL_OK || n_fix == 0) return st;
+    hipLaunchKernelGGL((backward_fix_kernel<T, V>), dim3((unsigned) fix_blocks, col_tiles(ncols)), block, 0, s,
+                       (const T *) overflow, fix_vertex, fix_start, (T *) gx, n_fix, ncols);
+    return dl_launch_status();
+}
+
 }  // namespace
+
+extern "C" int dl_logic_backward_chained(const void *x, const int32_t *verts, const int32_t *neuron, const uint8_t *flip,
+                                         const int32_t *dst, int64_t steps, const void *w, const void *grad_y,
+                                         int softmax_backward, const int32_t *fix_vertex, const int32_t *fix_start,
+                                         int64_t n_fix, void *grad_w, void *grad_x, void *overflow, int64_t in_dim,
+                                         int64_t out_dim, int64_t batch, double scale, int dtype, void *stream) {
+    if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
+    if (in_dim <= 0 || out_dim <= 0 || batch <= 0 || steps < out_dim || n_fix < 0 || n_fix > in_dim)
+        return DL_ERR_INVALID_ARGUMENT;
+    if (!x || !verts || !neuron || !flip || !dst || !w || !grad_y || !grad_w || !grad_x) return DL_ERR_INVALID_ARGUMENT;
+    if (n_fix > 0 && (!fix_vertex || !fix_start)) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    const bool sb = softmax_backward != 0;
+    switch (dtype) {
+    case DL_F16:
+        return backward_chain_t<__half>(x, verts, neuron, flip, dst, steps, w, grad_y, sb, fix_vertex, fix_start, n_fix,
+                                        grad_w, grad_x, overflow, in_dim, batch, scale, s);
+    case DL_F32:
+        return backward_chain_t<float>(x, verts, neuron, flip, dst, steps, w, grad_y, sb, fix_vertex, fix_start, n_fix,
+                                       grad_w, grad_x, overflow, in_dim, batch, scale, s);
+    default:
+        return backward_chain_t<double>(x, verts, neuron, flip, dst, steps, w, grad_y, sb, fix_vertex, fix_start, n_fix,
+                                        grad_w, grad_x, overflow, in_dim, batch, scale, s);
+    }
+}
 
 extern "C" int dl_logic_forward_chained(const void *x, const int32_t *verts, const int32_t *neuron, const uint8_t *flip,
                                         int64_t steps, const void *w, void *y, void *probs, int64_t in_dim,

@@ -218,6 +218,12 @@ class LogicLayerLogitsFunction(torch.autograd.Function):
         x, a, b, probs, given_x_indices_of_y_start, given_x_indices_of_y = ctx.saved_tensors
         grad_y = grad_y.contiguous()
         grad_logits = grad_x = None
+        if ctx.needs_input_grad[0] and ctx.needs_input_grad[3] and ctx.schedule is not None:
+            # one pass along the schedule yields both gradients
+            both = difflogic_cuda.backward_chained(x, probs, grad_y, ctx.schedule, ctx.grad_factor,
+                                                   softmax_backward=True)
+            if both is not None:
+                return both[1], None, None, both[0], None, None, None, None
         if ctx.needs_input_grad[0]:
             grad_x = difflogic_cuda.backward_x(x, a, b, probs, grad_y, given_x_indices_of_y_start,
                                                given_x_indices_of_y, ctx.grad_factor)

@@ -214,6 +214,48 @@ def backward_logits(x, a, b, grad_y, probs, schedule=None):
     return grad_logits
 
 
+def backward_chained(x, w, grad_y, schedule, scale=1.0, softmax_backward=False):
+    """backward_w (or backward_logits when ``softmax_backward``; ``w`` are then the probabilities
+    that forward_logits returned) and backward_x in one pass along ``schedule``.  Returns
+    (grad_w [out,16], grad_x [in,B]), or None where the fused pass does not apply (the caller
+    then uses the separate functions).  Not part of the reference's extension."""
+    for t, n in ((x, "x"), (w, "w"), (grad_y, "grad_y")):
+        _check_input(t, n)
+    code = _float_code(x, "logic_layer_cuda_backward")
+    if (x.dim() != 2 or grad_y.dim() != 2 or grad_y.shape[1] != x.shape[1] or grad_y.dtype != x.dtype
+            or w.shape != (grad_y.shape[0], 16) or w.dtype != x.dtype):
+        raise RuntimeError(f"expected x [in,B], w [out,16], grad_y [out,B] of one dtype, got {tuple(x.shape)}, "
+                           f"{tuple(w.shape)}, {tuple(grad_y.shape)}")
+    dev = _same_device(x, w, grad_y)
+    in_dim, batch = x.shape
+    out_dim = grad_y.shape[0]
+    if in_dim == 0 or out_dim == 0 or batch == 0:
+        return None
+    _check_schedule(schedule, in_dim, out_dim, dev)
+    dst, fix_vertex, fix_start, n_fix, rows = schedule.backward_plan()
+    if rows > in_dim * BACKWARD_CHAIN_MAX_OVERFLOW:
+        return None
+    grad_w = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
+    grad_x = torch.empty_like(x)
+    overflow = torch.empty((rows, batch), dtype=x.dtype, device=dev) if rows else None
+    with torch.cuda.device(dev):
+        st = _lib.load().dl_logic_backward_chained(
+            _p(x), _p(schedule.verts), _p(schedule.neuron), _p(schedule.flip), _p(dst), schedule.steps, _p(w),
+            _p(grad_y), 1 if softmax_backward else 0, _p(fix_vertex) if n_fix else None,
+            _p(fix_start) if n_fix else None, n_fix, _p(grad_w), _p(grad_x), _p(overflow) if rows else None, in_dim,
+            out_dim, batch, float(scale), code, _stream(dev))
+    if st == _lib.DL_ERR_TOO_LARGE:
+        return None
+    if st:
+        _raise(st, "logic_layer_cuda_backward_chained")
+    return grad_w, grad_x
+
+
+# backward_chained gives way to the separate kernels when the partial rows it would park in the
+# overflow buffer exceed this fraction of the input rows (wirings with many high-degree inputs).
+BACKWARD_CHAIN_MAX_OVERFLOW = 0.25
+
+
 def eval(x, a, b, w):  # noqa: A001  (the reference's name)
     """x [in,W] int words, w [out] uint8 gate ids -> y [out,W]   (difflogic.cpp:63-68)."""
     for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w")):
@@ -380,6 +422,32 @@ class EvalSchedule:
         self.neuron = torch.from_numpy(neuron[:steps].copy()).to(a.device)
         self.flip = torch.from_numpy(flip[:steps].copy()).to(a.device)
         self._wiring = (a, b)        # keeps the tensors (and their addresses) alive while cached
+        self._host = (verts[:steps + 1].copy(), neuron[:steps].copy())
+        self._backward = None
+
+    def backward_plan(self):
+        """(dst, fix_vertex, fix_start, n_fix, overflow_rows) for backward_chained, built on first
+        use: where each schedule position's grad_x row goes and which inputs are summed from
+        several partial rows afterwards."""
+        if self._backward is None:
+            import ctypes
+            import numpy as np
+            lib = _lib.load()
+            verts, neuron = self._host
+            dst = np.empty(self.steps + 1, dtype=np.int32)
+            fix_vertex = np.empty(self.in_dim, dtype=np.int32)
+            fix_start = np.empty(self.in_dim + 1, dtype=np.int32)
+            n_fix = ctypes.c_int64(0)
+            rows = lib.dl_backward_schedule_build(verts.ctypes.data, neuron.ctypes.data, self.steps, self.in_dim,
+                                                  dst.ctypes.data, fix_vertex.ctypes.data, fix_start.ctypes.data,
+                                                  ctypes.byref(n_fix))
+            if rows < 0:
+                _raise(-rows, "backward_schedule_build")
+            n = int(n_fix.value)
+            dev = self.verts.device
+            self._backward = (torch.from_numpy(dst).to(dev), torch.from_numpy(fix_vertex[:n].copy()).to(dev),
+                              torch.from_numpy(fix_start[:n + 1].copy()).to(dev), n, int(rows))
+        return self._backward
 
 
 _SCHEDULES = {}                      # (ptr a, ptr b, versions, in_dim) -> EvalSchedule, most recent last

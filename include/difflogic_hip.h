@@ -109,6 +109,33 @@ int dl_logic_backward_x(const void *x, const int64_t *a, const int64_t *b, const
                         int64_t in_dim, int64_t out_dim, int64_t batch, double scale, int dtype,
                         void *stream);
 
+/* backward_w and backward_x of one layer in a single pass along the schedule (the pair
+ * difflogic/difflogic.py:218,220): every neuron's input rows and grad_y row are read once and
+ * serve grad_w and both grad_x contributions.  No counterpart in the reference.
+ *   dl_backward_schedule_build()  HOST pointers.  From a schedule (verts [steps+1], neuron [steps])
+ *       writes dst [steps+1]: the grad_x row that schedule position p completes (-1: none;
+ *       >= in_dim: row dst - in_dim of the overflow buffer), and the fix-up list for inputs that
+ *       occur at several positions or at none: fix_vertex [<= in_dim], fix_start [<= in_dim + 1]
+ *       (overflow rows fix_start[i] .. fix_start[i+1]-1 are summed into grad_x[fix_vertex[i]]).
+ *       *n_fix receives the list's length; returns the number of overflow rows or a negated
+ *       dl_status.
+ *   dl_logic_backward_chained()   DEVICE pointers.  w [out,16]: the gate probabilities the forward
+ *       pass used.  softmax_backward = 0: grad_w as dl_logic_backward_w; else the gradient with
+ *       respect to the logits as dl_logic_backward_logits (w = its probs).  grad_x as
+ *       dl_logic_backward_x (same `scale`, same a == b rule) up to summation order.  overflow:
+ *       scratch of (overflow rows) x batch elements, 16-byte aligned; may be NULL when there are
+ *       none.  Returns DL_ERR_TOO_LARGE where it does not apply (see the chained entry points
+ *       above); the caller then uses the separate entry points. */
+int64_t dl_backward_schedule_build(const int32_t *verts, const int32_t *neuron, int64_t steps,
+                                   int64_t in_dim, int32_t *dst, int32_t *fix_vertex,
+                                   int32_t *fix_start, int64_t *n_fix);
+int dl_logic_backward_chained(const void *x, const int32_t *verts, const int32_t *neuron,
+                              const uint8_t *flip, const int32_t *dst, int64_t steps, const void *w,
+                              const void *grad_y, int softmax_backward, const int32_t *fix_vertex,
+                              const int32_t *fix_start, int64_t n_fix, void *grad_w, void *grad_x,
+                              void *overflow, int64_t in_dim, int64_t out_dim, int64_t batch,
+                              double scale, int dtype, void *stream);
+
 /* ---- GroupSum on the feature-major layout (training mode) ------------------------------- */
 
 /* Replaces the float branch of GroupSum.forward (difflogic/difflogic.py:195-196) for the

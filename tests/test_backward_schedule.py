@@ -1,0 +1,106 @@
+"""Host logic of the fused backward pass: the destinations that dl_backward_schedule_build derives
+from an evaluation schedule, checked by replaying the kernel's walk in numpy."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from difflogic_amd import _lib
+from oracle import connections as oc
+
+
+def _schedule(a, b, in_dim):
+    lib = _lib.load()
+    chunk = lib.dl_eval_schedule_chunk()
+    cap = lib.dl_eval_schedule_capacity(len(a), chunk)
+    verts = np.empty(cap + 1, np.int32)
+    neuron = np.empty(cap, np.int32)
+    flip = np.empty(cap, np.uint8)
+    steps = lib.dl_eval_schedule_build(a.ctypes.data, b.ctypes.data, in_dim, len(a), chunk, verts.ctypes.data,
+                                       neuron.ctypes.data, flip.ctypes.data)
+    assert steps >= len(a)
+    return verts[:steps + 1].copy(), neuron[:steps].copy(), flip[:steps].copy(), int(steps)
+
+
+def _plan(verts, neuron, steps, in_dim):
+    lib = _lib.load()
+    dst = np.empty(steps + 1, np.int32)
+    fix_vertex = np.empty(in_dim, np.int32)
+    fix_start = np.empty(in_dim + 1, np.int32)
+    n_fix = ctypes.c_int64(0)
+    rows = lib.dl_backward_schedule_build(verts.ctypes.data, neuron.ctypes.data, steps, in_dim, dst.ctypes.data,
+                                          fix_vertex.ctypes.data, fix_start.ctypes.data, ctypes.byref(n_fix))
+    assert rows >= 0
+    n = int(n_fix.value)
+    return dst, fix_vertex[:n], fix_start[:n + 1], int(rows)
+
+
+def _np(pair):
+    return tuple(np.asarray(t, dtype=np.int64) for t in pair)
+
+
+def _wirings():
+    import torch
+    torch.manual_seed(11)
+    rng = np.random.default_rng(5)
+    yield "random_square", 64, *_np(oc.random_connections(64, 64))
+    yield "unique_square", 50, *_np(oc.unique_connections(50, 50))
+    yield "random_wide", 20, *_np(oc.random_connections(20, 90))
+    a = rng.integers(0, 12, 30)
+    yield "self_loops_and_unused", 16, a, np.where(rng.random(30) < 0.3, a, rng.integers(0, 12, 30))
+
+
+@pytest.mark.parametrize("name,in_dim,a,b", list(_wirings()), ids=lambda v: v if isinstance(v, str) else None)
+def test_every_input_is_completed_exactly_once(name, in_dim, a, b):
+    a = np.ascontiguousarray(a, np.int64)
+    b = np.ascontiguousarray(b, np.int64)
+    verts, neuron, flip, steps = _schedule(a, b, in_dim)
+    dst, fix_vertex, fix_start, rows = _plan(verts, neuron, steps, in_dim)
+    # Replay: each neuron n hands one token (n, 'a') to input a[n] and (n, 'b') to input b[n]; position p
+    # receives the token of neuron[p-1] for its far end and of neuron[p] for its near end.
+    direct = [None] * in_dim
+    overflow = [None] * rows
+    for p in range(steps + 1):
+        tokens = []
+        if p > 0 and neuron[p - 1] >= 0:
+            n = neuron[p - 1]
+            tokens.append((n, "a" if flip[p - 1] else "b"))      # the step's new vertex is `a` when flipped
+        if p < steps and neuron[p] >= 0:
+            n = neuron[p]
+            tokens.append((n, "b" if flip[p] else "a"))          # the step's old vertex is `b` when flipped
+        for n, side in tokens:
+            assert (a if side == "a" else b)[n] == verts[p]
+        if not tokens:
+            assert dst[p] == -1
+            continue
+        if dst[p] < in_dim:
+            assert dst[p] == verts[p] and direct[dst[p]] is None
+            direct[dst[p]] = tokens
+        else:
+            assert overflow[dst[p] - in_dim] is None
+            overflow[dst[p] - in_dim] = (verts[p], tokens)
+    assert all(o is not None for o in overflow)
+    got = {v: sorted(t) for v, t in enumerate(direct) if t is not None}
+    assert len(set(fix_vertex.tolist())) == len(fix_vertex)
+    for i, v in enumerate(fix_vertex):
+        assert v not in got
+        parts = overflow[fix_start[i]:fix_start[i + 1]]
+        assert all(pv == v for pv, _ in parts)
+        got[int(v)] = sorted(t for _, ts in parts for t in ts)
+    assert fix_start[-1] == rows
+    want = {v: [] for v in range(in_dim)}
+    for n in range(len(a)):
+        want[int(a[n])].append((n, "a"))
+        want[int(b[n])].append((n, "b"))
+    assert got == {v: sorted(t) for v, t in want.items()}
+
+
+def test_rejects_out_of_range_vertices():
+    lib = _lib.load()
+    verts = np.array([0, 7], np.int32)
+    neuron = np.array([0], np.int32)
+    out = np.empty(4, np.int32)
+    n_fix = ctypes.c_int64(0)
+    st = lib.dl_backward_schedule_build(verts.ctypes.data, neuron.ctypes.data, 1, 4, out.ctypes.data, out.ctypes.data,
+                                        out.ctypes.data, ctypes.byref(n_fix))
+    assert st == -_lib.DL_ERR_INVALID_ARGUMENT

@@ -303,6 +303,76 @@ def test_chained_training_kernels_are_bit_identical(ext, dtype, in_dim, out_dim,
         assert torch.equal(y0, y1) and torch.equal(p0, p1) and torch.equal(g0, g1)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16])
+@pytest.mark.parametrize("in_dim,out_dim,batch,kind", [(64, 64, 256, "random"), (300, 300, 512, "random"),
+                                                       (50, 60, 1024, "unique"), (200, 200, 64, "unique"),
+                                                       (30, 47, 260, "any"), (5, 3, 64, "self"),
+                                                       (40, 20, 16, "sparse"), (20, 40, 8, "any")])
+@pytest.mark.parametrize("softmax_backward", [False, True])
+def test_fused_chained_backward_matches_separate_kernels(ext, monkeypatch, dtype, in_dim, out_dim, batch, kind,
+                                                         softmax_backward):
+    from oracle import connections as oc
+    monkeypatch.setattr(ext, "BACKWARD_CHAIN_MAX_OVERFLOW", 1e9)     # exercise the overflow rows on any wiring
+    g = torch.Generator().manual_seed(in_dim + batch)
+    torch.manual_seed(in_dim)
+    if kind == "random":
+        a, b = oc.random_connections(in_dim, out_dim)
+    elif kind == "unique":
+        a, b = oc.unique_connections(in_dim, out_dim)
+    elif kind == "self":
+        a, b = torch.tensor([1, 1, 2]), torch.tensor([1, 1, 2])
+    elif kind == "sparse":                                           # half of the inputs feed no neuron
+        a, b = torch.randint(0, in_dim // 2, (out_dim,), generator=g), torch.randint(0, in_dim // 2, (out_dim,),
+                                                                                    generator=g)
+    else:
+        a, b = torch.randint(0, in_dim, (out_dim,), generator=g), torch.randint(0, in_dim, (out_dim,), generator=g)
+    x = torch.rand(in_dim, batch, generator=g).to(dtype).cuda()
+    w = torch.softmax(torch.randn(out_dim, 16, generator=g), -1).to(dtype).cuda()
+    gy = torch.randn(out_dim, batch, generator=g).to(dtype).cuda()
+    start, idx = oc.reverse_index(a, b, in_dim)
+    a, b = a.cuda(), b.cuda()
+    start, idx = torch.as_tensor(start).cuda(), torch.as_tensor(idx).cuda()
+    sched = ext.schedule_for(a, b, in_dim)
+    scale = 1.5
+    both = ext.backward_chained(x, w, gy, sched, scale, softmax_backward=softmax_backward)
+    if batch * x.element_size() > 256 * 16 or batch * x.element_size() % 16:
+        # a wave holds at most 256 16-byte vectors of a row, and only whole ones
+        assert both is None
+        return
+    assert both is not None
+    gw, gx = both
+    want_gx = ext.backward_x(x, a, b, w, gy, start, idx, scale)
+    want_gw = ext.backward_logits(x, a, b, gy, w) if softmax_backward else ext.backward_w(x, a, b, gy)
+    # grad_w: same arithmetic and summation order as the unfused kernels
+    if dtype == torch.float16:
+        assert close(gw, want_gw.double(), 2e-3)[0]
+    else:
+        assert torch.equal(gw, want_gw)
+    # grad_x: the same terms summed in another order
+    rtol = {torch.float16: 4e-3, torch.float32: 1e-5, torch.float64: 1e-12}[dtype]
+    ok, err = close(gx, want_gx.double(), rtol)
+    assert ok, err
+    again = ext.backward_chained(x, w, gy, sched, scale, softmax_backward=softmax_backward)
+    assert torch.equal(again[0], gw) and torch.equal(again[1], gx)   # deterministic
+
+
+def test_fused_chained_backward_declines_where_it_does_not_apply(ext):
+    from oracle import connections as oc
+    torch.manual_seed(3)
+    a, b = oc.random_connections(16, 400)                            # degree 50: nearly every row would overflow
+    a, b = a.cuda(), b.cuda()
+    sched = ext.schedule_for(a, b, 16)
+    x, w, gy = torch.rand(16, 64).cuda(), torch.rand(400, 16).cuda(), torch.rand(400, 64).cuda()
+    assert ext.backward_chained(x, w, gy, sched) is None
+    a, b = oc.random_connections(64, 64)
+    a, b = a.cuda(), b.cuda()
+    sched = ext.schedule_for(a, b, 64)
+    x, w, gy = torch.rand(64, 6).cuda(), torch.rand(64, 16).cuda(), torch.rand(64, 6).cuda()
+    assert ext.backward_chained(x, w, gy, sched) is None             # rows are not whole 16-byte vectors
+    x, w, gy = torch.rand(64, 2048).cuda(), torch.rand(64, 16).cuda(), torch.rand(64, 2048).cuda()
+    assert ext.backward_chained(x, w, gy, sched) is None             # a wave cannot hold a whole row
+
+
 def test_layer_uses_schedule_for_wide_inputs():
     import difflogic_amd as dl
     torch.manual_seed(0)
@@ -315,3 +385,9 @@ def test_layer_uses_schedule_for_wide_inputs():
     ref = fo.layer_forward_sequential(x.detach().cpu().double(), wide.indices[0].cpu(), wide.indices[1].cpu(),
                                       torch.softmax(wide.weights.detach().cpu().double(), -1))
     assert close(y, ref)[0]
+    # the backward pass took the fused chained kernel; compare with autograd through the python formulation
+    xr = x.detach().cpu().double().requires_grad_()
+    wr = wide.weights.detach().cpu().double().requires_grad_()
+    fo.layer_forward_sequential(xr, wide.indices[0].cpu(), wide.indices[1].cpu(),
+                                torch.softmax(wr, -1)).square().sum().backward()
+    assert close(x.grad, xr.grad, 1e-4)[0] and close(wide.weights.grad, wr.grad, 1e-4)[0]
