@@ -417,7 +417,6 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_chain_kernel(const T *__rest
                                                                  T *__restrict__ probs, int64_t nchunks, int64_t ncols) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
-    static_assert(CHUNK % 2 == 0, "steps are processed in pairs");
     const int wave = dl_wave_in_block();
     const int lane = dl_lane();
     const int64_t c = (int64_t) blockIdx.x * 4 + wave;
@@ -430,26 +429,82 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_chain_kernel(const T *__rest
         const int64_t col = ct * DL_WAVE + lane;
         const bool live = col < ncols;
         const int64_t cl = live ? col : 0;
-        P prev = xv[(int64_t) verts[s0] * ncols + cl];
+        // every row of the chunk is requested before the first one is used
+        P rows[CHUNK + 1];
 #pragma unroll
-        for (int j = 0; j < CHUNK; j += 2) {
-            const int32_t v1 = verts[s0 + j + 1], v2 = verts[s0 + j + 2];
-            const int32_t n1 = neuron[s0 + j], n2 = neuron[s0 + j + 1];
-            const bool f1 = flip[s0 + j] != 0, f2 = flip[s0 + j + 1] != 0;
-            const P x1 = xv[(int64_t) v1 * ncols + cl], x2 = xv[(int64_t) v2 * ncols + cl];
-            C p00a, p10a, d0a, d1a, p00b, p10b, d0b, d1b;
-            neuron_corners<T, LOGITS>(w, n1 >= 0 ? n1 : 0, lane, n1 >= 0 && ct == 0, probs, p00a, p10a, d0a, d1a);
-            neuron_corners<T, LOGITS>(w, n2 >= 0 ? n2 : 0, lane, n2 >= 0 && ct == 0, probs, p00b, p10b, d0b, d1b);
-            P r1, r2;
+        for (int j = 0; j <= CHUNK; ++j) rows[j] = xv[(int64_t) verts[s0 + j] * ncols + cl];
+#pragma unroll
+        for (int j = 0; j < CHUNK; ++j) {
+            const int32_t n = neuron[s0 + j];
+            const bool f = flip[s0 + j] != 0;
+            C p00, p10, d0, d1;
+            neuron_corners<T, LOGITS>(w, n >= 0 ? n : 0, lane, n >= 0 && ct == 0, probs, p00, p10, d0, d1);
+            P r;
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-                const C u0 = up<T>(prev.v[e]), u1 = up<T>(x1.v[e]), u2 = up<T>(x2.v[e]);
-                r1.v[e] = down<T, C>(mix<C>(f1 ? u1 : u0, f1 ? u0 : u1, p00a, p10a, d0a, d1a));
-                r2.v[e] = down<T, C>(mix<C>(f2 ? u2 : u1, f2 ? u1 : u2, p00b, p10b, d0b, d1b));
+                const C u0 = up<T>(rows[j].v[e]), u1 = up<T>(rows[j + 1].v[e]);
+                r.v[e] = down<T, C>(mix<C>(f ? u1 : u0, f ? u0 : u1, p00, p10, d0, d1));
             }
-            if (live && n1 >= 0) yv[(int64_t) n1 * ncols + col] = r1;
-            if (live && n2 >= 0) yv[(int64_t) n2 * ncols + col] = r2;
-            prev = x2;
+            if (live && n >= 0) yv[(int64_t) n * ncols + col] = r;
+        }
+    }
+}
+
+// Forward along the schedule for rows of up to 256 vectors: one wave owns `chunk` steps and the
+// WHOLE row (lane l holds vectors l, l + 64, ...), so every gathered row is one contiguous
+// request, and the next step's row is requested before this step's arithmetic.
+template <typename T, int VEC, int CPL, bool LOGITS>
+__global__ __launch_bounds__(DL_BLOCK) void forward_chain_rows_kernel(const T *__restrict__ x,
+                                                                      const int32_t *__restrict__ verts,
+                                                                      const int32_t *__restrict__ neuron,
+                                                                      const uint8_t *__restrict__ flip,
+                                                                      const T *__restrict__ w, T *__restrict__ y,
+                                                                      T *__restrict__ probs, int64_t steps, int chunk,
+                                                                      int64_t ncols) {
+    typedef typename Acc<T>::type C;
+    typedef Pack<T, VEC> P;
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t s0 = ((int64_t) blockIdx.x * 4 + wave) * chunk;
+    if (s0 >= steps) return;
+    const int64_t s1 = s0 + chunk < steps ? s0 + chunk : steps;
+    const P *xv = reinterpret_cast<const P *>(x);
+    P *yv = reinterpret_cast<P *>(y);
+    P zero;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) zero.v[e] = down<T, C>((C) 0);
+    auto load_row = [&](int64_t row, P *out) {
+#pragma unroll
+        for (int q = 0; q < CPL; ++q) {
+            const int64_t col = lane + q * DL_WAVE;
+            out[q] = col < ncols ? xv[row * ncols + col] : zero;
+        }
+    };
+    P prev[CPL], cur[CPL], next[CPL];
+    load_row(verts[s0], prev);
+    load_row(verts[s0 + 1], cur);
+#pragma unroll 1
+    for (int64_t s = s0; s < s1; ++s) {
+        if (s + 1 < s1) load_row(verts[s + 2], next);
+        const int32_t n = neuron[s];
+        const bool f = flip[s] != 0;
+        C p00, p10, d0, d1;
+        neuron_corners<T, LOGITS>(w, n >= 0 ? n : 0, lane, n >= 0, probs, p00, p10, d0, d1);
+#pragma unroll
+        for (int q = 0; q < CPL; ++q) {
+            const int64_t col = lane + q * DL_WAVE;
+            P r;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const C u0 = up<T>(prev[q].v[e]), u1 = up<T>(cur[q].v[e]);
+                r.v[e] = down<T, C>(mix<C>(f ? u1 : u0, f ? u0 : u1, p00, p10, d0, d1));
+            }
+            if (n >= 0 && col < ncols) yv[(int64_t) n * ncols + col] = r;
+        }
+#pragma unroll
+        for (int q = 0; q < CPL; ++q) {
+            prev[q] = cur[q];
+            cur[q] = next[q];
         }
     }
 }
@@ -526,23 +581,23 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_w_chain_kernel(const T *__r
 // A vertex in the middle of a trail collects the share of the neuron before it (kept in
 // `carry`) and of the neuron after it and is written once: position p of the schedule goes to
 // row dst[p] (-1: nothing to write; >= in_dim: row dst[p] - in_dim of `overflow`, for vertices
-// that occur at several positions and are summed afterwards by backward_fix_kernel).  A chunk
-// owns positions [s0, s0 + CHUNK); it recomputes the last neuron of the chunk before it to get
+// that occur at several positions and are summed afterwards by backward_fix_kernel).  A wave
+// owns `chunk` positions [s0, s0 + chunk); it recomputes the last neuron of the chunk before it to get
 // the carry into its first position, so chunks do not exchange partial rows.
 // ------------------------------------------------------------------------------------------
-template <typename T, int VEC, int CPL, int CHUNK>
+template <typename T, int VEC, int CPL>
 __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
     const T *__restrict__ x, const int32_t *__restrict__ verts, const int32_t *__restrict__ neuron,
     const uint8_t *__restrict__ flip, const int32_t *__restrict__ dst, const T *__restrict__ w,
     const T *__restrict__ gy, const T *__restrict__ probs, T *__restrict__ gw, T *__restrict__ gx,
-    T *__restrict__ overflow, int64_t steps, int64_t in_dim, int64_t ncols, typename Acc<T>::type scale) {
+    T *__restrict__ overflow, int64_t steps, int chunk, int64_t in_dim, int64_t ncols, typename Acc<T>::type scale) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
     const int wave = dl_wave_in_block();
     const int lane = dl_lane();
-    const int64_t s0 = ((int64_t) blockIdx.x * 4 + wave) * CHUNK;
+    const int64_t s0 = ((int64_t) blockIdx.x * 4 + wave) * chunk;
     if (s0 >= steps) return;
-    const int64_t s1 = s0 + CHUNK < steps ? s0 + CHUNK : steps;
+    const int64_t s1 = s0 + chunk < steps ? s0 + chunk : steps;
     const P *xv = reinterpret_cast<const P *>(x);
     const P *gv = reinterpret_cast<const P *>(gy);
     P zero;
@@ -895,6 +950,15 @@ int group_sum_splits(int64_t out_dim, int64_t batch, int64_t k) {
 }
 
 #define DL_TRAIN_CHUNK 8     // must equal the chunk the schedule was built with (dl_eval_schedule_chunk)
+#define DL_FWD_ROWS_MIN 128  // vectors per row above which forward_chain_rows_kernel takes over
+
+// Steps per wave of the kernels in which a wave owns whole rows: long chunks re-read fewer rows at
+// their seams, short ones give more waves to hide latency with; keep about three waves per SIMD.
+int chain_chunk(int64_t steps) {
+    for (int chunk = 32; chunk > 8; chunk /= 2)
+        if (steps / chunk >= 3000) return chunk;
+    return 8;
+}
 
 template <typename T, bool LOGITS>
 int forward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, const uint8_t *flip, int64_t steps,
@@ -902,11 +966,25 @@ int forward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, 
     constexpr int V = Vec16<T>::n;
     if (batch % V != 0 || !dl_aligned(x, 16) || !dl_aligned(y, 16)) return DL_ERR_TOO_LARGE;
     const int64_t nchunks = steps / DL_TRAIN_CHUNK, ncols = batch / V;
+    const T *xp = (const T *) x, *wp = (const T *) w;
+    if (ncols > DL_FWD_ROWS_MIN && ncols <= 4 * DL_WAVE) {
+        // rows of 2-4 KB: a wave takes whole rows
+        const int chunk = chain_chunk(steps);
+        const int64_t blocks = dl_ceil_div(dl_ceil_div(steps, chunk), 4);
+        if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+        const dim3 grid((unsigned) blocks), block(DL_BLOCK);
+        if (ncols <= 2 * DL_WAVE)
+            hipLaunchKernelGGL((forward_chain_rows_kernel<T, V, 2, LOGITS>), grid, block, 0, s, xp, verts, neuron, flip, wp,
+                               (T *) y, (T *) probs, steps, chunk, ncols);
+        else
+            hipLaunchKernelGGL((forward_chain_rows_kernel<T, V, 4, LOGITS>), grid, block, 0, s, xp, verts, neuron, flip, wp,
+                               (T *) y, (T *) probs, steps, chunk, ncols);
+        return dl_launch_status();
+    }
     const int64_t blocks = dl_ceil_div(nchunks, 4);
     if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     hipLaunchKernelGGL((forward_chain_kernel<T, V, DL_TRAIN_CHUNK, LOGITS>), dim3((unsigned) blocks, col_tiles(ncols)),
-                       dim3(DL_BLOCK), 0, s, (const T *) x, verts, neuron, flip, (const T *) w, (T *) y, (T *) probs,
-                       nchunks, ncols);
+                       dim3(DL_BLOCK), 0, s, xp, verts, neuron, flip, wp, (T *) y, (T *) probs, nchunks, ncols);
     return dl_launch_status();
 }
 
@@ -932,8 +1010,6 @@ int backward_w_chain_t(const void *x, const int32_t *verts, const int32_t *neuro
     return dl_launch_status();
 }
 
-#define DL_BACKWARD_CHUNK 16   // steps per wave of backward_chain_kernel (any value: chunks recompute their carry-in)
-
 template <typename T>
 int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, const uint8_t *flip, const int32_t *dst,
                      int64_t steps, const void *w, const void *gy, bool softmax_backward, const int32_t *fix_vertex,
@@ -944,13 +1020,14 @@ int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron,
     if (batch % V != 0 || !dl_aligned(x, 16) || !dl_aligned(gy, 16) || !dl_aligned(gx, 16) || !dl_aligned(overflow, 16))
         return DL_ERR_TOO_LARGE;
     const int64_t ncols = batch / V;
-    const int64_t blocks = dl_ceil_div(dl_ceil_div(steps, DL_BACKWARD_CHUNK), 4), fix_blocks = dl_ceil_div(n_fix, 4);
+    const int chunk = chain_chunk(steps);
+    const int64_t blocks = dl_ceil_div(dl_ceil_div(steps, chunk), 4), fix_blocks = dl_ceil_div(n_fix, 4);
     if (blocks > 0x7fffffffLL || fix_blocks > 0x7fffffffLL || ncols > 4 * DL_WAVE) return DL_ERR_TOO_LARGE;
     const dim3 grid((unsigned) blocks), block(DL_BLOCK);
     const T *xp = (const T *) x, *wp = (const T *) w, *gp = (const T *) gy, *pp = softmax_backward ? wp : nullptr;
 #define DL_LAUNCH_BACKWARD_CHAIN(CPL)                                                                                   \
-    hipLaunchKernelGGL((backward_chain_kernel<T, V, CPL, DL_BACKWARD_CHUNK>), grid, block, 0, s, xp, verts, neuron, flip, \
-                       dst, wp, gp, pp, (T *) gw, (T *) gx, (T *) overflow, steps, in_dim, ncols, (C) scale)
+    hipLaunchKernelGGL((backward_chain_kernel<T, V, CPL>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp, pp, \
+                       (T *) gw, (T *) gx, (T *) overflow, steps, chunk, in_dim, ncols, (C) scale)
     if (ncols <= DL_WAVE)
         DL_LAUNCH_BACKWARD_CHAIN(1);
     else if (ncols <= 2 * DL_WAVE)
