@@ -189,7 +189,8 @@ def train_bench(args, torch, dl):
     """fp32 forward + backward of 784 -> 6 x 64000 -> GroupSum(10, tau 30), B = 512, 'unique'
     connections, grad_factor 1, CrossEntropy.  Reports the whole step (eager and replayed as one
     HIP graph) and each layer kernel timed alone (back-to-back launches on a 64000 -> 64000 layer,
-    forward and backward_w in their chained form, as the layer runs them)
+    forward and backward_w in their chained form; backward_chained is the single pass the layer
+    runs in place of backward_w + backward_x and is charged the bytes of both)
     against its algorithmic bytes: forward 4B(in+out)+80 out, backward_w 4B(in+out)+64 out,
     backward_x 4B(2 in+out)+64 out."""
     F, width, L, k, B = 784, 64000, 6, 10, 512
@@ -235,6 +236,9 @@ def train_bench(args, torch, dl):
         "forward_logits": (lambda: ext.forward_logits(xs, a, b, logits, sched), 4 * B * 2 * width + 80 * width),
         "backward_logits": (lambda: ext.backward_logits(xs, a, b, gy, probs, sched), 4 * B * 2 * width + 64 * width),
         "backward_x": (lambda: ext.backward_x(xs, a, b, probs, gy, start, idx), 4 * B * 3 * width + 64 * width),
+        # backward_logits + backward_x in one pass (what the layer runs when both gradients are needed)
+        "backward_chained": (lambda: ext.backward_chained(xs, probs, gy, sched, 1.0, softmax_backward=True),
+                             4 * B * 5 * width + 128 * width),
     }
     kernels = {}
     for name, (fn, by) in calls.items():

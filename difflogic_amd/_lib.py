@@ -22,6 +22,7 @@ _vp, _i64, _int, _dbl = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_
 SIGNATURES = {
     "dl_version": [],
     "dl_status_string": [_int],
+    "dl_last_hip_error": [],
     "dl_logic_forward": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "dl_logic_backward_w": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "dl_logic_forward_logits": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
@@ -48,7 +49,7 @@ SIGNATURES = {
     "dl_logic_eval_fused_groupbitsum_workspace_bytes": [_int, _i64, _i64, _int, _i64],
     "dl_logic_eval_fused_groupbitsum": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _i64, _vp, _vp],
 }
-_RESTYPES = {"dl_status_string": ctypes.c_char_p, "dl_group_sum_workspace_bytes": ctypes.c_int64,
+_RESTYPES = {"dl_status_string": ctypes.c_char_p, "dl_last_hip_error": ctypes.c_char_p, "dl_group_sum_workspace_bytes": ctypes.c_int64,
              "dl_logic_eval_fused_workspace_bytes": ctypes.c_int64,
              "dl_eval_schedule_capacity": ctypes.c_int64, "dl_eval_schedule_build": ctypes.c_int64,
              "dl_backward_schedule_build": ctypes.c_int64,
@@ -66,6 +67,10 @@ def load():
         raise ImportError(
             f"{LIB_PATH} is missing: the HIP kernel library has not been built. "
             "Run `python difflogic_amd/build.py` (needs hipcc); there is no fallback implementation.")
+    # torch first: its own copy of the HIP runtime must be the one in the process when the library's
+    # dependency on libamdhip64 is resolved.  Loaded the other way round, the process ends up with
+    # two runtimes and every launch from this library fails with "no ROCm-capable device".
+    import torch  # noqa: F401
     lib = ctypes.CDLL(LIB_PATH)
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)          # AttributeError if the symbol is not exported
@@ -76,4 +81,7 @@ def load():
 
 
 def status_string(status: int) -> str:
-    return load().dl_status_string(int(status)).decode()
+    text = load().dl_status_string(int(status)).decode()
+    if int(status) == DL_ERR_LAUNCH:
+        text += f" ({load().dl_last_hip_error().decode()})"
+    return text

@@ -12,7 +12,23 @@
 typedef uint32_t dl_u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t dl_u32x2 __attribute__((ext_vector_type(2)));
 
-static inline int dl_launch_status() { return hipGetLastError() == hipSuccess ? DL_OK : DL_ERR_LAUNCH; }
+// hipGetLastError() reports the last error of ANY earlier runtime call of this thread, including
+// harmless ones of the caller (an event query that answered "not ready"), so the error state is
+// cleared right before each launch and read right after it.
+#define DL_LAUNCH(kernel, grid, block, lds, stream, ...)                      \
+    do {                                                                      \
+        (void) hipGetLastError();                                             \
+        hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);    \
+    } while (0)
+
+extern thread_local int dl_last_hip_error_code;    // hipError_t of this thread's last refused launch (packed.hip)
+
+static inline int dl_launch_status() {
+    const hipError_t e = hipGetLastError();
+    if (e == hipSuccess) return DL_OK;
+    dl_last_hip_error_code = (int) e;
+    return DL_ERR_LAUNCH;
+}
 
 static inline int64_t dl_ceil_div(int64_t x, int64_t y) { return (x + y - 1) / y; }
 

@@ -298,7 +298,7 @@ int launch_eval(const void *x, const int64_t *a, const int64_t *b, const uint8_t
     if (ntiles > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     if (ctiles > 65535) ctiles = 65535;
     dim3 grid((unsigned) ntiles, (unsigned) ctiles);
-    hipLaunchKernelGGL((eval_kernel<V, NPW, ITERS>), grid, dim3(DL_BLOCK), 0, stream, (const V *) x, a, b, w, (V *) y,
+    DL_LAUNCH((eval_kernel<V, NPW, ITERS>), grid, dim3(DL_BLOCK), 0, stream, (const V *) x, a, b, w, (V *) y,
                        out_dim, ncols);
     return dl_launch_status();
 }
@@ -821,11 +821,11 @@ void launch_groupbitsum_v(const void *bits, int32_t *out, int64_t row_bytes, int
     const V *b = (const V *) bits;
     // NPH planes above weight 8 hold counts up to 16 * 2^NPH - 1.
     if (chunk < (16LL << 8))
-        hipLaunchKernelGGL((groupbitsum_kernel<V, 8>), grid, dim3(DL_BLOCK), 0, s, b, out, ncols, per_class, k, batch);
+        DL_LAUNCH((groupbitsum_kernel<V, 8>), grid, dim3(DL_BLOCK), 0, s, b, out, ncols, per_class, k, batch);
     else if (chunk < (16LL << 14))
-        hipLaunchKernelGGL((groupbitsum_kernel<V, 14>), grid, dim3(DL_BLOCK), 0, s, b, out, ncols, per_class, k, batch);
+        DL_LAUNCH((groupbitsum_kernel<V, 14>), grid, dim3(DL_BLOCK), 0, s, b, out, ncols, per_class, k, batch);
     else
-        hipLaunchKernelGGL((groupbitsum_kernel<V, 27>), grid, dim3(DL_BLOCK), 0, s, b, out, ncols, per_class, k, batch);
+        DL_LAUNCH((groupbitsum_kernel<V, 27>), grid, dim3(DL_BLOCK), 0, s, b, out, ncols, per_class, k, batch);
 }
 
 // Rows of whole 64-bit words, 8-byte aligned: 16-byte lanes where rows and base allow it.
@@ -852,7 +852,7 @@ int launch_count_fused_v(const void *x, const int32_t *leaves, const uint64_t *g
     const int64_t tiles = dl_ceil_div(ncols, DL_WAVE);
     const int64_t chunks_per_class = dl_ceil_div(per_class, DL_COUNT_ROWS);
     if (k * chunks_per_class > 0x7fffffffLL || tiles > 65535) return DL_ERR_TOO_LARGE;
-    hipLaunchKernelGGL((count_partial_kernel<V, TREE>), dim3((unsigned) (k * chunks_per_class), (unsigned) tiles),
+    DL_LAUNCH((count_partial_kernel<V, TREE>), dim3((unsigned) (k * chunks_per_class), (unsigned) tiles),
                        dim3(DL_BLOCK), 0, s, (const V *) x, leaves, gates, (V *) scratch, ncols, per_class,
                        chunks_per_class);
     int st = dl_launch_status();
@@ -861,13 +861,13 @@ int launch_count_fused_v(const void *x, const int32_t *leaves, const uint64_t *g
     // planes needed for counts up to per_class (pass 1 rounds a class up to whole chunks of 128)
     const int64_t top = chunks_per_class * DL_COUNT_ROWS;
     if (top < (1LL << 13))
-        hipLaunchKernelGGL((count_finish_kernel<V, 13>), grid, dim3(DL_BLOCK), 0, s, (const V *) scratch, out, ncols,
+        DL_LAUNCH((count_finish_kernel<V, 13>), grid, dim3(DL_BLOCK), 0, s, (const V *) scratch, out, ncols,
                            chunks_per_class, k, batch);
     else if (top < (1LL << 18))
-        hipLaunchKernelGGL((count_finish_kernel<V, 18>), grid, dim3(DL_BLOCK), 0, s, (const V *) scratch, out, ncols,
+        DL_LAUNCH((count_finish_kernel<V, 18>), grid, dim3(DL_BLOCK), 0, s, (const V *) scratch, out, ncols,
                            chunks_per_class, k, batch);
     else
-        hipLaunchKernelGGL((count_finish_kernel<V, 31>), grid, dim3(DL_BLOCK), 0, s, (const V *) scratch, out, ncols,
+        DL_LAUNCH((count_finish_kernel<V, 31>), grid, dim3(DL_BLOCK), 0, s, (const V *) scratch, out, ncols,
                            chunks_per_class, k, batch);
     return dl_launch_status();
 }
@@ -902,10 +902,10 @@ int compose_tree(int depth, const int64_t *const *a, const int64_t *const *b, co
     if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     const dim3 grid((unsigned) blocks), block(DL_BLOCK);
     switch (depth) {
-    case 1: hipLaunchKernelGGL(compose_tree_kernel<1>, grid, block, 0, s, t, *leaves, *gates, out_dim); break;
-    case 2: hipLaunchKernelGGL(compose_tree_kernel<2>, grid, block, 0, s, t, *leaves, *gates, out_dim); break;
-    case 3: hipLaunchKernelGGL(compose_tree_kernel<3>, grid, block, 0, s, t, *leaves, *gates, out_dim); break;
-    default: hipLaunchKernelGGL(compose_tree_kernel<4>, grid, block, 0, s, t, *leaves, *gates, out_dim); break;
+    case 1: DL_LAUNCH(compose_tree_kernel<1>, grid, block, 0, s, t, *leaves, *gates, out_dim); break;
+    case 2: DL_LAUNCH(compose_tree_kernel<2>, grid, block, 0, s, t, *leaves, *gates, out_dim); break;
+    case 3: DL_LAUNCH(compose_tree_kernel<3>, grid, block, 0, s, t, *leaves, *gates, out_dim); break;
+    default: DL_LAUNCH(compose_tree_kernel<4>, grid, block, 0, s, t, *leaves, *gates, out_dim); break;
     }
     return dl_launch_status();
 }
@@ -922,7 +922,7 @@ int launch_eval_tree(int depth, const void *x, const int32_t *leaves, const uint
     {                                                                                                                  \
         const int64_t ntiles = dl_ceil_div(out_dim, 4 * NPW * ITERS);                                                  \
         if (ntiles > 0x7fffffffLL) return DL_ERR_TOO_LARGE;                                                            \
-        hipLaunchKernelGGL((eval_tree_kernel<V, D, NPW, ITERS>), dim3((unsigned) ntiles, (unsigned) ctiles),           \
+        DL_LAUNCH((eval_tree_kernel<V, D, NPW, ITERS>), dim3((unsigned) ntiles, (unsigned) ctiles),           \
                            dim3(DL_BLOCK), 0, s, xv, leaves, gates, yv, out_dim, ncols);                               \
     }
     switch (depth) {
@@ -938,6 +938,10 @@ int launch_eval_tree(int depth, const void *x, const int32_t *leaves, const uint
 bool valid_bit_count(int bit_count) { return bit_count == 8 || bit_count == 16 || bit_count == 32 || bit_count == 64; }
 
 }  // namespace
+
+thread_local int dl_last_hip_error_code = 0;
+
+extern "C" const char *dl_last_hip_error(void) { return hipGetErrorString((hipError_t) dl_last_hip_error_code); }
 
 extern "C" int dl_logic_eval(const void *x, const int64_t *a, const int64_t *b, const uint8_t *w, void *y,
                              int64_t in_dim, int64_t out_dim, int64_t words, int bit_count, void *stream) {
@@ -970,12 +974,12 @@ extern "C" int dl_tensor_packbits(const uint8_t *t, void *out, int64_t features,
     if (vec) {
         int64_t gx = dl_ceil_div(out_row_bytes / 2, DL_BLOCK);
         if (gx > 65535) gx = 65535;
-        hipLaunchKernelGGL(packbits_vec16_kernel, dim3((unsigned) gx, gy), dim3(DL_BLOCK), 0, s, t, (uint8_t *) out,
+        DL_LAUNCH(packbits_vec16_kernel, dim3((unsigned) gx, gy), dim3(DL_BLOCK), 0, s, t, (uint8_t *) out,
                            features, batch, out_row_bytes);
     } else {
         int64_t gx = dl_ceil_div(out_row_bytes, DL_BLOCK);
         if (gx > 65535) gx = 65535;
-        hipLaunchKernelGGL(packbits_generic_kernel, dim3((unsigned) gx, gy), dim3(DL_BLOCK), 0, s, t,
+        DL_LAUNCH(packbits_generic_kernel, dim3((unsigned) gx, gy), dim3(DL_BLOCK), 0, s, t,
                            (uint8_t *) out, features, batch, out_row_bytes);
     }
     return dl_launch_status();
@@ -1000,17 +1004,17 @@ extern "C" int dl_tensor_packbits_batch_major(const uint8_t *x, void *out, int64
         const int64_t blocks = dl_ceil_div(dl_ceil_div(batch, 64), WC);
         if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
         const size_t lds = (size_t) (64 * features + features * WC * 8);
-        hipLaunchKernelGGL(packbits_batch_major_lds_kernel<WC>, dim3((unsigned) blocks), dim3(DL_BLOCK), lds, s, x,
+        DL_LAUNCH(packbits_batch_major_lds_kernel<WC>, dim3((unsigned) blocks), dim3(DL_BLOCK), lds, s, x,
                            (uint8_t *) out, batch, features, out_row_bytes);
     } else if (features % 4 == 0 && dl_aligned(x, 4)) {
         const int64_t gy = dl_ceil_div(features, 256);
         if (gy > 65535) return DL_ERR_TOO_LARGE;
-        hipLaunchKernelGGL(packbits_batch_major_kernel<4>, dim3((unsigned) gx, (unsigned) gy), dim3(DL_BLOCK), 0, s, x,
+        DL_LAUNCH(packbits_batch_major_kernel<4>, dim3((unsigned) gx, (unsigned) gy), dim3(DL_BLOCK), 0, s, x,
                            (uint8_t *) out, batch, features, out_row_bytes);
     } else {
         const int64_t gy = dl_ceil_div(features, 64);
         if (gy > 65535) return DL_ERR_TOO_LARGE;
-        hipLaunchKernelGGL(packbits_batch_major_kernel<1>, dim3((unsigned) gx, (unsigned) gy), dim3(DL_BLOCK), 0, s, x,
+        DL_LAUNCH(packbits_batch_major_kernel<1>, dim3((unsigned) gx, (unsigned) gy), dim3(DL_BLOCK), 0, s, x,
                            (uint8_t *) out, batch, features, out_row_bytes);
     }
     return dl_launch_status();
@@ -1037,7 +1041,7 @@ extern "C" int dl_groupbitsum(const void *b, int32_t *out, int64_t in_dim, int64
         int64_t gx = dl_ceil_div(batch, DL_BLOCK);
         if (gx > 0x7fffffffLL) gx = 0x7fffffffLL;
         const unsigned gy = (unsigned) (k < 65535 ? k : 65535);
-        hipLaunchKernelGGL(groupbitsum_generic_kernel, dim3((unsigned) gx, gy), dim3(DL_BLOCK), 0, s,
+        DL_LAUNCH(groupbitsum_generic_kernel, dim3((unsigned) gx, gy), dim3(DL_BLOCK), 0, s,
                            (const uint8_t *) b, out, row_bytes, per_class, k, batch);
     }
     return dl_launch_status();
@@ -1122,7 +1126,7 @@ int launch_eval_chain(int sub_depth, const void *x, const int32_t *sub_leaves, c
     {                                                                                                                  \
         const int64_t gx = dl_ceil_div(nchunks, 4 * ITERS);                                                            \
         if (gx > 0x7fffffffLL) return DL_ERR_TOO_LARGE;                                                                \
-        hipLaunchKernelGGL((eval_chain_kernel<V, DS, DL_EVAL_SCHEDULE_CHUNK, ITERS>),                                  \
+        DL_LAUNCH((eval_chain_kernel<V, DS, DL_EVAL_SCHEDULE_CHUNK, ITERS>),                                  \
                            dim3((unsigned) gx, (unsigned) ctiles), dim3(DL_BLOCK), 0, s, (const V *) x, sub_leaves,    \
                            sub_gates, verts, neuron, flip, w_top, (V *) y, nchunks, ncols);                            \
     }

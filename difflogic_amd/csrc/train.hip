@@ -737,11 +737,11 @@ int forward_t(const void *x, const int64_t *a, const int64_t *b, const void *w, 
     if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     constexpr int V = Vec16<T>::n;
     if (batch % V == 0 && dl_aligned(x, 16) && dl_aligned(y, 16)) {
-        hipLaunchKernelGGL((forward_kernel<T, V, NPW, LOGITS>), dim3((unsigned) blocks, col_tiles(batch / V)),
+        DL_LAUNCH((forward_kernel<T, V, NPW, LOGITS>), dim3((unsigned) blocks, col_tiles(batch / V)),
                            dim3(DL_BLOCK), 0, s, (const T *) x, a, b, (const T *) w, (T *) y, (T *) probs, out_dim,
                            batch / V);
     } else {
-        hipLaunchKernelGGL((forward_kernel<T, 1, NPW, LOGITS>), dim3((unsigned) blocks, col_tiles(batch)), dim3(DL_BLOCK),
+        DL_LAUNCH((forward_kernel<T, 1, NPW, LOGITS>), dim3((unsigned) blocks, col_tiles(batch)), dim3(DL_BLOCK),
                            0, s, (const T *) x, a, b, (const T *) w, (T *) y, (T *) probs, out_dim, batch);
     }
     return dl_launch_status();
@@ -762,13 +762,13 @@ int backward_w_t(const void *x, const int64_t *a, const int64_t *b, const void *
     const T *xp = (const T *) x, *gp = (const T *) gy, *pp = (const T *) probs;
     T *wp = (T *) gw;
     if (vec && split)
-        hipLaunchKernelGGL((backward_w_kernel<T, V, NPW, 4>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols);
+        DL_LAUNCH((backward_w_kernel<T, V, NPW, 4>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols);
     else if (vec)
-        hipLaunchKernelGGL((backward_w_kernel<T, V, NPW, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols);
+        DL_LAUNCH((backward_w_kernel<T, V, NPW, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols);
     else if (split)
-        hipLaunchKernelGGL((backward_w_kernel<T, 1, NPW, 4>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols);
+        DL_LAUNCH((backward_w_kernel<T, 1, NPW, 4>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols);
     else
-        hipLaunchKernelGGL((backward_w_kernel<T, 1, NPW, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols);
+        DL_LAUNCH((backward_w_kernel<T, 1, NPW, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols);
     return dl_launch_status();
 }
 
@@ -781,11 +781,11 @@ int backward_x_t(const void *x, const int64_t *a, const int64_t *b, const void *
     const int64_t blocks = dl_ceil_div(in_dim, 4);
     if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     if (batch % V == 0 && dl_aligned(x, 16) && dl_aligned(gy, 16) && dl_aligned(gx, 16)) {
-        hipLaunchKernelGGL((backward_x_kernel<T, V>), dim3((unsigned) blocks, col_tiles(batch / V)), dim3(DL_BLOCK), 0, s,
+        DL_LAUNCH((backward_x_kernel<T, V>), dim3((unsigned) blocks, col_tiles(batch / V)), dim3(DL_BLOCK), 0, s,
                            (const T *) x, a, b, (const T *) w, (const T *) gy, start, idx, (T *) gx, in_dim, batch / V,
                            (C) scale);
     } else {
-        hipLaunchKernelGGL((backward_x_kernel<T, 1>), dim3((unsigned) blocks, col_tiles(batch)), dim3(DL_BLOCK), 0, s,
+        DL_LAUNCH((backward_x_kernel<T, 1>), dim3((unsigned) blocks, col_tiles(batch)), dim3(DL_BLOCK), 0, s,
                            (const T *) x, a, b, (const T *) w, (const T *) gy, start, idx, (T *) gx, in_dim, batch,
                            (C) scale);
     }
@@ -905,16 +905,16 @@ int group_sum_forward_t(const void *x, void *y, void *workspace, int64_t out_dim
     if (gx > 0x7fffffffLL || k > 65535) return DL_ERR_TOO_LARGE;
     const dim3 grid((unsigned) gx, (unsigned) k, (unsigned) splits);
     if (vec)
-        hipLaunchKernelGGL((group_sum_partial_kernel<T, V>), grid, dim3(DL_BLOCK), 0, s, (const T *) x, (C *) workspace,
+        DL_LAUNCH((group_sum_partial_kernel<T, V>), grid, dim3(DL_BLOCK), 0, s, (const T *) x, (C *) workspace,
                            per_class, ncols, k, rows_per_split);
     else
-        hipLaunchKernelGGL((group_sum_partial_kernel<T, 1>), grid, dim3(DL_BLOCK), 0, s, (const T *) x, (C *) workspace,
+        DL_LAUNCH((group_sum_partial_kernel<T, 1>), grid, dim3(DL_BLOCK), 0, s, (const T *) x, (C *) workspace,
                            per_class, ncols, k, rows_per_split);
     int st = dl_launch_status();
     if (st != DL_OK) return st;
     const int64_t blocks = dl_ceil_div(batch, DL_WAVE);
     if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
-    hipLaunchKernelGGL((group_sum_finish_kernel<T>), dim3((unsigned) blocks, (unsigned) k), dim3(DL_BLOCK), 0, s,
+    DL_LAUNCH((group_sum_finish_kernel<T>), dim3((unsigned) blocks, (unsigned) k), dim3(DL_BLOCK), 0, s,
                        (const C *) workspace, (T *) y, batch, k, splits, (C) (1.0 / tau));
     return dl_launch_status();
 }
@@ -929,10 +929,10 @@ int group_sum_backward_t(const void *g, void *gx, int64_t out_dim, int64_t batch
     if (gxd > 0x7fffffffLL || gyd > 65535) return DL_ERR_TOO_LARGE;
     const dim3 grid((unsigned) gxd, (unsigned) gyd);
     if (vec)
-        hipLaunchKernelGGL((group_sum_backward_kernel<T, V>), grid, dim3(DL_BLOCK), 0, s, (const T *) g, (T *) gx, out_dim,
+        DL_LAUNCH((group_sum_backward_kernel<T, V>), grid, dim3(DL_BLOCK), 0, s, (const T *) g, (T *) gx, out_dim,
                            out_dim / k, ncols, k, (C) (1.0 / tau));
     else
-        hipLaunchKernelGGL((group_sum_backward_kernel<T, 1>), grid, dim3(DL_BLOCK), 0, s, (const T *) g, (T *) gx, out_dim,
+        DL_LAUNCH((group_sum_backward_kernel<T, 1>), grid, dim3(DL_BLOCK), 0, s, (const T *) g, (T *) gx, out_dim,
                            out_dim / k, ncols, k, (C) (1.0 / tau));
     return dl_launch_status();
 }
@@ -974,16 +974,16 @@ int forward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, 
         if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
         const dim3 grid((unsigned) blocks), block(DL_BLOCK);
         if (ncols <= 2 * DL_WAVE)
-            hipLaunchKernelGGL((forward_chain_rows_kernel<T, V, 2, LOGITS>), grid, block, 0, s, xp, verts, neuron, flip, wp,
+            DL_LAUNCH((forward_chain_rows_kernel<T, V, 2, LOGITS>), grid, block, 0, s, xp, verts, neuron, flip, wp,
                                (T *) y, (T *) probs, steps, chunk, ncols);
         else
-            hipLaunchKernelGGL((forward_chain_rows_kernel<T, V, 4, LOGITS>), grid, block, 0, s, xp, verts, neuron, flip, wp,
+            DL_LAUNCH((forward_chain_rows_kernel<T, V, 4, LOGITS>), grid, block, 0, s, xp, verts, neuron, flip, wp,
                                (T *) y, (T *) probs, steps, chunk, ncols);
         return dl_launch_status();
     }
     const int64_t blocks = dl_ceil_div(nchunks, 4);
     if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
-    hipLaunchKernelGGL((forward_chain_kernel<T, V, DL_TRAIN_CHUNK, LOGITS>), dim3((unsigned) blocks, col_tiles(ncols)),
+    DL_LAUNCH((forward_chain_kernel<T, V, DL_TRAIN_CHUNK, LOGITS>), dim3((unsigned) blocks, col_tiles(ncols)),
                        dim3(DL_BLOCK), 0, s, xp, verts, neuron, flip, wp, (T *) y, (T *) probs, nchunks, ncols);
     return dl_launch_status();
 }
@@ -999,13 +999,13 @@ int backward_w_chain_t(const void *x, const int32_t *verts, const int32_t *neuro
     const dim3 grid((unsigned) blocks), block(DL_BLOCK);
     const T *xp = (const T *) x, *gp = (const T *) gy, *pp = (const T *) probs;
     if (ncols <= DL_WAVE)
-        hipLaunchKernelGGL((backward_w_chain_kernel<T, V, 1, DL_TRAIN_CHUNK>), grid, block, 0, s, xp, verts, neuron, flip,
+        DL_LAUNCH((backward_w_chain_kernel<T, V, 1, DL_TRAIN_CHUNK>), grid, block, 0, s, xp, verts, neuron, flip,
                            gp, pp, (T *) gw, nchunks, ncols);
     else if (ncols <= 2 * DL_WAVE)
-        hipLaunchKernelGGL((backward_w_chain_kernel<T, V, 2, DL_TRAIN_CHUNK>), grid, block, 0, s, xp, verts, neuron, flip,
+        DL_LAUNCH((backward_w_chain_kernel<T, V, 2, DL_TRAIN_CHUNK>), grid, block, 0, s, xp, verts, neuron, flip,
                            gp, pp, (T *) gw, nchunks, ncols);
     else
-        hipLaunchKernelGGL((backward_w_chain_kernel<T, V, 4, DL_TRAIN_CHUNK>), grid, block, 0, s, xp, verts, neuron, flip,
+        DL_LAUNCH((backward_w_chain_kernel<T, V, 4, DL_TRAIN_CHUNK>), grid, block, 0, s, xp, verts, neuron, flip,
                            gp, pp, (T *) gw, nchunks, ncols);
     return dl_launch_status();
 }
@@ -1026,7 +1026,7 @@ int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron,
     const dim3 grid((unsigned) blocks), block(DL_BLOCK);
     const T *xp = (const T *) x, *wp = (const T *) w, *gp = (const T *) gy, *pp = softmax_backward ? wp : nullptr;
 #define DL_LAUNCH_BACKWARD_CHAIN(CPL)                                                                                   \
-    hipLaunchKernelGGL((backward_chain_kernel<T, V, CPL>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp, pp, \
+    DL_LAUNCH((backward_chain_kernel<T, V, CPL>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp, pp, \
                        (T *) gw, (T *) gx, (T *) overflow, steps, chunk, in_dim, ncols, (C) scale)
     if (ncols <= DL_WAVE)
         DL_LAUNCH_BACKWARD_CHAIN(1);
@@ -1037,7 +1037,7 @@ int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron,
 #undef DL_LAUNCH_BACKWARD_CHAIN
     int st = dl_launch_status();
     if (st != DL_OK || n_fix == 0) return st;
-    hipLaunchKernelGGL((backward_fix_kernel<T, V>), dim3((unsigned) fix_blocks, col_tiles(ncols)), block, 0, s,
+    DL_LAUNCH((backward_fix_kernel<T, V>), dim3((unsigned) fix_blocks, col_tiles(ncols)), block, 0, s,
                        (const T *) overflow, fix_vertex, fix_start, (T *) gx, n_fix, ncols);
     return dl_launch_status();
 }

@@ -34,7 +34,7 @@ typedef enum dl_status {
     DL_ERR_BIT_COUNT = 2,        /* bit_count not in {8, 16, 32, 64}                          */
     DL_ERR_NOT_DIVISIBLE = 3,    /* groupbitsum: in_dim not divisible by k                    */
     DL_ERR_DTYPE = 4,            /* dtype not one of dl_dtype                                 */
-    DL_ERR_LAUNCH = 5,           /* the HIP runtime refused the launch (see hipGetLastError)  */
+    DL_ERR_LAUNCH = 5,           /* the HIP runtime refused the launch (see dl_last_hip_error) */
     DL_ERR_TOO_LARGE = 6         /* a size exceeds what the entry point supports              */
 } dl_status;
 
@@ -43,6 +43,8 @@ typedef enum dl_dtype { DL_F16 = 0, DL_F32 = 1, DL_F64 = 2 } dl_dtype;
 /* Library version (major*10000 + minor*100 + patch) and a static message per status. */
 int dl_version(void);
 const char *dl_status_string(int status);
+/* HIP's description of the error behind the calling thread's last DL_ERR_LAUNCH. */
+const char *dl_last_hip_error(void);
 
 /* ---- training mode -------------------------------------------------------------------- */
 

@@ -70,3 +70,15 @@ def test_binding_rejects_cpu_tensors_and_bad_arguments():
         ext.groupbitsum(x, 0, 2)
     with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
         ext.tensor_packbits_cuda(torch.zeros(2, 8, dtype=torch.bool), 8)
+
+
+def test_library_shares_torchs_hip_runtime_whatever_the_import_order():
+    """Importing the package before torch must not bring a second HIP runtime into the process."""
+    import subprocess
+    import sys
+    code = ("import difflogic_amd, torch\n"
+            "libs = {l.split()[-1] for l in open('/proc/self/maps') if 'libamdhip64' in l}\n"
+            "print(len(libs), sorted(libs))")
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=ROOT, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert out.stdout.split()[0] == "1", out.stdout
