@@ -31,8 +31,9 @@ SIGNATURES = {
     "dl_logic_backward_w_chained": [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "dl_logic_backward_x": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _dbl, _int, _vp],
     "dl_backward_schedule_build": [_vp, _vp, _i64, _i64, _vp, _vp, _vp, ctypes.POINTER(_i64)],
-    "dl_logic_backward_chained": [_vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _int, _vp, _vp, _i64, _vp, _vp, _vp, _i64,
-                                  _i64, _i64, _dbl, _int, _vp],
+    "dl_logic_backward_chained": [_vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _int, _vp, _vp, _i64, _i64, _vp, _vp, _vp,
+                                  _i64, _i64, _i64, _dbl, _int, _vp],
+    "dl_logic_backward_chained_workspace_bytes": [_i64, _i64, _i64, _int],
     "dl_group_sum_workspace_bytes": [_i64, _i64, _i64, _int],
     "dl_group_sum_forward": [_vp, _vp, _vp, _i64, _i64, _i64, _dbl, _int, _vp],
     "dl_group_sum_backward": [_vp, _vp, _i64, _i64, _i64, _dbl, _int, _vp],
@@ -53,6 +54,7 @@ _RESTYPES = {"dl_status_string": ctypes.c_char_p, "dl_last_hip_error": ctypes.c_
              "dl_logic_eval_fused_workspace_bytes": ctypes.c_int64,
              "dl_eval_schedule_capacity": ctypes.c_int64, "dl_eval_schedule_build": ctypes.c_int64,
              "dl_backward_schedule_build": ctypes.c_int64,
+             "dl_logic_backward_chained_workspace_bytes": ctypes.c_int64,
              "dl_logic_eval_fused_groupbitsum_workspace_bytes": ctypes.c_int64}
 
 _lib = None

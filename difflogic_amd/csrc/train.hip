@@ -450,9 +450,10 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_chain_kernel(const T *__rest
     }
 }
 
-// Forward along the schedule for rows of up to 256 vectors: one wave owns `chunk` steps and the
-// WHOLE row (lane l holds vectors l, l + 64, ...), so every gathered row is one contiguous
-// request, and the next step's row is requested before this step's arithmetic.
+// Forward along the schedule for long rows: one wave owns `chunk` steps and a segment of
+// CPL * 64 consecutive vectors of the row (blockIdx.y picks the segment; lane l holds its vectors
+// l, l + 64, ...), so every gathered row is one contiguous request of up to 4 KB, and the next
+// step's row is requested before this step's arithmetic.
 template <typename T, int VEC, int CPL, bool LOGITS>
 __global__ __launch_bounds__(DL_BLOCK) void forward_chain_rows_kernel(const T *__restrict__ x,
                                                                       const int32_t *__restrict__ verts,
@@ -470,13 +471,14 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_chain_rows_kernel(const T *_
     const int64_t s1 = s0 + chunk < steps ? s0 + chunk : steps;
     const P *xv = reinterpret_cast<const P *>(x);
     P *yv = reinterpret_cast<P *>(y);
+    const int64_t col0 = (int64_t) blockIdx.y * (CPL * DL_WAVE);
     P zero;
 #pragma unroll
     for (int e = 0; e < VEC; ++e) zero.v[e] = down<T, C>((C) 0);
     auto load_row = [&](int64_t row, P *out) {
 #pragma unroll
         for (int q = 0; q < CPL; ++q) {
-            const int64_t col = lane + q * DL_WAVE;
+            const int64_t col = col0 + lane + q * DL_WAVE;
             out[q] = col < ncols ? xv[row * ncols + col] : zero;
         }
     };
@@ -489,10 +491,10 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_chain_rows_kernel(const T *_
         const int32_t n = neuron[s];
         const bool f = flip[s] != 0;
         C p00, p10, d0, d1;
-        neuron_corners<T, LOGITS>(w, n >= 0 ? n : 0, lane, n >= 0, probs, p00, p10, d0, d1);
+        neuron_corners<T, LOGITS>(w, n >= 0 ? n : 0, lane, n >= 0 && col0 == 0, probs, p00, p10, d0, d1);
 #pragma unroll
         for (int q = 0; q < CPL; ++q) {
-            const int64_t col = lane + q * DL_WAVE;
+            const int64_t col = col0 + lane + q * DL_WAVE;
             P r;
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
@@ -581,7 +583,9 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_w_chain_kernel(const T *__r
 // A vertex in the middle of a trail collects the share of the neuron before it (kept in
 // `carry`) and of the neuron after it and is written once: position p of the schedule goes to
 // row dst[p] (-1: nothing to write; >= in_dim: row dst[p] - in_dim of `overflow`, for vertices
-// that occur at several positions and are summed afterwards by backward_fix_kernel).  A wave
+// that occur at several positions and are summed afterwards by backward_fix_kernel).  Rows longer
+// than CPL * 64 vectors are cut into segments (blockIdx.y); the corner sums of the segments then
+// go to `partial` and backward_w_finish_kernel adds them.  A wave
 // owns `chunk` positions [s0, s0 + chunk); it recomputes the last neuron of the chunk before it to get
 // the carry into its first position, so chunks do not exchange partial rows.
 // ------------------------------------------------------------------------------------------
@@ -589,8 +593,9 @@ template <typename T, int VEC, int CPL>
 __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
     const T *__restrict__ x, const int32_t *__restrict__ verts, const int32_t *__restrict__ neuron,
     const uint8_t *__restrict__ flip, const int32_t *__restrict__ dst, const T *__restrict__ w,
-    const T *__restrict__ gy, const T *__restrict__ probs, T *__restrict__ gw, T *__restrict__ gx,
-    T *__restrict__ overflow, int64_t steps, int chunk, int64_t in_dim, int64_t ncols, typename Acc<T>::type scale) {
+    const T *__restrict__ gy, const T *__restrict__ probs, T *__restrict__ gw,
+    typename Acc<T>::type *__restrict__ partial, T *__restrict__ gx, T *__restrict__ overflow, int64_t steps, int chunk,
+    int64_t in_dim, int64_t out_dim, int64_t ncols, typename Acc<T>::type scale) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
     const int wave = dl_wave_in_block();
@@ -600,6 +605,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
     const int64_t s1 = s0 + chunk < steps ? s0 + chunk : steps;
     const P *xv = reinterpret_cast<const P *>(x);
     const P *gv = reinterpret_cast<const P *>(gy);
+    const int64_t col0 = (int64_t) blockIdx.y * (CPL * DL_WAVE);   // this wave's segment of the rows
     P zero;
 #pragma unroll
     for (int e = 0; e < VEC; ++e) zero.v[e] = down<T, C>((C) 0);
@@ -607,7 +613,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
     auto load_row = [&](const P *base, int64_t row, bool valid, P *out) {
 #pragma unroll
         for (int q = 0; q < CPL; ++q) {
-            const int64_t col = lane + q * DL_WAVE;
+            const int64_t col = col0 + lane + q * DL_WAVE;
             out[q] = (valid && col < ncols) ? base[row * ncols + col] : zero;
         }
     };
@@ -617,7 +623,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
                                : reinterpret_cast<P *>(overflow) + ((int64_t) row - in_dim) * ncols;
 #pragma unroll
         for (int q = 0; q < CPL; ++q) {
-            const int64_t col = lane + q * DL_WAVE;
+            const int64_t col = col0 + lane + q * DL_WAVE;
             P r;
 #pragma unroll
             for (int e = 0; e < VEC; ++e) r.v[e] = down<T, C>(val[q][e] * scale);
@@ -681,7 +687,12 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
         s01 = wave_sum(s01);
         s10 = wave_sum(s10);
         s11 = wave_sum(s11);
-        store_grad_w<T>(lane, valid, nn, s00, s01, s10, s11, probs, gw);
+        if (partial == nullptr) {
+            store_grad_w<T>(lane, valid, nn, s00, s01, s10, s11, probs, gw);
+        } else if (valid && lane < 4) {              // several segments: backward_w_finish_kernel adds them
+            const C mine = lane == 0 ? s00 : lane == 1 ? s01 : lane == 2 ? s10 : s11;
+            partial[((int64_t) blockIdx.y * out_dim + nn) * 4 + lane] = mine;
+        }
 #pragma unroll
         for (int q = 0; q < CPL; ++q) prev[q] = cur[q];
     }
@@ -720,6 +731,35 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_fix_kernel(const T *__restr
         for (int e = 0; e < VEC; ++e) res.v[e] = down<T, C>(acc[e]);
         out[v * ncols + col] = res;
     }
+}
+
+// grad_w from the per-segment corner sums of backward_chain_kernel, added in segment order.
+// One 16-lane row per neuron (4 neurons per wave).
+template <typename T>
+__global__ __launch_bounds__(DL_BLOCK) void backward_w_finish_kernel(const typename Acc<T>::type *__restrict__ partial,
+                                                                     const T *__restrict__ probs, T *__restrict__ gw,
+                                                                     int64_t out_dim, int segments) {
+    typedef typename Acc<T>::type C;
+    const int lane = dl_lane();
+    const int64_t n = ((int64_t) blockIdx.x * 4 + dl_wave_in_block()) * 4 + (lane >> 4);
+    const bool valid = n < out_dim;
+    const int gate = lane & 15;
+    C sum[4] = {(C) 0, (C) 0, (C) 0, (C) 0};
+    if (valid)
+        for (int g = 0; g < segments; ++g)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) sum[c] += partial[((int64_t) g * out_dim + n) * 4 + c];
+    C r = (C) 0;
+    if (gate & 8) r += sum[0];
+    if (gate & 4) r += sum[1];
+    if (gate & 2) r += sum[2];
+    if (gate & 1) r += sum[3];
+    if (probs != nullptr) {
+        const C p = valid ? up<T>(probs[n * 16 + gate]) : (C) 0;
+        const C dot = row16_sum(p * r);
+        r = p * (r - dot);
+    }
+    if (valid) gw[n * 16 + gate] = down<T, C>(r);
 }
 
 template <typename T> struct Vec16 { static constexpr int n = 16 / (int) sizeof(T); };
@@ -952,6 +992,11 @@ int group_sum_splits(int64_t out_dim, int64_t batch, int64_t k) {
 #define DL_TRAIN_CHUNK 8     // must equal the chunk the schedule was built with (dl_eval_schedule_chunk)
 #define DL_FWD_ROWS_MIN 128  // vectors per row above which forward_chain_rows_kernel takes over
 
+// Longest row (in 16-byte vectors) the whole-row kernels take: 16 segments of 256.
+#define DL_ROWS_MAX_VECTORS (16 * 4 * DL_WAVE)
+
+int row_segments(int64_t ncols) { return (int) dl_ceil_div(ncols, 4 * DL_WAVE); }
+
 // Steps per wave of the kernels in which a wave owns whole rows: long chunks re-read fewer rows at
 // their seams, short ones give more waves to hide latency with; keep about three waves per SIMD.
 int chain_chunk(int64_t steps) {
@@ -967,12 +1012,13 @@ int forward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, 
     if (batch % V != 0 || !dl_aligned(x, 16) || !dl_aligned(y, 16)) return DL_ERR_TOO_LARGE;
     const int64_t nchunks = steps / DL_TRAIN_CHUNK, ncols = batch / V;
     const T *xp = (const T *) x, *wp = (const T *) w;
-    if (ncols > DL_FWD_ROWS_MIN && ncols <= 4 * DL_WAVE) {
-        // rows of 2-4 KB: a wave takes whole rows
-        const int chunk = chain_chunk(steps);
+    if (ncols > DL_FWD_ROWS_MIN && ncols <= DL_ROWS_MAX_VECTORS) {
+        // rows of 2 KB and more: a wave takes whole rows, or segments of 4 KB
+        const int segments = row_segments(ncols);
+        const int chunk = chain_chunk(steps * segments);
         const int64_t blocks = dl_ceil_div(dl_ceil_div(steps, chunk), 4);
         if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
-        const dim3 grid((unsigned) blocks), block(DL_BLOCK);
+        const dim3 grid((unsigned) blocks, (unsigned) segments), block(DL_BLOCK);
         if (ncols <= 2 * DL_WAVE)
             DL_LAUNCH((forward_chain_rows_kernel<T, V, 2, LOGITS>), grid, block, 0, s, xp, verts, neuron, flip, wp,
                                (T *) y, (T *) probs, steps, chunk, ncols);
@@ -1010,24 +1056,37 @@ int backward_w_chain_t(const void *x, const int32_t *verts, const int32_t *neuro
     return dl_launch_status();
 }
 
+template <typename T> int64_t backward_partial_bytes(int64_t out_dim, int64_t batch) {
+    constexpr int V = Vec16<T>::n;
+    const int segments = batch % V == 0 ? row_segments(batch / V) : 1;
+    return segments > 1 ? (int64_t) segments * out_dim * 4 * (int64_t) sizeof(typename Acc<T>::type) : 0;
+}
+
 template <typename T>
 int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, const uint8_t *flip, const int32_t *dst,
                      int64_t steps, const void *w, const void *gy, bool softmax_backward, const int32_t *fix_vertex,
-                     const int32_t *fix_start, int64_t n_fix, void *gw, void *gx, void *overflow, int64_t in_dim,
-                     int64_t batch, double scale, hipStream_t s) {
+                     const int32_t *fix_start, int64_t n_fix, int64_t overflow_rows, void *gw, void *gx, void *workspace,
+                     int64_t in_dim, int64_t out_dim, int64_t batch, double scale, hipStream_t s) {
     typedef typename Acc<T>::type C;
     constexpr int V = Vec16<T>::n;
-    if (batch % V != 0 || !dl_aligned(x, 16) || !dl_aligned(gy, 16) || !dl_aligned(gx, 16) || !dl_aligned(overflow, 16))
+    if (batch % V != 0 || !dl_aligned(x, 16) || !dl_aligned(gy, 16) || !dl_aligned(gx, 16) || !dl_aligned(workspace, 16))
         return DL_ERR_TOO_LARGE;
     const int64_t ncols = batch / V;
-    const int chunk = chain_chunk(steps);
+    if (ncols > DL_ROWS_MAX_VECTORS) return DL_ERR_TOO_LARGE;
+    const int segments = row_segments(ncols);
+    // workspace: [segments x out x 4 corner sums (only with several segments)] [overflow rows]
+    const int64_t partial_bytes = backward_partial_bytes<T>(out_dim, batch);
+    if ((partial_bytes > 0 || overflow_rows > 0) && workspace == nullptr) return DL_ERR_INVALID_ARGUMENT;
+    C *partial = partial_bytes > 0 ? (C *) workspace : nullptr;
+    T *overflow = (T *) ((char *) workspace + partial_bytes);
+    const int chunk = chain_chunk(steps * segments);
     const int64_t blocks = dl_ceil_div(dl_ceil_div(steps, chunk), 4), fix_blocks = dl_ceil_div(n_fix, 4);
-    if (blocks > 0x7fffffffLL || fix_blocks > 0x7fffffffLL || ncols > 4 * DL_WAVE) return DL_ERR_TOO_LARGE;
-    const dim3 grid((unsigned) blocks), block(DL_BLOCK);
+    if (blocks > 0x7fffffffLL || fix_blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    const dim3 grid((unsigned) blocks, (unsigned) segments), block(DL_BLOCK);
     const T *xp = (const T *) x, *wp = (const T *) w, *gp = (const T *) gy, *pp = softmax_backward ? wp : nullptr;
-#define DL_LAUNCH_BACKWARD_CHAIN(CPL)                                                                                   \
-    DL_LAUNCH((backward_chain_kernel<T, V, CPL>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp, pp, \
-                       (T *) gw, (T *) gx, (T *) overflow, steps, chunk, in_dim, ncols, (C) scale)
+#define DL_LAUNCH_BACKWARD_CHAIN(CPL)                                                                                  \
+    DL_LAUNCH((backward_chain_kernel<T, V, CPL>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp, pp, (T *) gw, \
+              partial, (T *) gx, overflow, steps, chunk, in_dim, out_dim, ncols, (C) scale)
     if (ncols <= DL_WAVE)
         DL_LAUNCH_BACKWARD_CHAIN(1);
     else if (ncols <= 2 * DL_WAVE)
@@ -1036,21 +1095,42 @@ int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron,
         DL_LAUNCH_BACKWARD_CHAIN(4);
 #undef DL_LAUNCH_BACKWARD_CHAIN
     int st = dl_launch_status();
-    if (st != DL_OK || n_fix == 0) return st;
+    if (st != DL_OK) return st;
+    if (partial != nullptr) {
+        const int64_t fin_blocks = dl_ceil_div(out_dim, 16);
+        if (fin_blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+        DL_LAUNCH(backward_w_finish_kernel<T>, dim3((unsigned) fin_blocks), block, 0, s, (const C *) partial, pp, (T *) gw,
+                  out_dim, segments);
+        st = dl_launch_status();
+        if (st != DL_OK) return st;
+    }
+    if (n_fix == 0) return DL_OK;
     DL_LAUNCH((backward_fix_kernel<T, V>), dim3((unsigned) fix_blocks, col_tiles(ncols)), block, 0, s,
-                       (const T *) overflow, fix_vertex, fix_start, (T *) gx, n_fix, ncols);
+              (const T *) overflow, fix_vertex, fix_start, (T *) gx, n_fix, ncols);
     return dl_launch_status();
 }
 
 }  // namespace
 
+extern "C" int64_t dl_logic_backward_chained_workspace_bytes(int64_t overflow_rows, int64_t out_dim, int64_t batch,
+                                                             int dtype) {
+    if (overflow_rows < 0 || out_dim < 0 || batch < 0) return -DL_ERR_INVALID_ARGUMENT;
+    switch (dtype) {
+    case DL_F16: return backward_partial_bytes<__half>(out_dim, batch) + overflow_rows * batch * 2;
+    case DL_F32: return backward_partial_bytes<float>(out_dim, batch) + overflow_rows * batch * 4;
+    case DL_F64: return backward_partial_bytes<double>(out_dim, batch) + overflow_rows * batch * 8;
+    default: return -DL_ERR_DTYPE;
+    }
+}
+
 extern "C" int dl_logic_backward_chained(const void *x, const int32_t *verts, const int32_t *neuron, const uint8_t *flip,
                                          const int32_t *dst, int64_t steps, const void *w, const void *grad_y,
                                          int softmax_backward, const int32_t *fix_vertex, const int32_t *fix_start,
-                                         int64_t n_fix, void *grad_w, void *grad_x, void *overflow, int64_t in_dim,
-                                         int64_t out_dim, int64_t batch, double scale, int dtype, void *stream) {
+                                         int64_t n_fix, int64_t overflow_rows, void *grad_w, void *grad_x,
+                                         void *workspace, int64_t in_dim, int64_t out_dim, int64_t batch, double scale,
+                                         int dtype, void *stream) {
     if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
-    if (in_dim <= 0 || out_dim <= 0 || batch <= 0 || steps < out_dim || n_fix < 0 || n_fix > in_dim)
+    if (in_dim <= 0 || out_dim <= 0 || batch <= 0 || steps < out_dim || n_fix < 0 || n_fix > in_dim || overflow_rows < 0)
         return DL_ERR_INVALID_ARGUMENT;
     if (!x || !verts || !neuron || !flip || !dst || !w || !grad_y || !grad_w || !grad_x) return DL_ERR_INVALID_ARGUMENT;
     if (n_fix > 0 && (!fix_vertex || !fix_start)) return DL_ERR_INVALID_ARGUMENT;
@@ -1059,13 +1139,13 @@ extern "C" int dl_logic_backward_chained(const void *x, const int32_t *verts, co
     switch (dtype) {
     case DL_F16:
         return backward_chain_t<__half>(x, verts, neuron, flip, dst, steps, w, grad_y, sb, fix_vertex, fix_start, n_fix,
-                                        grad_w, grad_x, overflow, in_dim, batch, scale, s);
+                                        overflow_rows, grad_w, grad_x, workspace, in_dim, out_dim, batch, scale, s);
     case DL_F32:
         return backward_chain_t<float>(x, verts, neuron, flip, dst, steps, w, grad_y, sb, fix_vertex, fix_start, n_fix,
-                                       grad_w, grad_x, overflow, in_dim, batch, scale, s);
+                                       overflow_rows, grad_w, grad_x, workspace, in_dim, out_dim, batch, scale, s);
     default:
         return backward_chain_t<double>(x, verts, neuron, flip, dst, steps, w, grad_y, sb, fix_vertex, fix_start, n_fix,
-                                        grad_w, grad_x, overflow, in_dim, batch, scale, s);
+                                        overflow_rows, grad_w, grad_x, workspace, in_dim, out_dim, batch, scale, s);
     }
 }
 

@@ -237,13 +237,17 @@ def backward_chained(x, w, grad_y, schedule, scale=1.0, softmax_backward=False):
         return None
     grad_w = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
     grad_x = torch.empty_like(x)
-    overflow = torch.empty((rows, batch), dtype=x.dtype, device=dev) if rows else None
+    lib = _lib.load()
+    ws_bytes = lib.dl_logic_backward_chained_workspace_bytes(rows, out_dim, batch, code)
+    if ws_bytes < 0:
+        _raise(-ws_bytes, "logic_layer_cuda_backward_chained")
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
     with torch.cuda.device(dev):
-        st = _lib.load().dl_logic_backward_chained(
+        st = lib.dl_logic_backward_chained(
             _p(x), _p(schedule.verts), _p(schedule.neuron), _p(schedule.flip), _p(dst), schedule.steps, _p(w),
             _p(grad_y), 1 if softmax_backward else 0, _p(fix_vertex) if n_fix else None,
-            _p(fix_start) if n_fix else None, n_fix, _p(grad_w), _p(grad_x), _p(overflow) if rows else None, in_dim,
-            out_dim, batch, float(scale), code, _stream(dev))
+            _p(fix_start) if n_fix else None, n_fix, rows, _p(grad_w), _p(grad_x),
+            _p(workspace) if ws_bytes else None, in_dim, out_dim, batch, float(scale), code, _stream(dev))
     if st == _lib.DL_ERR_TOO_LARGE:
         return None
     if st:

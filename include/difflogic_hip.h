@@ -88,7 +88,7 @@ int dl_logic_backward_logits(const void *x, const int64_t *a, const int64_t *b, 
  *          backward - NULL: plain grad_w; else the softmax backward is chained
  *                     (as dl_logic_backward_logits).
  * Return DL_ERR_TOO_LARGE where the chained kernels do not apply (batch not a multiple of 16
- * bytes of elements, unaligned buffers; backward: rows longer than 256 vectors of 16 bytes);
+ * bytes of elements, unaligned buffers; backward_w: rows longer than 256 vectors of 16 bytes);
  * the caller then uses the unchained entry points. */
 int dl_logic_forward_chained(const void *x, const int32_t *verts, const int32_t *neuron,
                              const uint8_t *flip, int64_t steps, const void *w, void *y, void *probs,
@@ -124,19 +124,24 @@ int dl_logic_backward_x(const void *x, const int64_t *a, const int64_t *b, const
  *   dl_logic_backward_chained()   DEVICE pointers.  w [out,16]: the gate probabilities the forward
  *       pass used.  softmax_backward = 0: grad_w as dl_logic_backward_w; else the gradient with
  *       respect to the logits as dl_logic_backward_logits (w = its probs).  grad_x as
- *       dl_logic_backward_x (same `scale`, same a == b rule) up to summation order.  overflow:
- *       scratch of (overflow rows) x batch elements, 16-byte aligned; may be NULL when there are
- *       none.  Returns DL_ERR_TOO_LARGE where it does not apply (see the chained entry points
- *       above); the caller then uses the separate entry points. */
+ *       dl_logic_backward_x (same `scale`, same a == b rule) up to summation order.
+ *       overflow_rows: what dl_backward_schedule_build returned.  workspace: DEVICE scratch of
+ *       dl_logic_backward_chained_workspace_bytes(overflow_rows, out_dim, batch, dtype) bytes,
+ *       16-byte aligned (NULL if that is 0): the overflow rows and, for rows longer than 4 KB,
+ *       per-segment partial sums of grad_w.  Returns DL_ERR_TOO_LARGE where it does not apply
+ *       (batch not a multiple of 16 bytes of elements, unaligned buffers, rows longer than
+ *       64 KB); the caller then uses the separate entry points. */
 int64_t dl_backward_schedule_build(const int32_t *verts, const int32_t *neuron, int64_t steps,
                                    int64_t in_dim, int32_t *dst, int32_t *fix_vertex,
                                    int32_t *fix_start, int64_t *n_fix);
 int dl_logic_backward_chained(const void *x, const int32_t *verts, const int32_t *neuron,
                               const uint8_t *flip, const int32_t *dst, int64_t steps, const void *w,
                               const void *grad_y, int softmax_backward, const int32_t *fix_vertex,
-                              const int32_t *fix_start, int64_t n_fix, void *grad_w, void *grad_x,
-                              void *overflow, int64_t in_dim, int64_t out_dim, int64_t batch,
-                              double scale, int dtype, void *stream);
+                              const int32_t *fix_start, int64_t n_fix, int64_t overflow_rows,
+                              void *grad_w, void *grad_x, void *workspace, int64_t in_dim,
+                              int64_t out_dim, int64_t batch, double scale, int dtype, void *stream);
+int64_t dl_logic_backward_chained_workspace_bytes(int64_t overflow_rows, int64_t out_dim,
+                                                  int64_t batch, int dtype);
 
 /* ---- GroupSum on the feature-major layout (training mode) ------------------------------- */
 
