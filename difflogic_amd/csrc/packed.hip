@@ -437,31 +437,37 @@ __global__ __launch_bounds__(DL_BLOCK) void packbits_batch_major_kernel(const ui
     }
 }
 
-// Variant for narrow inputs (features % 16 == 0, staging + result tile within 64 KB of LDS): the 64 sample rows of one
-// word column are one contiguous block of the input, which the workgroup copies into LDS with
-// fully coalesced 16-byte loads (no partial cache lines however the rows fall), then every
-// thread folds one group of four features from LDS exactly as above.  WC word columns per
-// workgroup, so that a feature row is written in runs of 8 * WC bytes.
+// Variant for features % 16 == 0: the workgroup copies the 64 sample rows of one word column
+// (a slice of `slice` features of them when the rows are too long for LDS; consecutive workgroups
+// take the `nslices` slices of the same rows, so that the chip reads a contiguous region) into LDS with coalesced 16-byte loads, so no partial cache lines are fetched however
+// the rows fall, then every thread folds one group of four features from LDS exactly as above.
+// WC word columns per workgroup, so that a feature row is written in runs of 8 * WC bytes.
 template <int WC>
 __global__ __launch_bounds__(DL_BLOCK) void packbits_batch_major_lds_kernel(const uint8_t *__restrict__ x,
                                                                             uint8_t *__restrict__ out, int64_t batch,
-                                                                            int64_t features,
+                                                                            int64_t features, int slice, int nslices,
                                                                             int64_t out_row_bytes) {
     extern __shared__ __align__(16) uint8_t lds_raw[];
-    dl_u32x4 *stage = reinterpret_cast<dl_u32x4 *>(lds_raw);                        // 64 * features bytes
-    uint64_t *words = reinterpret_cast<uint64_t *>(lds_raw + 64 * features);         // [features][WC]
-    const int64_t w0 = (int64_t) blockIdx.x * WC;
-    const int groups = (int) (features / 4);                                         // dword columns
-    const int chunks = (int) (4 * features);                                         // 16-byte chunks per word column
+    dl_u32x4 *stage = reinterpret_cast<dl_u32x4 *>(lds_raw);                        // 64 * slice bytes
+    uint64_t *words = reinterpret_cast<uint64_t *>(lds_raw + 64 * slice);            // [slice][WC]
+    const int64_t w0 = (int64_t) (blockIdx.x / (unsigned) nslices) * WC;
+    const int64_t f0 = (int64_t) (blockIdx.x % (unsigned) nslices) * slice;
+    const int fs = (int) (features - f0 < slice ? features - f0 : slice);           // this slice's features
+    const int groups = fs / 4;                                                       // dword columns
+    const int per_row = fs / 16;                                                     // 16-byte chunks per sample
+    const int chunks = 64 * per_row;
 
     for (int wc = 0; wc < WC; ++wc) {
         const int64_t s0 = (w0 + wc) * 64;
         if (s0 >= batch) break;                                                      // uniform
-        const int64_t valid = (batch - s0 < 64 ? batch - s0 : 64) * features / 16;   // chunks holding real samples
-        const dl_u32x4 *src = reinterpret_cast<const dl_u32x4 *>(x + s0 * features);
+        const int rows = (int) (batch - s0 < 64 ? batch - s0 : 64);                  // real samples
+        const uint8_t *src = x + s0 * features + f0;
         __syncthreads();                                                             // previous column's readers are done
-        for (int i = threadIdx.x; i < chunks; i += DL_BLOCK)
-            stage[i] = i < valid ? __builtin_nontemporal_load(src + i) : dl_u32x4{0, 0, 0, 0};
+        for (int i = threadIdx.x; i < chunks; i += DL_BLOCK) {
+            const int r = i / per_row, c = i - r * per_row;
+            stage[i] = r < rows ? __builtin_nontemporal_load(reinterpret_cast<const dl_u32x4 *>(src + r * features) + c)
+                                : dl_u32x4{0, 0, 0, 0};
+        }
         __syncthreads();
         const uint32_t *flags = reinterpret_cast<const uint32_t *>(lds_raw);
         for (int g = threadIdx.x; g < groups; g += DL_BLOCK) {
@@ -491,10 +497,10 @@ __global__ __launch_bounds__(DL_BLOCK) void packbits_batch_major_lds_kernel(cons
     __syncthreads();
     // WC consecutive threads write the WC words of one feature row (out_row_bytes % 8 == 0 here)
     const int64_t total_words = out_row_bytes / 8;
-    for (int i = threadIdx.x; i < (int) features * WC; i += DL_BLOCK) {
+    for (int i = threadIdx.x; i < fs * WC; i += DL_BLOCK) {
         const int f = i / WC, wc = i - f * WC;
         if (w0 + wc < total_words)
-            *reinterpret_cast<uint64_t *>(out + (int64_t) f * out_row_bytes + (w0 + wc) * 8) = words[f * WC + wc];
+            *reinterpret_cast<uint64_t *>(out + (f0 + f) * out_row_bytes + (w0 + wc) * 8) = words[f * WC + wc];
     }
 }
 
@@ -998,14 +1004,27 @@ extern "C" int dl_tensor_packbits_batch_major(const uint8_t *x, void *out, int64
     if (out_row_bytes % 8 == 0 && !dl_aligned(out, 8)) return DL_ERR_INVALID_ARGUMENT;
     const int64_t gx = dl_ceil_div(dl_ceil_div(batch, 64), 16);
     if (gx > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
-    constexpr int WC = 2;
-    const bool fits_lds = 64 * features + features * WC * 8 <= 65536;      // default dynamic LDS limit
-    if (features % 16 == 0 && fits_lds && dl_aligned(x, 16) && out_row_bytes % 8 == 0) {
-        const int64_t blocks = dl_ceil_div(dl_ceil_div(batch, 64), WC);
+    if (features % 16 == 0 && dl_aligned(x, 16) && out_row_bytes % 8 == 0) {
+        // A workgroup stages a slice of the features: 64 bytes of LDS per feature + 8 * WC for the result tile.
+        // Small footprints (several workgroups per CU overlap their load, fold and store phases) measured
+        // fastest: slices of 128 features with 8 word columns where rows are whole 128-byte lines (every
+        // request is then a full cache line, and feature rows are written in 64-byte runs), otherwise slices
+        // of up to 400 features with 2 word columns.
+        const bool lines = features % 128 == 0;
+        const int wc = lines ? 8 : 2;
+        const int64_t max_slice = lines ? 128 : 400;
+        const int64_t want = dl_ceil_div(features, max_slice);
+        const int64_t slice = dl_ceil_div(dl_ceil_div(features, want), 16) * 16;
+        const int64_t nslices = dl_ceil_div(features, slice);
+        const int64_t blocks = dl_ceil_div(dl_ceil_div(batch, 64), wc) * nslices;
         if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
-        const size_t lds = (size_t) (64 * features + features * WC * 8);
-        DL_LAUNCH(packbits_batch_major_lds_kernel<WC>, dim3((unsigned) blocks), dim3(DL_BLOCK), lds, s, x,
-                           (uint8_t *) out, batch, features, out_row_bytes);
+        const size_t lds = (size_t) (64 * slice + slice * wc * 8);
+        if (wc == 2)
+            DL_LAUNCH(packbits_batch_major_lds_kernel<2>, dim3((unsigned) blocks), dim3(DL_BLOCK), lds, s, x,
+                      (uint8_t *) out, batch, features, (int) slice, (int) nslices, out_row_bytes);
+        else
+            DL_LAUNCH(packbits_batch_major_lds_kernel<8>, dim3((unsigned) blocks), dim3(DL_BLOCK), lds, s, x,
+                      (uint8_t *) out, batch, features, (int) slice, (int) nslices, out_row_bytes);
     } else if (features % 4 == 0 && dl_aligned(x, 4)) {
         const int64_t gy = dl_ceil_div(features, 256);
         if (gy > 65535) return DL_ERR_TOO_LARGE;

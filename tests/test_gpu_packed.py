@@ -46,7 +46,7 @@ def test_packbits_nonzero_bytes_count_as_true(ext):
 
 @pytest.mark.parametrize("bits", [8, 16, 32, 64])
 @pytest.mark.parametrize("B,F", [(1, 1), (7, 3), (64, 8), (65, 12), (1000, 7), (1024, 256), (4112, 260), (70000, 2),
-                                 (3000, 784), (130, 1028)])
+                                 (3000, 784), (130, 1028), (200, 816), (333, 832), (129, 1648), (700, 9216)])
 def test_packbits_batch_major(ext, bits, B, F):
     rng = np.random.default_rng(F * 131 + B + bits)
     x = rng.random((B, F)) < 0.3
