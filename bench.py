@@ -39,7 +39,7 @@ def parse():
     ap.add_argument("--features", type=int, default=784)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-train", action="store_true")
-    ap.add_argument("--cpu-sample-log2", type=int, default=17)
+    ap.add_argument("--cpu-sample-log2", type=int, default=18)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 4 plain device copies of 1 GiB (for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     return ap.parse_args()
