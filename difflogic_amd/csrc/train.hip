@@ -137,6 +137,40 @@ template <typename T> __device__ __forceinline__ void softmax16(const T *__restr
     for (int i = 0; i < 16; ++i) g[i] = lane_value(mine, i);
 }
 
+// Corner coefficients of FOUR neurons at once: the 16-lane row r of the wave works on neuron n[r]
+// (n[r] < 0: none), lane i of the row on gate i.  LOGITS: `w` holds logits, the row computes their
+// softmax (and stores it to `probs` if asked); otherwise `w` holds the probabilities.  The corner
+// sums are masked row sums whose association order is that of corners_of(), so the results are
+// bit-identical to it.  Returns, per neuron, the wave-uniform P00, P10, P01 - P00, P11 - P10.
+template <typename T, bool LOGITS>
+__device__ __forceinline__ void corners4(const T *__restrict__ w, const int32_t (&n)[4], int lane, bool store_probs,
+                                         T *__restrict__ probs, typename Acc<T>::type (&p00)[4],
+                                         typename Acc<T>::type (&p10)[4], typename Acc<T>::type (&d0)[4],
+                                         typename Acc<T>::type (&d1)[4]) {
+    typedef typename Acc<T>::type C;
+    const int row = lane >> 4, gate = lane & 15;
+    const int32_t mine = row == 0 ? n[0] : row == 1 ? n[1] : row == 2 ? n[2] : n[3];
+    const bool valid = mine >= 0;
+    const int64_t at = (int64_t) (valid ? mine : 0) * 16 + gate;
+    C p = up<T>(w[at]);
+    if (LOGITS) {
+        const C e = dl_exp(p - row16_max(p));
+        p = e / row16_sum(e);
+        if (store_probs && valid) probs[at] = down<T, C>(p);
+    }
+    const C zero = (C) 0;
+    const C q00 = row16_sum((gate & 8) ? p : zero), q01 = row16_sum((gate & 4) ? p : zero);
+    const C q10 = row16_sum((gate & 2) ? p : zero), q11 = row16_sum((gate & 1) ? p : zero);
+    const C e0 = q01 - q00, e1 = q11 - q10;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        p00[i] = lane_value(q00, 16 * i);
+        p10[i] = lane_value(q10, 16 * i);
+        d0[i] = lane_value(e0, 16 * i);
+        d1[i] = lane_value(e1, 16 * i);
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 // forward: one wave = NPW neurons x 64 vectors of the batch.
 // ------------------------------------------------------------------------------------------
@@ -154,27 +188,18 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_kernel(const T *__restrict__
     const int64_t n0 = ((int64_t) blockIdx.x * 4 + wave) * NPW;
     if (n0 >= out_dim) return;
 
+    static_assert(NPW == 4, "corners4 serves four neurons per wave");
     int64_t ia[NPW], ib[NPW];
     C p00[NPW], p10[NPW], d0[NPW], d1[NPW];
+    int32_t ids[NPW];
 #pragma unroll
     for (int j = 0; j < NPW; ++j) {
         const int64_t n = (n0 + j < out_dim) ? n0 + j : out_dim - 1;
         ia[j] = a[n];
         ib[j] = b[n];
-        Corners<C> c;
-        if (LOGITS) {
-            C g[16], mine;
-            softmax16<T>(w, n, lane, g, mine);
-            c = corners_of<C>(g);
-            if (blockIdx.y == 0 && n0 + j < out_dim && lane < 16) probs[n * 16 + lane] = down<T, C>(mine);
-        } else {
-            c = corners<T>(w, n);
-        }
-        p00[j] = c.p00;
-        p10[j] = c.p10;
-        d0[j] = c.p01 - c.p00;
-        d1[j] = c.p11 - c.p10;
+        ids[j] = n0 + j < out_dim ? (int32_t) (n0 + j) : -1;
     }
+    corners4<T, LOGITS>(w, ids, lane, blockIdx.y == 0, probs, p00, p10, d0, d1);
     const P *xv = reinterpret_cast<const P *>(x);
     P *yv = reinterpret_cast<P *>(y);
     for (int64_t col = (int64_t) blockIdx.y * DL_WAVE + lane; col < ncols; col += (int64_t) gridDim.y * DL_WAVE) {
@@ -421,6 +446,7 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_chain_kernel(const T *__rest
     const int lane = dl_lane();
     const int64_t c = (int64_t) blockIdx.x * 4 + wave;
     if (c >= nchunks) return;
+    static_assert(CHUNK % 4 == 0, "neurons are served four at a time");
     const int64_t s0 = c * CHUNK;
     const P *xv = reinterpret_cast<const P *>(x);
     P *yv = reinterpret_cast<P *>(y);
@@ -434,18 +460,24 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_chain_kernel(const T *__rest
 #pragma unroll
         for (int j = 0; j <= CHUNK; ++j) rows[j] = xv[(int64_t) verts[s0 + j] * ncols + cl];
 #pragma unroll
-        for (int j = 0; j < CHUNK; ++j) {
-            const int32_t n = neuron[s0 + j];
-            const bool f = flip[s0 + j] != 0;
-            C p00, p10, d0, d1;
-            neuron_corners<T, LOGITS>(w, n >= 0 ? n : 0, lane, n >= 0 && ct == 0, probs, p00, p10, d0, d1);
-            P r;
+        for (int j0 = 0; j0 < CHUNK; j0 += 4) {
+            int32_t n[4];
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-                const C u0 = up<T>(rows[j].v[e]), u1 = up<T>(rows[j + 1].v[e]);
-                r.v[e] = down<T, C>(mix<C>(f ? u1 : u0, f ? u0 : u1, p00, p10, d0, d1));
+            for (int i = 0; i < 4; ++i) n[i] = neuron[s0 + j0 + i];
+            C p00[4], p10[4], d0[4], d1[4];
+            corners4<T, LOGITS>(w, n, lane, ct == 0, probs, p00, p10, d0, d1);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int j = j0 + i;
+                const bool f = flip[s0 + j] != 0;
+                P r;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const C u0 = up<T>(rows[j].v[e]), u1 = up<T>(rows[j + 1].v[e]);
+                    r.v[e] = down<T, C>(mix<C>(f ? u1 : u0, f ? u0 : u1, p00[i], p10[i], d0[i], d1[i]));
+                }
+                if (live && n[i] >= 0) yv[(int64_t) n[i] * ncols + col] = r;
             }
-            if (live && n >= 0) yv[(int64_t) n * ncols + col] = r;
         }
     }
 }
@@ -486,27 +518,35 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_chain_rows_kernel(const T *_
     load_row(verts[s0], prev);
     load_row(verts[s0 + 1], cur);
 #pragma unroll 1
-    for (int64_t s = s0; s < s1; ++s) {
-        if (s + 1 < s1) load_row(verts[s + 2], next);
-        const int32_t n = neuron[s];
-        const bool f = flip[s] != 0;
-        C p00, p10, d0, d1;
-        neuron_corners<T, LOGITS>(w, n >= 0 ? n : 0, lane, n >= 0 && col0 == 0, probs, p00, p10, d0, d1);
+    for (int64_t g = s0; g < s1; g += 4) {           // four steps per trip: their corners are computed together
+        int32_t n[4];
 #pragma unroll
-        for (int q = 0; q < CPL; ++q) {
-            const int64_t col = col0 + lane + q * DL_WAVE;
-            P r;
+        for (int i = 0; i < 4; ++i) n[i] = g + i < s1 ? neuron[g + i] : -1;
+        C p00[4], p10[4], d0[4], d1[4];
+        corners4<T, LOGITS>(w, n, lane, col0 == 0, probs, p00, p10, d0, d1);
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-                const C u0 = up<T>(prev[q].v[e]), u1 = up<T>(cur[q].v[e]);
-                r.v[e] = down<T, C>(mix<C>(f ? u1 : u0, f ? u0 : u1, p00, p10, d0, d1));
+        for (int i = 0; i < 4; ++i) {
+            const int64_t s = g + i;
+            if (s < s1) {                            // wave-uniform
+                if (s + 1 < s1) load_row(verts[s + 2], next);
+                const bool f = flip[s] != 0;
+#pragma unroll
+                for (int q = 0; q < CPL; ++q) {
+                    const int64_t col = col0 + lane + q * DL_WAVE;
+                    P r;
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        const C u0 = up<T>(prev[q].v[e]), u1 = up<T>(cur[q].v[e]);
+                        r.v[e] = down<T, C>(mix<C>(f ? u1 : u0, f ? u0 : u1, p00[i], p10[i], d0[i], d1[i]));
+                    }
+                    if (n[i] >= 0 && col < ncols) yv[(int64_t) n[i] * ncols + col] = r;
+                }
+#pragma unroll
+                for (int q = 0; q < CPL; ++q) {
+                    prev[q] = cur[q];
+                    cur[q] = next[q];
+                }
             }
-            if (n >= 0 && col < ncols) yv[(int64_t) n * ncols + col] = r;
-        }
-#pragma unroll
-        for (int q = 0; q < CPL; ++q) {
-            prev[q] = cur[q];
-            cur[q] = next[q];
         }
     }
 }
@@ -652,17 +692,43 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
 #pragma unroll
             for (int e = 0; e < VEC; ++e) carry[q][e] = up<T>(g[q].v[e]) * dl_fma(up<T>(before[q].v[e]), dd, kv);
     }
-#pragma unroll 1
-    for (int64_t s = s0; s < s1; ++s) {
-        const int32_t n = neuron[s];
+    // The chunk's schedule entries are fetched once, one per lane (chunk <= 64), and handed out by
+    // readlane, so the step loop waits for no scalar loads; the rows of step i + 1 are requested
+    // before the arithmetic of step i.
+    const int cnt = (int) (s1 - s0);
+    const bool has = lane < cnt;
+    const int32_t sch_n = has ? neuron[s0 + lane] : -1;
+    const int32_t sch_v = has ? verts[s0 + 1 + lane] : 0;
+    const int32_t sch_d = has ? dst[s0 + lane] : -1;
+    const int32_t sch_f = has ? (int32_t) flip[s0 + lane] : 0;
+    const int gate = lane & 15;
+    // rows of step i: the new input row, the neuron's grad_y row (zero for a step without a neuron)
+    // and, in every 16-lane row, the neuron's 16 gate probabilities
+    auto fetch = [&](int i, P *row, P *grad, C &prob) {
+        const int32_t n = __builtin_amdgcn_readlane(sch_n, i);
         const bool valid = n >= 0;
         const int64_t nn = valid ? n : 0;
-        const bool f = flip[s] != 0;
-        P cur[CPL], g[CPL];
-        load_row(xv, verts[s + 1], true, cur);
-        load_row(gv, nn, valid, g);                  // zero gradient for a step without a neuron
-        const Corners<C> k = corners<T>(w, nn);
-        const C d0 = k.p01 - k.p00, dd = (k.p11 - k.p10) - d0, da = k.p10 - k.p00;
+        load_row(xv, __builtin_amdgcn_readlane(sch_v, i), true, row);
+        load_row(gv, nn, valid, grad);
+        prob = up<T>(w[nn * 16 + gate]);
+    };
+    P cur[CPL], g[CPL];
+    C pw;
+    fetch(0, cur, g, pw);
+#pragma unroll 1
+    for (int i = 0; i < cnt; ++i) {
+        P ncur[CPL], ng[CPL];
+        C npw = (C) 0;
+        if (i + 1 < cnt) fetch(i + 1, ncur, ng, npw);
+        const int32_t n = __builtin_amdgcn_readlane(sch_n, i);
+        const bool valid = n >= 0;
+        const int64_t nn = valid ? n : 0;
+        const bool f = __builtin_amdgcn_readlane(sch_f, i) != 0;
+        // corner sums of the probabilities, in the association order of corners_of()
+        const C zc = (C) 0;
+        const C p00 = lane_value(row16_sum((gate & 8) ? pw : zc), 0), p01 = lane_value(row16_sum((gate & 4) ? pw : zc), 0);
+        const C p10 = lane_value(row16_sum((gate & 2) ? pw : zc), 0), p11 = lane_value(row16_sum((gate & 1) ? pw : zc), 0);
+        const C d0 = p01 - p00, dd = (p11 - p10) - d0, da = p10 - p00;
         const C ku = f ? d0 : da, kv = f ? da : d0;
         C s00 = (C) 0, s01 = (C) 0, s10 = (C) 0, s11 = (C) 0;
         C out[CPL][VEC];
@@ -682,19 +748,35 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
                 carry[q][e] = gg * dl_fma(u0, dd, kv);
             }
         }
-        store_row(dst[s], out);
+        store_row(__builtin_amdgcn_readlane(sch_d, i), out);
         s00 = wave_sum(s00);
         s01 = wave_sum(s01);
         s10 = wave_sum(s10);
         s11 = wave_sum(s11);
         if (partial == nullptr) {
-            store_grad_w<T>(lane, valid, nn, s00, s01, s10, s11, probs, gw);
+            // as store_grad_w, with the probabilities already at hand
+            C r = (C) 0;
+            if (lane & 8) r += s00;
+            if (lane & 4) r += s01;
+            if (lane & 2) r += s10;
+            if (lane & 1) r += s11;
+            if (probs != nullptr) {
+                const C pr = (valid && lane < 16) ? pw : zc;
+                const C dot = row16_sum(pr * r);
+                r = pr * (r - dot);
+            }
+            if (valid && lane < 16) gw[nn * 16 + lane] = down<T, C>(r);
         } else if (valid && lane < 4) {              // several segments: backward_w_finish_kernel adds them
             const C mine = lane == 0 ? s00 : lane == 1 ? s01 : lane == 2 ? s10 : s11;
             partial[((int64_t) blockIdx.y * out_dim + nn) * 4 + lane] = mine;
         }
 #pragma unroll
-        for (int q = 0; q < CPL; ++q) prev[q] = cur[q];
+        for (int q = 0; q < CPL; ++q) {
+            prev[q] = cur[q];
+            cur[q] = ncur[q];
+            g[q] = ng[q];
+        }
+        pw = npw;
     }
     if (s1 == steps) store_row(dst[steps], carry);   // the schedule's last position
 }
