@@ -1111,6 +1111,13 @@ int forward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, 
     }
     const int64_t blocks = dl_ceil_div(nchunks, 4);
     if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    if (V >= 2 && ncols <= DL_WAVE / 2) {
+        // short rows: 8-byte vectors put a row on all 64 lanes instead of half of them
+        constexpr int H = V >= 2 ? V / 2 : 1;
+        DL_LAUNCH((forward_chain_kernel<T, H, DL_TRAIN_CHUNK, LOGITS>), dim3((unsigned) blocks, 1), dim3(DL_BLOCK), 0, s, xp,
+                  verts, neuron, flip, wp, (T *) y, (T *) probs, nchunks, 2 * ncols);
+        return dl_launch_status();
+    }
     DL_LAUNCH((forward_chain_kernel<T, V, DL_TRAIN_CHUNK, LOGITS>), dim3((unsigned) blocks, col_tiles(ncols)),
                        dim3(DL_BLOCK), 0, s, xp, verts, neuron, flip, wp, (T *) y, (T *) probs, nchunks, ncols);
     return dl_launch_status();
@@ -1166,15 +1173,18 @@ int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron,
     if (blocks > 0x7fffffffLL || fix_blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     const dim3 grid((unsigned) blocks, (unsigned) segments), block(DL_BLOCK);
     const T *xp = (const T *) x, *wp = (const T *) w, *gp = (const T *) gy, *pp = softmax_backward ? wp : nullptr;
-#define DL_LAUNCH_BACKWARD_CHAIN(CPL)                                                                                  \
-    DL_LAUNCH((backward_chain_kernel<T, V, CPL>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp, pp, (T *) gw, \
-              partial, (T *) gx, overflow, steps, chunk, in_dim, out_dim, ncols, (C) scale)
-    if (ncols <= DL_WAVE)
-        DL_LAUNCH_BACKWARD_CHAIN(1);
+    constexpr int H = V >= 2 ? V / 2 : 1;
+#define DL_LAUNCH_BACKWARD_CHAIN(VV, CPL, NC)                                                                              \
+    DL_LAUNCH((backward_chain_kernel<T, VV, CPL>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp, pp, (T *) gw, \
+              partial, (T *) gx, overflow, steps, chunk, in_dim, out_dim, NC, (C) scale)
+    if (V >= 2 && ncols <= DL_WAVE / 2)
+        DL_LAUNCH_BACKWARD_CHAIN(H, 1, 2 * ncols);   // short rows: 8-byte vectors use all 64 lanes
+    else if (ncols <= DL_WAVE)
+        DL_LAUNCH_BACKWARD_CHAIN(V, 1, ncols);
     else if (ncols <= 2 * DL_WAVE)
-        DL_LAUNCH_BACKWARD_CHAIN(2);
+        DL_LAUNCH_BACKWARD_CHAIN(V, 2, ncols);
     else
-        DL_LAUNCH_BACKWARD_CHAIN(4);
+        DL_LAUNCH_BACKWARD_CHAIN(V, 4, ncols);
 #undef DL_LAUNCH_BACKWARD_CHAIN
     int st = dl_launch_status();
     if (st != DL_OK) return st;

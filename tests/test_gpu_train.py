@@ -339,7 +339,9 @@ def test_fused_chained_backward_matches_separate_kernels(ext, monkeypatch, dtype
     if batch * x.element_size() % 16:                               # rows must be whole 16-byte vectors
         assert both is None
         return
-    one_segment = batch * x.element_size() <= 256 * 16               # longer rows are cut into segments
+    # rows of 33..256 16-byte vectors are summed in the order of the unfused kernel; shorter rows use
+    # 8-byte vectors and longer ones are cut into segments (same terms, another order)
+    one_segment = 32 * 16 < batch * x.element_size() <= 256 * 16
     assert both is not None
     gw, gx = both
     want_gx = ext.backward_x(x, a, b, w, gy, start, idx, scale)
