@@ -123,20 +123,6 @@ __device__ __forceinline__ double lane_value(double v, int i) {
     return __builtin_bit_cast(double, ((uint64_t) hi << 32) | lo);
 }
 
-// softmax over neuron n's 16 gate logits, exp(l - max) / sum.  Lane i of every 16-lane row works
-// on gate i & 15 (one exp and one division per lane, row-wide max and sum by DPP); the 16
-// probabilities are then broadcast as wave-uniform values g[0..15], and `mine` is lane's own.
-template <typename T> __device__ __forceinline__ void softmax16(const T *__restrict__ logits, int64_t n, int lane,
-                                                                typename Acc<T>::type (&g)[16],
-                                                                typename Acc<T>::type &mine) {
-    typedef typename Acc<T>::type C;
-    const C l = up<T>(logits[n * 16 + (lane & 15)]);
-    const C e = dl_exp(l - row16_max(l));
-    mine = e / row16_sum(e);
-#pragma unroll
-    for (int i = 0; i < 16; ++i) g[i] = lane_value(mine, i);
-}
-
 // Corner coefficients of FOUR neurons at once: the 16-lane row r of the wave works on neuron n[r]
 // (n[r] < 0: none), lane i of the row on gate i.  LOGITS: `w` holds logits, the row computes their
 // softmax (and stores it to `probs` if asked); otherwise `w` holds the probabilities.  The corner
@@ -412,27 +398,6 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_x_kernel(const T *__restric
 // fp64 results are bit-identical (fp16 outputs can differ in the last bit, where the compiler
 // folds the final conversion into a fused multiply-add in one kernel and not in the other).
 // ------------------------------------------------------------------------------------------
-template <typename T, bool LOGITS>
-__device__ __forceinline__ void neuron_corners(const T *__restrict__ w, int64_t n, int lane, bool store_probs,
-                                               T *__restrict__ probs, typename Acc<T>::type &p00,
-                                               typename Acc<T>::type &p10, typename Acc<T>::type &d0,
-                                               typename Acc<T>::type &d1) {
-    typedef typename Acc<T>::type C;
-    Corners<C> c;
-    if (LOGITS) {
-        C g[16], mine;
-        softmax16<T>(w, n, lane, g, mine);
-        c = corners_of<C>(g);
-        if (store_probs && lane < 16) probs[n * 16 + lane] = down<T, C>(mine);
-    } else {
-        c = corners<T>(w, n);
-    }
-    p00 = c.p00;
-    p10 = c.p10;
-    d0 = c.p01 - c.p00;
-    d1 = c.p11 - c.p10;
-}
-
 template <typename T, int VEC, int CHUNK, bool LOGITS>
 __global__ __launch_bounds__(DL_BLOCK) void forward_chain_kernel(const T *__restrict__ x,
                                                                  const int32_t *__restrict__ verts,
