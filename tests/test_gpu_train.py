@@ -396,3 +396,42 @@ def test_layer_uses_schedule_for_wide_inputs():
     fo.layer_forward_sequential(xr, wide.indices[0].cpu(), wide.indices[1].cpu(),
                                 torch.softmax(wr, -1)).square().sum().backward()
     assert close(x.grad, xr.grad, 1e-4)[0] and close(wide.weights.grad, wr.grad, 1e-4)[0]
+
+
+def test_chained_layer_matches_the_python_formulation_on_random_wirings(monkeypatch):
+    """LogicLayer with its schedule forced on (chained forward, one-pass backward), against the
+    fp64 python formulation with autograd, over random wirings of every awkward kind: inputs
+    that feed no neuron, many neurons on one input, neurons wired twice to one input, one
+    neuron, rows shorter and longer than a wave."""
+    import difflogic_amd as dl
+    monkeypatch.setattr(dl.LogicLayer, "_CHAIN_MIN_IN_DIM", 0)
+    monkeypatch.setattr(dl.LogicLayer, "_CHAIN_MIN_OUT_DIM", 0)
+    monkeypatch.setattr(dl.difflogic_cuda, "BACKWARD_CHAIN_MAX_OVERFLOW", 1e9)
+    pick = torch.Generator().manual_seed(99)
+    for case in range(40):
+        in_dim = int(torch.randint(1, 60, (1,), generator=pick))
+        out_dim = int(torch.randint(max(1, (in_dim + 1) // 2), 130, (1,), generator=pick))
+        batch = [4, 8, 20, 64, 100, 128, 256, 260, 512, 1024, 1028, 2048][case % 12]
+        grad_factor = [1.0, 2.0, 0.5][case % 3]
+        layer = dl.LogicLayer(in_dim, out_dim, grad_factor=grad_factor)
+        kind = case % 4
+        a = torch.randint(0, in_dim, (out_dim,), generator=pick)
+        b = torch.randint(0, in_dim, (out_dim,), generator=pick)
+        if kind == 1:                                   # a few inputs carry everything
+            a, b = a % max(1, in_dim // 4), b % max(1, in_dim // 4)
+        elif kind == 2:                                 # self loops
+            b = torch.where(torch.rand(out_dim, generator=pick) < 0.3, a, b)
+        layer.set_connections(a, b)
+        assert layer._train_schedule() is not None
+        x = torch.rand(batch, in_dim, generator=pick).cuda().requires_grad_()
+        gy = torch.randn(batch, out_dim, generator=pick)
+        y = layer(x)
+        (y * gy.cuda()).sum().backward()
+        xr = x.detach().cpu().double().requires_grad_()
+        wr = layer.weights.detach().cpu().double().requires_grad_()
+        yr = fo.layer_forward_sequential(xr, a, b, torch.softmax(wr, -1))
+        (yr * gy.double()).sum().backward()
+        tag = (case, in_dim, out_dim, batch, kind)
+        assert close(y, yr)[0], tag
+        assert close(layer.weights.grad, wr.grad, 2 * RTOL)[0], tag
+        assert close(x.grad, grad_factor * xr.grad, 2 * RTOL)[0], tag
