@@ -293,36 +293,44 @@ def train_bench(args, torch, dl):
 def train_cpu_baseline(torch):
     """Full training step (forward, CrossEntropy, backward, Adam lr 0.01) of the python
     implementation restated in oracle/float_oracle.py: 784 -> 4 x 8000 -> GroupSum(10, tau 10),
-    B = 128, 'random' connections; median of 5 steps after 2 warm-ups, 1 thread."""
+    B = 128, 'random' connections; median of 5 steps after 2 warm-ups, at 1 thread (the figure
+    reported) and at torch's default thread count."""
     from oracle import connections as oc
     from oracle import float_oracle as fo
-    threads = torch.get_num_threads()
-    torch.set_num_threads(1)
-    try:
-        torch.manual_seed(0)
-        layers, d = [], 784
-        for _ in range(4):
-            lg = torch.randn(8000, 16, requires_grad=True)
-            a, b = oc.random_connections(d, 8000)
-            layers.append((a, b, lg))
-            d = 8000
-        net = fo.PythonNet(layers, 10, 10.0)
-        opt = torch.optim.Adam([l[2] for l in layers], lr=0.01)
-        x = (torch.rand(128, 784) < 0.2).float()
-        y = torch.randint(0, 10, (128,))
+    torch.manual_seed(0)
+    layers, d = [], 784
+    for _ in range(4):
+        lg = torch.randn(8000, 16, requires_grad=True)
+        a, b = oc.random_connections(d, 8000)
+        layers.append((a, b, lg))
+        d = 8000
+    net = fo.PythonNet(layers, 10, 10.0)
+    opt = torch.optim.Adam([l[2] for l in layers], lr=0.01)
+    x = (torch.rand(128, 784) < 0.2).float()
+    y = torch.randint(0, 10, (128,))
+
+    def median_step():
         times = []
-        for i in range(7):
+        for _ in range(7):
             t0 = time.perf_counter()
             loss = torch.nn.functional.cross_entropy(net(x), y)
             opt.zero_grad()
             loss.backward()
             opt.step()
             times.append(time.perf_counter() - t0)
-        med = statistics.median(times[2:])
+        return statistics.median(times[2:])
+
+    threads = torch.get_num_threads()
+    all_threads = median_step()                      # torch's default thread count
+    torch.set_num_threads(1)                         # what the reference's drivers pin (experiments/main.py:17)
+    try:
+        med = median_step()
     finally:
         torch.set_num_threads(threads)
     return {"value": round(4 * 8000 * 128 / med, 1), "unit": "neuron-samples/s", "cores": 1, "kind": "port",
-            "sample": "784->4x8000 B=128 full step (fwd+CE+bwd+Adam), median of 5, %.3f s/step" % med}
+            "sample": "784->4x8000 B=128 full step (fwd+CE+bwd+Adam), median of 5, %.3f s/step" % med,
+            "default_threads": {"value": round(4 * 8000 * 128 / all_threads, 1), "cores": threads,
+                                "s_per_step": round(all_threads, 4)}}
 
 
 def main():
