@@ -4,6 +4,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <tuple>
+#include <utility>
+
 #include "difflogic_hip.h"
 
 #define DL_WAVE 64
@@ -12,21 +15,36 @@
 typedef uint32_t dl_u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t dl_u32x2 __attribute__((ext_vector_type(2)));
 
-// hipGetLastError() reports the last error of ANY earlier runtime call of this thread, including
-// harmless ones of the caller (an event query that answered "not ready"), so the error state is
-// cleared right before each launch and read right after it.
-#define DL_LAUNCH(kernel, grid, block, lds, stream, ...)                      \
-    do {                                                                      \
-        (void) hipGetLastError();                                             \
-        hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);    \
-    } while (0)
-
+// Launches go through hipLaunchKernel, whose return value is the launch's own verdict; the
+// runtime's per-thread "last error" (which also holds harmless results of the caller's earlier
+// calls, such as an event query that answered "not ready") is neither read nor cleared.
 extern thread_local int dl_last_hip_error_code;    // hipError_t of this thread's last refused launch (packed.hip)
+extern thread_local int dl_launch_result;          // hipError_t of this thread's last DL_LAUNCH (packed.hip)
 
+template <typename... P, size_t... I, typename... A>
+inline hipError_t dl_launch_impl(void (*kernel)(P...), dim3 grid, dim3 block, size_t lds, hipStream_t stream,
+                                 std::index_sequence<I...>, A &&... args) {
+    std::tuple<P...> params{static_cast<P>(args)...};             // the kernel's own parameter types
+    void *ptrs[] = {static_cast<void *>(&std::get<I>(params))...};
+    return hipLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, ptrs, lds, stream);
+}
+
+template <typename... P, typename... A>
+inline void dl_launch(void (*kernel)(P...), dim3 grid, dim3 block, size_t lds, hipStream_t stream, A &&... args) {
+    static_assert(sizeof...(P) == sizeof...(A), "argument count differs from the kernel's parameter count");
+    const hipError_t e = dl_launch_impl(kernel, grid, block, lds, stream, std::index_sequence_for<P...>(), args...);
+    if (dl_launch_result == (int) hipSuccess) dl_launch_result = (int) e;   // the first failure is the one reported
+}
+
+#define DL_LAUNCH(kernel, grid, block, lds, stream, ...) dl_launch(kernel, grid, block, lds, stream, __VA_ARGS__)
+
+// Status of the launch(es) since the last call: DL_OK, or DL_ERR_LAUNCH with the HIP error kept
+// for dl_last_hip_error().
 static inline int dl_launch_status() {
-    const hipError_t e = hipGetLastError();
-    if (e == hipSuccess) return DL_OK;
-    dl_last_hip_error_code = (int) e;
+    const int e = dl_launch_result;
+    dl_launch_result = (int) hipSuccess;
+    if (e == (int) hipSuccess) return DL_OK;
+    dl_last_hip_error_code = e;
     return DL_ERR_LAUNCH;
 }
 

@@ -946,6 +946,7 @@ bool valid_bit_count(int bit_count) { return bit_count == 8 || bit_count == 16 |
 }  // namespace
 
 thread_local int dl_last_hip_error_code = 0;
+thread_local int dl_launch_result = 0;
 
 extern "C" const char *dl_last_hip_error(void) { return hipGetErrorString((hipError_t) dl_last_hip_error_code); }
 
