@@ -12,7 +12,9 @@
  * - Index tables `a`, `b` hold values in [0, in_dim); `start`/`idx` are the CSR reverse
  *   index the reference builds at difflogic/difflogic.py:60-69.  The kernels trust them.
  * - Every function returns a dl_status (0 = success).  Nothing here calls exit().
- * - Functions are re-entrant; there is no global state.
+ * - Functions are re-entrant; the only state is a per-thread record of the last refused
+ *   launch's HIP error (dl_last_hip_error).  Kernels are launched with hipLaunchKernel and its
+ *   return value is what is reported; the runtime's per-thread last error is not touched.
  *
  * Each entry point replaces one function of the reference's extension module
  * `difflogic_cuda` (difflogic/cuda/difflogic.cpp:45-84); the comment above each declaration
