@@ -48,7 +48,9 @@ SIGNATURES = {
     "dl_eval_schedule_build": [_vp, _vp, _i64, _i64, _int, _vp, _vp, _vp],
     "dl_logic_eval_chained": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _int, _vp, _vp],
     "dl_logic_eval_fused_groupbitsum_workspace_bytes": [_int, _i64, _i64, _int, _i64],
-    "dl_logic_eval_fused_groupbitsum": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _i64, _vp, _vp],
+    "dl_logic_eval_fused_groupbitsum": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _i64, _vp, _vp, _vp],
+    "dl_count_group": [],
+    "dl_count_order_build": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp],
 }
 _RESTYPES = {"dl_status_string": ctypes.c_char_p, "dl_last_hip_error": ctypes.c_char_p, "dl_group_sum_workspace_bytes": ctypes.c_int64,
              "dl_logic_eval_fused_workspace_bytes": ctypes.c_int64,

@@ -111,12 +111,13 @@ struct TreeTables {
 };
 
 template <int D>
-__global__ __launch_bounds__(DL_BLOCK) void compose_tree_kernel(TreeTables t, int32_t *__restrict__ leaves,
+__global__ __launch_bounds__(DL_BLOCK) void compose_tree_kernel(TreeTables t, const int32_t *__restrict__ order,
+                                                                int32_t *__restrict__ leaves,
                                                                 uint64_t *__restrict__ gates, int64_t out_dim) {
     const int64_t n = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x;
     if (n >= out_dim) return;
     int64_t nodes[1 << D];
-    nodes[0] = n;
+    nodes[0] = order ? (int64_t) order[n] : n;        // slot n of the composites describes this neuron
     uint64_t packed = 0;
 #pragma unroll
     for (int r = 0; r < D; ++r) {                  // r = distance from the root; layer index D-1-r
@@ -889,7 +890,8 @@ int launch_count_fused(const void *x, const int32_t *leaves, const uint64_t *gat
 // Validates the description of a fused group and launches the composite builder.
 // dims = {in_dim, width of layer 0, ..., width of layer depth-1} (host array).
 int compose_tree(int depth, const int64_t *const *a, const int64_t *const *b, const uint8_t *const *w,
-                 const int64_t *dims, void *workspace, int32_t **leaves, uint64_t **gates, hipStream_t s) {
+                 const int64_t *dims, const int32_t *order, void *workspace, int32_t **leaves, uint64_t **gates,
+                 hipStream_t s) {
     if (depth < 1 || depth > DL_MAX_FUSE_DEPTH || !a || !b || !w || !dims || !workspace) return DL_ERR_INVALID_ARGUMENT;
     TreeTables t;
     for (int l = 0; l < depth; ++l) {
@@ -908,10 +910,10 @@ int compose_tree(int depth, const int64_t *const *a, const int64_t *const *b, co
     if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     const dim3 grid((unsigned) blocks), block(DL_BLOCK);
     switch (depth) {
-    case 1: DL_LAUNCH(compose_tree_kernel<1>, grid, block, 0, s, t, *leaves, *gates, out_dim); break;
-    case 2: DL_LAUNCH(compose_tree_kernel<2>, grid, block, 0, s, t, *leaves, *gates, out_dim); break;
-    case 3: DL_LAUNCH(compose_tree_kernel<3>, grid, block, 0, s, t, *leaves, *gates, out_dim); break;
-    default: DL_LAUNCH(compose_tree_kernel<4>, grid, block, 0, s, t, *leaves, *gates, out_dim); break;
+    case 1: DL_LAUNCH(compose_tree_kernel<1>, grid, block, 0, s, t, order, *leaves, *gates, out_dim); break;
+    case 2: DL_LAUNCH(compose_tree_kernel<2>, grid, block, 0, s, t, order, *leaves, *gates, out_dim); break;
+    case 3: DL_LAUNCH(compose_tree_kernel<3>, grid, block, 0, s, t, order, *leaves, *gates, out_dim); break;
+    default: DL_LAUNCH(compose_tree_kernel<4>, grid, block, 0, s, t, order, *leaves, *gates, out_dim); break;
     }
     return dl_launch_status();
 }
@@ -1085,7 +1087,7 @@ extern "C" int dl_logic_eval_fused(const void *x, int depth, const int64_t *cons
     hipStream_t s = (hipStream_t) stream;
     int32_t *leaves;
     uint64_t *gates;
-    const int st = compose_tree(depth, a, b, w, dims, workspace, &leaves, &gates, s);
+    const int st = compose_tree(depth, a, b, w, dims, nullptr, workspace, &leaves, &gates, s);
     if (st != DL_OK) return st;
     if (mis % 16 == 0) return launch_eval_tree<dl_u32x4>(depth, x, leaves, gates, y, dims[depth], row_bytes, s);
     return launch_eval_tree<dl_u32x2>(depth, x, leaves, gates, y, dims[depth], row_bytes, s);
@@ -1094,7 +1096,7 @@ extern "C" int dl_logic_eval_fused(const void *x, int depth, const int64_t *cons
 extern "C" int dl_logic_eval_fused_groupbitsum(const void *x, int depth, const int64_t *const *a,
                                                const int64_t *const *b, const uint8_t *const *w, const int64_t *dims,
                                                int32_t *out, int64_t words, int bit_count, int64_t pad_len, int64_t k,
-                                               void *workspace, void *stream) {
+                                               const int32_t *order, void *workspace, void *stream) {
     if (!valid_bit_count(bit_count)) return DL_ERR_BIT_COUNT;
     if (depth < 1 || depth > 2 || !dims || words < 0 || k <= 0 || pad_len < 0) return DL_ERR_INVALID_ARGUMENT;
     const int64_t out_dim = dims[depth];
@@ -1111,7 +1113,7 @@ extern "C" int dl_logic_eval_fused_groupbitsum(const void *x, int depth, const i
     hipStream_t s = (hipStream_t) stream;
     int32_t *leaves;
     uint64_t *gates;
-    const int st = compose_tree(depth, a, b, w, dims, workspace, &leaves, &gates, s);
+    const int st = compose_tree(depth, a, b, w, dims, order, workspace, &leaves, &gates, s);
     if (st != DL_OK) return st;
     // scratch for the partial counters follows the flattened wiring in the workspace
     const int64_t tables = dl_logic_eval_fused_workspace_bytes(depth, out_dim);
@@ -1120,6 +1122,8 @@ extern "C" int dl_logic_eval_fused_groupbitsum(const void *x, int depth, const i
         return launch_count_fused<1>(x, leaves, gates, scratch, out, row_bytes, per_class, k, batch, s);
     return launch_count_fused<2>(x, leaves, gates, scratch, out, row_bytes, per_class, k, batch, s);
 }
+
+extern "C" int dl_count_group(void) { return DL_COUNT_ROWS; }
 
 extern "C" int64_t dl_logic_eval_fused_groupbitsum_workspace_bytes(int depth, int64_t out_dim, int64_t words,
                                                                     int bit_count, int64_t k) {
@@ -1177,7 +1181,7 @@ extern "C" int dl_logic_eval_chained(const void *x, int depth, const int64_t *co
     int32_t *sub_leaves = nullptr;
     uint64_t *sub_gates = nullptr;
     if (depth > 1) {                                 // flatten the layers below the top one, per vertex
-        const int st = compose_tree(depth - 1, a, b, w, dims, workspace, &sub_leaves, &sub_gates, s);
+        const int st = compose_tree(depth - 1, a, b, w, dims, nullptr, workspace, &sub_leaves, &sub_gates, s);
         if (st != DL_OK) return st;
     }
     const int64_t nchunks = steps / DL_EVAL_SCHEDULE_CHUNK;

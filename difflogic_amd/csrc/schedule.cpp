@@ -13,6 +13,7 @@
 // neuron[s] = -1 marks a load-only step (start of a trail, or padding to whole chunks).
 #include <stdint.h>
 
+#include <algorithm>
 #include <vector>
 
 #include "difflogic_hip.h"
@@ -133,4 +134,83 @@ extern "C" int64_t dl_backward_schedule_build(const int32_t *verts, const int32_
     }
     *n_fix = entries;
     return rows;
+}
+
+// Order in which dl_logic_eval_fused_groupbitsum walks the neurons of each class.  The count of a
+// class does not depend on the order of its neurons, but the cache traffic does: a workgroup of
+// the fused count kernel handles `group` consecutive neurons, and an input row that several of
+// them read is fetched from beyond the L2 cache once instead of once per reader.  Neurons of a
+// class are therefore collected breadth-first along shared input rows (the leaves of the
+// depth-1 or depth-2 gate tree: a_low == NULL means the top layer reads the rows directly), so
+// that readers of one row fall into one group wherever the class allows it.
+//   order [out_dim]: a permutation of the neurons that maps every class onto itself.
+extern "C" int dl_count_order_build(const int64_t *a_top, const int64_t *b_top, const int64_t *a_low,
+                                    const int64_t *b_low, int64_t rows, int64_t mid_dim, int64_t out_dim, int64_t k,
+                                    int group, int32_t *order) {
+    if (!a_top || !b_top || !order || (!a_low) != (!b_low) || rows <= 0 || out_dim < 0 || k <= 0 || group <= 0)
+        return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim % k != 0) return DL_ERR_NOT_DIVISIBLE;
+    if (rows > 0x7fffffffLL || out_dim > 0x7fffffffLL || mid_dim > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    const int nl = a_low ? 4 : 2;
+    const int64_t top_in = a_low ? mid_dim : rows;
+    std::vector<int32_t> leaf((size_t) (out_dim * nl));
+    for (int64_t n = 0; n < out_dim; ++n) {
+        const int64_t u = a_top[n], v = b_top[n];
+        if (u < 0 || u >= top_in || v < 0 || v >= top_in) return DL_ERR_INVALID_ARGUMENT;
+        int64_t l[4] = {u, v, 0, 0};
+        if (a_low) {
+            l[0] = a_low[u];
+            l[1] = b_low[u];
+            l[2] = a_low[v];
+            l[3] = b_low[v];
+        }
+        for (int i = 0; i < nl; ++i) {
+            if (l[i] < 0 || l[i] >= rows) return DL_ERR_INVALID_ARGUMENT;
+            leaf[(size_t) (n * nl + i)] = (int32_t) l[i];
+        }
+    }
+    const int64_t per_class = out_dim / k;
+    std::vector<int64_t> start((size_t) rows + 1);
+    std::vector<int32_t> readers((size_t) (per_class * nl)), queue;
+    std::vector<uint8_t> taken((size_t) per_class);
+    for (int64_t c = 0; c < k; ++c) {
+        const int64_t n0 = c * per_class;
+        // readers of every row within this class (CSR)
+        std::fill(start.begin(), start.end(), 0);
+        for (int64_t i = 0; i < per_class * nl; ++i) ++start[(size_t) leaf[(size_t) (n0 * nl + i)] + 1];
+        for (int64_t r = 0; r < rows; ++r) start[(size_t) r + 1] += start[(size_t) r];
+        {
+            std::vector<int64_t> fill(start.begin(), start.end() - 1);
+            for (int64_t i = 0; i < per_class; ++i)
+                for (int j = 0; j < nl; ++j) readers[(size_t) fill[(size_t) leaf[(size_t) ((n0 + i) * nl + j)]]++] = (int32_t) i;
+        }
+        std::fill(taken.begin(), taken.end(), 0);
+        int64_t placed = 0, seed = 0;
+        while (placed < per_class) {
+            while (taken[(size_t) seed]) ++seed;
+            // one group: breadth-first from the first free neuron; what is left in the queue when the
+            // group is full goes back to the pool
+            queue.assign(1, (int32_t) seed);
+            taken[(size_t) seed] = 1;
+            size_t head = 0;
+            int in_group = 0;
+            while (head < queue.size() && in_group < group) {
+                const int32_t i = queue[head++];
+                order[n0 + placed++] = (int32_t) (n0 + i);
+                ++in_group;
+                for (int j = 0; j < nl; ++j) {
+                    const int32_t r = leaf[(size_t) ((n0 + i) * nl + j)];
+                    for (int64_t q = start[(size_t) r]; q < start[(size_t) r + 1]; ++q) {
+                        const int32_t other = readers[(size_t) q];
+                        if (!taken[(size_t) other]) {
+                            taken[(size_t) other] = 1;
+                            queue.push_back(other);
+                        }
+                    }
+                }
+            }
+            for (; head < queue.size(); ++head) taken[(size_t) queue[head]] = 0;
+        }
+    }
+    return DL_OK;
 }

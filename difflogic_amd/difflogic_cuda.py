@@ -500,10 +500,45 @@ def eval_chained(x, layers, schedule=None):
     return y
 
 
-def eval_fused_groupbitsum(x, layers, pad_len, k):
+_COUNT_ORDERS = {}                   # wiring tensors + k -> device order, most recent last
+_COUNT_ORDERS_MAX = 16
+
+
+def count_order_for(layers, in_dim, k):
+    """Cached neuron order for eval_fused_groupbitsum over ``layers`` (the net's last one or two
+    layers, [(a, b, w), ...]): neurons of a class that read the same input rows are walked by
+    the same workgroup.  Built on the host from the wiring alone; rebuilt when the index tensors
+    are replaced or modified."""
+    import numpy as np
+    idx = [t for a, b, _ in layers for t in (a, b)]
+    key = tuple((t.data_ptr(), t._version, t.shape[0]) for t in idx) + (int(in_dim), int(k))
+    hit = _COUNT_ORDERS.pop(key, None)
+    if hit is None:
+        lib = _lib.load()
+        host = [np.ascontiguousarray(t.detach().cpu().numpy(), dtype=np.int64) for t in idx]
+        out_dim = host[-1].shape[0]
+        order = np.empty(out_dim, dtype=np.int32)
+        if len(layers) == 2:
+            low_a, low_b, top_a, top_b = (h.ctypes.data for h in host)
+            mid = host[0].shape[0]
+        else:
+            (top_a, top_b), low_a, low_b, mid = (h.ctypes.data for h in host), None, None, 0
+        st = lib.dl_count_order_build(top_a, top_b, low_a, low_b, int(in_dim), mid, out_dim, int(k),
+                                      lib.dl_count_group(), order.ctypes.data)
+        if st:
+            _raise(st, "count_order_build")
+        hit = (torch.from_numpy(order).to(idx[0].device), idx)      # idx keeps the keyed tensors alive
+        while len(_COUNT_ORDERS) >= _COUNT_ORDERS_MAX:
+            _COUNT_ORDERS.pop(next(iter(_COUNT_ORDERS)))
+    _COUNT_ORDERS[key] = hit
+    return hit[0]
+
+
+def eval_fused_groupbitsum(x, layers, pad_len, k, order=None):
     """groupbitsum(eval(... eval(x, layer 0) ..., last layer), pad_len, k) for the net's last
     one or two layers without materialising their output.  Not part of the reference's
-    extension.  Falls back to the separate kernels where the fused one does not apply."""
+    extension.  Falls back to the separate kernels where the fused one does not apply.
+    ``order`` (see count_order_for) changes the cache traffic, not the result."""
     dev, bits, depth, pa, pb, pw, pdims, dims = _fused_args(x, layers)
     if depth > MAX_FUSE_DEPTH_COUNT:
         raise RuntimeError(f"at most {MAX_FUSE_DEPTH_COUNT} layers can be fused with the count, got {depth}")
@@ -513,6 +548,9 @@ def eval_fused_groupbitsum(x, layers, pad_len, k):
     batch = words * bits - int(pad_len)
     if pad_len < 0 or batch < 0:
         raise RuntimeError(f"pad_len ({pad_len}) has to be in [0, {words * bits}]")
+    if order is not None and (order.dtype != torch.int32 or order.shape != (out_dim,) or order.device != dev
+                              or not order.is_contiguous()):
+        raise RuntimeError(f"expected order to be a contiguous int32 [{out_dim}] tensor on {dev}")
     if 0 in dims:
         st = _lib.DL_ERR_TOO_LARGE
     else:
@@ -521,7 +559,9 @@ def eval_fused_groupbitsum(x, layers, pad_len, k):
         ws = torch.empty(max(2, -(-nbytes // 8)), dtype=torch.int64, device=dev)
         with torch.cuda.device(dev):
             st = _lib.load().dl_logic_eval_fused_groupbitsum(_p(x), depth, pa, pb, pw, pdims, _p(out), words, bits,
-                                                             int(pad_len), int(k), _p(ws), _stream(dev))
+                                                             int(pad_len), int(k),
+                                                             _p(order) if order is not None else None, _p(ws),
+                                                             _stream(dev))
     if st == _lib.DL_ERR_TOO_LARGE:
         return groupbitsum(eval_fused(x, layers), pad_len, k)
     if st:

@@ -104,3 +104,46 @@ def test_rejects_out_of_range_vertices():
     st = lib.dl_backward_schedule_build(verts.ctypes.data, neuron.ctypes.data, 1, 4, out.ctypes.data, out.ctypes.data,
                                         out.ctypes.data, ctypes.byref(n_fix))
     assert st == -_lib.DL_ERR_INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("depth", [1, 2])
+@pytest.mark.parametrize("rows,mid,out,k", [(40, 60, 60, 3), (16, 30, 20, 10), (9, 5, 7, 7), (100, 200, 500, 10)])
+def test_count_order_is_a_class_preserving_permutation_that_gathers_readers(depth, rows, mid, out, k):
+    """dl_count_order_build: every class is permuted onto itself, and walking a class in that order
+    never needs more distinct input rows per workgroup than the natural order (that is its purpose)."""
+    lib = _lib.load()
+    rng = np.random.default_rng(rows + out + depth)
+    top_in = mid if depth == 2 else rows
+    a_top = rng.integers(0, top_in, out).astype(np.int64)
+    b_top = rng.integers(0, top_in, out).astype(np.int64)
+    a_low = rng.integers(0, rows, mid).astype(np.int64) if depth == 2 else None
+    b_low = rng.integers(0, rows, mid).astype(np.int64) if depth == 2 else None
+    order = np.full(out, -1, np.int32)
+    group = 4
+    st = lib.dl_count_order_build(a_top.ctypes.data, b_top.ctypes.data, a_low.ctypes.data if depth == 2 else None,
+                                  b_low.ctypes.data if depth == 2 else None, rows, mid if depth == 2 else 0, out, k, group,
+                                  order.ctypes.data)
+    if out % k:
+        assert st == _lib.DL_ERR_NOT_DIVISIBLE
+        return
+    assert st == 0
+    per = out // k
+    for c in range(k):
+        assert sorted(order[c * per:(c + 1) * per].tolist()) == list(range(c * per, (c + 1) * per))
+    if depth == 2:
+        leaves = np.stack([a_low[a_top], b_low[a_top], a_low[b_top], b_low[b_top]], 1)
+    else:
+        leaves = np.stack([a_top, b_top], 1)
+
+    def distinct(seq):
+        return sum(len(np.unique(leaves[seq[c * per + g:min(c * per + g + group, (c + 1) * per)]]))
+                   for c in range(k) for g in range(0, per, group))
+    assert distinct(order) <= distinct(np.arange(out))
+
+
+def test_count_order_rejects_bad_wiring():
+    lib = _lib.load()
+    a = np.array([0, 5], np.int64)
+    order = np.empty(2, np.int32)
+    assert lib.dl_count_order_build(a.ctypes.data, a.ctypes.data, None, None, 4, 0, 2, 1, 4,
+                                    order.ctypes.data) == _lib.DL_ERR_INVALID_ARGUMENT

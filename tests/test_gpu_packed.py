@@ -260,6 +260,11 @@ def test_fused_eval_groupbitsum(ext, bits, in_dim, widths, W, k, pad):
     assert got.dtype == torch.int32 and tuple(got.shape) == want.shape
     assert np.array_equal(got.cpu().numpy(), want)
     assert torch.equal(got, ext.groupbitsum(ext.eval_fused(_dev(x), dev_layers), pad, k))
+    # walking the neurons in the cache-friendly order changes nothing
+    order = ext.count_order_for(dev_layers, in_dim, k)
+    assert order.dtype == torch.int32 and sorted(order.tolist()) == list(range(widths[-1]))
+    assert torch.equal(got, ext.eval_fused_groupbitsum(_dev(x), dev_layers, pad, k, order))
+    assert ext.count_order_for(dev_layers, in_dim, k) is order          # cached per wiring
 
 
 def test_lazy_pack_tensor_keeps_t_current():
