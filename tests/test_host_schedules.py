@@ -1,5 +1,7 @@
-"""Host logic of the fused backward pass: the destinations that dl_backward_schedule_build derives
-from an evaluation schedule, checked by replaying the kernel's walk in numpy."""
+"""Host-side planning code of the C-ABI library (no GPU): the evaluation schedule (trails of a
+layer's wiring), the destinations that dl_backward_schedule_build derives from it for the
+one-pass backward, checked by replaying the kernel's walk in numpy, and the neuron order of the
+fused count."""
 import ctypes
 
 import numpy as np
@@ -147,3 +149,32 @@ def test_count_order_rejects_bad_wiring():
     order = np.empty(2, np.int32)
     assert lib.dl_count_order_build(a.ctypes.data, a.ctypes.data, None, None, 4, 0, 2, 1, 4,
                                     order.ctypes.data) == _lib.DL_ERR_INVALID_ARGUMENT
+
+
+def test_schedules_of_random_multigraphs():
+    """Many small random wirings (parallel edges, self loops, isolated inputs): every neuron is
+    scheduled exactly once between its two inputs, chunks are whole, and the backward plan gives
+    every input its tokens exactly once (the replay of test_every_input_is_completed_exactly_once)."""
+    rng = np.random.default_rng(2024)
+    for _ in range(300):
+        in_dim = int(rng.integers(1, 40))
+        out_dim = int(rng.integers(0, 80))
+        a = rng.integers(0, in_dim, out_dim).astype(np.int64)
+        b = rng.integers(0, in_dim, out_dim).astype(np.int64)
+        if out_dim == 0:
+            a = np.zeros(1, np.int64)[:0]
+            b = a.copy()
+        verts, neuron, flip, steps = _schedule(a, b, in_dim) if out_dim else (np.zeros(1, np.int32), np.zeros(0, np.int32),
+                                                                             np.zeros(0, np.uint8), 0)
+        assert steps % 8 == 0 and steps <= 2 * out_dim + 16
+        seen = np.zeros(out_dim, int)
+        for s in range(steps):
+            n = neuron[s]
+            if n < 0:
+                continue
+            seen[n] += 1
+            u, v = verts[s], verts[s + 1]
+            assert (a[n], b[n]) == ((v, u) if flip[s] else (u, v))
+        assert (seen == 1).all()
+        if out_dim:
+            test_every_input_is_completed_exactly_once("random", in_dim, a, b)
