@@ -821,7 +821,7 @@ int forward_t(const void *x, const int64_t *a, const int64_t *b, const void *w, 
               int64_t batch, hipStream_t s) {
     constexpr int NPW = 4;
     const int64_t blocks = dl_ceil_div(out_dim, 4 * NPW);
-    if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    if (out_dim > 0x7fffffffLL) return DL_ERR_TOO_LARGE;     // neuron ids travel as int32 inside the kernel
     constexpr int V = Vec16<T>::n;
     if (batch % V == 0 && dl_aligned(x, 16) && dl_aligned(y, 16)) {
         DL_LAUNCH((forward_kernel<T, V, NPW, LOGITS>), dim3((unsigned) blocks, col_tiles(batch / V)),
