@@ -9,6 +9,9 @@ differently:
   compact interpreter loop evaluates them; compiles in well under a second at any size and runs
   at about the speed of the unrolled code built with -O0.
 
+``num_threads`` other than 1 (0 = all cores) spreads the blocks of ``num_bits`` samples over OpenMP
+threads (compiled with ``-fopenmp``); the reference's generated code is single-threaded.
+
 Both variants export ``apply_logic_gate_net(bool const *inp, int *out, size_t len)`` with the
 reference's meaning: ``inp`` holds ``len`` blocks of ``num_bits`` samples x ``num_inputs`` bools
 (sample-major), ``out`` receives ``num_classes`` int32 bit counts per sample.
@@ -37,13 +40,15 @@ _GATE_EXPR = ("(T) 0", "a & b", "a & ~b", "a", "b & ~a", "b", "a ^ b", "a | b", 
 
 class CompiledLogicNet(torch.nn.Module):
     def __init__(self, model: torch.nn.Sequential, device="cpu", num_bits=64, cpu_compiler="gcc", verbose=False,
-                 mode=None):
+                 mode=None, num_threads=1):
         super().__init__()
         self.model = model
         self.device = device
         self.num_bits = num_bits
         self.cpu_compiler = cpu_compiler
         self.mode = mode
+        self.num_threads = int(num_threads)      # 1: single-threaded like the reference; 0: all cores (OpenMP)
+        assert self.num_threads >= 0, num_threads
         assert cpu_compiler in ["clang", "gcc"], cpu_compiler
         assert num_bits in [8, 16, 32, 64]
         assert mode in [None, "unrolled", "table"], mode
@@ -87,13 +92,20 @@ class CompiledLogicNet(torch.nn.Module):
         n_last = len(self.layers[-1][0])
         per_class = n_last // self.num_classes
         planes = max(1, math.ceil(math.log2(n_last / self.num_classes + 1)))
+        omp_region = omp_for = ""
+        if self.num_threads != 1:               # every thread owns its buffers; blocks are independent
+            omp_region = "#pragma omp parallel" + (f" num_threads({self.num_threads})" if self.num_threads > 1 else "")
+            omp_for = "#pragma omp for schedule(static)"
         return f"""
 void apply_logic_gate_net(bool const *inp, int *out, size_t len) {{
     enum {{ F = {self.num_inputs}, BITS = {bits}, NOUT = {n_last}, K = {self.num_classes},
            PER_CLASS = {per_class}, PLANES = {planes} }};
+{omp_region}
+    {{
     T *words = malloc(sizeof(T) * F);
     T *gates = malloc(sizeof(T) * NOUT);
-    for (size_t blk = 0; blk < len; ++blk) {{
+{omp_for}
+    for (long long blk = 0; blk < (long long) len; ++blk) {{
         bool const *rows = inp + blk * (size_t) F * BITS;
         for (size_t f = 0; f < F; ++f) {{                    /* sample s of the block -> bit s */
             T w = 0;
@@ -121,6 +133,7 @@ void apply_logic_gate_net(bool const *inp, int *out, size_t len) {{
     }}
     free(words);
     free(gates);
+    }}
 }}
 """
 
@@ -183,7 +196,8 @@ void apply_logic_gate_net(bool const *inp, int *out, size_t len) {{
         if verbose:
             print("C code created ({} mode, {} lines) at {}".format(self._resolved_mode(), code.count("\n") + 1, c_path))
         t0 = time.time()
-        out = subprocess.run([self.cpu_compiler, "-shared", "-fPIC", "-O{}".format(opt_level), "-o", so_path, c_path])
+        flags = ["-shared", "-fPIC", "-O{}".format(opt_level)] + (["-fopenmp"] if self.num_threads != 1 else [])
+        out = subprocess.run([self.cpu_compiler, *flags, "-o", so_path, c_path])
         if out.returncode != 0:
             raise RuntimeError(f"compilation exited with error code {out.returncode}")
         print("Compiling finished in {:.3f} seconds.".format(time.time() - t0))

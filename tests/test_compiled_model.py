@@ -55,3 +55,18 @@ def test_default_mode_and_checks():
         dl.CompiledLogicNet(model, num_bits=12)
     with pytest.raises(AssertionError):
         dl.CompiledLogicNet(model)(np.zeros((4, 10), bool))                    # not compiled yet
+
+
+@pytest.mark.parametrize("mode", ["unrolled", "table"])
+def test_openmp_variant_equals_single_threaded(mode):
+    rng = np.random.default_rng(3)
+    layers = random_layers(rng, 24, [96, 96, 60])
+    model = build_model(24, layers, 6, device="cpu")
+    x = rng.random((64 * 37 + 11, 24)) < 0.5
+    want = po.net_eval_bitwise(x, layers, 6)
+    for threads in (0, 3):
+        net = dl.CompiledLogicNet(model, num_bits=64, mode=mode, num_threads=threads)
+        assert "#pragma omp parallel" in net.get_c_code()
+        net.compile(opt_level=1)
+        assert np.array_equal(net(x).numpy(), want), (mode, threads)
+    assert "omp" not in dl.CompiledLogicNet(model, mode=mode).get_c_code()        # the reference's single-threaded form
