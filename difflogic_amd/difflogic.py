@@ -102,9 +102,10 @@ class LogicLayer(torch.nn.Module):
                                                       self._train_schedule()).transpose(0, 1)
             w = torch.nn.functional.softmax(self.weights, dim=-1).to(x.dtype)
             return LogicLayerCudaFunction.apply(x, a, b, w, *tail).transpose(0, 1)
+        # eval mode: the discretised net on float inputs (no gradients)
         w = torch.nn.functional.one_hot(self.weights.argmax(-1), 16).to(x.dtype)
         with torch.no_grad():
-            return LogicLayerCudaFunction.apply(x, a, b, w, *tail).transpose(0, 1)
+            return difflogic_cuda.forward(x, a, b, w, self._train_schedule()).transpose(0, 1)
 
     def forward_cuda_eval(self, x: PackBitsTensor):
         """Packed inference.  Updates ``x`` in place (as the reference rebinds ``x.t``) and

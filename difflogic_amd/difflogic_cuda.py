@@ -68,8 +68,10 @@ def _p(t):
     return ctypes.c_void_p(t.data_ptr())
 
 
-def forward(x, a, b, w):
-    """x [in,B], a/b [out] int64, w [out,16] -> y [out,B]   (difflogic.cpp:46-51)."""
+def forward(x, a, b, w, schedule=None):
+    """x [in,B], a/b [out] int64, w [out,16] -> y [out,B]   (difflogic.cpp:46-51).
+    ``schedule`` (an EvalSchedule of (a, b); not in the reference) selects the chained kernel:
+    same result, one gathered input row per neuron instead of two."""
     for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w")):
         _check_input(t, n)
     code = _float_code(x, "logic_layer_cuda_forward")
@@ -82,8 +84,16 @@ def forward(x, a, b, w):
     dev = _same_device(x, a, b, w)
     in_dim, batch = x.shape
     y = torch.empty((out_dim, batch), dtype=x.dtype, device=dev)
+    lib = _lib.load()
     with torch.cuda.device(dev):
-        st = _lib.load().dl_logic_forward(_p(x), _p(a), _p(b), _p(w), _p(y), in_dim, out_dim, batch, code, _stream(dev))
+        st = _lib.DL_ERR_TOO_LARGE
+        if schedule is not None and out_dim > 0 and batch > 0:
+            _check_schedule(schedule, in_dim, out_dim, dev)
+            st = lib.dl_logic_forward_chained(_p(x), _p(schedule.verts), _p(schedule.neuron), _p(schedule.flip),
+                                              schedule.steps, _p(w), _p(y), None, in_dim, out_dim, batch, code,
+                                              _stream(dev))
+        if st == _lib.DL_ERR_TOO_LARGE:
+            st = lib.dl_logic_forward(_p(x), _p(a), _p(b), _p(w), _p(y), in_dim, out_dim, batch, code, _stream(dev))
     if st:
         _raise(st, "logic_layer_cuda_forward")
     return y

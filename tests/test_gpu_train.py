@@ -396,6 +396,13 @@ def test_layer_uses_schedule_for_wide_inputs():
     fo.layer_forward_sequential(xr, wide.indices[0].cpu(), wide.indices[1].cpu(),
                                 torch.softmax(wr, -1)).square().sum().backward()
     assert close(x.grad, xr.grad, 1e-4)[0] and close(wide.weights.grad, wr.grad, 1e-4)[0]
+    # eval mode on float inputs takes the chained forward too: exact 0/1 results of the discretised gates
+    wide.eval()
+    xb = (torch.rand(64, 5000, device="cuda") < 0.5).float()
+    ye = wide(xb)
+    onehot = torch.nn.functional.one_hot(wide.weights.argmax(-1), 16).double().cpu()
+    want = fo.layer_forward_sequential(xb.cpu().double(), wide.indices[0].cpu(), wide.indices[1].cpu(), onehot)
+    assert torch.equal(ye.cpu().double(), want) and not ye.requires_grad
 
 
 def test_chained_layer_matches_the_python_formulation_on_random_wirings(monkeypatch):
