@@ -337,7 +337,7 @@ def main():
     args = parse()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the path shards along the batch without "
-              "communication; see DESIGN.md); --gpus %d is not supported" % args.gpus, file=sys.stderr)
+              "communication); --gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
     import torch
 
