@@ -258,16 +258,22 @@ __global__ __launch_bounds__(DL_BLOCK) void eval_chain_kernel(const V *__restric
         if (col >= ncols) continue;
         const V *xcol = x + col;
         V *ycol = y + col;
+        if (c_first >= nchunks) continue;
+        // the wave's chunks follow each other in the schedule: only the first vertex of the first
+        // one is evaluated on its own, after that every step's left input is the step before's right
+        V prev;
+        {
+            Subtree<V, DS> first;
+            first.locate(verts[c_first * CHUNK], sub_leaves, sub_gates);
+            V leaves0[G];
+            first.gather(xcol, ncols, leaves0);
+            prev = TreeFold<V, DS>::run(leaves0, first.gates);
+        }
 #pragma unroll 1
         for (int it = 0; it < ITERS; ++it) {
             const int64_t c = c_first + it;
             if (c >= nchunks) break;
             const int64_t s0 = c * CHUNK;
-            Subtree<V, DS> first;
-            first.locate(verts[s0], sub_leaves, sub_gates);
-            V leaves0[G];
-            first.gather(xcol, ncols, leaves0);
-            V prev = TreeFold<V, DS>::run(leaves0, first.gates);
 #pragma unroll
             for (int j = 0; j < CHUNK; j += 2) {
                 Subtree<V, DS> ta, tb;
@@ -1154,11 +1160,19 @@ int launch_eval_chain(int sub_depth, const void *x, const int32_t *sub_leaves, c
                            dim3((unsigned) gx, (unsigned) ctiles), dim3(DL_BLOCK), 0, s, (const V *) x, sub_leaves,    \
                            sub_gates, verts, neuron, flip, w_top, (V *) y, nchunks, ncols);                            \
     }
+    // Two consecutive chunks per wave halve the vertices that are evaluated only to seed a chain, but
+    // also the workgroups per column tile; deep subtrees want enough of those to keep the chip on few
+    // column tiles (whose input rows are what the L2 caches hold).
+    const bool pair = sub_depth <= 1 || nchunks >= 4096;
     switch (sub_depth) {
     case 0: DL_CHAIN_LAUNCH(0, 2) break;
     case 1: DL_CHAIN_LAUNCH(1, 2) break;
-    case 2: DL_CHAIN_LAUNCH(2, 1) break;
-    default: DL_CHAIN_LAUNCH(3, 1) break;
+    case 2:
+        if (pair) DL_CHAIN_LAUNCH(2, 2) else DL_CHAIN_LAUNCH(2, 1)
+        break;
+    default:
+        if (pair) DL_CHAIN_LAUNCH(3, 2) else DL_CHAIN_LAUNCH(3, 1)
+        break;
     }
 #undef DL_CHAIN_LAUNCH
     return dl_launch_status();
