@@ -53,8 +53,32 @@ def _same_device(*tensors):
     return dev
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(dev):
+    """torch's current stream on ``dev`` as the void* the C ABI takes."""
+    if _raw_stream is not None and dev.index is not None:
+        return ctypes.c_void_p(_raw_stream(dev.index))           # no Stream object on the hot path
     return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def _on(dev):
+    """Device guard for a launch: nothing to do when ``dev`` is already current."""
+    if dev.index is None or torch.cuda.current_device() == dev.index:
+        return _NO_GUARD
+    return torch.cuda.device(dev)
 
 
 def _raise(status, what):
@@ -85,7 +109,7 @@ def forward(x, a, b, w, schedule=None):
     in_dim, batch = x.shape
     y = torch.empty((out_dim, batch), dtype=x.dtype, device=dev)
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _lib.DL_ERR_TOO_LARGE
         if schedule is not None and out_dim > 0 and batch > 0:
             _check_schedule(schedule, in_dim, out_dim, dev)
@@ -113,7 +137,7 @@ def backward_w(x, a, b, grad_y):
     dev = _same_device(x, a, b, grad_y)
     in_dim, batch = x.shape
     grad_w = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _lib.load().dl_logic_backward_w(_p(x), _p(a), _p(b), _p(grad_y), _p(grad_w), in_dim, out_dim, batch, code,
                                              _stream(dev))
     if st:
@@ -141,7 +165,7 @@ def backward_x(x, a, b, w, grad_y, given_x_indices_of_y_start, given_x_indices_o
     _check_index(given_x_indices_of_y, "given_x_indices_of_y", 2 * out_dim)
     dev = _same_device(x, a, b, w, grad_y, given_x_indices_of_y_start, given_x_indices_of_y)
     grad_x = torch.empty_like(x)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _lib.load().dl_logic_backward_x(_p(x), _p(a), _p(b), _p(w), _p(grad_y), _p(given_x_indices_of_y_start),
                                              _p(given_x_indices_of_y), _p(grad_x), in_dim, out_dim, batch,
                                              float(scale), code, _stream(dev))
@@ -170,7 +194,7 @@ def forward_logits(x, a, b, logits, schedule=None):
     y = torch.empty((out_dim, batch), dtype=x.dtype, device=dev)
     probs = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _lib.DL_ERR_TOO_LARGE
         if schedule is not None and out_dim > 0:
             _check_schedule(schedule, in_dim, out_dim, dev)
@@ -209,7 +233,7 @@ def backward_logits(x, a, b, grad_y, probs, schedule=None):
     in_dim, batch = x.shape
     grad_logits = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _lib.DL_ERR_TOO_LARGE
         if schedule is not None and out_dim > 0 and batch > 0:
             _check_schedule(schedule, in_dim, out_dim, dev)
@@ -252,7 +276,7 @@ def backward_chained(x, w, grad_y, schedule, scale=1.0, softmax_backward=False):
     if ws_bytes < 0:
         _raise(-ws_bytes, "logic_layer_cuda_backward_chained")
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = lib.dl_logic_backward_chained(
             _p(x), _p(schedule.verts), _p(schedule.neuron), _p(schedule.flip), _p(dst), schedule.steps, _p(w),
             _p(grad_y), 1 if softmax_backward else 0, _p(fix_vertex) if n_fix else None,
@@ -285,7 +309,7 @@ def eval(x, a, b, w):  # noqa: A001  (the reference's name)
     dev = _same_device(x, a, b, w)
     in_dim, words = x.shape
     y = torch.empty((out_dim, words), dtype=x.dtype, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _lib.load().dl_logic_eval(_p(x), _p(a), _p(b), _p(w), _p(y), in_dim, out_dim, words, bits, _stream(dev))
     if st:
         _raise(st, "logic_layer_cuda_eval")
@@ -303,7 +327,7 @@ def tensor_packbits_cuda(t, bit_count):
     words = -(-batch // bit_count)
     out = torch.empty((features, words), dtype=_BITS_TO_DTYPE[bit_count], device=t.device)
     pad = ctypes.c_int64(0)
-    with torch.cuda.device(t.device):
+    with _on(t.device):
         st = _lib.load().dl_tensor_packbits(_p(t), _p(out), features, batch, bit_count, ctypes.byref(pad),
                                             _stream(t.device))
     if st:
@@ -324,7 +348,7 @@ def tensor_packbits_batch_major(x, bit_count):
     words = -(-batch // bit_count)
     out = torch.empty((features, words), dtype=_BITS_TO_DTYPE[bit_count], device=x.device)
     pad = ctypes.c_int64(0)
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         st = _lib.load().dl_tensor_packbits_batch_major(_p(x), _p(out), batch, features, bit_count, ctypes.byref(pad),
                                                         _stream(x.device))
     if st:
@@ -345,7 +369,7 @@ def groupbitsum(b, pad_len, k):
     if pad_len < 0 or batch < 0:
         raise RuntimeError(f"pad_len ({pad_len}) has to be in [0, {words * bits}]")
     out = torch.empty((batch, k), dtype=torch.int32, device=b.device)
-    with torch.cuda.device(b.device):
+    with _on(b.device):
         st = _lib.load().dl_groupbitsum(_p(b), _p(out), in_dim, words, bits, int(pad_len), int(k), _stream(b.device))
     if st:
         _raise(st, "groupbitsum")
@@ -399,7 +423,7 @@ def eval_fused(x, layers):
     else:
         y = torch.empty((dims[-1], words), dtype=x.dtype, device=dev)
         ws = _fused_workspace(depth, dims[-1], dev)
-        with torch.cuda.device(dev):
+        with _on(dev):
             st = _lib.load().dl_logic_eval_fused(_p(x), depth, pa, pb, pw, pdims, _p(y), words, bits, _p(ws),
                                                  _stream(dev))
     if st == _lib.DL_ERR_TOO_LARGE:
@@ -499,7 +523,7 @@ def eval_chained(x, layers, schedule=None):
                            f"{dims[-2]}->{dims[-1]}")
     y = torch.empty((dims[-1], words), dtype=x.dtype, device=dev)
     ws = _fused_workspace(depth - 1, dims[-2], dev) if depth > 1 else None
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _lib.load().dl_logic_eval_chained(_p(x), depth, pa, pb, pw, pdims, _p(schedule.verts), _p(schedule.neuron),
                                                _p(schedule.flip), schedule.steps, _p(y), words, bits,
                                                _p(ws) if ws is not None else None, _stream(dev))
@@ -567,7 +591,7 @@ def eval_fused_groupbitsum(x, layers, pad_len, k, order=None):
         out = torch.empty((batch, k), dtype=torch.int32, device=dev)
         nbytes = _lib.load().dl_logic_eval_fused_groupbitsum_workspace_bytes(depth, out_dim, words, bits, int(k))
         ws = torch.empty(max(2, -(-nbytes // 8)), dtype=torch.int64, device=dev)
-        with torch.cuda.device(dev):
+        with _on(dev):
             st = _lib.load().dl_logic_eval_fused_groupbitsum(_p(x), depth, pa, pb, pw, pdims, _p(out), words, bits,
                                                              int(pad_len), int(k),
                                                              _p(order) if order is not None else None, _p(ws),
@@ -593,7 +617,7 @@ def group_sum_forward(x, k, tau):
     y = torch.empty((batch, k), dtype=x.dtype, device=x.device)
     ws = torch.empty(max(1, lib.dl_group_sum_workspace_bytes(out_dim, batch, k, code)), dtype=torch.uint8,
                      device=x.device)
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         st = lib.dl_group_sum_forward(_p(x), _p(y), _p(ws), out_dim, batch, int(k), float(tau), code, _stream(x.device))
     if st:
         _raise(st, "group_sum_forward")
@@ -608,7 +632,7 @@ def group_sum_backward(grad_y, out_dim, tau):
     if k <= 0 or out_dim % k != 0:
         raise ValueError(f"in_dim ({out_dim}) has to be divisible by k ({k}) but it is not")
     grad_x = torch.empty((out_dim, batch), dtype=grad_y.dtype, device=grad_y.device)
-    with torch.cuda.device(grad_y.device):
+    with _on(grad_y.device):
         st = _lib.load().dl_group_sum_backward(_p(grad_y), _p(grad_x), out_dim, batch, int(k), float(tau), code,
                                                _stream(grad_y.device))
     if st:
