@@ -13,8 +13,11 @@ DL_ERR_NOT_DIVISIBLE = 3
 DL_ERR_DTYPE = 4
 DL_ERR_LAUNCH = 5
 DL_ERR_TOO_LARGE = 6
+DL_ERR_SCRATCH_LIMIT = 7
 
 DL_F16, DL_F32, DL_F64 = 0, 1, 2
+
+DL_STATIC_SCRATCH_BYTES = 64 << 20      # include/difflogic_hip.h
 
 _vp, _i64, _int, _dbl = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_double
 
@@ -49,6 +52,7 @@ SIGNATURES = {
     "dl_logic_eval_chained": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _int, _vp, _vp],
     "dl_logic_eval_fused_groupbitsum_workspace_bytes": [_int, _i64, _i64, _int, _i64],
     "dl_logic_eval_fused_groupbitsum": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _i64, _vp, _vp, _vp],
+    "dl_logic_eval_fused_groupbitsum_noalloc": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _i64, _vp, _vp],
     "dl_count_group": [],
     "dl_count_order_build": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp],
 }

@@ -6,6 +6,8 @@
 // 8/16/32/64-bit word types and the widest vector access the row length allows is used.
 #include "dl_common.h"
 
+#include <mutex>
+
 namespace {
 
 // ------------------------------------------------------------------------------------------
@@ -1130,6 +1132,63 @@ extern "C" int dl_logic_eval_fused_groupbitsum(const void *x, int depth, const i
 }
 
 extern "C" int dl_count_group(void) { return DL_COUNT_ROWS; }
+
+// ------------------------------------------------------------------------------------------
+// dl_logic_eval_fused_groupbitsum for callers that cannot allocate (code under HIP graph capture,
+// serving loops, harnesses that forbid hipMalloc): the workspace of the allocating entry point
+// (flattened wiring + the bit-sliced partial counters the first pass hands to the second) lives in
+// a file-scope device array.  Each GPU holds its own copy of the array at its own address, looked
+// up once per device; host code only ever uses that looked-up address, never the array's name.
+// Nothing in the array has to start at zero: compose_tree_kernel rewrites the wiring tables and
+// pass 1 writes every counter that pass 2 reads.
+// ------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[DL_STATIC_SCRATCH_BYTES];
+
+#define DL_MAX_DEVICES 64
+static void *scratch_address[DL_MAX_DEVICES];      // per device: where that GPU's copy of `scratch` lives
+static std::mutex scratch_mutex;
+
+// Address of the current device's copy of `scratch` (looked up on the first call per device).
+static int static_scratch(void **ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        dl_last_hip_error_code = (int) e;
+        return DL_ERR_LAUNCH;
+    }
+    if (dev < 0 || dev >= DL_MAX_DEVICES) return DL_ERR_TOO_LARGE;
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_address[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            dl_last_hip_error_code = (int) (e != hipSuccess ? e : hipErrorInvalidSymbol);
+            return DL_ERR_LAUNCH;
+        }
+        scratch_address[dev] = p;
+    }
+    *ptr = scratch_address[dev];
+    return DL_OK;
+}
+
+extern "C" int dl_logic_eval_fused_groupbitsum_noalloc(const void *x, int depth, const int64_t *const *a,
+                                                       const int64_t *const *b, const uint8_t *const *w,
+                                                       const int64_t *dims, int32_t *out, int64_t words, int bit_count,
+                                                       int64_t pad_len, int64_t k, const int32_t *order, void *stream) {
+    if (!valid_bit_count(bit_count)) return DL_ERR_BIT_COUNT;
+    if (depth < 1 || depth > 2 || !dims || words < 0 || k <= 0 || pad_len < 0) return DL_ERR_INVALID_ARGUMENT;
+    const int64_t out_dim = dims[depth];
+    if (out_dim <= 0) return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim % k != 0) return DL_ERR_NOT_DIVISIBLE;
+    const int64_t row_bytes = words * (bit_count / 8);
+    if (row_bytes % 8 != 0) return DL_ERR_TOO_LARGE;          // rows of whole 64-bit words only, as the allocating call
+    const int64_t need = dl_logic_eval_fused_groupbitsum_workspace_bytes(depth, out_dim, words, bit_count, k);
+    if (need > (int64_t) DL_STATIC_SCRATCH_BYTES) return DL_ERR_SCRATCH_LIMIT;
+    void *ws = nullptr;
+    const int st = static_scratch(&ws);
+    if (st != DL_OK) return st;
+    return dl_logic_eval_fused_groupbitsum(x, depth, a, b, w, dims, out, words, bit_count, pad_len, k, order, ws, stream);
+}
 
 extern "C" int64_t dl_logic_eval_fused_groupbitsum_workspace_bytes(int depth, int64_t out_dim, int64_t words,
                                                                     int bit_count, int64_t k) {

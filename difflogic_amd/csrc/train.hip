@@ -1391,6 +1391,7 @@ extern "C" const char *dl_status_string(int status) {
     case DL_ERR_DTYPE: return "dtype has to be DL_F16, DL_F32 or DL_F64";
     case DL_ERR_LAUNCH: return "HIP refused the kernel launch";
     case DL_ERR_TOO_LARGE: return "size exceeds what this entry point supports";
+    case DL_ERR_SCRATCH_LIMIT: return "the call needs more than the library's static scratch array (DL_STATIC_SCRATCH_BYTES)";
     default: return "unknown status";
     }
 }

@@ -603,6 +603,38 @@ def eval_fused_groupbitsum(x, layers, pad_len, k, order=None):
     return out
 
 
+def eval_fused_groupbitsum_noalloc(x, layers, pad_len, k, out, order=None):
+    """eval_fused_groupbitsum into the caller's ``out`` (int32 [batch, k], contiguous) through the
+    entry point that allocates no device memory: its workspace is a static device array of
+    ``_lib.DL_STATIC_SCRATCH_BYTES`` inside the library (one copy per GPU, shared by all calls on
+    that GPU, so calls must not overlap in time on one GPU).  Raises RuntimeError when the call
+    needs more scratch than that or when rows are not whole 64-bit words; there is no fallback.
+    Not part of the reference's extension."""
+    dev, bits, depth, pa, pb, pw, pdims, dims = _fused_args(x, layers)
+    if depth > MAX_FUSE_DEPTH_COUNT:
+        raise RuntimeError(f"at most {MAX_FUSE_DEPTH_COUNT} layers can be fused with the count, got {depth}")
+    out_dim, words = dims[-1], x.shape[1]
+    if k <= 0 or out_dim % k != 0:
+        raise ValueError(f"in_dim ({out_dim}) has to be divisible by k ({k}) but it is not")
+    batch = words * bits - int(pad_len)
+    if pad_len < 0 or batch < 0:
+        raise RuntimeError(f"pad_len ({pad_len}) has to be in [0, {words * bits}]")
+    _check_input(out, "out")
+    if out.dtype != torch.int32 or tuple(out.shape) != (batch, k) or out.device != dev:
+        raise RuntimeError(f"expected out to be int32 [{batch}, {k}] on {dev}, got {out.dtype} {tuple(out.shape)}")
+    if order is not None and (order.dtype != torch.int32 or order.shape != (out_dim,) or order.device != dev
+                              or not order.is_contiguous()):
+        raise RuntimeError(f"expected order to be a contiguous int32 [{out_dim}] tensor on {dev}")
+    with _on(dev):
+        st = _lib.load().dl_logic_eval_fused_groupbitsum_noalloc(_p(x), depth, pa, pb, pw, pdims, _p(out), words, bits,
+                                                                 int(pad_len), int(k),
+                                                                 _p(order) if order is not None else None,
+                                                                 _stream(dev))
+    if st:
+        _raise(st, "logic_layer_cuda_eval_fused_groupbitsum_noalloc")
+    return out
+
+
 def group_sum_forward(x, k, tau):
     """Feature-major GroupSum: x [out,B] -> [B,k] = per-class sums over neurons / tau
     (difflogic/difflogic.py:195-196 on the layout the layer kernels produce)."""

@@ -4,7 +4,8 @@
  * Conventions
  * -----------
  * - Every pointer is a DEVICE pointer on the current HIP device unless stated otherwise.
- *   The library never allocates, frees or synchronises: the caller owns all buffers
+ *   The library never allocates, frees or synchronises (dl_logic_eval_fused_groupbitsum_noalloc
+ *   owns one static device array, see there): the caller owns all buffers
  *   (inputs are read-only, outputs are fully overwritten) and orders work through the
  *   `stream` argument (a hipStream_t passed as void*; NULL = the null stream).
  * - All matrices are feature-major and batch-contiguous: element (row f, column r) of an
@@ -37,7 +38,8 @@ typedef enum dl_status {
     DL_ERR_NOT_DIVISIBLE = 3,    /* groupbitsum: in_dim not divisible by k                    */
     DL_ERR_DTYPE = 4,            /* dtype not one of dl_dtype                                 */
     DL_ERR_LAUNCH = 5,           /* the HIP runtime refused the launch (see dl_last_hip_error) */
-    DL_ERR_TOO_LARGE = 6         /* a size exceeds what the entry point supports              */
+    DL_ERR_TOO_LARGE = 6,        /* a size exceeds what the entry point supports              */
+    DL_ERR_SCRATCH_LIMIT = 7     /* the call needs more than DL_STATIC_SCRATCH_BYTES of scratch */
 } dl_status;
 
 typedef enum dl_dtype { DL_F16 = 0, DL_F32 = 1, DL_F64 = 2 } dl_dtype;
@@ -253,6 +255,28 @@ int dl_logic_eval_fused_groupbitsum(const void *x, int depth, const int64_t *con
                                     const int64_t *dims, int32_t *out, int64_t words, int bit_count,
                                     int64_t pad_len, int64_t k, const int32_t *order, void *workspace,
                                     void *stream);
+
+/* dl_logic_eval_fused_groupbitsum without a workspace argument, for callers that cannot allocate
+ * device memory: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  It has no counterpart in the reference (whose functions allocate their outputs and
+ * scratch through torch, difflogic/cuda/difflogic_kernel.cu:316,518,615,688).  The workspace is a
+ * static device array of DL_STATIC_SCRATCH_BYTES inside the library; every GPU the library runs
+ * on holds its own copy until the process ends.  The call allocates and frees nothing and runs
+ * the same kernels as dl_logic_eval_fused_groupbitsum, with the same arguments, results and
+ * status codes, plus:
+ *   DL_ERR_SCRATCH_LIMIT  dl_logic_eval_fused_groupbitsum_workspace_bytes(depth, dims[depth],
+ *                         words, bit_count, k) exceeds DL_STATIC_SCRATCH_BYTES (split the batch);
+ *   DL_ERR_TOO_LARGE      rows are not whole 64-bit words (no per-layer fallback exists here).
+ * The first call on a device looks the array's address up (make it outside a graph capture).
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different
+ * streams or threads) race; calls ordered on one stream do not.  Nothing in the array needs to be
+ * cleared between calls. */
+#define DL_STATIC_SCRATCH_BYTES (64u << 20)
+int dl_logic_eval_fused_groupbitsum_noalloc(const void *x, int depth, const int64_t *const *a,
+                                            const int64_t *const *b, const uint8_t *const *w,
+                                            const int64_t *dims, int32_t *out, int64_t words,
+                                            int bit_count, int64_t pad_len, int64_t k,
+                                            const int32_t *order, void *stream);
 
 #ifdef __cplusplus
 }
