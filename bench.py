@@ -7,14 +7,34 @@ one pass of the whole path over the batch, starting from a bool [B, 784] tensor 
 HBM: PackBitsTensor (transpose + pack, 64-bit words) -> six LogicLayers (evaluated in fused
 groups) -> GroupSum bit counts [B, 10] int32.
 
-Prints ONE JSON line.  `roofline` describes the dominant launch (the one that takes the most
-time per step): its algorithmic bytes (per layer 8*W*(in+out) + 17*out, summed over the layers a
-fused launch replaces) divided by the launch duration measured with events on the launch stream
-inside the timed region.  `cpu_baseline`
-times the CPU oracle (single thread, like the reference's generated C) on a bounded sample.
-`extra.train` reports the fp32 forward+backward path (784 -> 6 x 64000, B = 512).
+Prints ONE JSON line.
+
+`roofline` describes the dominant launch (the one that takes the most time per step), timed with
+events on the launch stream inside the timed region.  A fused launch replaces several layers and
+moves fewer bytes than their algorithmic sum, so two figures are kept apart:
+  * `achieved` / `frac`: bytes the launch really moved between the L2 caches and the memory fabric
+    (`traffic`, from the committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary of this very
+    kernel source, see profiles/packed_kernel_traffic.json) divided by the launch time, against
+    the 8 TB/s HBM peak; `bound` names the resource the counters show as binding;
+  * `alg_GBps` / `alg_over_peak`: the algorithmic bytes (per layer 8*W*(in+out) + 17*out, summed
+    over the layers the launch replaces, plus 8*W*out + 4*k*B for the count) divided by the same
+    time.  This ratio can exceed 1 for a fused launch and is not a bandwidth.
+When the committed traffic summary was taken from other kernel sources than the built ones,
+`traffic` is null, a warning goes to stderr, and `achieved`/`frac` fall back to null.
+
+`cpu_baseline` times the CPU oracle (single thread, like the reference's generated C) on a bounded
+sample.  `extra.configs` holds the other BASELINE configurations: C2 and C4 (packed inference,
+checked bit-exactly against the CPU interpreter on the first 4096 samples of the full-batch
+result), C3 and C5 (fp32 training forward+backward, with and without the Adam step, eager and as a
+replayed HIP graph) and C1 on the GPU next to the CPU python-implementation step.
+
+`python bench.py --ceilings` instead measures plain streaming and gather kernels (the practical
+ceilings the kernels are compared with) and prints them as one JSON line.
 """
 import argparse
+import ctypes
+import gc
+import hashlib
 import json
 import os
 import statistics
@@ -26,6 +46,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "packed_kernel_traffic.json")
+# what the measured traffic of the packed launches depends on: the kernels and the launch plan
+TRAFFIC_SOURCES = ("difflogic_amd/csrc/packed.hip", "difflogic_amd/csrc/schedule.cpp", "difflogic_amd/csrc/dl_common.h",
+                   "difflogic_amd/packbitstensor.py")
 
 
 def parse():
@@ -38,33 +62,71 @@ def parse():
     ap.add_argument("--layers", type=int, default=6)
     ap.add_argument("--features", type=int, default=784)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-train", action="store_true")
+    ap.add_argument("--no-train", action="store_true", help="skip the training configurations (C1, C3, C5)")
+    ap.add_argument("--no-configs", action="store_true", help="skip the other packed configurations (C2, C4)")
+    ap.add_argument("--only", default="", help="comma list out of c1,c2,c3,c4,c5: run only these extra configurations")
     ap.add_argument("--cpu-sample-log2", type=int, default=18)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 4 plain device copies of 1 GiB (for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE)")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="measure streaming read/write/copy and row-gather ceilings instead of the benchmark")
     return ap.parse_args()
+
+
+def source_hash():
+    """sha256 over the sources the packed launches' traffic depends on."""
+    h = hashlib.sha256()
+    for rel in TRAFFIC_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(rel.encode() + b"\0" + f.read() + b"\0")
+    return h.hexdigest()[:16]
 
 
 def eval_layer_bytes(in_dim, out_dim, words):
     return 8 * words * (in_dim + out_dim) + 17 * out_dim
 
 
-def packed_bench(args, torch, dl):
-    F, width, L, k = args.features, args.width, args.layers, 10
-    B = 1 << args.batch_log2
-    W = B // 64
-    torch.manual_seed(0)
-    mods, d = [torch.nn.Flatten()], F
-    for _ in range(L):
-        mods.append(dl.LogicLayer(d, width, connections="random"))
-        d = width
-    model = torch.nn.Sequential(*mods, dl.GroupSum(k, 30.0)).eval()
-    g = torch.Generator(device="cuda").manual_seed(1)
-    x = torch.rand(B, F, device="cuda", generator=g) < 0.2
+# ------------------------------------------------------------------------------------------
+# packed inference
+# ------------------------------------------------------------------------------------------
 
+def bernoulli_input(torch, B, F, seed):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    return torch.rand(B, F, device="cuda", generator=g) < 0.2
+
+
+def thresholded_input(torch, B, seed, as_float=False):
+    """3x32x32 uniform values thresholded at 1/4, 2/4, 3/4 and concatenated on the channel axis
+    (experiments/main.py:57 with 3 thresholds): [B, 9216]."""
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    out = torch.empty(B, 9216, dtype=torch.float32 if as_float else torch.bool, device="cuda")
+    step = 1 << 14
+    for s in range(0, B, step):
+        u = torch.rand(min(step, B - s), 3, 32, 32, device="cuda", generator=g)
+        bits = torch.cat([u > (i + 1) / 4 for i in range(3)], dim=1).flatten(1)
+        out[s:s + step] = bits.float() if as_float else bits
+    return out
+
+
+def packed_model(torch, dl, F, widths, k, seed=0, connections="random"):
+    torch.manual_seed(seed)
+    mods, d = [torch.nn.Flatten()], F
+    for w in widths:
+        mods.append(dl.LogicLayer(d, w, connections=connections))
+        d = w
+    return torch.nn.Sequential(*mods, dl.GroupSum(k, 30.0)).eval()
+
+
+def packed_run(torch, dl, model, x, k, steps, warmup):
+    """Times `steps` passes of pack -> layers -> counts over x; returns (samples/s, ms per step,
+    per-launch table, last output).  Every binding call of the path is bracketed by events on the
+    launch stream."""
+    B, F = x.shape
+    W = B // 64
     ext = dl.difflogic_cuda
     names = ("tensor_packbits_batch_major", "eval", "eval_fused", "eval_chained", "eval_fused_groupbitsum",
-             "groupbitsum")
+             "eval_chained_groupbitsum", "eval_net_lds", "groupbitsum")
+    names = tuple(n for n in names if hasattr(ext, n))
     real = {n: getattr(ext, n) for n in names}
     launches = []          # (kernel label, algorithmic bytes, start_event, end_event)
     record = {"on": False}
@@ -80,9 +142,10 @@ def packed_bench(args, torch, dl):
             return "eval %d->%d" % (a[0].shape[0], a[3].shape[0]), eval_layer_bytes(a[0].shape[0], a[3].shape[0], W)
         dims = [a[0].shape[0]] + [l[2].shape[0] for l in a[1]]
         by = sum(eval_layer_bytes(i, o, W) for i, o in zip(dims[:-1], dims[1:]))
-        label = "%s x%d %s" % (name if name != "eval_fused_groupbitsum" else "eval_fused", len(a[1]),
-                               "->".join(str(d) for d in dims))
-        if name == "eval_fused_groupbitsum":
+        counted = name in ("eval_fused_groupbitsum", "eval_chained_groupbitsum", "eval_net_lds")
+        base = {"eval_fused_groupbitsum": "eval_fused", "eval_chained_groupbitsum": "eval_chained"}.get(name, name)
+        label = "%s x%d %s" % (base, len(a[1]), "->".join(str(d) for d in dims))
+        if counted:
             by += 8 * W * dims[-1] + 4 * k * B
             label += " +groupbitsum"
         return label, by
@@ -107,12 +170,16 @@ def packed_bench(args, torch, dl):
             return model(dl.PackBitsTensor(x, bit_count=64))
 
     try:
-        for _ in range(args.warmup):
+        t_first = time.perf_counter()
+        out = step()
+        torch.cuda.synchronize()
+        first_call_ms = (time.perf_counter() - t_first) * 1e3       # includes the host-side schedule / order builds
+        for _ in range(max(0, warmup - 1)):
             out = step()
         torch.cuda.synchronize()
         record["on"] = True
         t0 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(steps):
             out = step()
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
@@ -121,109 +188,231 @@ def packed_bench(args, torch, dl):
             setattr(ext, n, real[n])
         record["on"] = False
 
-    ms_per_step = elapsed / args.steps * 1e3
     per_kernel = {}
     for label, by, s, e in launches:
         d = per_kernel.setdefault(label, {"n": 0, "ms": 0.0, "bytes": by})
         d["n"] += 1
         d["ms"] += s.elapsed_time(e)
+    return B * steps / elapsed, elapsed / steps * 1e3, per_kernel, out, first_call_ms
+
+
+def kernel_table(per_kernel, steps):
+    return {kk: {"avg_ms": round(v["ms"] / v["n"], 4), "launches_per_step": v["n"] / steps,
+                 "algorithmic_GB": round(v["bytes"] / 1e9, 3),
+                 "alg_GBps": round(v["bytes"] / (v["ms"] / v["n"] * 1e-3) / 1e9, 1)}
+            for kk, v in per_kernel.items()}
+
+
+def load_traffic():
+    """The committed rocprofv3 --pmc summary of the packed launches, or ({}, note) when it was
+    taken from other kernel sources than the ones in the tree."""
+    if not os.path.exists(TRAFFIC_JSON):
+        return {}, "no traffic summary committed"
+    with open(TRAFFIC_JSON) as f:
+        table = json.load(f)
+    have, want = table.get("_source_hash"), source_hash()
+    if have != want:
+        note = ("profiles/packed_kernel_traffic.json was measured on kernel sources %s, the tree has %s: traffic "
+                "not reported; re-run the --pmc passes named in profiles/packed_path_hbm_traffic.txt" % (have, want))
+        print("bench.py: WARNING: " + note, file=sys.stderr)
+        return {}, note
+    return table, None
+
+
+def packed_headline(args, torch, dl):
+    F, width, L, k = args.features, args.width, args.layers, 10
+    B = 1 << args.batch_log2
+    model = packed_model(torch, dl, F, [width] * L, k)
+    x = bernoulli_input(torch, B, F, 1)
+    value, ms_per_step, per_kernel, out, first_ms = packed_run(torch, dl, model, x, k, args.steps, args.warmup)
+
     # dominant kernel = the launch kind that takes the most time in a step
     dom = max(per_kernel, key=lambda kk: per_kernel[kk]["ms"])
     avg_ms = per_kernel[dom]["ms"] / per_kernel[dom]["n"]
     alg = per_kernel[dom]["bytes"]
-    achieved = alg / (avg_ms * 1e-3) / 1e9
-    total_alg = sum(v["bytes"] * v["n"] for v in per_kernel.values()) / args.steps
+    alg_gbps = alg / (avg_ms * 1e-3) / 1e9
+    table, note = load_traffic()
+    entry = table.get(dom) or {}
+    traffic = entry.get("hbm_bytes_per_launch")
+    achieved = traffic / (avg_ms * 1e-3) / 1e9 if traffic else None
     roofline = {
-        "bound": "hbm", "kernel": dom,
-        "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-        "traffic": load_traffic(dom), "algorithmic_bytes_per_launch": int(alg), "avg_launch_ms": round(avg_ms, 4),
-        "launches_timed": per_kernel[dom]["n"],
+        "bound": entry.get("bound", "hbm") if traffic else "hbm (traffic of this build not measured)",
+        "kernel": dom,
+        "achieved": round(achieved, 1) if achieved else None, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4) if achieved else None,
+        "traffic": traffic,
+        "achieved_is": "measured L2<->fabric bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a plain "
+                       "copy) / launch time; reads served by the Infinity Cache are included",
+        "algorithmic_bytes_per_launch": int(alg), "alg_GBps": round(alg_gbps, 1),
+        "alg_over_peak": round(alg_gbps / HBM_PEAK_GBS, 4),
+        "avg_launch_ms": round(avg_ms, 4), "launches_timed": per_kernel[dom]["n"],
+        "fully_fused_floor_bytes_per_sample": F // 8 + 4 * k,
     }
+    if note:
+        roofline["traffic_note"] = note
+    total_alg = sum(v["bytes"] * v["n"] for v in per_kernel.values()) / args.steps
+    kernels = kernel_table(per_kernel, args.steps)
+    for label, row in kernels.items():
+        e = table.get(label)
+        if e and e.get("hbm_bytes_per_launch"):
+            row["traffic_GB"] = round(e["hbm_bytes_per_launch"] / 1e9, 3)
+            row["traffic_GBps"] = round(e["hbm_bytes_per_launch"] / (row["avg_ms"] * 1e-3) / 1e9, 1)
+            row["bound"] = e.get("bound")
     info = {
-        "kernels": {kk: {"avg_ms": round(v["ms"] / v["n"], 4), "launches_per_step": v["n"] / args.steps,
-                         "algorithmic_GB": round(v["bytes"] / 1e9, 3),
-                         "GBps_algorithmic": round(v["bytes"] / (v["ms"] / v["n"] * 1e-3) / 1e9, 1)}
-                    for kk, v in per_kernel.items()},
+        "kernels": kernels,
         "path_algorithmic_GB_per_step": round(total_alg / 1e9, 2),
-        "path_GBps_algorithmic": round(total_alg / (ms_per_step * 1e-3) / 1e9, 1),
+        "path_alg_GBps": round(total_alg / (ms_per_step * 1e-3) / 1e9, 1),
+        "first_call_ms": round(first_ms, 1),
         "checksum": int(out.sum().item()),
     }
-    return B * args.steps / elapsed, ms_per_step, roofline, info, model, x
+    return value, ms_per_step, roofline, info, model, x, out
 
 
-def load_traffic(kernel_label):
-    """HBM-side bytes per launch of the dominant kernel from the committed rocprofv3 --pmc summary
-    (profiles/packed_kernel_traffic.json, keyed by the launch label), or None when that launch
-    has not been measured."""
-    p = os.path.join(ROOT, "profiles", "packed_kernel_traffic.json")
-    if os.path.exists(p):
-        with open(p) as f:
-            entry = json.load(f).get(kernel_label)
-        if entry:
-            return entry.get("hbm_bytes_per_launch")
-    return None
-
-
-def cpu_baseline(args, model, x, dl):
-    """The oracle's table-driven C interpreter (same per-word arithmetic as the C the reference
-    generates), one thread, on the first 2^cpu_sample_log2 samples of the batch."""
+def net_tables(model, dl):
     import numpy as np
+    return [(m.indices[0].cpu().numpy(), m.indices[1].cpu().numpy(),
+             m.weights.argmax(-1).to("cpu").numpy().astype(np.uint8)) for m in model if isinstance(m, dl.LogicLayer)]
 
+
+def cpu_baseline(args, model, x, out, dl):
+    """The oracle's table-driven C interpreter (same per-word arithmetic as the C the reference
+    generates), one thread, on the first 2^cpu_sample_log2 samples of the batch; the GPU's
+    full-batch result is compared with it on those samples."""
     from oracle import interp
-    layers = [(m.indices[0].cpu().numpy(), m.indices[1].cpu().numpy(),
-               m.weights.argmax(-1).to("cpu").numpy().astype(np.uint8)) for m in model if isinstance(m, dl.LogicLayer)]
+    layers = net_tables(model, dl)
     n = min(1 << args.cpu_sample_log2, x.shape[0])
     xs = x[:n].cpu().numpy()
     interp.net_eval(xs[:64], layers, 10)            # load the library, touch the tables
     t0 = time.perf_counter()
     want = interp.net_eval(xs, layers, 10, threads=1)
     dt = time.perf_counter() - t0
-    with __import__("torch").no_grad():
-        got = model(dl.PackBitsTensor(x[:n], bit_count=64)).cpu().numpy()
+    got = out[:n].cpu().numpy()
     return {"value": round(n / dt, 1), "unit": "samples/s", "cores": 1, "kind": "port",
             "sample": "first %d of %d samples, same net; oracle/c/packed_interp.c, 1 thread, %.1f s" % (n, x.shape[0], dt),
             "gpu_matches_cpu_on_sample": bool((got == want).all())}
 
 
-def train_bench(args, torch, dl):
-    """fp32 forward + backward of 784 -> 6 x 64000 -> GroupSum(10, tau 30), B = 512, 'unique'
-    connections, grad_factor 1, CrossEntropy.  Reports the whole step (eager and replayed as one
-    HIP graph) and each layer kernel timed alone (back-to-back launches on a 64000 -> 64000 layer,
-    forward and backward_w in their chained form; backward_chained is the single pass the layer
-    runs in place of backward_w + backward_x and is charged the bytes of both)
-    against its algorithmic bytes: forward 4B(in+out)+80 out, backward_w 4B(in+out)+64 out,
-    backward_x 4B(2 in+out)+64 out."""
-    F, width, L, k, B = 784, 64000, 6, 10, 512
+def packed_config(torch, dl, name, F, widths, B, x, check_cpu):
+    """One of the other packed configurations: samples/s, per-launch times, and the first 4096
+    samples of the full-batch result compared with the CPU interpreter."""
+    k = 10
+    model = packed_model(torch, dl, F, widths, k)
+    value, ms, per_kernel, out, first_ms = packed_run(torch, dl, model, x, k, steps=5, warmup=2)
+    W = B // 64
+    dims = [F] + list(widths)
+    alg = sum(eval_layer_bytes(i, o, W) for i, o in zip(dims[:-1], dims[1:])) + 8 * W * dims[-1] + 4 * k * B
+    res = {"workload": name, "dtype": "int64", "samples_per_s": round(value, 1), "ms_per_step": round(ms, 4),
+           "algorithmic_GB_per_step_without_pack": round(alg / 1e9, 2),
+           "alg_over_peak": round(alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+           "first_call_ms": round(first_ms, 1), "kernels": kernel_table(per_kernel, 5),
+           "checksum": int(out.sum().item())}
+    if check_cpu:
+        from oracle import interp
+        n = 4096
+        t0 = time.perf_counter()
+        want = interp.net_eval(x[:n].cpu().numpy(), net_tables(model, dl), k, threads=1)
+        dt = time.perf_counter() - t0
+        res["bit_exact_vs_cpu_interpreter"] = {"samples": n, "equal": bool((out[:n].cpu().numpy() == want).all()),
+                                               "cpu_samples_per_s": round(n / dt, 1)}
+    del model, out
+    return res
+
+
+# ------------------------------------------------------------------------------------------
+# fp32 training
+# ------------------------------------------------------------------------------------------
+
+def train_alg_bytes(dims, B):
+    """forward 4B(in+out)+80 out, backward_w 4B(in+out)+64 out per layer; backward_x 4B(2 in+out)+64 out
+    for every layer but the first."""
+    alg = sum(4 * B * (i + o) + 80 * o + 4 * B * (i + o) + 64 * o for i, o in zip(dims[:-1], dims[1:]))
+    return alg + sum(4 * B * (2 * i + o) + 64 * o for i, o in zip(dims[1:-1], dims[2:]))
+
+
+def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor, x, steps, warmup):
+    """fp32 training step of one configuration with CrossEntropy: forward+backward and
+    forward+backward+Adam(lr 0.01, torch's fused multi-tensor kernel), each eager and replayed as
+    one HIP graph."""
+    from difflogic_amd.graphs import GraphedTrainStep
     torch.manual_seed(0)
     mods, d = [torch.nn.Flatten()], F
-    for _ in range(L):
-        mods.append(dl.LogicLayer(d, width, connections="unique"))
-        d = width
-    model = torch.nn.Sequential(*mods, dl.GroupSum(k, 30.0)).train()
+    for w in widths:
+        mods.append(dl.LogicLayer(d, w, connections=connections, grad_factor=grad_factor))
+        d = w
+    model = torch.nn.Sequential(*mods, dl.GroupSum(k, tau)).train()
     g = torch.Generator(device="cuda").manual_seed(2)
-    x = (torch.rand(B, F, device="cuda", generator=g) < 0.2).float()
     labels = torch.randint(0, k, (B,), device="cuda", generator=g)
     loss_fn = torch.nn.CrossEntropyLoss()
-    steps, warmup = max(5, args.steps), max(3, args.warmup)
+    neuron_samples = sum(widths) * B
+    alg = train_alg_bytes([F] + list(widths), B)
 
-    def step():
+    def timeit(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            last = fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps, last
+
+    def report(sec, loss):
+        return {"neuron_samples_per_s": round(neuron_samples / sec, 1), "ms_per_step": round(sec * 1e3, 4),
+                "alg_GBps": round(alg / sec / 1e9, 1), "frac_hbm_algorithmic": round(alg / sec / 1e9 / HBM_PEAK_GBS, 4),
+                "loss": round(float(loss), 6)}
+
+    def fwd_bwd():
         model.zero_grad(set_to_none=True)
         loss = loss_fn(model(x), labels)
         loss.backward()
         return loss
 
-    for _ in range(warmup):
-        step()
+    res = {"workload": name, "dtype": "f32", "algorithmic_GB_per_step": round(alg / 1e9, 3)}
+    sec, loss = timeit(fwd_bwd)
+    res["fwd_bwd_eager"] = report(sec, loss.item())
+    # Drop every reference to the eager autograd graph before capturing: gradient-accumulation
+    # nodes kept alive by `loss` belong to the default stream and would be replayed into the
+    # capture stream's backward.
+    del loss
+    model.zero_grad(set_to_none=True)
+    gc.collect()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        loss = step()
-    torch.cuda.synchronize()
-    eager = (time.perf_counter() - t0) / steps
-    eager_loss = loss.item()
+    graphed = GraphedTrainStep(model, loss_fn, x, labels)
+    sec, loss = timeit(graphed.step)
+    res["fwd_bwd_graph"] = report(sec, loss.item())
+    del graphed, loss
+    gc.collect()
 
-    # each layer kernel alone, 20 launches back to back on one square layer
+    # with the optimizer step (experiments/main.py:169,174-181).  The weights move, so the loss differs per step.
+    opt = torch.optim.Adam(model.parameters(), lr=0.01, fused=True, capturable=True)
+
+    def full_step():
+        opt.zero_grad(set_to_none=True)
+        loss = loss_fn(model(x), labels)
+        loss.backward()
+        opt.step()
+        return loss
+
+    sec, loss = timeit(full_step)
+    res["fwd_bwd_adam_eager"] = report(sec, loss.item())
+    del loss
+    opt.zero_grad(set_to_none=True)
+    gc.collect()
+    torch.cuda.synchronize()
+    graphed = GraphedTrainStep(model, loss_fn, x, labels, optimizer=opt)
+    sec, loss = timeit(graphed.step)
+    res["fwd_bwd_adam_graph"] = report(sec, loss.item())
+    del graphed, loss, opt
+    gc.collect()
+    return res, model
+
+
+def train_kernels_alone(torch, dl, model, B, width):
+    """Each layer kernel timed alone (back-to-back launches on a 64000 -> 64000 layer, forward and
+    backward_w in their chained form; backward_chained is the single pass the layer runs in place
+    of backward_w + backward_x and is charged the bytes of both) against its algorithmic bytes."""
     ext = dl.difflogic_cuda
+    g = torch.Generator(device="cuda").manual_seed(3)
     layer = model[2]
     a, b = layer.indices
     xs = torch.rand(width, B, device="cuda", generator=g)
@@ -236,7 +425,6 @@ def train_bench(args, torch, dl):
         "forward_logits": (lambda: ext.forward_logits(xs, a, b, logits, sched), 4 * B * 2 * width + 80 * width),
         "backward_logits": (lambda: ext.backward_logits(xs, a, b, gy, probs, sched), 4 * B * 2 * width + 64 * width),
         "backward_x": (lambda: ext.backward_x(xs, a, b, probs, gy, start, idx), 4 * B * 3 * width + 64 * width),
-        # backward_logits + backward_x in one pass (what the layer runs when both gradients are needed)
         "backward_chained": (lambda: ext.backward_chained(xs, probs, gy, sched, 1.0, softmax_backward=True),
                              4 * B * 5 * width + 128 * width),
     }
@@ -251,43 +439,9 @@ def train_bench(args, torch, dl):
         e.record()
         torch.cuda.synchronize()
         us = s.elapsed_time(e) / 20 * 1e3
-        kernels[name] = {"us_per_launch": round(us, 2), "GBps_algorithmic": round(by / (us * 1e-6) / 1e9, 1),
-                         "frac_hbm": round(by / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
-    del xs, gy
-
-    # Drop every reference to the eager autograd graph before capturing: gradient-accumulation
-    # nodes kept alive by `loss` belong to the default stream and would be replayed into the
-    # capture stream's backward.
-    del loss
-    model.zero_grad(set_to_none=True)
-    import gc
-    gc.collect()
-    torch.cuda.synchronize()
-    from difflogic_amd.graphs import GraphedTrainStep
-    graphed = GraphedTrainStep(model, loss_fn, x, labels)
-    for _ in range(warmup):
-        graphed.step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        gl = graphed.step()
-    torch.cuda.synchronize()
-    replay = (time.perf_counter() - t0) / steps
-
-    dims = [F] + [width] * L
-    alg = sum(4 * B * (i + o) + 80 * o + 4 * B * (i + o) + 64 * o for i, o in zip(dims[:-1], dims[1:]))
-    alg += sum(4 * B * (2 * i + o) + 64 * o for i, o in zip(dims[1:-1], dims[2:]))     # no backward_x for layer 1
-    neuron_samples = L * width * B
-    return {
-        "workload": "fp32 fwd+bwd 784->6x64000->GroupSum(10,tau=30), B=512, connections=unique, CrossEntropy",
-        "dtype": "f32", "algorithmic_GB_per_step": round(alg / 1e9, 3),
-        "graph_replay": {"neuron_samples_per_s": round(neuron_samples / replay, 1), "ms_per_step": round(replay * 1e3, 4),
-                         "GBps_algorithmic": round(alg / replay / 1e9, 1),
-                         "frac_hbm": round(alg / replay / 1e9 / HBM_PEAK_GBS, 4), "loss": round(gl.item(), 6)},
-        "eager": {"neuron_samples_per_s": round(neuron_samples / eager, 1), "ms_per_step": round(eager * 1e3, 4),
-                  "loss": round(eager_loss, 6)},
-        "kernels_alone_64000x64000": kernels,
-    }
+        kernels[name] = {"us_per_launch": round(us, 2), "alg_GBps": round(by / (us * 1e-6) / 1e9, 1),
+                         "frac_hbm_algorithmic": round(by / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+    return kernels
 
 
 def train_cpu_baseline(torch):
@@ -333,6 +487,71 @@ def train_cpu_baseline(torch):
                                 "s_per_step": round(all_threads, 4)}}
 
 
+# ------------------------------------------------------------------------------------------
+# practical ceilings
+# ------------------------------------------------------------------------------------------
+
+def ceilings(torch):
+    """Streaming read / write / copy over 8 GiB buffers and row gathers with the gate kernels'
+    access pattern (64 lanes x 16 bytes per gathered row, column-tile-major dispatch) from an
+    input that stays L2-resident per column tile (784 rows) and from one that does not (64000
+    rows, served by the fabric / Infinity Cache).  GB/s, best of the grid sizes tried."""
+    from difflogic_amd import build
+    lib = ctypes.CDLL(build.CEILINGS_LIB_PATH)
+    vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    lib.dlc_stream.argtypes = [i32, vp, vp, i64, i32, vp]
+    lib.dlc_gather.argtypes = [vp, vp, i64, i64, i32, vp, vp]
+    stream = vp(torch.cuda.current_stream().cuda_stream)
+
+    def timed(fn, iters):
+        for _ in range(2):
+            fn()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(iters):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) / iters * 1e-3
+
+    nbytes = 8 << 30                            # also holds the 64000 x 128 KB matrix of the gather test
+    a = torch.empty(nbytes, dtype=torch.uint8, device="cuda").fill_(1)
+    b = torch.empty(nbytes, dtype=torch.uint8, device="cuda").fill_(2)
+    res = {"buffer_GiB": nbytes >> 30}
+    for mode, key, moved in ((0, "stream_read", nbytes), (1, "stream_write", nbytes), (2, "stream_copy", 2 * nbytes)):
+        best = {}
+        for grid in (2048, 8192, 32768):
+            def fn():
+                st = lib.dlc_stream(mode, vp(a.data_ptr()), vp(b.data_ptr()), nbytes, grid, stream)
+                assert st == 0, st
+            best[grid] = round(moved / timed(fn, 5) / 1e9, 1)
+        res[key + "_GBps"] = max(best.values())
+        res[key + "_by_grid"] = best
+    t = timed(lambda: b[:1 << 30].copy_(a[:1 << 30]), 5)
+    res["runtime_copy_1GiB_GBps"] = round(2 * (1 << 30) / t / 1e9, 1)
+    del b
+
+    W = 16384                                   # row = 128 KB, as in the headline workload
+    out_rows = 64000
+    g = torch.Generator(device="cuda").manual_seed(0)
+    sink = torch.zeros(16, dtype=torch.uint8, device="cuda")
+    for rows, key in ((784, "gather_l2_resident_784_rows"), (64000, "gather_fabric_64000_rows")):
+        assert rows * W * 8 <= a.numel(), "the gathered matrix must fit the buffer"
+        x = a[:rows * W * 8]
+        for gathers in (2, 4, 8):
+            if rows == 64000 and gathers == 8:
+                continue
+            idx = torch.randint(0, rows, (out_rows * gathers,), device="cuda", generator=g, dtype=torch.int32)
+            assert 0 <= int(idx.min()) and int(idx.max()) < rows and x.numel() == rows * W * 8
+
+            def fn():
+                st = lib.dlc_gather(vp(x.data_ptr()), vp(idx.data_ptr()), out_rows, W * 8, gathers, vp(sink.data_ptr()), stream)
+                assert st == 0, st
+            sec = timed(fn, 3)
+            res["%s_x%d_GBps" % (key, gathers)] = round(out_rows * gathers * W * 8 / sec / 1e9, 1)
+    return res
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -344,6 +563,11 @@ def main():
     import difflogic_amd as dl
     assert torch.cuda.is_available(), "bench.py needs the GPU"
 
+    if args.ceilings:
+        print(json.dumps({"metric": "practical ceilings on this GPU", "unit": "GB/s", "hbm_peak_GBps": HBM_PEAK_GBS,
+                          "device": torch.cuda.get_device_name(0), **ceilings(torch)}))
+        return
+
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
         dst = torch.empty_like(src)
@@ -351,7 +575,7 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    value, ms, roofline, info, model, x = packed_bench(args, torch, dl)
+    value, ms, roofline, info, model, x, out = packed_headline(args, torch, dl)
     result = {
         "metric": "packed-eval samples/s (784->6x64k)", "value": round(value, 1), "unit": "samples/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
@@ -362,14 +586,57 @@ def main():
                    "connections": "random", "seed": 0},
         "roofline": roofline,
     }
-    result["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(args, model, x, dl)
+    result["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(args, model, x, out, dl)
     extra = dict(info)
-    del model, x
+    del model, x, out
+    gc.collect()
     torch.cuda.empty_cache()
-    if not args.no_train:
-        extra["train"] = train_bench(args, torch, dl)
+
+    only = {c for c in args.only.lower().split(",") if c}
+    want = lambda c, group_off: (c in only) if only else not group_off      # noqa: E731
+    configs = {}
+    check = not args.no_cpu_baseline
+    if want("c2", args.no_configs):
+        B = 1 << 20
+        configs["C2"] = packed_config(torch, dl, "packed inference 784->6x8000->GroupSum(10), batch 2^20, int64 words",
+                                      784, [8000] * 6, B, bernoulli_input(torch, B, 784, 1), check)
+        torch.cuda.empty_cache()
+    if want("c4", args.no_configs):
+        B = 1 << 18
+        configs["C4"] = packed_config(torch, dl, "packed inference 9216->4x256000->GroupSum(10), batch 2^18, int64 words, "
+                                      "thresholded-uniform input", 9216, [256000] * 4, B, thresholded_input(torch, B, 1),
+                                      check)
+        torch.cuda.empty_cache()
+    steps, warmup = max(5, args.steps), max(3, args.warmup)
+    if want("c3", args.no_train):
+        B = 512
+        x = bernoulli_input(torch, B, 784, 2).float()
+        configs["C3"], model = train_config(
+            torch, dl, "fp32 train 784->6x64000->GroupSum(10,tau=30), B=512, connections=unique, CrossEntropy",
+            784, [64000] * 6, 10, 30.0, B, "unique", 1.0, x, steps, warmup)
+        configs["C3"]["kernels_alone_64000x64000"] = train_kernels_alone(torch, dl, model, B, 64000)
+        del model, x
+        gc.collect()
+        torch.cuda.empty_cache()
+    if want("c5", args.no_train):
+        B = 1024
+        x = thresholded_input(torch, B, 2, as_float=True)
+        configs["C5"], model = train_config(
+            torch, dl, "fp32 train 9216->12x128000->GroupSum(10,tau=100), B=1024, connections=random, grad_factor=2, "
+            "thresholded-uniform input, CrossEntropy", 9216, [128000] * 12, 10, 100.0, B, "random", 2.0, x, steps, warmup)
+        del model, x
+        gc.collect()
+        torch.cuda.empty_cache()
+    if want("c1", args.no_train):
+        B = 128
+        x = bernoulli_input(torch, B, 784, 2).float()
+        configs["C1"], model = train_config(
+            torch, dl, "fp32 train 784->4x8000->GroupSum(10,tau=10), B=128, connections=random, CrossEntropy",
+            784, [8000] * 4, 10, 10.0, B, "random", 1.0, x, max(steps, 50), warmup)
+        del model, x
         if not args.no_cpu_baseline:
-            extra["train"]["cpu_baseline"] = train_cpu_baseline(torch)
+            configs["C1"]["cpu_baseline"] = train_cpu_baseline(torch)
+    extra["configs"] = configs
     result["extra"] = extra
     print(json.dumps(result))
 

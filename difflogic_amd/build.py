@@ -13,6 +13,10 @@ INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB_NAME = "libdifflogic_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
 SOURCES = ("packed.hip", "train.hip", "schedule.cpp")
+# streaming / gather microbenchmarks for `bench.py --ceilings`: a library of their own, never
+# loaded by the package
+CEILINGS_LIB_PATH = os.path.join(HERE, "libdl_ceilings.so")
+CEILINGS_SOURCES = ("ceilings.hip",)
 
 HIPCC_FLAGS = (
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared", "-fvisibility=default",
@@ -31,9 +35,16 @@ def hipcc_path():
 
 
 def build_library(verbose=False):
-    """Compiles every kernel source into one shared library next to this file."""
+    """Compiles every kernel source into one shared library next to this file, and the
+    measurement helpers into a second one."""
+    _compile(SOURCES, LIB_PATH, verbose)
+    _compile(CEILINGS_SOURCES, CEILINGS_LIB_PATH, verbose)
+    return LIB_PATH
+
+
+def _compile(sources, out_path, verbose):
     cmd = [hipcc_path(), *HIPCC_FLAGS, f"-I{INCLUDE}", f"-I{CSRC}",
-           *[os.path.join(CSRC, s) for s in SOURCES], "-o", LIB_PATH + ".tmp"]
+           *[os.path.join(CSRC, s) for s in sources], "-o", out_path + ".tmp"]
     if verbose:
         print(" ".join(cmd))
     proc = subprocess.run(cmd, capture_output=True, text=True)
@@ -44,8 +55,8 @@ def build_library(verbose=False):
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
-    os.replace(LIB_PATH + ".tmp", LIB_PATH)
-    return LIB_PATH
+    os.replace(out_path + ".tmp", out_path)
+    return out_path
 
 
 if __name__ == "__main__":
