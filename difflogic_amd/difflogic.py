@@ -131,13 +131,9 @@ class LogicLayer(torch.nn.Module):
         return difflogic_cuda.schedule_for(self.indices[0], self.indices[1], self.in_dim)
 
     def _gate_ids(self):
-        """uint8 [out_dim] argmax gate per neuron, recomputed only when ``weights`` changed."""
-        key = (self.weights.data_ptr(), self.weights._version)
-        cached = getattr(self, "_gate_ids_cache", None)
-        if cached is None or cached[0] != key:
-            cached = (key, self.weights.detach().argmax(-1).to(torch.uint8))
-            self._gate_ids_cache = cached
-        return cached[1]
+        """uint8 [out_dim] argmax gate per neuron.  Recomputed on every call like the reference
+        (difflogic/difflogic.py:146): a cache could not see writes through ``weights.data``."""
+        return self.weights.detach().argmax(-1).to(torch.uint8)
 
     def extra_repr(self):
         return "{}, {}, {}".format(self.in_dim, self.out_dim, "train" if self.training else "eval")

@@ -459,7 +459,6 @@ class EvalSchedule:
         self.verts = torch.from_numpy(verts[:steps + 1].copy()).to(a.device)
         self.neuron = torch.from_numpy(neuron[:steps].copy()).to(a.device)
         self.flip = torch.from_numpy(flip[:steps].copy()).to(a.device)
-        self._wiring = (a, b)        # keeps the tensors (and their addresses) alive while cached
         self._host = (verts[:steps + 1].copy(), neuron[:steps].copy())
         self._backward = None
 
@@ -488,21 +487,55 @@ class EvalSchedule:
         return self._backward
 
 
-_SCHEDULES = {}                      # (ptr a, ptr b, versions, in_dim) -> EvalSchedule, most recent last
-_SCHEDULES_MAX = 64
+class _WiringCache:
+    """Results derived from wiring tensors (schedules, count orders), kept only while those
+    tensors are alive: an entry holds weak references to its tensors and is dropped when one of
+    them is collected, so a freed tensor's address can never be mistaken for a new tensor at the
+    same address, and nothing is pinned beyond the wiring's own lifetime.  The key also carries
+    the tensors' version counters, so in-place edits of the wiring rebuild the entry (writes
+    through ``.data`` are invisible to the counter: replace the tensors instead).  Thread-safe."""
+
+    def __init__(self):
+        import threading
+        self._lock = threading.Lock()
+        self._entries = {}
+
+    def get(self, tensors, extra, build):
+        import weakref
+        key = tuple((t.data_ptr(), t._version, t.shape[0]) for t in tensors) + tuple(extra)
+        with self._lock:
+            hit = self._entries.get(key)
+            if hit is not None and all(r() is t for r, t in zip(hit[0], tensors)):
+                return hit[1]
+        value = build()
+
+        def drop(_ref, key=key, cache=weakref.ref(self)):
+            me = cache()
+            if me is not None:
+                with me._lock:
+                    me._entries.pop(key, None)
+
+        with self._lock:
+            # stale versions of the same tensors go: one entry per set of live tensors
+            n = len(tensors)
+            same = lambda k: (len(k) == len(key) and k[n:] == key[n:]                           # noqa: E731
+                              and all(u[0] == v[0] for u, v in zip(k[:n], key[:n])))
+            for old in [k for k in self._entries if same(k)]:
+                del self._entries[old]
+            self._entries[key] = (tuple(weakref.ref(t, drop) for t in tensors), value)
+        return value
+
+    def __len__(self):
+        return len(self._entries)
+
+
+_SCHEDULES = _WiringCache()
 
 
 def schedule_for(a, b, in_dim):
-    """The cached EvalSchedule of the wiring (a, b), rebuilt when the tensors are replaced or
-    modified in place."""
-    key = (a.data_ptr(), b.data_ptr(), a._version, b._version, int(in_dim), a.shape[0])
-    sched = _SCHEDULES.pop(key, None)
-    if sched is None:
-        sched = EvalSchedule(a, b, in_dim)
-        while len(_SCHEDULES) >= _SCHEDULES_MAX:
-            _SCHEDULES.pop(next(iter(_SCHEDULES)))
-    _SCHEDULES[key] = sched
-    return sched
+    """The cached EvalSchedule of the wiring (a, b): lives as long as the tensors do, rebuilt when
+    they are replaced or modified in place."""
+    return _SCHEDULES.get((a, b), (int(in_dim),), lambda: EvalSchedule(a, b, in_dim))
 
 
 def eval_chained(x, layers, schedule=None):
@@ -534,20 +567,18 @@ def eval_chained(x, layers, schedule=None):
     return y
 
 
-_COUNT_ORDERS = {}                   # wiring tensors + k -> device order, most recent last
-_COUNT_ORDERS_MAX = 16
+_COUNT_ORDERS = _WiringCache()
 
 
 def count_order_for(layers, in_dim, k):
     """Cached neuron order for eval_fused_groupbitsum over ``layers`` (the net's last one or two
     layers, [(a, b, w), ...]): neurons of a class that read the same input rows are walked by
-    the same workgroup.  Built on the host from the wiring alone; rebuilt when the index tensors
-    are replaced or modified."""
-    import numpy as np
+    the same workgroup.  Built on the host from the wiring alone; lives as long as the index
+    tensors do and is rebuilt when they are replaced or modified in place."""
     idx = [t for a, b, _ in layers for t in (a, b)]
-    key = tuple((t.data_ptr(), t._version, t.shape[0]) for t in idx) + (int(in_dim), int(k))
-    hit = _COUNT_ORDERS.pop(key, None)
-    if hit is None:
+
+    def build():
+        import numpy as np
         lib = _lib.load()
         host = [np.ascontiguousarray(t.detach().cpu().numpy(), dtype=np.int64) for t in idx]
         out_dim = host[-1].shape[0]
@@ -561,11 +592,9 @@ def count_order_for(layers, in_dim, k):
                                       lib.dl_count_group(), order.ctypes.data)
         if st:
             _raise(st, "count_order_build")
-        hit = (torch.from_numpy(order).to(idx[0].device), idx)      # idx keeps the keyed tensors alive
-        while len(_COUNT_ORDERS) >= _COUNT_ORDERS_MAX:
-            _COUNT_ORDERS.pop(next(iter(_COUNT_ORDERS)))
-    _COUNT_ORDERS[key] = hit
-    return hit[0]
+        return torch.from_numpy(order).to(idx[0].device)
+
+    return _COUNT_ORDERS.get(tuple(idx), (int(in_dim), int(k)), build)
 
 
 def eval_fused_groupbitsum(x, layers, pad_len, k, order=None):

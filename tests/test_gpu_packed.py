@@ -352,3 +352,24 @@ def test_schedule_follows_in_place_wiring_changes():
     with torch.no_grad():
         got2 = model(dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=64)).cpu().numpy()
     assert np.array_equal(got2, interp.net_eval(x, layers2, 10, threads=4))
+
+
+def test_packed_inference_follows_weight_writes_through_data():
+    """``layer.weights.data.copy_(...)`` (no version bump) between two packed evaluations: the second
+    one uses the new gates."""
+    import difflogic_amd as dl
+    rng = np.random.default_rng(12)
+    F = 40
+    layers = random_layers(rng, F, [80, 80, 60])
+    x = rng.random((200, F)) < 0.5
+    model = build_model(F, layers, 10).eval()
+    xd = torch.as_tensor(x).cuda()
+    with torch.no_grad():
+        got = model(dl.PackBitsTensor(xd, bit_count=64)).cpu().numpy()
+    assert np.array_equal(got, interp.net_eval(x, layers, 10))
+    layers2 = [(a, b, ((op.astype(np.int64) * 7 + 3) % 16).astype(np.uint8)) for a, b, op in layers]
+    for m, (_, _, op) in zip([model[1], model[2], model[3]], layers2):
+        m.weights.data.copy_(torch.nn.functional.one_hot(torch.as_tensor(op).long(), 16).float())
+    with torch.no_grad():
+        got2 = model(dl.PackBitsTensor(xd, bit_count=64)).cpu().numpy()
+    assert np.array_equal(got2, interp.net_eval(x, layers2, 10))

@@ -2,15 +2,17 @@
 restated on CPU).
 
 Tolerance: fp32 results must satisfy |got - want| <= 1e-5 * max|want| + 1e-5 * |want|
-(1e-5 relative, with the tensor's scale as the floor for entries that cancel to ~0).  The
-oracle value is computed in fp32 like the reference's python implementation; an fp64 oracle
-run bounds both."""
+(1e-5 relative, with the tensor's scale as the floor for entries that cancel to ~0) against the
+python implementation evaluated in fp64.  Gradients that are long fp32 sums are held to the
+error budget of tests.helpers.within_budget instead: the same bound, or the distance of the
+fp32 python implementation itself from the fp64 value on the same case, whichever is larger.
+No test widens the 1e-5 beyond that."""
 import numpy as np
 import pytest
 import torch
 
 from oracle import float_oracle as fo
-from tests.helpers import build_model, random_layers
+from tests.helpers import build_model, random_layers, within_budget
 
 pytestmark = pytest.mark.gpu
 
@@ -164,26 +166,31 @@ def test_train_step_matches_python_implementation(conn, grad_factor, batch):
     x = (torch.rand(batch, F) < 0.2).float()
     labels = torch.randint(0, k, (batch,))
 
-    logits = [l.weights.detach().cpu().clone().requires_grad_(True) for l in layers]
-    oracle = fo.PythonNet([(l.indices[0].cpu(), l.indices[1].cpu(), lg) for l, lg in zip(layers, logits)], k, tau,
-                          grad_factor)
-    xo = x.clone().requires_grad_(True)
-    want_out = oracle(xo, training=True)
-    want_loss = torch.nn.functional.cross_entropy(want_out, labels)
-    want_loss.backward()
+    def python_impl(dtype):
+        """(logits, loss, [grad per layer], grad_x) of the CPU python implementation in ``dtype``."""
+        lg = [l.weights.detach().cpu().to(dtype).requires_grad_(True) for l in layers]
+        net = fo.PythonNet([(l.indices[0].cpu(), l.indices[1].cpu(), w) for l, w in zip(layers, lg)], k, tau, grad_factor)
+        xo = x.detach().clone().to(dtype).requires_grad_(True)
+        out = net(xo, training=True)
+        loss = torch.nn.functional.cross_entropy(out, labels)
+        loss.backward()
+        return out.detach(), loss.detach(), [w.grad for w in lg], xo.grad
 
-    xg = x.cuda().requires_grad_(True)
+    out32, loss32, gw32, gx32 = python_impl(torch.float32)
+    out64, loss64, gw64, gx64 = python_impl(torch.float64)
+
+    xg = x.detach().cuda().requires_grad_(True)
     got_out = model(xg)
     got_loss = torch.nn.functional.cross_entropy(got_out, labels.cuda())
     got_loss.backward()
 
-    assert close(got_out, want_out)[0]
-    assert abs(got_loss.item() - want_loss.item()) <= RTOL * abs(want_loss.item())
-    for l, lg in zip(layers, logits):
-        ok, err = close(l.weights.grad, lg.grad, 2e-5)
-        assert ok, err
-    ok, err = close(xg.grad, xo.grad, 2e-5)
-    assert ok, err
+    assert close(got_out, out64)[0] and close(got_out, out32)[0]
+    assert abs(got_loss.item() - loss64.item()) <= RTOL * abs(loss64.item())
+    for l, w64, w32 in zip(layers, gw64, gw32):
+        ok, rep = within_budget(l.weights.grad, w64, w32)
+        assert ok, rep
+    ok, rep = within_budget(xg.grad, gx64, gx32)
+    assert ok, rep
 
 
 def test_eval_mode_and_state_dict_round_trip():
@@ -261,8 +268,15 @@ def test_logits_entry_points(ext, dtype, rtol, in_dim, out_dim, batch):
     yy = fo.layer_forward_sequential(xq.double().t(), a, b, torch.softmax(lw, -1))
     want_g, = torch.autograd.grad(yy, lw, gq.double().t())
     got_g = ext.backward_logits(xq.cuda(), a.cuda(), b.cuda(), gq.cuda(), probs)
-    ok, err = close(got_g, want_g, 2 * rtol)
-    assert ok, err
+    if dtype == torch.float32:            # the python formulation in fp32 sets the budget
+        l32 = lq.clone().requires_grad_(True)
+        y32 = fo.layer_forward_sequential(xq.t(), a, b, torch.softmax(l32, -1))
+        ref_g, = torch.autograd.grad(y32, l32, gq.t())
+        ok, rep = within_budget(got_g, want_g, ref_g)
+        assert ok, rep
+    else:
+        ok, err = close(got_g, want_g, rtol)
+        assert ok, err
     assert torch.equal(got_g, ext.backward_logits(xq.cuda(), a.cuda(), b.cuda(), gq.cuda(), probs))
 
 
@@ -395,7 +409,14 @@ def test_layer_uses_schedule_for_wide_inputs():
     wr = wide.weights.detach().cpu().double().requires_grad_()
     fo.layer_forward_sequential(xr, wide.indices[0].cpu(), wide.indices[1].cpu(),
                                 torch.softmax(wr, -1)).square().sum().backward()
-    assert close(x.grad, xr.grad, 1e-4)[0] and close(wide.weights.grad, wr.grad, 1e-4)[0]
+    x32 = x.detach().cpu().requires_grad_()
+    w32 = wide.weights.detach().cpu().requires_grad_()
+    fo.layer_forward_sequential(x32, wide.indices[0].cpu(), wide.indices[1].cpu(),
+                                torch.softmax(w32, -1)).square().sum().backward()
+    ok, rep = within_budget(x.grad, xr.grad, x32.grad)
+    assert ok, rep
+    ok, rep = within_budget(wide.weights.grad, wr.grad, w32.grad)
+    assert ok, rep
     # eval mode on float inputs takes the chained forward too: exact 0/1 results of the discretised gates
     wide.eval()
     xb = (torch.rand(64, 5000, device="cuda") < 0.5).float()
@@ -438,7 +459,46 @@ def test_chained_layer_matches_the_python_formulation_on_random_wirings(monkeypa
         wr = layer.weights.detach().cpu().double().requires_grad_()
         yr = fo.layer_forward_sequential(xr, a, b, torch.softmax(wr, -1))
         (yr * gy.double()).sum().backward()
+        x32 = x.detach().cpu().requires_grad_()
+        w32 = layer.weights.detach().cpu().requires_grad_()
+        (fo.layer_forward_sequential(x32, a, b, torch.softmax(w32, -1)) * gy).sum().backward()
         tag = (case, in_dim, out_dim, batch, kind)
         assert close(y, yr)[0], tag
-        assert close(layer.weights.grad, wr.grad, 2 * RTOL)[0], tag
-        assert close(x.grad, grad_factor * xr.grad, 2 * RTOL)[0], tag
+        ok, rep = within_budget(layer.weights.grad, wr.grad, w32.grad)
+        assert ok, (tag, rep)
+        ok, rep = within_budget(x.grad, grad_factor * xr.grad, grad_factor * x32.grad)
+        assert ok, (tag, rep)
+
+
+@pytest.mark.parametrize("dtype,rtol", [(torch.float16, 4e-3), (torch.float64, 1e-5)])
+def test_layer_module_with_half_and_double_activations(dtype, rtol):
+    """The reference's --training-bit-count 16 / 64 (experiments/main.py:19-23,286): the input is
+    cast to half / double while the weights stay fp32, so LogicLayer takes the
+    softmax-in-torch + LogicLayerCudaFunction route (difflogic/difflogic.py:123-126,205-221).
+    Outputs and both gradients against the same formulation on CPU (fp64 arithmetic on the
+    values as rounded to ``dtype``, the fp32 softmax and the casts as autograd sees them)."""
+    import difflogic_amd as dl
+    torch.manual_seed(5)
+    in_dim, out_dim, batch = 48, 120, 264
+    layer = dl.LogicLayer(in_dim, out_dim, grad_factor=1.5).train()
+    a, b = layer.indices[0].cpu(), layer.indices[1].cpu()
+    g = torch.Generator().manual_seed(6)
+    x = torch.rand(batch, in_dim, generator=g).to(dtype)
+    gy = torch.randn(batch, out_dim, generator=g).to(dtype)
+
+    xg = x.cuda().requires_grad_()
+    y = layer(xg)
+    assert y.dtype == dtype and y.shape == (batch, out_dim)
+    (y * gy.cuda()).sum().backward()
+    assert layer.weights.grad.dtype == torch.float32 and xg.grad.dtype == dtype
+
+    w32 = layer.weights.detach().cpu().requires_grad_()
+    xr = x.double().requires_grad_()
+    wq = torch.softmax(w32, -1).to(dtype).double()
+    yr = fo.layer_forward_sequential(xr, a, b, wq)
+    (yr * gy.double()).sum().backward()
+    assert close(y, yr.to(dtype), rtol)[0]
+    ok, err = close(xg.grad, 1.5 * xr.grad, rtol)
+    assert ok, err
+    ok, err = close(layer.weights.grad, w32.grad, rtol)
+    assert ok, err

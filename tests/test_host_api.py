@@ -121,3 +121,48 @@ def test_group_planner():
     # a wide net over few inputs: deep first group (its gathers hit in L2), pairs afterwards
     assert plan_groups([784] + [64000] * 6, True)[0] >= 3
     assert plan_groups([64000] * 5, False) == [2, 2]
+
+
+def test_gate_ids_follow_writes_through_data():
+    """The packed path's gate ids are the argmax of the weights as they are now: writes through
+    ``weights.data`` do not bump the tensor's version counter, so nothing may be cached on it."""
+    torch.manual_seed(3)
+    layer = dl.LogicLayer(12, 20, device="cpu")
+    before = layer._gate_ids()
+    assert before.dtype == torch.uint8 and torch.equal(before.long(), layer.weights.detach().argmax(-1))
+    version = layer.weights._version
+    new_ids = (before.long() + 5) % 16
+    layer.weights.data.copy_(torch.nn.functional.one_hot(new_ids, 16).float())
+    assert layer.weights._version == version                       # the write was invisible to autograd ...
+    assert torch.equal(layer._gate_ids().long(), new_ids)          # ... and still shows
+    layer.weights.data[0, :] = 0
+    layer.weights.data[0, 9] = 1
+    assert int(layer._gate_ids()[0]) == 9
+
+
+def test_wiring_cache_lives_and_dies_with_its_tensors():
+    import gc
+
+    from difflogic_amd.difflogic_cuda import _WiringCache
+    cache = _WiringCache()
+    a, b = torch.arange(6), torch.arange(6)
+    built = []
+
+    def build():
+        built.append(len(built))
+        return object()
+
+    v = cache.get((a, b), (7,), build)
+    assert cache.get((a, b), (7,), build) is v and built == [0]
+    assert cache.get((a, b), (8,), build) is not v and len(cache) == 2       # another in_dim: another entry
+    a[0] = 3                                                                 # in-place edit: rebuilt, old entry gone
+    v2 = cache.get((a, b), (7,), build)
+    assert v2 is not v and len(cache) == 2
+    c = a.clone()                                                            # equal values, other tensor
+    assert cache.get((c, b), (7,), build) is not v2 and len(cache) == 3
+    del a, c
+    gc.collect()
+    assert len(cache) == 0                                                   # nothing outlives the wiring
+    # a new tensor that happens to reuse a freed address is never served a dead tensor's entry
+    a = torch.arange(6)
+    assert cache.get((a, b), (7,), build) is not v2
