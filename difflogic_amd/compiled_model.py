@@ -165,14 +165,15 @@ void apply_logic_gate_net(bool const *inp, int *out, size_t len) {{
         gate_fn += [f"\tcase {i}: return (T) ({e});" for i, e in enumerate(_GATE_EXPR[:15])]
         gate_fn += ["\tdefault: return (T) ~(T) 0;", "\t}", "}", ""]
         widest = max(widths)
-        body += [f"\tT *cur = malloc(sizeof(T) * {widest}), *nxt = malloc(sizeof(T) * {widest}), *tmp;",
-                 "\tT const *src = inp;"]
+        # the two layer buffers are per-thread statics: no allocation per block of samples
+        body += [f"\tstatic __thread T buf0[{widest}], buf1[{widest}];",
+                 "\tT *cur = buf0, *nxt = buf1, *tmp;", "\tT const *src = inp;"]
         for li, w in enumerate(widths):
             dst = "out" if li == len(widths) - 1 else "nxt"
             body.append(f"\tfor (int n = 0; n < {w}; ++n) {dst}[n] = gate(src[A{li}[n]], src[B{li}[n]], G{li}[n]);")
             if li != len(widths) - 1:
                 body.append("\ttmp = cur; cur = nxt; nxt = tmp; src = cur;")
-        body += ["\tfree(cur);", "\tfree(nxt);", "}"]
+        body += ["}"]
         return "\n".join(head + tables + [""] + gate_fn + body) + self._driver_code()
 
     # ------------------------------------------------------------------ build / load / call
@@ -189,8 +190,10 @@ void apply_logic_gate_net(bool const *inp, int *out, size_t len) {{
         ``apply_logic_gate_net``; ``save_lib_path`` keeps a copy of the shared library."""
         assert self.device == "cpu", "Device {} not supported.".format(self.device)
         code = self.get_c_code()
-        self._lib_dir = tempfile.mkdtemp(prefix="difflogic_amd_compiled_")
-        c_path, so_path = os.path.join(self._lib_dir, "net.c"), os.path.join(self._lib_dir, "net.so")
+        # held on the object (replacing the directory of an earlier compile()) and removed with it;
+        # the bound library stays usable after the file is gone
+        self._lib_dir = tempfile.TemporaryDirectory(prefix="difflogic_amd_compiled_")
+        c_path, so_path = os.path.join(self._lib_dir.name, "net.c"), os.path.join(self._lib_dir.name, "net.so")
         with open(c_path, "w") as f:
             f.write(code)
         if verbose:

@@ -159,12 +159,18 @@ class GroupSum(torch.nn.Module):
         self.tau = tau
         self.device = device
 
+    # grid limits of dl_group_sum_forward / dl_group_sum_backward (one grid row per class, one per 64
+    # neurons); beyond them the torch formulation below runs, in forward and backward alike
+    _HIP_MAX_K = 65535
+    _HIP_MAX_OUT_DIM = 65535 * 64
+
     def forward(self, x):
         if isinstance(x, PackBitsTensor):
             return x.group_sum(self.k)
         assert x.shape[-1] % self.k == 0, (x.shape, self.k)
         if (x.is_cuda and x.dim() == 2 and x.dtype in (torch.float16, torch.float32, torch.float64)
-                and x.numel() > 0 and x.stride(0) == 1 and x.stride(1) == x.shape[0]):
+                and x.numel() > 0 and x.stride(0) == 1 and x.stride(1) == x.shape[0]
+                and self.k <= self._HIP_MAX_K and x.shape[1] <= self._HIP_MAX_OUT_DIM):
             # the transposed view a 'cuda' LogicLayer returns: sum on the feature-major storage
             return GroupSumCudaFunction.apply(x.transpose(0, 1), self.k, float(self.tau))
         return x.reshape(*x.shape[:-1], self.k, x.shape[-1] // self.k).sum(-1) / self.tau
