@@ -53,6 +53,9 @@ SIGNATURES = {
     "dl_logic_eval_fused_groupbitsum_workspace_bytes": [_int, _i64, _i64, _int, _i64],
     "dl_logic_eval_fused_groupbitsum": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _i64, _vp, _vp, _vp],
     "dl_logic_eval_fused_groupbitsum_noalloc": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _i64, _vp, _vp],
+    "dl_logic_net_lds_max_width": [],
+    "dl_logic_net_lds_workspace_bytes": [_int, _vp],
+    "dl_logic_net_lds_groupbitsum": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _i64, _vp, _vp],
     "dl_count_group": [],
     "dl_count_order_build": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp],
 }
@@ -61,7 +64,8 @@ _RESTYPES = {"dl_status_string": ctypes.c_char_p, "dl_last_hip_error": ctypes.c_
              "dl_eval_schedule_capacity": ctypes.c_int64, "dl_eval_schedule_build": ctypes.c_int64,
              "dl_backward_schedule_build": ctypes.c_int64,
              "dl_logic_backward_chained_workspace_bytes": ctypes.c_int64,
-             "dl_logic_eval_fused_groupbitsum_workspace_bytes": ctypes.c_int64}
+             "dl_logic_eval_fused_groupbitsum_workspace_bytes": ctypes.c_int64,
+             "dl_logic_net_lds_max_width": ctypes.c_int64, "dl_logic_net_lds_workspace_bytes": ctypes.c_int64}
 
 _lib = None
 

@@ -12,7 +12,7 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB_NAME = "libdifflogic_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ("packed.hip", "train.hip", "schedule.cpp")
+SOURCES = ("packed.hip", "lds_net.hip", "train.hip", "schedule.cpp")
 # streaming / gather microbenchmarks for `bench.py --ceilings`: a library of their own, never
 # loaded by the package
 CEILINGS_LIB_PATH = os.path.join(HERE, "libdl_ceilings.so")

@@ -632,6 +632,41 @@ def eval_fused_groupbitsum(x, layers, pad_len, k, order=None):
     return out
 
 
+MAX_NET_DEPTH = 16          # layers dl_logic_net_lds_groupbitsum can carry through LDS
+
+
+def net_lds_max_width():
+    """Widest layer (and input) the LDS-resident whole-net kernel takes."""
+    return int(_lib.load().dl_logic_net_lds_max_width())
+
+
+def eval_net_lds(x, layers, pad_len, k):
+    """groupbitsum(eval(... eval(x, layer 0) ..., last layer), pad_len, k) for a whole narrow net
+    (every layer and the input at most net_lds_max_width() wide, at most MAX_NET_DEPTH layers) in
+    one kernel that keeps the activations in LDS.  Returns None where it does not apply (the
+    caller then uses the streaming kernels).  Not part of the reference's extension."""
+    dev, bits, depth, pa, pb, pw, pdims, dims = _fused_args(x, layers)
+    out_dim, words = dims[-1], x.shape[1]
+    if k <= 0 or out_dim % k != 0:
+        raise ValueError(f"in_dim ({out_dim}) has to be divisible by k ({k}) but it is not")
+    batch = words * bits - int(pad_len)
+    if pad_len < 0 or batch < 0:
+        raise RuntimeError(f"pad_len ({pad_len}) has to be in [0, {words * bits}]")
+    if depth > MAX_NET_DEPTH or 0 in dims or max(dims) > net_lds_max_width():
+        return None
+    lib = _lib.load()
+    out = torch.empty((batch, k), dtype=torch.int32, device=dev)
+    ws = torch.empty(max(1, lib.dl_logic_net_lds_workspace_bytes(depth, pdims) // 4), dtype=torch.int32, device=dev)
+    with _on(dev):
+        st = lib.dl_logic_net_lds_groupbitsum(_p(x), depth, pa, pb, pw, pdims, _p(out), words, bits, int(pad_len),
+                                              int(k), _p(ws), _stream(dev))
+    if st == _lib.DL_ERR_TOO_LARGE:
+        return None
+    if st:
+        _raise(st, "logic_net_lds_groupbitsum")
+    return out
+
+
 def eval_fused_groupbitsum_noalloc(x, layers, pad_len, k, out, order=None):
     """eval_fused_groupbitsum into the caller's ``out`` (int32 [batch, k], contiguous) through the
     entry point that allocates no device memory: its workspace is a static device array of

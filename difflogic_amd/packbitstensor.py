@@ -56,6 +56,18 @@ def plan_groups(dims, count_at_end):
     return best[n][1]
 
 
+def lds_tail(dims):
+    """Number of layers at the end of the net (``dims`` = [in_dim, width_1, ..., width_L]) that the
+    LDS-resident whole-net kernel takes together with the count: the longest run of trailing layers
+    whose input and widths all fit its buffer, if that run is at least two layers long (a single
+    layer gains nothing over the streaming kernel fused with the count)."""
+    limit = difflogic_cuda.net_lds_max_width()
+    n = 0
+    while n < len(dims) - 1 and n < difflogic_cuda.MAX_NET_DEPTH and max(dims[len(dims) - 2 - n:]) <= limit:
+        n += 1
+    return n if n >= 2 else 0
+
+
 class PackBitsTensor:
     """``.t`` is int{bit_count} [features, ceil(B / bit_count)]; bit i of word c of a row is
     sample ``bit_count*c + i``; ``.pad_len`` samples at the end of the last word are padding.
@@ -118,6 +130,16 @@ class PackBitsTensor:
         if self._pending:
             if self.features % k != 0:
                 raise ValueError(f"in_dim ({self.features}) has to be divisible by k ({k}) but it is not")
+            dims = self._dims()
+            tail = lds_tail(dims)
+            if tail:
+                # the narrow end of the net runs resident in LDS; what lies before it streams
+                head = len(self._pending) - tail
+                if head:
+                    self._run_groups(plan_groups(dims[:head + 1], count_at_end=False))
+                out = difflogic_cuda.eval_net_lds(self._t, self._pending, self.pad_len, k)
+                if out is not None:
+                    return out
             groups = plan_groups(self._dims(), count_at_end=True)
             self._run_groups(groups[:-1])
             # the last group stays pending: the object's state does not change by counting

@@ -256,6 +256,25 @@ int dl_logic_eval_fused_groupbitsum(const void *x, int depth, const int64_t *con
                                     int64_t pad_len, int64_t k, const int32_t *order, void *workspace,
                                     void *stream);
 
+/* A whole narrow net and its `groupbitsum` in one kernel that keeps the activations in LDS (the
+ * per-layer loop difflogic/difflogic.py:147 over every layer of the model, then
+ * difflogic/packbitstensor.py:22): a workgroup carries a few 64-bit word columns of the packed
+ * input through all `depth` layers and counts the last layer's outputs per class; memory sees
+ * the packed input once and the counts once.  No counterpart in the reference.  Arguments as
+ * dl_logic_eval_fused_groupbitsum, with depth up to 16; result identical to dl_groupbitsum after
+ * `depth` calls of dl_logic_eval.
+ *   Applies when dims[0..depth] <= dl_logic_net_lds_max_width() and rows are whole 64-bit words
+ *   (8-byte aligned x); otherwise DL_ERR_TOO_LARGE is returned and the caller uses the streaming
+ *   entry points.
+ *   workspace DEVICE scratch of dl_logic_net_lds_workspace_bytes(depth, dims) bytes, 4-byte
+ *             aligned: one 32-bit record per gate, rebuilt by every call. */
+int64_t dl_logic_net_lds_max_width(void);
+int64_t dl_logic_net_lds_workspace_bytes(int depth, const int64_t *dims);
+int dl_logic_net_lds_groupbitsum(const void *x, int depth, const int64_t *const *a,
+                                 const int64_t *const *b, const uint8_t *const *w,
+                                 const int64_t *dims, int32_t *out, int64_t words, int bit_count,
+                                 int64_t pad_len, int64_t k, void *workspace, void *stream);
+
 /* dl_logic_eval_fused_groupbitsum without a workspace argument, for callers that cannot allocate
  * device memory: code under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc.  It has no counterpart in the reference (whose functions allocate their outputs and

@@ -373,3 +373,87 @@ def test_packed_inference_follows_weight_writes_through_data():
     with torch.no_grad():
         got2 = model(dl.PackBitsTensor(xd, bit_count=64)).cpu().numpy()
     assert np.array_equal(got2, interp.net_eval(x, layers2, 10))
+
+
+@pytest.mark.parametrize("bits,in_dim,widths,W,k,pad", [
+    (64, 30, [60], 1, 3, 0),                              # a single layer: straight into the class phase
+    (64, 30, [60, 90], 1, 3, 0), (64, 50, [100, 640], 7, 10, 63), (64, 33, [66, 130, 77, 130], 129, 2, 1),
+    (32, 20, [40, 64], 6, 4, 3), (8, 12, [24, 24, 24], 16, 3, 2), (16, 20, [40, 40], 12, 5, 0),
+    (64, 784, [8000] * 6, 9, 10, 5),                      # C2's net: 2 columns per workgroup, odd column count
+    (64, 784, [4000] * 3, 11, 10, 0),                     # 4 columns per workgroup, 3 columns left over
+    (64, 6000, [3000, 10240, 3000], 3, 3, 7),             # widest supported layer; input wider than the last layer
+    (64, 100, [300, 4096], 5, 2, 0),                      # 2048 neurons per class: 8 counter planes per lane
+    (64, 64, [128, 1920], 2, 2, 11),                      # 960 per class: the most 4 planes per lane hold
+    (64, 64, [128, 2048], 2, 2, 11),                      # 1024 per class: 16 per lane, needs the fifth plane
+    (64, 40, [80, 400], 4, 40, 9),                        # more classes than waves
+    (64, 5, [3, 3, 3, 3, 3, 3, 3, 3, 3, 3, 3, 3, 3, 3, 3, 4], 2, 2, 0),     # 16 layers
+])
+def test_net_lds_groupbitsum(ext, bits, in_dim, widths, W, k, pad):
+    """The LDS-resident whole-net kernel against the oracle (eval per layer, then groupbitsum) and
+    against the streaming kernels."""
+    rng = np.random.default_rng(in_dim + W + k + widths[-1] + len(widths))
+    x = rng.integers(np.iinfo(NP_WORD[bits]).min, np.iinfo(NP_WORD[bits]).max, (in_dim, W), dtype=NP_WORD[bits],
+                     endpoint=True)
+    layers, dev_layers = _chain(rng, in_dim, widths)
+    y = x
+    for a, b, op in layers:
+        y = po.eval_layer(y, a, b, op)
+    want = po.groupbitsum(y, pad, k)
+    got = ext.eval_net_lds(_dev(x), dev_layers, pad, k)
+    if W * bits % 64:
+        assert got is None                                # rows are not whole 64-bit words
+        return
+    assert got is not None and got.dtype == torch.int32 and tuple(got.shape) == want.shape
+    assert np.array_equal(got.cpu().numpy(), want)
+    t = _dev(x)
+    for lay in dev_layers:
+        t = ext.eval(t, *lay)
+    assert torch.equal(got, ext.groupbitsum(t, pad, k))
+
+
+def test_net_lds_every_gate_and_saturated_counts(ext):
+    """All 16 gates on all four input pairs through the per-lane mask path, and a class whose
+    every neuron is true for every sample (the count reaches the class size in every lane)."""
+    t = np.array([[0, 0, 1, 1], [0, 1, 0, 1]], dtype=bool)
+    x, pad = po.packbits(t, 64)
+    l1 = (np.zeros(16, np.int64), np.ones(16, np.int64), np.arange(16).astype(np.uint8))
+    want = po.groupbitsum(po.eval_layer(x, *l1), pad, 16)
+    l0 = (np.array([0, 1]), np.array([1, 0]), np.array([3, 3], dtype=np.uint8))        # gate 3 = a: rows stay as they are
+    got = ext.eval_net_lds(_dev(x), [tuple(_dev(v) for v in l0), tuple(_dev(v) for v in l1)], pad, 16)
+    assert np.array_equal(got.cpu().numpy(), want)
+    ones = (np.zeros(5000, np.int64), np.zeros(5000, np.int64), np.full(5000, 15, np.uint8))
+    xs = np.zeros((3, 5), dtype=np.int64)
+    got = ext.eval_net_lds(_dev(xs), [tuple(_dev(v) for v in ones), tuple(_dev(v) for v in ones)], 3, 2)
+    assert got.shape == (317, 2) and bool((got == 2500).all())
+
+
+def test_net_lds_declines_what_does_not_fit(ext):
+    rng = np.random.default_rng(2)
+    layers, dev_layers = _chain(rng, 30, [60, 10241])
+    assert ext.eval_net_lds(_dev(np.zeros((30, 2), np.int64)), dev_layers, 0, 1) is None        # too wide
+    layers, dev_layers = _chain(rng, 30, [40] * 17)
+    assert ext.eval_net_lds(_dev(np.zeros((30, 2), np.int64)), dev_layers, 0, 1) is None        # too deep
+    with pytest.raises(ValueError):
+        ext.eval_net_lds(_dev(np.zeros((30, 2), np.int64)), dev_layers, 0, 3)                   # 40 % 3
+
+
+def test_pack_tensor_runs_narrow_tail_in_lds(monkeypatch):
+    """PackBitsTensor.group_sum hands the narrow end of a net to the LDS kernel (the wide head
+    streams), and the result equals the oracle's."""
+    import difflogic_amd as dl
+    from difflogic_amd import packbitstensor as pbt
+    assert pbt.lds_tail([784, 8000, 8000, 8000]) == 3 and pbt.lds_tail([784, 64000, 64000]) == 0
+    assert pbt.lds_tail([784, 64000, 8000, 8000]) == 0 and pbt.lds_tail([784, 64000, 8000, 8000, 8000]) == 2
+    assert pbt.lds_tail([20000, 8000, 8000]) == 0 and pbt.lds_tail([784, 8000]) == 0
+    rng = np.random.default_rng(31)
+    F, widths = 40, [12000, 6000, 3000, 1500]
+    layers = random_layers(rng, F, widths)
+    x = rng.random((300, F)) < 0.4
+    model = build_model(F, layers, 10).eval()
+    calls = []
+    real = dl.difflogic_cuda.eval_net_lds
+    monkeypatch.setattr(dl.difflogic_cuda, "eval_net_lds", lambda *a, **kw: calls.append(len(a[1])) or real(*a, **kw))
+    with torch.no_grad():
+        got = model(dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=64)).cpu().numpy()
+    assert calls == [2]                                   # 6000 -> 3000 -> 1500 in LDS; what reads the 12000 rows streams
+    assert np.array_equal(got, interp.net_eval(x, layers, 10))
