@@ -50,25 +50,37 @@ __global__ __launch_bounds__(DL_BLOCK) void compose_net_kernel(NetWiring t, uint
 // COLS 64-bit words as 2 * COLS dwords
 template <int COLS> struct Row { uint32_t d[2 * COLS]; };
 
-template <int COLS> __device__ __forceinline__ Row<COLS> lds_row(const dl_u32x4 *act, uint32_t row) {
+// act[] is addressed in units of one row (8 * COLS bytes): 16-byte accesses for COLS >= 2, one
+// 8-byte access for COLS = 1
+template <int COLS> __device__ __forceinline__ Row<COLS> lds_row(const void *act, uint32_t row) {
     Row<COLS> r;
+    if constexpr (COLS == 1) {
+        const dl_u32x2 v = static_cast<const dl_u32x2 *>(act)[row];
+        r.d[0] = v.x, r.d[1] = v.y;
+    } else {
 #pragma unroll
-    for (int q = 0; q < COLS / 2; ++q) {
-        const dl_u32x4 v = act[row * (COLS / 2) + q];
-        r.d[4 * q] = v.x, r.d[4 * q + 1] = v.y, r.d[4 * q + 2] = v.z, r.d[4 * q + 3] = v.w;
+        for (int q = 0; q < COLS / 2; ++q) {
+            const dl_u32x4 v = static_cast<const dl_u32x4 *>(act)[row * (COLS / 2) + q];
+            r.d[4 * q] = v.x, r.d[4 * q + 1] = v.y, r.d[4 * q + 2] = v.z, r.d[4 * q + 3] = v.w;
+        }
     }
     return r;
 }
 
-template <int COLS> __device__ __forceinline__ void lds_store(dl_u32x4 *act, uint32_t row, const Row<COLS> &r) {
+template <int COLS> __device__ __forceinline__ void lds_store(void *act, uint32_t row, const Row<COLS> &r) {
+    if constexpr (COLS == 1) {
+        static_cast<dl_u32x2 *>(act)[row] = dl_u32x2{r.d[0], r.d[1]};
+    } else {
 #pragma unroll
-    for (int q = 0; q < COLS / 2; ++q)
-        act[row * (COLS / 2) + q] = dl_u32x4{r.d[4 * q], r.d[4 * q + 1], r.d[4 * q + 2], r.d[4 * q + 3]};
+        for (int q = 0; q < COLS / 2; ++q)
+            static_cast<dl_u32x4 *>(act)[row * (COLS / 2) + q] =
+                dl_u32x4{r.d[4 * q], r.d[4 * q + 1], r.d[4 * q + 2], r.d[4 * q + 3]};
+    }
 }
 
 // gate id = truth table (f(0,0) f(0,1) f(1,0) f(1,1)), MSB first; masks are per lane here
 template <int COLS>
-__device__ __forceinline__ Row<COLS> gate_rows(const dl_u32x4 *act, uint32_t rec) {
+__device__ __forceinline__ Row<COLS> gate_rows(const void *act, uint32_t rec) {
     const uint32_t ia = rec & ((1u << DL_NET_ID_BITS) - 1), ib = (rec >> DL_NET_ID_BITS) & ((1u << DL_NET_ID_BITS) - 1);
     const uint32_t m00 = 0u - ((rec >> 31) & 1u), m01 = 0u - ((rec >> 30) & 1u);
     const uint32_t m10 = 0u - ((rec >> 29) & 1u), m11 = 0u - ((rec >> 28) & 1u);
@@ -81,6 +93,13 @@ __device__ __forceinline__ Row<COLS> gate_rows(const dl_u32x4 *act, uint32_t rec
         y.d[i] = (a.d[i] & hi) | (~a.d[i] & lo);
     }
     return y;
+}
+
+// carry-save adder on dwords: a + b + c = 2 * carry + sum, bit by bit
+__device__ __forceinline__ void csa32(uint32_t &carry, uint32_t &sum, uint32_t a, uint32_t b, uint32_t c) {
+    const uint32_t u = a ^ b;
+    carry = (a & b) | (u & c);
+    sum = u ^ c;
 }
 
 // a (NP planes, one dword each) += b (NP planes); the sum takes NP + 1 planes
@@ -140,7 +159,7 @@ __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint
                                                                       const uint32_t *__restrict__ rec, NetShape net,
                                                                       int32_t *__restrict__ out, int64_t ncols,
                                                                       int64_t per_class, int64_t k, int64_t batch) {
-    extern __shared__ __align__(16) dl_u32x4 act[];            // [rows][COLS / 2]
+    extern __shared__ __align__(16) uint8_t act[];             // [rows][COLS] 64-bit words
     const int tid = (int) threadIdx.x;
     const int64_t col0 = (int64_t) blockIdx.x * COLS;
 
@@ -156,7 +175,11 @@ __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint
     }
     __syncthreads();
 
-    // every layer but the last: act <- layer(act)
+    // every layer but the last: act <- layer(act).  The records of the next layer are requested
+    // before this layer's barrier, so their latency overlaps the exchange through LDS.
+    // every layer but the last: act <- layer(act).  (Measured: the hidden layers are bound by LDS
+    // throughput, bank conflicts of the random row reads included, not by its latency: putting all
+    // of a thread's reads in flight together is no faster than this gate-by-gate form.)
     for (int l = 0; l + 1 < net.depth; ++l) {
         const uint32_t *tab = rec + net.offset[l];
         const int width = net.width[l];
@@ -183,29 +206,47 @@ __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint
     const int wave = dl_wave_in_block(), lane = dl_lane();
     const uint32_t *tab = rec + net.offset[net.depth - 1];
     for (int64_t cls = wave; cls < k; cls += DL_NET_THREADS / DL_WAVE) {
-        uint32_t pl[COLS][2][NP0];                               // [column][lo / hi dword][plane]
+        uint32_t pl[2 * COLS][NP0];                              // [dword of the row][plane]
 #pragma unroll
-        for (int j = 0; j < COLS; ++j)
+        for (int i = 0; i < 2 * COLS; ++i)
 #pragma unroll
-            for (int p = 0; p < NP0; ++p) pl[j][0][p] = pl[j][1][p] = 0;
-        for (int64_t i = lane; i < per_class; i += DL_WAVE) {
-            const Row<COLS> y = gate_rows<COLS>(act, tab[cls * per_class + i]);
+            for (int p = 0; p < NP0; ++p) pl[i][p] = 0;
+        // four neurons at a time: their records are requested together, their output words are
+        // compressed by a carry-save tree into one word of weight 4 that ripples into the planes
+        // above; neurons past the end of the class contribute zero words
+        const uint32_t *ctab = tab + cls * per_class;
+        for (int64_t i0 = lane; i0 < per_class; i0 += 4 * DL_WAVE) {
+            uint32_t r4[4], live[4];
 #pragma unroll
-            for (int j = 0; j < COLS; ++j)
+            for (int u = 0; u < 4; ++u) {
+                const int64_t i = i0 + u * DL_WAVE;
+                live[u] = i < per_class ? ~0u : 0u;
+                r4[u] = ctab[i < per_class ? i : per_class - 1];
+            }
+            Row<COLS> y[4];
 #pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    uint32_t carry = y.d[2 * j + h];
+            for (int u = 0; u < 4; ++u) {
+                y[u] = gate_rows<COLS>(act, r4[u]);
 #pragma unroll
-                    for (int p = 0; p < NP0; ++p) {              // counter += one bit per sample
-                        const uint32_t old = pl[j][h][p];
-                        pl[j][h][p] = old ^ carry;
-                        carry = old & carry;
-                    }
+                for (int i = 0; i < 2 * COLS; ++i) y[u].d[i] &= live[u];
+            }
+#pragma unroll
+            for (int i = 0; i < 2 * COLS; ++i) {
+                uint32_t t2a, t2b, carry;
+                csa32(t2a, pl[i][0], pl[i][0], y[0].d[i], y[1].d[i]);
+                csa32(t2b, pl[i][0], pl[i][0], y[2].d[i], y[3].d[i]);
+                csa32(carry, pl[i][1], pl[i][1], t2a, t2b);
+#pragma unroll
+                for (int p = 2; p < NP0; ++p) {                  // counter += carry * 4
+                    const uint32_t old = pl[i][p];
+                    pl[i][p] = old ^ carry;
+                    carry = old & carry;
                 }
+            }
         }
 #pragma unroll
         for (int j = 0; j < COLS; ++j) {
-            const int32_t count = lanes_count<NP0>(pl[j][0], pl[j][1], lane);
+            const int32_t count = lanes_count<NP0>(pl[2 * j], pl[2 * j + 1], lane);
             const int64_t sample = (col0 + j) * 64 + lane;
             if (col0 + j < ncols && sample < batch) out[sample * k + cls] = count;
         }
