@@ -56,6 +56,11 @@ SIGNATURES = {
     "dl_logic_net_lds_max_width": [],
     "dl_logic_net_lds_workspace_bytes": [_int, _vp],
     "dl_logic_net_lds_groupbitsum": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _i64, _vp, _vp],
+    "dl_count_chain_padded_steps": [_i64],
+    "dl_count_chain_plan_build": [_vp, _i64, _i64, _i64, _vp, _vp, ctypes.POINTER(_int)],
+    "dl_logic_eval_chained_groupbitsum_workspace_bytes": [_i64, _int, _i64, _int, _i64],
+    "dl_logic_eval_chained_groupbitsum": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _int, _vp,
+                                          _i64, _int, _i64, _i64, _vp, _vp],
     "dl_count_group": [],
     "dl_count_order_build": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp],
 }
@@ -65,6 +70,8 @@ _RESTYPES = {"dl_status_string": ctypes.c_char_p, "dl_last_hip_error": ctypes.c_
              "dl_backward_schedule_build": ctypes.c_int64,
              "dl_logic_backward_chained_workspace_bytes": ctypes.c_int64,
              "dl_logic_eval_fused_groupbitsum_workspace_bytes": ctypes.c_int64,
+             "dl_count_chain_padded_steps": ctypes.c_int64, "dl_count_chain_plan_build": ctypes.c_int64,
+             "dl_logic_eval_chained_groupbitsum_workspace_bytes": ctypes.c_int64,
              "dl_logic_net_lds_max_width": ctypes.c_int64, "dl_logic_net_lds_workspace_bytes": ctypes.c_int64}
 
 _lib = None

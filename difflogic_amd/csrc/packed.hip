@@ -8,6 +8,8 @@
 
 #include <mutex>
 
+#include "count_chain.h"
+
 namespace {
 
 // ------------------------------------------------------------------------------------------
@@ -778,6 +780,152 @@ __global__ __launch_bounds__(DL_BLOCK) void count_partial_kernel(const V *__rest
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// Count fused with the last one or two layers, the top layer walked along its evaluation
+// schedule (schedule.cpp): consecutive top-layer neurons share an input vertex, whose value stays
+// in registers, so a neuron costs 2^DS gathered rows instead of 2^(DS+1) (DS = 1: the vertex is a
+// neuron of the layer below, a gate over two rows of x; DS = 0: a row of x itself).
+//
+// Consecutive neurons of a trail belong to arbitrary classes, so a wave cannot keep one counter.
+// Instead a workgroup of DL_CC_WAVES waves proceeds in blocks: every wave walks DL_CC_WAVE_STEPS
+// steps of its own contiguous range of the schedule and parks each output vector in LDS, at a
+// slot (precomputed per wiring) that sorts the block's outputs by class; after a barrier the wave
+// that owns a class reads that class's run of slots and adds it to bit-sliced counters it keeps
+// in registers for the whole workgroup (DL_CC_PLANES planes: the plan guarantees at most 255
+// neurons of a class per workgroup).  The counters go to the same partial-plane layout that
+// count_finish_kernel sums: one "chunk" per workgroup.
+//
+// Per step the wave reads one 16-byte record (wave-uniform: a scalar load) that a small kernel
+// composes per call from the schedule and the current gate ids:
+//   rec[i + 1] = { la, lb, sub gate | top gate << 4 | slot << 8 } for step i, rec[0] for the
+//   vertex before step 0; a wave that starts at step f seeds its chain from rec[f].
+// ------------------------------------------------------------------------------------------
+template <int DS>
+__global__ __launch_bounds__(DL_BLOCK) void compose_count_chain_kernel(TreeTables t, const int32_t *__restrict__ verts,
+                                                                       const int32_t *__restrict__ neuron,
+                                                                       const uint8_t *__restrict__ flip,
+                                                                       const uint8_t *__restrict__ slot, int64_t steps,
+                                                                       int64_t padded, dl_u32x4 *__restrict__ rec) {
+    const int64_t i = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x;      // record index: step i - 1
+    if (i > padded) return;
+    const int64_t v = verts[i < steps ? i : steps];                        // vertex reached by step i - 1
+    uint32_t la, lb = 0, bits = 0;
+    if (DS == 1) {
+        la = (uint32_t) t.a[0][v];
+        lb = (uint32_t) t.b[0][v];
+        bits = t.w[0][v] & 15u;
+    } else {
+        la = (uint32_t) v;
+    }
+    uint32_t where = 255;
+    if (i >= 1) {
+        const int64_t s = i - 1;
+        where = slot[s];
+        if (s < steps && neuron[s] >= 0) {
+            uint32_t top = t.w[DS][neuron[s]] & 15u;
+            if (flip[s]) top = swap_gate_inputs(top);
+            bits |= top << 4;
+        }
+    }
+    rec[i] = dl_u32x4{la, lb, bits | (where << 8), 0u};
+}
+
+template <typename V, int DS, int CPW>
+__global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(const V *__restrict__ x,
+                                                                            const dl_u32x4 *__restrict__ rec,
+                                                                            const uint16_t *__restrict__ runs,
+                                                                            V *__restrict__ partial, int64_t ncols,
+                                                                            int64_t k, int64_t nwg, int blocks) {
+    __shared__ V stage[DL_CC_BLOCK][DL_WAVE];
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t g = blockIdx.x;
+    const int64_t col = (int64_t) blockIdx.y * DL_WAVE + lane;
+    const bool live = col < ncols;
+    const V *xcol = x + (live ? col : 0);
+    // the wave's range of the schedule: [0] = seed, [1 + j] = its step j
+    const dl_u32x4 *wrec = rec + (g * DL_CC_WAVES + wave) * (int64_t) (DL_CC_WAVE_STEPS * blocks);
+
+    auto vertex = [&](V ra, V rb, uint32_t bits) -> V {
+        if (DS == 1) return gate_apply<V>(ra, rb, gate_masks(bits & 15u));
+        return ra;
+    };
+    V prev;
+    {
+        const dl_u32x4 r = wrec[0];
+        const V ra = xcol[(int64_t) r.x * ncols];
+        const V rb = DS == 1 ? xcol[(int64_t) r.y * ncols] : ra;
+        prev = vertex(ra, rb, r.z);
+    }
+    V cnt[CPW][DL_CC_PLANES];
+#pragma unroll
+    for (int i = 0; i < CPW; ++i)
+#pragma unroll
+        for (int p = 0; p < DL_CC_PLANES; ++p) cnt[i][p] = Words<V>::zero();
+
+#pragma unroll 1
+    for (int b = 0; b < blocks; ++b) {
+        // phase A: walk DL_CC_WAVE_STEPS steps, four at a time (their rows are requested together)
+#pragma unroll
+        for (int h = 0; h < DL_CC_WAVE_STEPS; h += 4) {
+            dl_u32x4 r[4];
+            V ra[4], rb[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                r[j] = wrec[1 + b * DL_CC_WAVE_STEPS + h + j];
+                ra[j] = xcol[(int64_t) r[j].x * ncols];
+                if (DS == 1) rb[j] = xcol[(int64_t) r[j].y * ncols];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const V cur = vertex(ra[j], DS == 1 ? rb[j] : ra[j], r[j].z);
+                const uint32_t where = (r[j].z >> 8) & 255u;
+                if (where != 255u) stage[where][lane] = gate_apply<V>(prev, cur, gate_masks((r[j].z >> 4) & 15u));
+                prev = cur;
+            }
+        }
+        __syncthreads();
+        // phase B: the owner of a class adds that class's run of parked outputs to its counters
+#pragma unroll
+        for (int i = 0; i < CPW; ++i) {
+            const int64_t cls = wave + i * DL_CC_WAVES;
+            if (cls < k) {
+                const uint32_t run = runs[(g * blocks + b) * k + cls];
+                const int start = (int) (run & 255u), n = (int) (run >> 8);
+#pragma unroll 1
+                for (int q = 0; q < n; q += 4) {
+                    V v[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int at = start + q + u;
+                        const V parked = stage[at < DL_CC_BLOCK ? at : DL_CC_BLOCK - 1][lane];
+                        v[u] = q + u < n ? parked : Words<V>::zero();
+                    }
+                    V carry = csa_quad(cnt[i][0], cnt[i][1], v);          // weight 4
+#pragma unroll
+                    for (int p = 2; p < DL_CC_PLANES; ++p) {
+                        const V old = cnt[i][p];
+                        cnt[i][p] = old ^ carry;
+                        carry = old & carry;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (live) {
+#pragma unroll
+        for (int i = 0; i < CPW; ++i) {
+            const int64_t cls = wave + i * DL_CC_WAVES;
+            if (cls < k) {
+                V *dst = partial + ((((int64_t) blockIdx.y * k + cls) * nwg + g) * DL_CC_PLANES) * DL_WAVE + lane;
+#pragma unroll
+                for (int p = 0; p < DL_CC_PLANES; ++p) __builtin_nontemporal_store(cnt[i][p], dst + (int64_t) p * DL_WAVE);
+            }
+        }
+    }
+}
+
 template <typename V, int NP>
 __global__ __launch_bounds__(DL_BLOCK) void count_finish_kernel(const V *__restrict__ partial, int32_t *__restrict__ out,
                                                                 int64_t ncols, int64_t chunks_per_class, int64_t k,
@@ -1263,4 +1411,111 @@ extern "C" int dl_logic_eval_chained(const void *x, int depth, const int64_t *co
                                            nchunks, row_bytes, s);
     return launch_eval_chain<dl_u32x2>(depth - 1, x, sub_leaves, sub_gates, verts, neuron, flip, w[depth - 1], y, nchunks,
                                        row_bytes, s);
+}
+
+// ---- count fused with the last layers, walked along the evaluation schedule ----------------
+static_assert(DL_CC_PLANES == DL_COUNT_PLANES, "count_finish_kernel reads DL_COUNT_PLANES planes per chunk");
+static_assert(DL_CC_BLOCK <= 255, "slots are bytes, 255 = none");
+
+namespace {
+
+int64_t count_chain_partial_bytes(int64_t padded_steps, int blocks, int64_t k, int64_t row_bytes) {
+    const int64_t vec = row_bytes % 16 == 0 ? 16 : 8;
+    const int64_t tiles = dl_ceil_div(row_bytes / vec, DL_WAVE);
+    return tiles * k * (padded_steps / (DL_CC_BLOCK * blocks)) * DL_CC_PLANES * DL_WAVE * vec;
+}
+
+bool valid_cc_blocks(int blocks) { return blocks == 1 || blocks == 2 || blocks == 4 || blocks == 8 || blocks == 16; }
+
+template <typename V, int DS>
+int launch_count_chain(const void *x, const dl_u32x4 *rec, const uint16_t *runs, void *partial, int32_t *out,
+                       int64_t row_bytes, int64_t padded_steps, int blocks, int64_t per_class, int64_t k, int64_t batch,
+                       hipStream_t s) {
+    const int64_t ncols = row_bytes / (int64_t) sizeof(V);
+    const int64_t tiles = dl_ceil_div(ncols, DL_WAVE);
+    const int64_t nwg = padded_steps / (DL_CC_BLOCK * blocks);
+    if (nwg > 0x7fffffffLL || tiles > 65535) return DL_ERR_TOO_LARGE;
+    const dim3 grid((unsigned) nwg, (unsigned) tiles), block(DL_CC_WAVES * DL_WAVE);
+    if (k <= DL_CC_WAVES)
+        DL_LAUNCH((count_chain_kernel<V, DS, 1>), grid, block, 0, s, (const V *) x, rec, runs, (V *) partial, ncols, k, nwg,
+                  blocks);
+    else
+        DL_LAUNCH((count_chain_kernel<V, DS, 2>), grid, block, 0, s, (const V *) x, rec, runs, (V *) partial, ncols, k, nwg,
+                  blocks);
+    int st = dl_launch_status();
+    if (st != DL_OK) return st;
+    const dim3 fgrid((unsigned) tiles, (unsigned) k);
+    if (per_class < (1LL << 13))
+        DL_LAUNCH((count_finish_kernel<V, 13>), fgrid, dim3(DL_BLOCK), 0, s, (const V *) partial, out, ncols, nwg, k, batch);
+    else if (per_class < (1LL << 18))
+        DL_LAUNCH((count_finish_kernel<V, 18>), fgrid, dim3(DL_BLOCK), 0, s, (const V *) partial, out, ncols, nwg, k, batch);
+    else
+        DL_LAUNCH((count_finish_kernel<V, 31>), fgrid, dim3(DL_BLOCK), 0, s, (const V *) partial, out, ncols, nwg, k, batch);
+    return dl_launch_status();
+}
+
+}  // namespace
+
+extern "C" int64_t dl_logic_eval_chained_groupbitsum_workspace_bytes(int64_t padded_steps, int blocks, int64_t words,
+                                                                      int bit_count, int64_t k) {
+    if (padded_steps < 0 || padded_steps % DL_CC_MAX_WG_STEPS != 0 || !valid_cc_blocks(blocks) || words < 0 || k <= 0 ||
+        !valid_bit_count(bit_count))
+        return 0;
+    const int64_t row_bytes = words * (bit_count / 8);
+    if (row_bytes % 8 != 0) return 0;
+    return (padded_steps + 1) * 16 + count_chain_partial_bytes(padded_steps, blocks, k, row_bytes);
+}
+
+extern "C" int dl_logic_eval_chained_groupbitsum(const void *x, int depth, const int64_t *const *a, const int64_t *const *b,
+                                                 const uint8_t *const *w, const int64_t *dims, const int32_t *verts,
+                                                 const int32_t *neuron, const uint8_t *flip, int64_t steps,
+                                                 const uint8_t *slot, const uint16_t *runs, int64_t padded_steps,
+                                                 int blocks, int32_t *out, int64_t words, int bit_count, int64_t pad_len,
+                                                 int64_t k, void *workspace, void *stream) {
+    if (!valid_bit_count(bit_count)) return DL_ERR_BIT_COUNT;
+    if (depth < 1 || depth > 2 || !dims || !w || words < 0 || k <= 0 || pad_len < 0 || steps < 0 || padded_steps < steps ||
+        padded_steps % DL_CC_MAX_WG_STEPS != 0 || !valid_cc_blocks(blocks))
+        return DL_ERR_INVALID_ARGUMENT;
+    const int64_t out_dim = dims[depth];
+    if (out_dim <= 0 || steps < out_dim) return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim % k != 0) return DL_ERR_NOT_DIVISIBLE;
+    const int64_t batch = words * bit_count - pad_len;
+    if (batch < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (batch == 0) return DL_OK;
+    if (!out || !x || !verts || !neuron || !flip || !slot || !runs || !workspace) return DL_ERR_INVALID_ARGUMENT;
+    for (int l = 0; l < depth; ++l)
+        if (!w[l] || (l + 1 < depth && (!a || !b || !a[l] || !b[l])) || dims[l] <= 0) return DL_ERR_INVALID_ARGUMENT;
+    const int64_t per_class = out_dim / k;
+    const int64_t row_bytes = words * (bit_count / 8);
+    if (row_bytes % 8 != 0 || !dl_aligned(x, 8) || k > DL_CC_MAX_CLASSES || per_class > 0x7fffffffLL ||
+        dims[0] > 0x7fffffffLL || padded_steps > 0x7ffffff0LL)
+        return DL_ERR_TOO_LARGE;
+    if (!dl_aligned(workspace, 16)) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+
+    TreeTables t;
+    for (int l = 0; l < DL_MAX_FUSE_DEPTH; ++l) t.a[l] = t.b[l] = nullptr, t.w[l] = nullptr;
+    for (int l = 0; l < depth; ++l) {
+        t.a[l] = a ? a[l] : nullptr;
+        t.b[l] = b ? b[l] : nullptr;
+        t.w[l] = w[l];
+    }
+    dl_u32x4 *rec = (dl_u32x4 *) workspace;
+    void *partial = (char *) workspace + (padded_steps + 1) * 16;
+    const dim3 cgrid((unsigned) dl_ceil_div(padded_steps + 1, DL_BLOCK));
+    if (depth == 2)
+        DL_LAUNCH(compose_count_chain_kernel<1>, cgrid, dim3(DL_BLOCK), 0, s, t, verts, neuron, flip, slot, steps,
+                  padded_steps, rec);
+    else
+        DL_LAUNCH(compose_count_chain_kernel<0>, cgrid, dim3(DL_BLOCK), 0, s, t, verts, neuron, flip, slot, steps,
+                  padded_steps, rec);
+    const int st = dl_launch_status();
+    if (st != DL_OK) return st;
+    const bool wide = row_bytes % 16 == 0 && dl_aligned(x, 16);
+    if (depth == 2) {
+        if (wide) return launch_count_chain<dl_u32x4, 1>(x, rec, runs, partial, out, row_bytes, padded_steps, blocks, per_class, k, batch, s);
+        return launch_count_chain<uint64_t, 1>(x, rec, runs, partial, out, row_bytes, padded_steps, blocks, per_class, k, batch, s);
+    }
+    if (wide) return launch_count_chain<dl_u32x4, 0>(x, rec, runs, partial, out, row_bytes, padded_steps, blocks, per_class, k, batch, s);
+    return launch_count_chain<uint64_t, 0>(x, rec, runs, partial, out, row_bytes, padded_steps, blocks, per_class, k, batch, s);
 }

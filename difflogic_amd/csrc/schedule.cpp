@@ -16,6 +16,7 @@
 #include <algorithm>
 #include <vector>
 
+#include "count_chain.h"
 #include "difflogic_hip.h"
 
 extern "C" int64_t dl_eval_schedule_capacity(int64_t out_dim, int chunk) {
@@ -213,4 +214,75 @@ extern "C" int dl_count_order_build(const int64_t *a_top, const int64_t *b_top, 
         }
     }
     return DL_OK;
+}
+
+// Plan for dl_logic_eval_chained_groupbitsum: the count kernel walks the top layer along the
+// evaluation schedule, so consecutive outputs belong to arbitrary classes.  A workgroup of
+// DL_CC_WAVES waves owns 64 * blocks consecutive steps (a contiguous range per wave) and proceeds
+// in `blocks` blocks of DL_CC_BLOCK outputs (DL_CC_WAVE_STEPS per wave): every wave parks its
+// outputs of the block in LDS at a slot that sorts the block by class, and the wave that owns a
+// class then reads that class's run of slots and adds it to its bit-sliced counters.
+//   slot [padded]           LDS slot of step s within its block, 255 = the step has no output
+//   runs [padded / 64 * k]  per block and class: first slot | number of slots << 8
+//   *blocks                 blocks per workgroup: the largest of 16, 8, 4, 2, 1 for which no
+//                           workgroup counts more than 255 neurons of one class (its counters have
+//                           DL_CC_PLANES planes); fewer blocks mean more partial counters
+// where step s of workgroup g, wave w, block b, position j is
+// g*64*blocks + w*8*blocks + b*DL_CC_WAVE_STEPS + j.  Returns the padded step count (a multiple of
+// DL_CC_MAX_WG_STEPS; steps past `steps` have no output), or -DL_ERR_TOO_LARGE for more classes
+// than the kernel's waves can own.
+extern "C" int64_t dl_count_chain_padded_steps(int64_t steps) {
+    if (steps < 0) return -DL_ERR_INVALID_ARGUMENT;
+    return (steps + DL_CC_MAX_WG_STEPS - 1) / DL_CC_MAX_WG_STEPS * DL_CC_MAX_WG_STEPS;
+}
+
+static bool count_chain_plan(const int32_t *neuron, int64_t steps, int64_t per_class, int64_t k, int blocks,
+                             int64_t padded, uint8_t *slot, uint16_t *runs) {
+    const int64_t wg_steps = (int64_t) DL_CC_BLOCK * blocks, span = (int64_t) DL_CC_WAVE_STEPS * blocks;
+    std::vector<int64_t> total((size_t) k);
+    for (int64_t g = 0; g < padded / wg_steps; ++g) {
+        std::fill(total.begin(), total.end(), 0);
+        for (int64_t b = 0; b < blocks; ++b) {
+            // class of every output of the block, in (wave, position) order
+            int64_t cls[DL_CC_BLOCK], where[DL_CC_BLOCK];
+            int count[DL_CC_MAX_CLASSES] = {0};
+            for (int64_t w = 0; w < DL_CC_WAVES; ++w)
+                for (int64_t j = 0; j < DL_CC_WAVE_STEPS; ++j) {
+                    const int64_t s = g * wg_steps + w * span + b * DL_CC_WAVE_STEPS + j;
+                    const int64_t i = w * DL_CC_WAVE_STEPS + j;
+                    where[i] = s;
+                    cls[i] = (s < steps && neuron[s] >= 0) ? neuron[s] / per_class : -1;
+                    if (cls[i] >= 0) ++count[cls[i]];
+                }
+            int first[DL_CC_MAX_CLASSES];
+            int at = 0;
+            uint16_t *run = runs + (g * blocks + b) * k;
+            for (int64_t c = 0; c < k; ++c) {
+                first[c] = at;
+                run[c] = (uint16_t) (at | (count[c] << 8));
+                at += count[c];
+                total[(size_t) c] += count[c];
+            }
+            for (int64_t i = 0; i < DL_CC_BLOCK; ++i) slot[where[i]] = cls[i] < 0 ? 255 : (uint8_t) first[cls[i]]++;
+        }
+        for (int64_t c = 0; c < k; ++c)
+            if (total[(size_t) c] >= (1 << DL_CC_PLANES)) return false;
+    }
+    return true;
+}
+
+extern "C" int64_t dl_count_chain_plan_build(const int32_t *neuron, int64_t steps, int64_t out_dim, int64_t k,
+                                             uint8_t *slot, uint16_t *runs, int *blocks) {
+    if (!neuron || !slot || !runs || !blocks || steps < 0 || out_dim <= 0 || k <= 0) return -DL_ERR_INVALID_ARGUMENT;
+    if (out_dim % k != 0) return -DL_ERR_NOT_DIVISIBLE;
+    if (k > DL_CC_MAX_CLASSES) return -DL_ERR_TOO_LARGE;
+    for (int64_t s = 0; s < steps; ++s)
+        if (neuron[s] >= out_dim) return -DL_ERR_INVALID_ARGUMENT;
+    const int64_t padded = dl_count_chain_padded_steps(steps);
+    for (int nb = DL_CC_MAX_BLOCKS; nb >= 1; nb /= 2)       // one block holds 64 outputs: always fits
+        if (count_chain_plan(neuron, steps, out_dim / k, k, nb, padded, slot, runs)) {
+            *blocks = nb;
+            return padded;
+        }
+    return -DL_ERR_TOO_LARGE;
 }

@@ -461,6 +461,32 @@ class EvalSchedule:
         self.flip = torch.from_numpy(flip[:steps].copy()).to(a.device)
         self._host = (verts[:steps + 1].copy(), neuron[:steps].copy())
         self._backward = None
+        self._count_plans = {}
+
+    def count_plan(self, k):
+        """(slot, runs, padded_steps, blocks) plan for eval_chained_groupbitsum with ``k`` classes (slot,
+        runs on the device), built on first use per k; None where the chained count does not
+        apply (too many classes)."""
+        if k not in self._count_plans:
+            import numpy as np
+            lib = _lib.load()
+            _, neuron = self._host
+            padded = lib.dl_count_chain_padded_steps(self.steps)
+            slot = np.empty(max(1, padded), dtype=np.uint8)
+            runs = np.empty(max(1, padded // 64 * k), dtype=np.uint16)
+            blocks = ctypes.c_int(0)
+            got = lib.dl_count_chain_plan_build(neuron.ctypes.data, self.steps, self.out_dim, int(k), slot.ctypes.data,
+                                                runs.ctypes.data, ctypes.byref(blocks))
+            if got == -_lib.DL_ERR_TOO_LARGE:
+                self._count_plans[k] = None
+            elif got < 0:
+                _raise(-got, "count_chain_plan_build")
+            else:
+                dev = self.verts.device
+                # uint16 has no torch dtype on every build: the table travels as int16 with the same bits
+                self._count_plans[k] = (torch.from_numpy(slot).to(dev), torch.from_numpy(runs.view(np.int16)).to(dev),
+                                        int(got), int(blocks.value))
+        return self._count_plans[k]
 
     def backward_plan(self):
         """(dst, fix_vertex, fix_start, n_fix, overflow_rows) for backward_chained, built on first
@@ -595,6 +621,47 @@ def count_order_for(layers, in_dim, k):
         return torch.from_numpy(order).to(idx[0].device)
 
     return _COUNT_ORDERS.get(tuple(idx), (int(in_dim), int(k)), build)
+
+
+def eval_chained_groupbitsum(x, layers, pad_len, k, schedule=None):
+    """Same result as ``eval_fused_groupbitsum(x, layers, pad_len, k)`` for the net's last one or
+    two layers; the top layer is walked along ``schedule`` (default: the cached schedule of its
+    wiring), which halves the rows gathered per neuron.  Returns None where it does not apply
+    (the caller then uses eval_fused_groupbitsum).  Not part of the reference's extension."""
+    dev, bits, depth, pa, pb, pw, pdims, dims = _fused_args(x, layers)
+    if depth > MAX_FUSE_DEPTH_COUNT:
+        raise RuntimeError(f"at most {MAX_FUSE_DEPTH_COUNT} layers can be fused with the count, got {depth}")
+    out_dim, words = dims[-1], x.shape[1]
+    if k <= 0 or out_dim % k != 0:
+        raise ValueError(f"in_dim ({out_dim}) has to be divisible by k ({k}) but it is not")
+    batch = words * bits - int(pad_len)
+    if pad_len < 0 or batch < 0:
+        raise RuntimeError(f"pad_len ({pad_len}) has to be in [0, {words * bits}]")
+    if 0 in dims or batch == 0 or (words * bits) % 64:
+        return None
+    if schedule is None:
+        schedule = schedule_for(layers[-1][0], layers[-1][1], dims[-2])
+    if schedule.in_dim != dims[-2] or schedule.out_dim != dims[-1] or schedule.verts.device != dev:
+        raise RuntimeError(f"schedule is for a {schedule.in_dim}->{schedule.out_dim} layer on {schedule.verts.device}, "
+                           f"the group ends in {dims[-2]}->{dims[-1]} on {dev}")
+    plan = schedule.count_plan(int(k))
+    if plan is None:
+        return None
+    slot, runs, padded, blocks = plan
+    lib = _lib.load()
+    out = torch.empty((batch, k), dtype=torch.int32, device=dev)
+    nbytes = lib.dl_logic_eval_chained_groupbitsum_workspace_bytes(padded, blocks, words, bits, int(k))
+    ws = torch.empty(max(2, -(-nbytes // 8)), dtype=torch.int64, device=dev)
+    with _on(dev):
+        st = lib.dl_logic_eval_chained_groupbitsum(_p(x), depth, pa, pb, pw, pdims, _p(schedule.verts),
+                                                   _p(schedule.neuron), _p(schedule.flip), schedule.steps, _p(slot),
+                                                   _p(runs), padded, blocks, _p(out), words, bits, int(pad_len), int(k),
+                                                   _p(ws), _stream(dev))
+    if st == _lib.DL_ERR_TOO_LARGE:
+        return None
+    if st:
+        _raise(st, "logic_layer_cuda_eval_chained_groupbitsum")
+    return out
 
 
 def eval_fused_groupbitsum(x, layers, pad_len, k, order=None):

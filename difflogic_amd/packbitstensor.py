@@ -143,6 +143,9 @@ class PackBitsTensor:
             groups = plan_groups(self._dims(), count_at_end=True)
             self._run_groups(groups[:-1])
             # the last group stays pending: the object's state does not change by counting
+            out = difflogic_cuda.eval_chained_groupbitsum(self._t, self._pending, self.pad_len, k)
+            if out is not None:
+                return out
             order = difflogic_cuda.count_order_for(self._pending, self._t.shape[0], k)
             return difflogic_cuda.eval_fused_groupbitsum(self._t, self._pending, self.pad_len, k, order)
         return difflogic_cuda.groupbitsum(self._t, self.pad_len, k)

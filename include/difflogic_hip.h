@@ -256,6 +256,40 @@ int dl_logic_eval_fused_groupbitsum(const void *x, int depth, const int64_t *con
                                     int64_t pad_len, int64_t k, const int32_t *order, void *workspace,
                                     void *stream);
 
+/* dl_logic_eval_fused_groupbitsum with the top layer walked along its evaluation schedule (as
+ * dl_logic_eval_chained walks it): consecutive neurons share an input vertex whose value stays in
+ * registers, so a neuron of a depth-2 group costs two gathered rows of x instead of four (depth 1:
+ * one instead of two).  Same result as dl_logic_eval_fused_groupbitsum.  No counterpart in the
+ * reference.
+ *   verts, neuron, flip, steps   DEVICE copies of the top layer's schedule (dl_eval_schedule_build)
+ *   dl_count_chain_padded_steps()  HOST: steps rounded up to whole workgroups
+ *   dl_count_chain_plan_build()    HOST pointers.  From the schedule's neuron [steps], out_dim and k
+ *       writes slot [padded] and runs [padded / 64 * k]: where every workgroup parks the outputs
+ *       of a block so that they are sorted by class, and each class's run of slots; and *blocks:
+ *       how many blocks of 64 steps a workgroup walks (16 at most; fewer where a workgroup would
+ *       otherwise count more than 255 neurons of one class).  Returns padded, or a negated
+ *       dl_status: -DL_ERR_TOO_LARGE for k > 16 (the caller then uses
+ *       dl_logic_eval_fused_groupbitsum).
+ *   slot, runs, padded_steps, blocks   that plan (slot, runs: DEVICE copies)
+ *   workspace DEVICE scratch of dl_logic_eval_chained_groupbitsum_workspace_bytes(...) bytes,
+ *             16-byte aligned: one 16-byte record per step (composed per call from the schedule
+ *             and the current gate ids) and the bit-sliced partial counters.
+ * depth is 1 or 2; a, b are read for the layer below the top one only (a[0], b[0] at depth 2).
+ * DL_ERR_TOO_LARGE: rows are not whole 64-bit words or k > 16. */
+int64_t dl_count_chain_padded_steps(int64_t steps);
+int64_t dl_count_chain_plan_build(const int32_t *neuron, int64_t steps, int64_t out_dim, int64_t k,
+                                  uint8_t *slot, uint16_t *runs, int *blocks);
+int64_t dl_logic_eval_chained_groupbitsum_workspace_bytes(int64_t padded_steps, int blocks,
+                                                          int64_t words, int bit_count, int64_t k);
+int dl_logic_eval_chained_groupbitsum(const void *x, int depth, const int64_t *const *a,
+                                      const int64_t *const *b, const uint8_t *const *w,
+                                      const int64_t *dims, const int32_t *verts,
+                                      const int32_t *neuron, const uint8_t *flip, int64_t steps,
+                                      const uint8_t *slot, const uint16_t *runs,
+                                      int64_t padded_steps, int blocks, int32_t *out,
+                                      int64_t words, int bit_count, int64_t pad_len, int64_t k,
+                                      void *workspace, void *stream);
+
 /* A whole narrow net and its `groupbitsum` in one kernel that keeps the activations in LDS (the
  * per-layer loop difflogic/difflogic.py:147 over every layer of the model, then
  * difflogic/packbitstensor.py:22): a workgroup carries a few 64-bit word columns of the packed

@@ -457,3 +457,55 @@ def test_pack_tensor_runs_narrow_tail_in_lds(monkeypatch):
         got = model(dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=64)).cpu().numpy()
     assert calls == [2]                                   # 6000 -> 3000 -> 1500 in LDS; what reads the 12000 rows streams
     assert np.array_equal(got, interp.net_eval(x, layers, 10))
+
+
+@pytest.mark.parametrize("in_dim,widths,W,k,pad,kind", [
+    (30, [60], 1, 3, 0, "any"), (50, [640], 70, 10, 63, "any"), (33, [130], 129, 2, 1, "any"),
+    (64, [64], 3, 16, 0, "random"), (100, [40000], 2, 2, 11, "any"),
+    (30, [60, 90], 1, 3, 0, "any"), (50, [100, 640], 70, 10, 63, "any"), (33, [66, 130], 129, 2, 1, "any"),
+    (784, [8000, 8000], 33, 10, 5, "random"), (784, [8000, 8000], 32, 10, 0, "unique"),
+    (300, [3000, 3000], 16, 1, 0, "random"),               # one class: every output lands in one counter
+    (20, [40, 64], 4, 16, 3, "self"), (40, [80, 2400], 2, 12, 0, "any"),
+])
+def test_chained_groupbitsum(ext, in_dim, widths, W, k, pad, kind):
+    """The count walked along the evaluation schedule against the oracle and the unchained
+    fused count, for 16-byte and 8-byte lanes, ragged batches and every kind of wiring."""
+    from oracle import connections as oc
+    rng = np.random.default_rng(in_dim + W + k + widths[-1])
+    x = rng.integers(np.iinfo(np.int64).min, np.iinfo(np.int64).max, (in_dim, W), dtype=np.int64, endpoint=True)
+    layers = random_layers(rng, in_dim, widths)
+    top_in = in_dim if len(widths) == 1 else widths[-2]
+    torch.manual_seed(k)
+    if kind == "random":
+        ta, tb = oc.random_connections(top_in, widths[-1])
+    elif kind == "unique":
+        ta, tb = oc.unique_connections(top_in, widths[-1])
+    elif kind == "self":
+        ta = torch.as_tensor(layers[-1][0])
+        tb = ta.clone()
+    else:
+        ta, tb = torch.as_tensor(layers[-1][0]), torch.as_tensor(layers[-1][1])
+    layers[-1] = (np.asarray(ta), np.asarray(tb), layers[-1][2])
+    dev_layers = [tuple(_dev(t) for t in l) for l in layers]
+    y = x
+    for a, b, op in layers:
+        y = po.eval_layer(y, a, b, op)
+    want = po.groupbitsum(y, pad, k)
+    got = ext.eval_chained_groupbitsum(_dev(x), dev_layers, pad, k)
+    assert got is not None and got.dtype == torch.int32 and tuple(got.shape) == want.shape
+    assert np.array_equal(got.cpu().numpy(), want)
+    assert torch.equal(got, ext.eval_fused_groupbitsum(_dev(x), dev_layers, pad, k))
+
+
+def test_chained_groupbitsum_declines_where_it_does_not_apply(ext):
+    rng = np.random.default_rng(3)
+    layers, dev_layers = _chain(rng, 30, [60, 170])
+    x = _dev(rng.integers(0, 1 << 62, (30, 2), dtype=np.int64))
+    assert ext.eval_chained_groupbitsum(x, dev_layers, 0, 17) is None                 # more classes than the waves own
+    # 3000 neurons on one trail: with 12 classes (250 each) a workgroup walks 16 blocks, with one class only 2
+    a = torch.arange(3000) % 2999
+    b = (torch.arange(3000) + 1) % 2999
+    sched = ext.schedule_for(_dev(a.numpy()), _dev(b.numpy()), 2999)
+    assert sched.count_plan(12)[3] == 16 and sched.count_plan(1)[3] == 2 and sched.count_plan(20) is None
+    x32 = torch.zeros((30, 3), dtype=torch.int32, device="cuda")
+    assert ext.eval_chained_groupbitsum(x32, dev_layers, 0, 10) is None               # rows are not whole 64-bit words
