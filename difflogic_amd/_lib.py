@@ -49,6 +49,7 @@ SIGNATURES = {
     "dl_eval_schedule_chunk": [],
     "dl_eval_schedule_capacity": [_i64, _int],
     "dl_eval_schedule_build": [_vp, _vp, _i64, _i64, _int, _vp, _vp, _vp],
+    "dl_logic_eval_chained_workspace_bytes": [_int, _i64, _i64],
     "dl_logic_eval_chained": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _int, _vp, _vp],
     "dl_logic_eval_fused_groupbitsum_workspace_bytes": [_int, _i64, _i64, _int, _i64],
     "dl_logic_eval_fused_groupbitsum": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _i64, _vp, _vp, _vp],
@@ -70,6 +71,7 @@ _RESTYPES = {"dl_status_string": ctypes.c_char_p, "dl_last_hip_error": ctypes.c_
              "dl_backward_schedule_build": ctypes.c_int64,
              "dl_logic_backward_chained_workspace_bytes": ctypes.c_int64,
              "dl_logic_eval_fused_groupbitsum_workspace_bytes": ctypes.c_int64,
+             "dl_logic_eval_chained_workspace_bytes": ctypes.c_int64,
              "dl_count_chain_padded_steps": ctypes.c_int64, "dl_count_chain_plan_build": ctypes.c_int64,
              "dl_logic_eval_chained_groupbitsum_workspace_bytes": ctypes.c_int64,
              "dl_logic_net_lds_max_width": ctypes.c_int64, "dl_logic_net_lds_workspace_bytes": ctypes.c_int64}

@@ -300,6 +300,113 @@ __global__ __launch_bounds__(DL_BLOCK) void eval_chain_kernel(const V *__restric
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// eval_chain_kernel with everything a step needs in ONE record, composed per call by a small
+// kernel from the schedule, the flattened subtrees and the current gate ids:
+//   rec[i + 1] for step i (rec[0]: the vertex before step 0, from which a wave starting at step 0
+//   seeds its chain; a wave starting at step f seeds from rec[f]):
+//     leaf[2^DS]  the subtree's rows, already multiplied by the row length in vectors
+//     gates       the subtree's gate ids (4 bits each, fold order) | top gate << 28, the top gate
+//                 with its inputs swapped where the schedule says so
+//     out         the output row times the row length in vectors, 0xffffffff = no output
+// so that a step costs one wide scalar load instead of a chain of dependent ones (vertex ->
+// subtree tables, neuron -> gate id, flip), and every gather is a scalar row base plus the lane's
+// constant 32-bit offset.  Applies when rows * row length and out_dim * row length fit 32 bits.
+// ------------------------------------------------------------------------------------------
+template <int DS> struct alignas(DS == 3 ? 64 : DS == 2 ? 32 : 16) StepRec {
+    uint32_t leaf[1 << DS];
+    uint32_t gates;
+    uint32_t out;
+};
+static_assert(sizeof(StepRec<3>) == 64 && sizeof(StepRec<2>) == 32 && sizeof(StepRec<1>) == 16 && sizeof(StepRec<0>) == 16,
+              "records are whole scalar-load units");
+
+template <int DS>
+__global__ __launch_bounds__(DL_BLOCK) void compose_steps_kernel(const int32_t *__restrict__ sub_leaves,
+                                                                 const uint64_t *__restrict__ sub_gates,
+                                                                 const int32_t *__restrict__ verts,
+                                                                 const int32_t *__restrict__ neuron,
+                                                                 const uint8_t *__restrict__ flip,
+                                                                 const uint8_t *__restrict__ w_top, int64_t steps,
+                                                                 uint32_t ncols, StepRec<DS> *__restrict__ rec) {
+    const int64_t i = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x;      // record index: step i - 1
+    if (i > steps) return;
+    const int64_t v = verts[i];
+    StepRec<DS> r;
+    uint32_t gates = 0;
+    if (DS == 0) {
+        r.leaf[0] = (uint32_t) v * ncols;
+    } else {
+        gates = (uint32_t) sub_gates[v];
+#pragma unroll
+        for (int g = 0; g < (1 << DS); ++g) r.leaf[g] = (uint32_t) sub_leaves[v * (1 << DS) + g] * ncols;
+    }
+    r.out = 0xffffffffu;
+    if (i >= 1 && neuron[i - 1] >= 0) {
+        const int32_t n = neuron[i - 1];
+        uint32_t top = w_top[n] & 15u;
+        if (flip[i - 1]) top = swap_gate_inputs(top);
+        gates |= top << 28;
+        r.out = (uint32_t) n * ncols;
+    }
+    r.gates = gates;
+    rec[i] = r;
+}
+
+// One wave = STEPS consecutive steps x 64 vectors; dispatch order as eval_kernel.  BUF: x is at
+// most 4 GiB and is read through a buffer resource, whose loads take the row's byte offset as a
+// scalar operand next to the lane's constant offset: no vector instruction per gather.
+template <typename V, int DS, int STEPS, bool BUF>
+__global__ __launch_bounds__(DL_BLOCK) void eval_steps_kernel(const V *__restrict__ x, const StepRec<DS> *__restrict__ rec,
+                                                              V *__restrict__ y, int64_t nsteps, int64_t ncols,
+                                                              uint32_t x_bytes) {
+    constexpr int G = 1 << DS;
+    static_assert(STEPS % 2 == 0, "steps are processed in pairs");
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t first = ((int64_t) blockIdx.x * 4 + wave) * STEPS;
+    if (first >= nsteps) return;
+    const StepRec<DS> *wrec = rec + first;                 // [0] = seed, [1 + j] = the wave's step j
+
+    for (int64_t ct = blockIdx.y; ct * DL_WAVE < ncols; ct += gridDim.y) {
+        const uint32_t col = (uint32_t) (ct * DL_WAVE) + (uint32_t) lane;
+        if (col >= ncols) continue;
+        auto row = [&](uint32_t start) -> V {                                  // scalar row base + the lane's offset
+            if constexpr (BUF && sizeof(V) == 16) {
+                const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *) x, 0, (int) x_bytes, 0x00027000);
+                return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int) (col * 16u), (int) (start * 16u), 0));
+            } else {
+                return (x + start)[col];
+            }
+        };
+        V prev;
+        {
+            const StepRec<DS> r = wrec[0];
+            V leaves0[G];
+#pragma unroll
+            for (int g = 0; g < G; ++g) leaves0[g] = row(r.leaf[g]);
+            prev = TreeFold<V, DS>::run(leaves0, r.gates);
+        }
+#pragma unroll 1
+        for (int j = 0; j < STEPS; j += 2) {
+            if (first + j >= nsteps) break;                // the schedule is a whole number of step pairs
+            const StepRec<DS> ra = wrec[1 + j], rb = wrec[2 + j];
+            V la[G], lb[G];
+#pragma unroll
+            for (int g = 0; g < G; ++g) la[g] = row(ra.leaf[g]);
+#pragma unroll
+            for (int g = 0; g < G; ++g) lb[g] = row(rb.leaf[g]);
+            const V va = TreeFold<V, DS>::run(la, ra.gates);
+            const V vb = TreeFold<V, DS>::run(lb, rb.gates);
+            if (ra.out != 0xffffffffu)
+                __builtin_nontemporal_store(gate_apply<V>(prev, va, gate_masks(ra.gates >> 28)), (y + ra.out) + col);
+            if (rb.out != 0xffffffffu)
+                __builtin_nontemporal_store(gate_apply<V>(va, vb, gate_masks(rb.gates >> 28)), (y + rb.out) + col);
+            prev = vb;
+        }
+    }
+}
+
 template <typename V, int NPW, int ITERS>
 int launch_eval(const void *x, const int64_t *a, const int64_t *b, const uint8_t *w, void *y, int64_t out_dim,
                 int64_t row_bytes, hipStream_t stream) {
@@ -1385,6 +1492,39 @@ int launch_eval_chain(int sub_depth, const void *x, const int32_t *sub_leaves, c
     return dl_launch_status();
 }
 
+template <typename V, int DS>
+int launch_eval_steps(const void *x, const int32_t *sub_leaves, const uint64_t *sub_gates, const int32_t *verts,
+                      const int32_t *neuron, const uint8_t *flip, const uint8_t *w_top, void *y, void *records,
+                      int64_t steps, int64_t row_bytes, int64_t x_bytes, hipStream_t s) {
+    constexpr int STEPS = 16;
+    const int64_t ncols = row_bytes / (int64_t) sizeof(V);
+    StepRec<DS> *rec = (StepRec<DS> *) records;
+    DL_LAUNCH(compose_steps_kernel<DS>, dim3((unsigned) dl_ceil_div(steps + 1, DL_BLOCK)), dim3(DL_BLOCK), 0, s, sub_leaves,
+              sub_gates, verts, neuron, flip, w_top, steps, (uint32_t) ncols, rec);
+    const int st = dl_launch_status();
+    if (st != DL_OK) return st;
+    int64_t ctiles = dl_ceil_div(ncols, DL_WAVE);
+    if (ctiles > 65535) ctiles = 65535;
+    const int64_t gx = dl_ceil_div(steps, 4 * STEPS);
+    if (gx > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    const dim3 grid((unsigned) gx, (unsigned) ctiles);
+    if (x_bytes <= 0xffffffffLL)
+        DL_LAUNCH((eval_steps_kernel<V, DS, STEPS, true>), grid, dim3(DL_BLOCK), 0, s, (const V *) x, rec, (V *) y, steps,
+                  ncols, (uint32_t) x_bytes);
+    else
+        DL_LAUNCH((eval_steps_kernel<V, DS, STEPS, false>), grid, dim3(DL_BLOCK), 0, s, (const V *) x, rec, (V *) y, steps,
+                  ncols, 0u);
+    return dl_launch_status();
+}
+
+static int64_t step_record_bytes(int sub_depth) { return sub_depth == 3 ? 64 : sub_depth == 2 ? 32 : 16; }
+
+extern "C" int64_t dl_logic_eval_chained_workspace_bytes(int depth, int64_t sub_dim, int64_t steps) {
+    if (depth < 1 || depth > DL_MAX_FUSE_DEPTH || sub_dim < 0 || steps < 0) return 0;
+    const int64_t tables = depth > 1 ? dl_logic_eval_fused_workspace_bytes(depth - 1, sub_dim) : 0;
+    return ((tables + 63) / 64) * 64 + (steps + 1) * step_record_bytes(depth - 1);
+}
+
 extern "C" int dl_logic_eval_chained(const void *x, int depth, const int64_t *const *a, const int64_t *const *b,
                                      const uint8_t *const *w, const int64_t *dims, const int32_t *verts,
                                      const int32_t *neuron, const uint8_t *flip, int64_t steps, void *y, int64_t words,
@@ -1404,6 +1544,19 @@ extern "C" int dl_logic_eval_chained(const void *x, int depth, const int64_t *co
     if (depth > 1) {                                 // flatten the layers below the top one, per vertex
         const int st = compose_tree(depth - 1, a, b, w, dims, nullptr, workspace, &sub_leaves, &sub_gates, s);
         if (st != DL_OK) return st;
+    }
+    // one record per step where the pre-multiplied row offsets fit 32 bits (16-byte lanes only)
+    const int64_t ncols16 = row_bytes / 16;
+    if (mis % 16 == 0 && workspace && dl_aligned(workspace, 64) && dims[0] * ncols16 < 0xffffffffLL && dims[depth] * ncols16 < 0xffffffffLL) {
+        const int64_t tables = depth > 1 ? dl_logic_eval_fused_workspace_bytes(depth - 1, dims[depth - 1]) : 0;
+        void *records = (char *) workspace + ((tables + 63) / 64) * 64;
+        const uint8_t *w_top = w[depth - 1];
+        switch (depth - 1) {
+        case 0: return launch_eval_steps<dl_u32x4, 0>(x, sub_leaves, sub_gates, verts, neuron, flip, w_top, y, records, steps, row_bytes, dims[0] * row_bytes, s);
+        case 1: return launch_eval_steps<dl_u32x4, 1>(x, sub_leaves, sub_gates, verts, neuron, flip, w_top, y, records, steps, row_bytes, dims[0] * row_bytes, s);
+        case 2: return launch_eval_steps<dl_u32x4, 2>(x, sub_leaves, sub_gates, verts, neuron, flip, w_top, y, records, steps, row_bytes, dims[0] * row_bytes, s);
+        default: return launch_eval_steps<dl_u32x4, 3>(x, sub_leaves, sub_gates, verts, neuron, flip, w_top, y, records, steps, row_bytes, dims[0] * row_bytes, s);
+        }
     }
     const int64_t nchunks = steps / DL_EVAL_SCHEDULE_CHUNK;
     if (mis % 16 == 0)

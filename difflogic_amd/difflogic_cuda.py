@@ -581,7 +581,8 @@ def eval_chained(x, layers, schedule=None):
         raise RuntimeError(f"schedule is for a {schedule.in_dim}->{schedule.out_dim} layer, the group ends in "
                            f"{dims[-2]}->{dims[-1]}")
     y = torch.empty((dims[-1], words), dtype=x.dtype, device=dev)
-    ws = _fused_workspace(depth - 1, dims[-2], dev) if depth > 1 else None
+    nbytes = _lib.load().dl_logic_eval_chained_workspace_bytes(depth, dims[-2], schedule.steps)
+    ws = torch.empty(max(1, -(-nbytes // 8)), dtype=torch.int64, device=dev)      # torch aligns allocations to 512 bytes
     with _on(dev):
         st = _lib.load().dl_logic_eval_chained(_p(x), depth, pa, pb, pw, pdims, _p(schedule.verts), _p(schedule.neuron),
                                                _p(schedule.flip), schedule.steps, _p(y), words, bits,

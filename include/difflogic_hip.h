@@ -219,12 +219,14 @@ int dl_logic_eval_fused(const void *x, int depth, const int64_t *const *a, const
  *                                 neuron [steps] (-1 = no output at this step), flip [steps];
  *                                 returns the number of steps, or a negated dl_status.
  *   dl_logic_eval_chained()       as dl_logic_eval_fused plus the DEVICE schedule arrays; workspace
- *                                 of dl_logic_eval_fused_workspace_bytes(depth-1, dims[depth-1])
- *                                 bytes (none needed for depth 1). */
+ *                                 of dl_logic_eval_chained_workspace_bytes(depth, dims[depth-1],
+ *                                 steps) bytes, 64-byte aligned: the flattened subtrees and one
+ *                                 record per step, both rebuilt by every call. */
 int dl_eval_schedule_chunk(void);
 int64_t dl_eval_schedule_capacity(int64_t out_dim, int chunk);
 int64_t dl_eval_schedule_build(const int64_t *a, const int64_t *b, int64_t in_dim, int64_t out_dim,
                                int chunk, int32_t *verts, int32_t *neuron, uint8_t *flip);
+int64_t dl_logic_eval_chained_workspace_bytes(int depth, int64_t sub_dim, int64_t steps);
 int dl_logic_eval_chained(const void *x, int depth, const int64_t *const *a, const int64_t *const *b,
                           const uint8_t *const *w, const int64_t *dims, const int32_t *verts,
                           const int32_t *neuron, const uint8_t *flip, int64_t steps, void *y,
