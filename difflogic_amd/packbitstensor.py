@@ -5,9 +5,20 @@ import torch
 
 from . import difflogic_cuda
 
-# Inputs with at most this many rows stay resident in the L2 caches while a 1 KB column tile of
-# all neurons is swept, so gathers from them are cheap and deeper fusion pays off.
-_L2_RESIDENT_ROWS = 2048
+# ---------------------------------------------------------------------------------------------
+# Launch planning.  The cost of a fused group is modelled from the bytes it moves through each
+# level of the memory system, at the rates plain kernels with the same access pattern sustain on
+# MI355X (`python bench.py --ceilings`; profiles/ceilings_mi355x.txt), so the plan follows the
+# shapes (rows, widths, words per row) instead of constants fitted to one workload.
+# ---------------------------------------------------------------------------------------------
+_L2_GATHER_RATE = 31e12      # B/s: row gathers + stores through the L2s when the input tile stays L2-resident
+_FABRIC_RATE = 7.5e12        # B/s: row gathers + stores between the L2s and Infinity Cache / HBM
+_WRITE_RATE = 6.1e12         # B/s: streaming stores to HBM
+_COUNT_EFFICIENCY = 0.87     # the count kernels reach this fraction of the fabric rate (barriers between phases)
+_TILE_BYTES = 1024           # one wave covers 64 lanes x 16 bytes of a row
+_L2_RESIDENT_BYTES = 4 << 20     # input tiles (rows x 1 KB each) in flight up to this size are re-read from L2 (4 MB per XCD)
+_LDS_GATE_WORD_SECONDS = 9.4e-13     # LDS-resident whole-net kernel: seconds per gate and 64-sample word
+_LAUNCH_SECONDS = 3e-6       # per kernel on the stream; decides between plans for small batches only
 
 
 def _chained(depth):
@@ -15,57 +26,84 @@ def _chained(depth):
     return depth >= 2
 
 
-def plan_groups(dims, count_at_end):
+def group_cost(rows_in, out, depth, words, counted):
+    """Modelled seconds of one fused group: `depth` layers from `rows_in` input rows to `out` output
+    rows of `words` 64-bit words, ending in the per-class count when `counted`."""
+    row_bytes = 8.0 * words
+    if counted:                                    # walked along the schedule: one seed per 128 steps
+        gathers = (1 << (depth - 1)) * (1 + 1 / 128) * out
+    elif _chained(depth):                          # one seed per 16 steps
+        gathers = (1 << (depth - 1)) * (1 + 1 / 16) * out
+    else:
+        gathers = (1 << depth) * out
+    gathered = gathers * row_bytes
+    written = 0.0 if counted else out * row_bytes
+    # The chip sweeps all output rows of one 1 KB column tile before the next, but a narrow layer
+    # does not fill it: several tiles are then in flight and their input rows share the L2s.
+    steps_per_workgroup = 1024 if counted else 64
+    resident_workgroups = 512 if counted else 2048
+    tiles_in_flight = max(1.0, resident_workgroups * steps_per_workgroup / max(out, 1))
+    hit = min(1.0, _L2_RESIDENT_BYTES / (rows_in * _TILE_BYTES * tiles_in_flight))     # share of gathers served by L2
+    through_l2 = (hit * gathered + written) / _L2_GATHER_RATE
+    beyond_l2 = ((1 - hit) * gathered + written) / (_WRITE_RATE if hit == 1.0 else _FABRIC_RATE)
+    t = max(through_l2, beyond_l2) + 0.3 * min(through_l2, beyond_l2)                  # the two overlap only in part
+    if counted:
+        t /= _COUNT_EFFICIENCY
+        t += 2 * (out / 128.0) * row_bytes / _FABRIC_RATE                # partial counters: written, then read once
+    # kernels on the stream: the per-call table builders, the group's kernel, the count's second pass
+    return t + _LAUNCH_SECONDS * (3 if counted or _chained(depth) else 1)
+
+
+def plan_groups(dims, count_at_end, words=16384):
     """Splits consecutive layers into fused groups.
 
-    ``dims`` = [in_dim, width_1, ..., width_L].  Returns a list of group sizes summing to L; when
-    ``count_at_end`` the last group is the one fused with the bit count.  Chosen by dynamic
-    programming over a traffic model: a group of depth D gathers 2^D rows per output neuron,
-    2^(D-1) when it runs chained, from L2 when its input has few rows and through the memory fabric
-    otherwise, and writes one row per output neuron unless it ends in the count."""
+    ``dims`` = [in_dim, width_1, ..., width_L]; ``words`` = 64-bit words per row.  Returns a list of
+    group sizes summing to L; when ``count_at_end`` the last group is the one fused with the bit
+    count.  Chosen by dynamic programming over group_cost."""
     n = len(dims) - 1
     if n == 0:
         return []
-
-    def cost(first, depth, last):
-        # milliseconds per 64000 rows of 16384 words, fitted to launches measured on MI355X
-        rows_in, out = dims[first], dims[first + depth]
-        counted = last and count_at_end
-        gathers = (1 << depth) * out
-        if _chained(depth) and not counted:
-            gathers = gathers * 9 / 16             # half, plus one extra subtree per chunk of 8
-        written = 0 if counted else out
-        if rows_in <= _L2_RESIDENT_ROWS:           # gathers hit in L2; writes stream to HBM
-            t = max(1.5 * written, 0.3 * gathers + 0.5 * out)
-        else:                                      # L2 <-> fabric traffic, with the HBM copy rate as floor
-            t = max(1.1 * (gathers + written), 1.68 * (rows_in + written))
-        if counted:
-            t += 0.2 * out                         # second pass over the partial counters
-        return t
-
     best = [(0.0, [])] + [None] * n    # best[i] = (cost, groups) for the first i layers
     for i in range(1, n + 1):
         for depth in range(1, min(i, difflogic_cuda.MAX_FUSE_DEPTH) + 1):
-            last = i == n
-            if last and count_at_end and depth > difflogic_cuda.MAX_FUSE_DEPTH_COUNT:
+            counted = i == n and count_at_end
+            if counted and depth > difflogic_cuda.MAX_FUSE_DEPTH_COUNT:
                 continue
             prev = best[i - depth]
-            c = prev[0] + cost(i - depth, depth, last)
+            c = prev[0] + group_cost(dims[i - depth], dims[i], depth, words, counted)
             if best[i] is None or c < best[i][0]:
                 best[i] = (c, prev[1] + [depth])
     return best[n][1]
 
 
-def lds_tail(dims):
-    """Number of layers at the end of the net (``dims`` = [in_dim, width_1, ..., width_L]) that the
-    LDS-resident whole-net kernel takes together with the count: the longest run of trailing layers
-    whose input and widths all fit its buffer, if that run is at least two layers long (a single
-    layer gains nothing over the streaming kernel fused with the count)."""
+def plan_cost(dims, groups, count_at_end, words=16384):
+    """Modelled seconds of running ``groups`` (as plan_groups returns them) over ``dims``."""
+    t, pos = 0.0, 0
+    for j, depth in enumerate(groups):
+        t += group_cost(dims[pos], dims[pos + depth], depth, words, count_at_end and j == len(groups) - 1)
+        pos += depth
+    return t
+
+
+def lds_cost(dims, words):
+    """Modelled seconds of the LDS-resident whole-net kernel over all of ``dims``."""
+    return sum(dims[1:]) * words * _LDS_GATE_WORD_SECONDS + 2 * _LAUNCH_SECONDS
+
+
+def lds_tail(dims, words=16384):
+    """Number of layers at the end of the net (``dims`` = [in_dim, width_1, ..., width_L]) to run
+    in the LDS-resident whole-net kernel together with the count: the longest run of trailing
+    layers whose input and widths all fit its buffer, if the model prices it below the streaming
+    plan for the same layers (0 otherwise)."""
     limit = difflogic_cuda.net_lds_max_width()
     n = 0
     while n < len(dims) - 1 and n < difflogic_cuda.MAX_NET_DEPTH and max(dims[len(dims) - 2 - n:]) <= limit:
         n += 1
-    return n if n >= 2 else 0
+    if n == 0:
+        return 0
+    tail = dims[len(dims) - 1 - n:]
+    streaming = plan_cost(tail, plan_groups(tail, True, words), True, words)
+    return n if lds_cost(tail, words) < streaming else 0
 
 
 class PackBitsTensor:
@@ -98,6 +136,10 @@ class PackBitsTensor:
         """Number of rows ``.t`` has (after the deferred layers)."""
         return self._pending[-1][2].shape[0] if self._pending else self._t.shape[0]
 
+    def _words64(self):
+        """Row length in 64-bit words (what the planner's byte counts are based on)."""
+        return max(1, self._t.shape[1] * self.bit_count // 64)
+
     def _dims(self):
         return [self._t.shape[0]] + [w.shape[0] for _, _, w in self._pending]
 
@@ -112,7 +154,7 @@ class PackBitsTensor:
     @property
     def t(self):
         if self._pending:
-            self._run_groups(plan_groups(self._dims(), count_at_end=False))
+            self._run_groups(plan_groups(self._dims(), False, self._words64()))
         return self._t
 
     @t.setter
@@ -131,16 +173,16 @@ class PackBitsTensor:
             if self.features % k != 0:
                 raise ValueError(f"in_dim ({self.features}) has to be divisible by k ({k}) but it is not")
             dims = self._dims()
-            tail = lds_tail(dims)
+            tail = lds_tail(dims, self._words64())
             if tail:
                 # the narrow end of the net runs resident in LDS; what lies before it streams
                 head = len(self._pending) - tail
                 if head:
-                    self._run_groups(plan_groups(dims[:head + 1], count_at_end=False))
+                    self._run_groups(plan_groups(dims[:head + 1], False, self._words64()))
                 out = difflogic_cuda.eval_net_lds(self._t, self._pending, self.pad_len, k)
                 if out is not None:
                     return out
-            groups = plan_groups(self._dims(), count_at_end=True)
+            groups = plan_groups(self._dims(), True, self._words64())
             self._run_groups(groups[:-1])
             # the last group stays pending: the object's state does not change by counting
             out = difflogic_cuda.eval_chained_groupbitsum(self._t, self._pending, self.pad_len, k)

@@ -443,8 +443,8 @@ def test_pack_tensor_runs_narrow_tail_in_lds(monkeypatch):
     import difflogic_amd as dl
     from difflogic_amd import packbitstensor as pbt
     assert pbt.lds_tail([784, 8000, 8000, 8000]) == 3 and pbt.lds_tail([784, 64000, 64000]) == 0
-    assert pbt.lds_tail([784, 64000, 8000, 8000]) == 0 and pbt.lds_tail([784, 64000, 8000, 8000, 8000]) == 2
-    assert pbt.lds_tail([20000, 8000, 8000]) == 0 and pbt.lds_tail([784, 8000]) == 0
+    assert pbt.lds_tail([784, 64000, 8000, 8000]) == 1 and pbt.lds_tail([784, 64000, 8000, 8000, 8000]) == 2
+    assert pbt.lds_tail([20000, 12000, 12000]) == 0 and pbt.lds_tail([784, 8000]) == 1
     rng = np.random.default_rng(31)
     F, widths = 40, [12000, 6000, 3000, 1500]
     layers = random_layers(rng, F, widths)

@@ -178,3 +178,32 @@ def test_schedules_of_random_multigraphs():
         assert (seen == 1).all()
         if out_dim:
             test_every_input_is_completed_exactly_once("random", in_dim, a, b)
+
+
+def test_launch_plan_follows_the_traffic_model():
+    """plan_groups / lds_tail choose from modelled bytes and measured rates, not from constants
+    fitted to one workload: the plans measured fastest on MI355X for the three packed BASELINE
+    configurations come out, and the model prices them within 25 % of the measured times."""
+    from difflogic_amd import packbitstensor as pbt
+    headline, c2, c4 = [784] + [64000] * 6, [784] + [8000] * 6, [9216] + [256000] * 4
+    assert pbt.plan_groups(headline, True, 16384) == [4, 2] and pbt.lds_tail(headline, 16384) == 0
+    assert pbt.plan_groups(c4, True, 4096) == [2, 2] and pbt.lds_tail(c4, 4096) == 0
+    assert pbt.lds_tail(c2, 16384) == 6                       # the whole narrow net runs resident in LDS
+    # measured launch times in ms (bench.py on MI355X): 4-layer prefix + 2 layers with the count
+    measured = {"headline": (headline, [4, 2], 16384, 2.83 + 2.89), "C4": (c4, [2, 2], 4096, 3.18 + 2.94)}
+    for name, (dims, groups, words, ms) in measured.items():
+        model = pbt.plan_cost(dims, groups, True, words) * 1e3
+        assert abs(model - ms) <= 0.25 * ms, (name, model, ms)
+    assert abs(pbt.lds_cost(c2, 16384) * 1e3 - 0.75) <= 0.25 * 0.75
+    # single groups against their measured times: 784 -> 64000 prefixes of depth 2, 3, 4 and square 64000-wide groups
+    for depth, ms in ((2, 1.50), (3, 1.95), (4, 2.83)):
+        assert abs(pbt.group_cost(784, 64000, depth, 16384, False) * 1e3 - ms) <= 0.25 * ms, depth
+    assert abs(pbt.group_cost(64000, 64000, 1, 16384, False) * 1e3 - 3.37) <= 0.25 * 3.37
+    assert abs(pbt.group_cost(64000, 64000, 2, 16384, False) * 1e3 - 3.71) <= 0.25 * 3.71
+    # the model scales with the row length: the plan of a 16x shorter batch is the same, its cost 16x lower (up to
+    # the per-launch overhead: 6 kernels x 3 us)
+    assert pbt.plan_groups(headline, True, 1024) == [4, 2]
+    assert abs(pbt.plan_cost(headline, [4, 2], True, 1024) * 16 - pbt.plan_cost(headline, [4, 2], True, 16384)) < 6 * 3e-6 * 16
+    # a net whose last layers are narrow hands exactly those to the LDS kernel
+    assert pbt.lds_tail([784, 64000, 8000, 8000, 8000], 16384) == 2
+    assert pbt.plan_groups([784], True) == []
