@@ -65,6 +65,8 @@ def parse():
     ap.add_argument("--no-train", action="store_true", help="skip the training configurations (C1, C3, C5)")
     ap.add_argument("--no-configs", action="store_true", help="skip the other packed configurations (C2, C4)")
     ap.add_argument("--only", default="", help="comma list out of c1,c2,c3,c4,c5: run only these extra configurations")
+    ap.add_argument("--skip-headline", action="store_true",
+                    help="profiling aid: run only the configurations selected with --only and print their results")
     ap.add_argument("--cpu-sample-log2", type=int, default=18)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 4 plain device copies of 1 GiB (for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE)")
@@ -552,46 +554,8 @@ def ceilings(torch):
     return res
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        print("bench.py: this build runs on one GPU only (the path shards along the batch without "
-              "communication); --gpus %d is not supported" % args.gpus, file=sys.stderr)
-        sys.exit(2)
-    import torch
-
-    import difflogic_amd as dl
-    assert torch.cuda.is_available(), "bench.py needs the GPU"
-
-    if args.ceilings:
-        print(json.dumps({"metric": "practical ceilings on this GPU", "unit": "GB/s", "hbm_peak_GBps": HBM_PEAK_GBS,
-                          "device": torch.cuda.get_device_name(0), **ceilings(torch)}))
-        return
-
-    if args.calibrate_copy:
-        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
-        dst = torch.empty_like(src)
-        for _ in range(4):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
-    value, ms, roofline, info, model, x, out = packed_headline(args, torch, dl)
-    result = {
-        "metric": "packed-eval samples/s (784->6x64k)", "value": round(value, 1), "unit": "samples/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int64", "data": "synthetic",
-        "config": {"workload": "packed inference %d->%dx%d->GroupSum(10), batch 2^%d, int64 words, bool input "
-                               "resident in HBM; step = pack + %d gate layers + groupbitsum"
-                               % (args.features, args.layers, args.width, args.batch_log2, args.layers),
-                   "connections": "random", "seed": 0},
-        "roofline": roofline,
-    }
-    result["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(args, model, x, out, dl)
-    extra = dict(info)
-    del model, x, out
-    gc.collect()
-    torch.cuda.empty_cache()
-
+def extra_configs(args, torch, dl):
+    """The other BASELINE configurations (C1 .. C5), each optional."""
     only = {c for c in args.only.lower().split(",") if c}
     want = lambda c, group_off: (c in only) if only else not group_off      # noqa: E731
     configs = {}
@@ -636,7 +600,53 @@ def main():
         del model, x
         if not args.no_cpu_baseline:
             configs["C1"]["cpu_baseline"] = train_cpu_baseline(torch)
-    extra["configs"] = configs
+    return configs
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (the path shards along the batch without "
+              "communication); --gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    import difflogic_amd as dl
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+
+    if args.ceilings:
+        print(json.dumps({"metric": "practical ceilings on this GPU", "unit": "GB/s", "hbm_peak_GBps": HBM_PEAK_GBS,
+                          "device": torch.cuda.get_device_name(0), **ceilings(torch)}))
+        return
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    if args.skip_headline:
+        print(json.dumps({"metric": "extra configurations only (--skip-headline)", "extra": {"configs": extra_configs(args, torch, dl)}}))
+        return
+    value, ms, roofline, info, model, x, out = packed_headline(args, torch, dl)
+    result = {
+        "metric": "packed-eval samples/s (784->6x64k)", "value": round(value, 1), "unit": "samples/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int64", "data": "synthetic",
+        "config": {"workload": "packed inference %d->%dx%d->GroupSum(10), batch 2^%d, int64 words, bool input "
+                               "resident in HBM; step = pack + %d gate layers + groupbitsum"
+                               % (args.features, args.layers, args.width, args.batch_log2, args.layers),
+                   "connections": "random", "seed": 0},
+        "roofline": roofline,
+    }
+    result["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(args, model, x, out, dl)
+    extra = dict(info)
+    del model, x, out
+    gc.collect()
+    torch.cuda.empty_cache()
+
+    extra["configs"] = extra_configs(args, torch, dl)
     result["extra"] = extra
     print(json.dumps(result))
 
