@@ -363,49 +363,58 @@ def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor
                 "alg_GBps": round(alg / sec / 1e9, 1), "frac_hbm_algorithmic": round(alg / sec / 1e9 / HBM_PEAK_GBS, 4),
                 "loss": round(float(loss), 6)}
 
-    def fwd_bwd():
-        model.zero_grad(set_to_none=True)
-        loss = loss_fn(model(x), labels)
-        loss.backward()
-        return loss
-
     res = {"workload": name, "dtype": "f32", "algorithmic_GB_per_step": round(alg / 1e9, 3)}
-    sec, loss = timeit(fwd_bwd)
-    res["fwd_bwd_eager"] = report(sec, loss.item())
-    # Drop every reference to the eager autograd graph before capturing: gradient-accumulation
-    # nodes kept alive by `loss` belong to the default stream and would be replayed into the
-    # capture stream's backward.
-    del loss
-    model.zero_grad(set_to_none=True)
-    gc.collect()
-    torch.cuda.synchronize()
-    graphed = GraphedTrainStep(model, loss_fn, x, labels)
-    sec, loss = timeit(graphed.step)
-    res["fwd_bwd_graph"] = report(sec, loss.item())
-    del graphed, loss
-    gc.collect()
 
-    # with the optimizer step (experiments/main.py:169,174-181).  The weights move, so the loss differs per step.
-    opt = torch.optim.Adam(model.parameters(), lr=0.01, fused=True, capturable=True)
+    def measure(net, out):
+        """forward+backward and forward+backward+Adam of `net`, eager and as a replayed HIP graph."""
+        def fwd_bwd():
+            net.zero_grad(set_to_none=True)
+            loss = loss_fn(net(x), labels)
+            loss.backward()
+            return loss
 
-    def full_step():
+        sec, loss = timeit(fwd_bwd)
+        out["fwd_bwd_eager"] = report(sec, loss.item())
+        # Drop every reference to the eager autograd graph before capturing: gradient-accumulation
+        # nodes kept alive by `loss` belong to the default stream and would be replayed into the
+        # capture stream's backward.
+        del loss
+        net.zero_grad(set_to_none=True)
+        gc.collect()
+        torch.cuda.synchronize()
+        graphed = GraphedTrainStep(net, loss_fn, x, labels)
+        sec, loss = timeit(graphed.step)
+        out["fwd_bwd_graph"] = report(sec, loss.item())
+        del graphed, loss
+        gc.collect()
+
+        # with the optimizer step (experiments/main.py:169,174-181).  The weights move, so the loss differs per step.
+        opt = torch.optim.Adam(net.parameters(), lr=0.01, fused=True, capturable=True)
+
+        def full_step():
+            opt.zero_grad(set_to_none=True)
+            loss = loss_fn(net(x), labels)
+            loss.backward()
+            opt.step()
+            return loss
+
+        sec, loss = timeit(full_step)
+        out["fwd_bwd_adam_eager"] = report(sec, loss.item())
+        del loss
         opt.zero_grad(set_to_none=True)
-        loss = loss_fn(model(x), labels)
-        loss.backward()
-        opt.step()
-        return loss
+        gc.collect()
+        torch.cuda.synchronize()
+        graphed = GraphedTrainStep(net, loss_fn, x, labels, optimizer=opt)
+        sec, loss = timeit(graphed.step)
+        out["fwd_bwd_adam_graph"] = report(sec, loss.item())
+        del graphed, loss, opt
+        gc.collect()
 
-    sec, loss = timeit(full_step)
-    res["fwd_bwd_adam_eager"] = report(sec, loss.item())
-    del loss
-    opt.zero_grad(set_to_none=True)
-    gc.collect()
-    torch.cuda.synchronize()
-    graphed = GraphedTrainStep(model, loss_fn, x, labels, optimizer=opt)
-    sec, loss = timeit(graphed.step)
-    res["fwd_bwd_adam_graph"] = report(sec, loss.item())
-    del graphed, loss, opt
-    gc.collect()
+    # the model as a user of the reference writes it, then with the last LogicLayer and GroupSum merged
+    # (difflogic_amd.fuse_group_sum: same parameters; the Adam steps above moved them, so the losses differ)
+    measure(model, res)
+    res["fused_group_sum"] = {}
+    measure(dl.fuse_group_sum(model).train(), res["fused_group_sum"])
     return res, model
 
 

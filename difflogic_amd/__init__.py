@@ -2,7 +2,8 @@
 
 Same Python API as the reference package (difflogic/__init__.py:1-3): ``LogicLayer``,
 ``GroupSum``, ``PackBitsTensor`` and ``CompiledLogicNet``; ``difflogic_amd.difflogic_cuda`` stands in for the
-reference's extension module of that name.  Importing the package loads
+reference's extension module of that name.  ``fuse_group_sum`` (not in the reference) merges a
+model's last LogicLayer with the GroupSum after it for training.  Importing the package loads
 libdifflogic_hip.so; it raises ImportError if the library has not been built.
 """
 from . import _lib
@@ -10,8 +11,9 @@ from . import _lib
 _lib.load()
 
 from . import difflogic_cuda  # noqa: E402
-from .difflogic import GroupSum, LogicLayer  # noqa: E402
+from .difflogic import FusedLogicLayerGroupSum, GroupSum, LogicLayer, fuse_group_sum  # noqa: E402
 from .packbitstensor import PackBitsTensor  # noqa: E402
 from .compiled_model import CompiledLogicNet  # noqa: E402
 
-__all__ = ["LogicLayer", "GroupSum", "PackBitsTensor", "CompiledLogicNet", "difflogic_cuda"]
+__all__ = ["LogicLayer", "GroupSum", "PackBitsTensor", "CompiledLogicNet", "difflogic_cuda", "fuse_group_sum",
+           "FusedLogicLayerGroupSum"]

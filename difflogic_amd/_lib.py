@@ -40,6 +40,11 @@ SIGNATURES = {
     "dl_group_sum_workspace_bytes": [_i64, _i64, _i64, _int],
     "dl_group_sum_forward": [_vp, _vp, _vp, _i64, _i64, _i64, _dbl, _int, _vp],
     "dl_group_sum_backward": [_vp, _vp, _i64, _i64, _i64, _dbl, _int, _vp],
+    "dl_logic_forward_group_sum": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _dbl, _int, _vp],
+    "dl_logic_backward_logits_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp],
+    "dl_logic_backward_x_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _dbl, _int, _vp],
+    "dl_logic_backward_chained_grouped": [_vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _int, _vp, _vp, _i64, _i64, _vp, _vp,
+                                          _vp, _i64, _i64, _i64, _i64, _dbl, _int, _vp],
     "dl_logic_eval": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "dl_tensor_packbits": [_vp, _vp, _i64, _i64, _int, ctypes.POINTER(_i64), _vp],
     "dl_tensor_packbits_batch_major": [_vp, _vp, _i64, _i64, _int, ctypes.POINTER(_i64), _vp],

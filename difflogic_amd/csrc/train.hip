@@ -151,6 +151,14 @@ __device__ __forceinline__ double row16_max(double v) {
     return v;
 }
 
+// Row of the gradient matrix that belongs to neuron n.  gdiv == 0: grad_y is [out_dim, batch] and
+// the row is n.  gdiv > 0: the layer feeds a GroupSum and grad_y is its [k, batch] gradient (already
+// divided by tau): all gdiv = out_dim / k neurons of a class share one row, and the broadcast
+// [out_dim, batch] matrix is never materialised.
+__device__ __forceinline__ int64_t grad_row(int64_t n, int64_t gdiv) {
+    return gdiv ? (int64_t) ((uint32_t) n / (uint32_t) gdiv) : n;
+}
+
 // Corner coefficients of FOUR neurons at once: the 16-lane row r of the wave works on neuron n[r]
 // (n[r] < 0: none), lane i of the row on gate i.  LOGITS: `w` holds logits, the row computes their
 // softmax (and stores it to `probs` if asked); otherwise `w` holds the probabilities.  The corner
@@ -273,7 +281,8 @@ template <typename T, int VEC, int NPW, int WPN>
 __global__ __launch_bounds__(DL_BLOCK) void backward_w_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
                                                               const int64_t *__restrict__ b,
                                                               const T *__restrict__ gy, const T *__restrict__ probs,
-                                                              T *__restrict__ gw, int64_t out_dim, int64_t ncols) {
+                                                              T *__restrict__ gw, int64_t out_dim, int64_t ncols,
+                                                              int64_t gdiv) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
     __shared__ C partial[4][NPW][4];
@@ -290,9 +299,10 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_w_kernel(const T *__restric
         int64_t ia[NPW], ib[NPW], nn[NPW];
 #pragma unroll
         for (int j = 0; j < NPW; ++j) {
-            nn[j] = (n0 + j < out_dim) ? n0 + j : out_dim - 1;
-            ia[j] = a[nn[j]];
-            ib[j] = b[nn[j]];
+            const int64_t n = (n0 + j < out_dim) ? n0 + j : out_dim - 1;
+            ia[j] = a[n];
+            ib[j] = b[n];
+            nn[j] = grad_row(n, gdiv);
         }
         const P *xv = reinterpret_cast<const P *>(x);
         const P *gv = reinterpret_cast<const P *>(gy);
@@ -369,7 +379,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_x_kernel(const T *__restric
                                                               const int64_t *__restrict__ start,
                                                               const int64_t *__restrict__ idx, T *__restrict__ gx,
                                                               int64_t in_dim, int64_t ncols,
-                                                              typename Acc<T>::type scale) {
+                                                              typename Acc<T>::type scale, int64_t gdiv) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
     const int wave = dl_wave_in_block();
@@ -391,8 +401,8 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_x_kernel(const T *__restric
             const int64_t nA = idx[e], nB = two ? idx[e + 1] : nA;
             const int64_t iaA = a[nA], ibA = b[nA], iaB = a[nB], ibB = b[nB];
             const bool isaA = iaA == c, isaB = iaB == c;
-            const P gA = gv[nA * ncols + col], oA = xv[(isaA ? ibA : iaA) * ncols + col];
-            const P gB = gv[nB * ncols + col], oB = xv[(isaB ? ibB : iaB) * ncols + col];
+            const P gA = gv[grad_row(nA, gdiv) * ncols + col], oA = xv[(isaA ? ibA : iaA) * ncols + col];
+            const P gB = gv[grad_row(nB, gdiv) * ncols + col], oB = xv[(isaB ? ibB : iaB) * ncols + col];
             const Corners<C> kA = corners<T>(w, nA), kB = corners<T>(w, nB);
             {
                 const C d0 = kA.p01 - kA.p00, d1 = kA.p11 - kA.p10, dd = d1 - d0, da = kA.p10 - kA.p00;
@@ -549,7 +559,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_w_chain_kernel(const T *__r
                                                                     const uint8_t *__restrict__ flip,
                                                                     const T *__restrict__ gy,
                                                                     const T *__restrict__ probs, T *__restrict__ gw,
-                                                                    int64_t nchunks, int64_t ncols) {
+                                                                    int64_t nchunks, int64_t ncols, int64_t gdiv) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
     const int wave = dl_wave_in_block();
@@ -578,7 +588,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_w_chain_kernel(const T *__r
         const bool f = flip[s0 + j] != 0;
         P cur[CPL], g[CPL];
         load_row(xv, verts[s0 + j + 1], cur);
-        load_row(gv, n >= 0 ? n : 0, g);
+        load_row(gv, grad_row(n >= 0 ? n : 0, gdiv), g);
         C s00 = (C) 0, s01 = (C) 0, s10 = (C) 0, s11 = (C) 0;
 #pragma unroll
         for (int q = 0; q < CPL; ++q) {
@@ -622,7 +632,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
     const uint8_t *__restrict__ flip, const int32_t *__restrict__ dst, const T *__restrict__ w,
     const T *__restrict__ gy, const T *__restrict__ probs, T *__restrict__ gw,
     typename Acc<T>::type *__restrict__ partial, T *__restrict__ gx, T *__restrict__ overflow, int64_t steps, int chunk,
-    int64_t in_dim, int64_t out_dim, int64_t ncols, typename Acc<T>::type scale) {
+    int64_t in_dim, int64_t out_dim, int64_t ncols, typename Acc<T>::type scale, int64_t gdiv) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
     const int wave = dl_wave_in_block();
@@ -670,7 +680,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
         const bool f = flip[s0 - 1] != 0;
         P before[CPL], g[CPL];
         load_row(xv, verts[s0 - 1], true, before);
-        load_row(gv, n, true, g);
+        load_row(gv, grad_row(n, gdiv), true, g);
         const Corners<C> k = corners<T>(w, n);
         const C d0 = k.p01 - k.p00, dd = (k.p11 - k.p10) - d0, da = k.p10 - k.p00;
         const C kv = f ? da : d0;
@@ -696,7 +706,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
         const bool valid = n >= 0;
         const int64_t nn = valid ? n : 0;
         load_row(xv, __builtin_amdgcn_readlane(sch_v, i), true, row);
-        load_row(gv, nn, valid, grad);
+        load_row(gv, grad_row(nn, gdiv), valid, grad);
         prob = up<T>(w[nn * 16 + gate]);
     };
     P cur[CPL], g[CPL];
@@ -855,7 +865,7 @@ int forward_t(const void *x, const int64_t *a, const int64_t *b, const void *w, 
 
 template <typename T>
 int backward_w_t(const void *x, const int64_t *a, const int64_t *b, const void *gy, const void *probs, void *gw,
-                 int64_t out_dim, int64_t batch, hipStream_t s) {
+                 int64_t out_dim, int64_t batch, hipStream_t s, int64_t gdiv = 0) {
     constexpr int NPW = 2;
     constexpr int V = Vec16<T>::n;
     const bool vec = batch % V == 0 && dl_aligned(x, 16) && dl_aligned(gy, 16);
@@ -868,20 +878,20 @@ int backward_w_t(const void *x, const int64_t *a, const int64_t *b, const void *
     const T *xp = (const T *) x, *gp = (const T *) gy, *pp = (const T *) probs;
     T *wp = (T *) gw;
     if (vec && split)
-        DL_LAUNCH((backward_w_kernel<T, V, NPW, 4>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols);
+        DL_LAUNCH((backward_w_kernel<T, V, NPW, 4>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv);
     else if (vec)
-        DL_LAUNCH((backward_w_kernel<T, V, NPW, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols);
+        DL_LAUNCH((backward_w_kernel<T, V, NPW, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv);
     else if (split)
-        DL_LAUNCH((backward_w_kernel<T, 1, NPW, 4>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols);
+        DL_LAUNCH((backward_w_kernel<T, 1, NPW, 4>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv);
     else
-        DL_LAUNCH((backward_w_kernel<T, 1, NPW, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols);
+        DL_LAUNCH((backward_w_kernel<T, 1, NPW, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv);
     return dl_launch_status();
 }
 
 template <typename T>
 int backward_x_t(const void *x, const int64_t *a, const int64_t *b, const void *w, const void *gy,
                  const int64_t *start, const int64_t *idx, void *gx, int64_t in_dim, int64_t batch, double scale,
-                 hipStream_t s) {
+                 hipStream_t s, int64_t gdiv = 0) {
     typedef typename Acc<T>::type C;
     constexpr int V = Vec16<T>::n;
     const int64_t blocks = dl_ceil_div(in_dim, 4);
@@ -889,11 +899,11 @@ int backward_x_t(const void *x, const int64_t *a, const int64_t *b, const void *
     if (batch % V == 0 && dl_aligned(x, 16) && dl_aligned(gy, 16) && dl_aligned(gx, 16)) {
         DL_LAUNCH((backward_x_kernel<T, V>), dim3((unsigned) blocks, col_tiles(batch / V)), dim3(DL_BLOCK), 0, s,
                            (const T *) x, a, b, (const T *) w, (const T *) gy, start, idx, (T *) gx, in_dim, batch / V,
-                           (C) scale);
+                           (C) scale, gdiv);
     } else {
         DL_LAUNCH((backward_x_kernel<T, 1>), dim3((unsigned) blocks, col_tiles(batch)), dim3(DL_BLOCK), 0, s,
                            (const T *) x, a, b, (const T *) w, (const T *) gy, start, idx, (T *) gx, in_dim, batch,
-                           (C) scale);
+                           (C) scale, gdiv);
     }
     return dl_launch_status();
 }
@@ -941,6 +951,76 @@ __global__ __launch_bounds__(DL_BLOCK) void group_sum_partial_kernel(const T *__
     for (int e = 0; e < VEC; ++e) lds[wave][lane * VEC + e] = acc[e];
     __syncthreads();
     if (wave == 0 && col < ncols) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const int i = lane * VEC + e;
+            const C sum = (lds[0][i] + lds[1][i]) + (lds[2][i] + lds[3][i]);
+            partial[((int64_t) split * k + cls) * (ncols * VEC) + col * VEC + e] = sum;
+        }
+    }
+}
+
+// The last LogicLayer and GroupSum in one pass: pass 1 of the sum above with the rows computed on
+// the fly, y[n, r] = layer(x)[n, r] for the neurons of the class block, so the layer's output
+// (and, in the backward pass, the broadcast gradient) never exists in memory.  Grid and partial
+// layout as group_sum_partial_kernel; a wave takes four consecutive neurons at a time (their
+// corner coefficients are computed together), the workgroup's waves interleave groups of four.
+// LOGITS: `w` holds logits; the probabilities go to `probs` (column tile 0 only).
+template <typename T, int VEC, bool LOGITS>
+__global__ __launch_bounds__(DL_BLOCK) void forward_group_sum_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
+                                                                     const int64_t *__restrict__ b, const T *__restrict__ w,
+                                                                     T *__restrict__ probs,
+                                                                     typename Acc<T>::type *__restrict__ partial,
+                                                                     int64_t per_class, int64_t ncols, int64_t k,
+                                                                     int64_t rows_per_split) {
+    typedef typename Acc<T>::type C;
+    typedef Pack<T, VEC> P;
+    __shared__ C lds[4][DL_WAVE * VEC];
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t col = (int64_t) blockIdx.x * DL_WAVE + lane;
+    const bool live = col < ncols;
+    const int64_t cls = blockIdx.y, split = blockIdx.z;
+    int64_t r0 = split * rows_per_split, r1 = r0 + rows_per_split;
+    if (r1 > per_class) r1 = per_class;
+    const P *xv = reinterpret_cast<const P *>(x) + (live ? col : 0);
+    C acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = (C) 0;
+    for (int64_t r = r0 + 4 * wave; r < r1; r += 16) {           // uniform per wave
+        int64_t ia[4], ib[4];
+        int32_t ids[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const bool valid = r + j < r1;
+            const int64_t n = cls * per_class + (valid ? r + j : r);
+            ia[j] = a[n];
+            ib[j] = b[n];
+            ids[j] = valid ? (int32_t) n : -1;
+        }
+        C p00[4], p10[4], d0[4], d1[4];
+        corners4<T, LOGITS>(w, ids, lane, blockIdx.x == 0, probs, p00, p10, d0, d1);
+        P va[4], vb[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            va[j] = xv[ia[j] * ncols];
+            vb[j] = xv[ib[j] * ncols];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (ids[j] >= 0) {                                   // uniform
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    // rounded to T like the stored activation would have been
+                    acc[e] += up<T>(down<T, C>(mix<C>(up<T>(va[j].v[e]), up<T>(vb[j].v[e]), p00[j], p10[j], d0[j], d1[j])));
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) lds[wave][lane * VEC + e] = acc[e];
+    __syncthreads();
+    if (wave == 0 && live) {
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
             const int i = lane * VEC + e;
@@ -1043,6 +1123,39 @@ int group_sum_backward_t(const void *g, void *gx, int64_t out_dim, int64_t batch
     return dl_launch_status();
 }
 
+int group_sum_splits(int64_t out_dim, int64_t batch, int64_t k);
+
+template <typename T>
+int forward_group_sum_t(const void *x, const int64_t *a, const int64_t *b, const void *w, void *probs, void *y,
+                        void *workspace, int64_t out_dim, int64_t batch, int64_t k, double tau, hipStream_t s) {
+    typedef typename Acc<T>::type C;
+    constexpr int V = Vec16<T>::n;
+    const int splits = group_sum_splits(out_dim, batch, k);
+    const int64_t per_class = out_dim / k;
+    const int64_t rows_per_split = dl_ceil_div(dl_ceil_div(per_class, splits), 16) * 16;     // whole groups of four per wave
+    const bool vec = batch % V == 0 && dl_aligned(x, 16);
+    const int64_t ncols = vec ? batch / V : batch;
+    const int64_t gx = dl_ceil_div(ncols, DL_WAVE);
+    if (gx > 0x7fffffffLL || k > 65535 || out_dim > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    const dim3 grid((unsigned) gx, (unsigned) k, (unsigned) splits);
+    const T *xp = (const T *) x, *wp = (const T *) w;
+#define DL_LAUNCH_FGS(VV, LG)                                                                                               \
+    DL_LAUNCH((forward_group_sum_kernel<T, VV, LG>), grid, dim3(DL_BLOCK), 0, s, xp, a, b, wp, (T *) probs, (C *) workspace, \
+              per_class, ncols, k, rows_per_split)
+    if (vec && probs) DL_LAUNCH_FGS(V, true);
+    else if (vec) DL_LAUNCH_FGS(V, false);
+    else if (probs) DL_LAUNCH_FGS(1, true);
+    else DL_LAUNCH_FGS(1, false);
+#undef DL_LAUNCH_FGS
+    int st = dl_launch_status();
+    if (st != DL_OK) return st;
+    const int64_t blocks = dl_ceil_div(batch, DL_WAVE);
+    if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    DL_LAUNCH((group_sum_finish_kernel<T>), dim3((unsigned) blocks, (unsigned) k), dim3(DL_BLOCK), 0, s,
+                       (const C *) workspace, (T *) y, batch, k, splits, (C) (1.0 / tau));
+    return dl_launch_status();
+}
+
 // Number of row splits per class: enough workgroups to fill the chip, at least 64 rows each.
 int group_sum_splits(int64_t out_dim, int64_t batch, int64_t k) {
     const int64_t per_class = out_dim / k;
@@ -1109,7 +1222,7 @@ int forward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, 
 
 template <typename T>
 int backward_w_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, const uint8_t *flip, int64_t steps,
-                       const void *gy, const void *probs, void *gw, int64_t batch, hipStream_t s) {
+                       const void *gy, const void *probs, void *gw, int64_t batch, hipStream_t s, int64_t gdiv = 0) {
     constexpr int V = Vec16<T>::n;
     if (batch % V != 0 || !dl_aligned(x, 16) || !dl_aligned(gy, 16)) return DL_ERR_TOO_LARGE;
     const int64_t nchunks = steps / DL_TRAIN_CHUNK, ncols = batch / V;
@@ -1119,13 +1232,13 @@ int backward_w_chain_t(const void *x, const int32_t *verts, const int32_t *neuro
     const T *xp = (const T *) x, *gp = (const T *) gy, *pp = (const T *) probs;
     if (ncols <= DL_WAVE)
         DL_LAUNCH((backward_w_chain_kernel<T, V, 1, DL_TRAIN_CHUNK>), grid, block, 0, s, xp, verts, neuron, flip,
-                           gp, pp, (T *) gw, nchunks, ncols);
+                           gp, pp, (T *) gw, nchunks, ncols, gdiv);
     else if (ncols <= 2 * DL_WAVE)
         DL_LAUNCH((backward_w_chain_kernel<T, V, 2, DL_TRAIN_CHUNK>), grid, block, 0, s, xp, verts, neuron, flip,
-                           gp, pp, (T *) gw, nchunks, ncols);
+                           gp, pp, (T *) gw, nchunks, ncols, gdiv);
     else
         DL_LAUNCH((backward_w_chain_kernel<T, V, 4, DL_TRAIN_CHUNK>), grid, block, 0, s, xp, verts, neuron, flip,
-                           gp, pp, (T *) gw, nchunks, ncols);
+                           gp, pp, (T *) gw, nchunks, ncols, gdiv);
     return dl_launch_status();
 }
 
@@ -1139,7 +1252,7 @@ template <typename T>
 int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, const uint8_t *flip, const int32_t *dst,
                      int64_t steps, const void *w, const void *gy, bool softmax_backward, const int32_t *fix_vertex,
                      const int32_t *fix_start, int64_t n_fix, int64_t overflow_rows, void *gw, void *gx, void *workspace,
-                     int64_t in_dim, int64_t out_dim, int64_t batch, double scale, hipStream_t s) {
+                     int64_t in_dim, int64_t out_dim, int64_t batch, double scale, hipStream_t s, int64_t gdiv = 0) {
     typedef typename Acc<T>::type C;
     constexpr int V = Vec16<T>::n;
     if (batch % V != 0 || !dl_aligned(x, 16) || !dl_aligned(gy, 16) || !dl_aligned(gx, 16) || !dl_aligned(workspace, 16))
@@ -1160,7 +1273,7 @@ int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron,
     constexpr int H = V >= 2 ? V / 2 : 1;
 #define DL_LAUNCH_BACKWARD_CHAIN(VV, CPL, NC)                                                                              \
     DL_LAUNCH((backward_chain_kernel<T, VV, CPL>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp, pp, (T *) gw, \
-              partial, (T *) gx, overflow, steps, chunk, in_dim, out_dim, NC, (C) scale)
+              partial, (T *) gx, overflow, steps, chunk, in_dim, out_dim, NC, (C) scale, gdiv)
     if (V >= 2 && ncols <= DL_WAVE / 2)
         DL_LAUNCH_BACKWARD_CHAIN(H, 1, 2 * ncols);   // short rows: 8-byte vectors use all 64 lanes
     else if (ncols <= DL_WAVE)
@@ -1377,6 +1490,90 @@ extern "C" int dl_group_sum_backward(const void *grad_y, void *grad_x, int64_t o
     case DL_F16: return group_sum_backward_t<__half>(grad_y, grad_x, out_dim, batch, k, tau, s);
     case DL_F32: return group_sum_backward_t<float>(grad_y, grad_x, out_dim, batch, k, tau, s);
     default: return group_sum_backward_t<double>(grad_y, grad_x, out_dim, batch, k, tau, s);
+    }
+}
+
+// ---- the last LogicLayer fused with GroupSum (training mode) --------------------------------
+
+extern "C" int dl_logic_forward_group_sum(const void *x, const int64_t *a, const int64_t *b, const void *w, void *probs,
+                                          void *y, void *workspace, int64_t in_dim, int64_t out_dim, int64_t batch,
+                                          int64_t k, double tau, int dtype, void *stream) {
+    if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
+    if (in_dim <= 0 || out_dim <= 0 || batch <= 0 || k <= 0 || !(tau != 0.0)) return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim % k != 0) return DL_ERR_NOT_DIVISIBLE;
+    if (!x || !a || !b || !w || !y || !workspace) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    switch (dtype) {
+    case DL_F16: return forward_group_sum_t<__half>(x, a, b, w, probs, y, workspace, out_dim, batch, k, tau, s);
+    case DL_F32: return forward_group_sum_t<float>(x, a, b, w, probs, y, workspace, out_dim, batch, k, tau, s);
+    default: return forward_group_sum_t<double>(x, a, b, w, probs, y, workspace, out_dim, batch, k, tau, s);
+    }
+}
+
+static int grouped_args(int64_t in_dim, int64_t out_dim, int64_t batch, int64_t k, int dtype) {
+    if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
+    if (in_dim <= 0 || out_dim <= 0 || batch <= 0 || k <= 0) return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim % k != 0) return DL_ERR_NOT_DIVISIBLE;
+    if (out_dim > 0xffffffffLL) return DL_ERR_TOO_LARGE;          // class of a neuron by 32-bit division
+    return DL_OK;
+}
+
+extern "C" int dl_logic_backward_logits_grouped(const void *x, const int64_t *a, const int64_t *b, const void *grad_cls,
+                                                const void *probs, void *grad_w, int64_t in_dim, int64_t out_dim,
+                                                int64_t batch, int64_t k, int dtype, void *stream) {
+    const int st = grouped_args(in_dim, out_dim, batch, k, dtype);
+    if (st != DL_OK) return st;
+    if (!x || !a || !b || !grad_cls || !grad_w) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    const int64_t per_class = out_dim / k;
+    switch (dtype) {
+    case DL_F16: return backward_w_t<__half>(x, a, b, grad_cls, probs, grad_w, out_dim, batch, s, per_class);
+    case DL_F32: return backward_w_t<float>(x, a, b, grad_cls, probs, grad_w, out_dim, batch, s, per_class);
+    default: return backward_w_t<double>(x, a, b, grad_cls, probs, grad_w, out_dim, batch, s, per_class);
+    }
+}
+
+extern "C" int dl_logic_backward_x_grouped(const void *x, const int64_t *a, const int64_t *b, const void *w,
+                                           const void *grad_cls, const int64_t *start, const int64_t *idx, void *grad_x,
+                                           int64_t in_dim, int64_t out_dim, int64_t batch, int64_t k, double scale,
+                                           int dtype, void *stream) {
+    const int st = grouped_args(in_dim, out_dim, batch, k, dtype);
+    if (st != DL_OK) return st;
+    if (!x || !a || !b || !w || !grad_cls || !start || !idx || !grad_x) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    const int64_t per_class = out_dim / k;
+    switch (dtype) {
+    case DL_F16: return backward_x_t<__half>(x, a, b, w, grad_cls, start, idx, grad_x, in_dim, batch, scale, s, per_class);
+    case DL_F32: return backward_x_t<float>(x, a, b, w, grad_cls, start, idx, grad_x, in_dim, batch, scale, s, per_class);
+    default: return backward_x_t<double>(x, a, b, w, grad_cls, start, idx, grad_x, in_dim, batch, scale, s, per_class);
+    }
+}
+
+extern "C" int dl_logic_backward_chained_grouped(const void *x, const int32_t *verts, const int32_t *neuron,
+                                                 const uint8_t *flip, const int32_t *dst, int64_t steps, const void *w,
+                                                 const void *grad_cls, int softmax_backward, const int32_t *fix_vertex,
+                                                 const int32_t *fix_start, int64_t n_fix, int64_t overflow_rows,
+                                                 void *grad_w, void *grad_x, void *workspace, int64_t in_dim,
+                                                 int64_t out_dim, int64_t batch, int64_t k, double scale, int dtype,
+                                                 void *stream) {
+    const int st = grouped_args(in_dim, out_dim, batch, k, dtype);
+    if (st != DL_OK) return st;
+    if (steps < out_dim || n_fix < 0 || n_fix > in_dim || overflow_rows < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (!x || !verts || !neuron || !flip || !dst || !w || !grad_cls || !grad_w || !grad_x) return DL_ERR_INVALID_ARGUMENT;
+    if (n_fix > 0 && (!fix_vertex || !fix_start)) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    const bool sb = softmax_backward != 0;
+    const int64_t per_class = out_dim / k;
+    switch (dtype) {
+    case DL_F16:
+        return backward_chain_t<__half>(x, verts, neuron, flip, dst, steps, w, grad_cls, sb, fix_vertex, fix_start, n_fix,
+                                        overflow_rows, grad_w, grad_x, workspace, in_dim, out_dim, batch, scale, s, per_class);
+    case DL_F32:
+        return backward_chain_t<float>(x, verts, neuron, flip, dst, steps, w, grad_cls, sb, fix_vertex, fix_start, n_fix,
+                                       overflow_rows, grad_w, grad_x, workspace, in_dim, out_dim, batch, scale, s, per_class);
+    default:
+        return backward_chain_t<double>(x, verts, neuron, flip, dst, steps, w, grad_cls, sb, fix_vertex, fix_start, n_fix,
+                                        overflow_rows, grad_w, grad_x, workspace, in_dim, out_dim, batch, scale, s, per_class);
     }
 }
 

@@ -247,3 +247,88 @@ class GroupSumCudaFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_y):
         return difflogic_cuda.group_sum_backward(grad_y.contiguous(), ctx.out_dim, ctx.tau), None, None
+
+
+class LogicLayerGroupSumFunction(torch.autograd.Function):
+    """The last LogicLayer and the GroupSum after it as one autograd node: feature-major input
+    [in, B] and gate logits -> class scores [B, k].  Neither the layer's [out, B] output nor the
+    broadcast gradient GroupSum's backward would return is ever materialised."""
+
+    @staticmethod
+    def forward(ctx, x, a, b, logits, given_x_indices_of_y_start, given_x_indices_of_y, grad_factor, schedule, k, tau):
+        y, probs = difflogic_cuda.forward_group_sum(x, a, b, logits.detach().contiguous(), k, tau)
+        ctx.save_for_backward(x, a, b, probs, given_x_indices_of_y_start, given_x_indices_of_y)
+        ctx.grad_factor, ctx.schedule, ctx.tau = grad_factor, schedule, tau
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        x, a, b, probs, start, idx = ctx.saved_tensors
+        grad_cls = (grad_y / ctx.tau).t().contiguous()                 # [k, B]: a few KB
+        grad_logits, grad_x = difflogic_cuda.backward_group_sum(
+            x, a, b, probs, grad_cls, start, idx, ctx.schedule, ctx.grad_factor,
+            want_x=ctx.needs_input_grad[0], want_w=ctx.needs_input_grad[3])
+        return grad_x, None, None, grad_logits, None, None, None, None, None, None
+
+
+class FusedLogicLayerGroupSum(torch.nn.Module):
+    """``GroupSum(LogicLayer(x))`` as one module (see fuse_group_sum).  Holds the two original
+    modules; the LogicLayer's ``weights`` stay registered under their own name, so the
+    state_dict of a fused ``nn.Sequential`` has the keys of the unfused one.  Takes the fused kernels
+    in training mode on float inputs; everything else (eval mode, PackBitsTensor, dtypes that
+    differ from the weights') runs the two modules one after the other."""
+
+    def __init__(self, layer: LogicLayer, group_sum: GroupSum):
+        super().__init__()
+        assert isinstance(layer, LogicLayer) and isinstance(group_sum, GroupSum)
+        self.weights = layer.weights                                    # same Parameter, same key as before
+        object.__setattr__(self, "layer", layer)                        # not registered: no second state_dict entry
+        object.__setattr__(self, "group_sum", group_sum)
+
+    def train(self, mode=True):
+        self.layer.train(mode)
+        self.group_sum.train(mode)
+        return super().train(mode)
+
+    def _apply(self, fn, recurse=True):
+        self.layer._apply(fn)
+        self.group_sum._apply(fn)
+        super()._apply(fn, recurse)
+        self.weights = self.layer.weights
+        return self
+
+    def forward(self, x):
+        layer, gs = self.layer, self.group_sum
+        if (isinstance(x, PackBitsTensor) or not self.training or layer.implementation != "cuda" or not x.is_cuda
+                or x.ndim != 2 or x.dtype != layer.weights.dtype or x.shape[0] == 0 or layer.out_dim % gs.k != 0
+                or gs.k > GroupSum._HIP_MAX_K):
+            return gs(layer(x))
+        xt = x.transpose(0, 1).contiguous()
+        assert xt.shape[0] == layer.in_dim, (xt.shape, layer.in_dim)
+        a, b = layer.indices
+        return LogicLayerGroupSumFunction.apply(xt, a, b, layer.weights, layer.given_x_indices_of_y_start,
+                                                layer.given_x_indices_of_y, float(layer.grad_factor),
+                                                layer._train_schedule(), int(gs.k), float(gs.tau))
+
+    def extra_repr(self):
+        return "{}, {}".format(self.layer.extra_repr(), self.group_sum.extra_repr())
+
+
+class _GroupSumDone(torch.nn.Module):
+    """Stands where the GroupSum stood after fuse_group_sum: the module before it already summed."""
+
+    def forward(self, x):
+        return x
+
+
+def fuse_group_sum(model: torch.nn.Sequential) -> torch.nn.Sequential:
+    """Returns a ``nn.Sequential`` in which every ``LogicLayer`` directly followed by a ``GroupSum``
+    (normally the model's last two modules) is replaced by one fused module, which in training
+    saves writing and re-reading the layer's output and GroupSum's broadcast gradient.  Module
+    positions, parameters and state_dict keys are unchanged; the input model is not modified and
+    shares its parameters with the result."""
+    mods = list(model)
+    for i in range(len(mods) - 1):
+        if isinstance(mods[i], LogicLayer) and isinstance(mods[i + 1], GroupSum) and mods[i].implementation == "cuda":
+            mods[i], mods[i + 1] = FusedLogicLayerGroupSum(mods[i], mods[i + 1]), _GroupSumDone()
+    return torch.nn.Sequential(*mods)

@@ -767,6 +767,89 @@ def eval_fused_groupbitsum_noalloc(x, layers, pad_len, k, out, order=None):
     return out
 
 
+def forward_group_sum(x, a, b, logits, k, tau):
+    """``group_sum_forward(forward_logits(x, a, b, logits)[0], k, tau)`` without the layer's output
+    ever being written: returns (sums [B, k], probs [out, 16]).  Not part of the reference's
+    extension."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (logits, "logits")):
+        _check_input(t, n)
+    code = _float_code(x, "logic_layer_cuda_forward")
+    if x.dim() != 2 or logits.dim() != 2 or logits.shape[1] != 16 or logits.dtype != x.dtype or 0 in x.shape:
+        raise RuntimeError(f"expected x [in>0,B>0] and logits [out,16] of one dtype, got {tuple(x.shape)} {x.dtype}, "
+                           f"{tuple(logits.shape)} {logits.dtype}")
+    out_dim = logits.shape[0]
+    if k <= 0 or out_dim == 0 or out_dim % k != 0:
+        raise ValueError(f"in_dim ({out_dim}) has to be divisible by k ({k}) but it is not")
+    _check_index(a, "a", out_dim)
+    _check_index(b, "b", out_dim)
+    dev = _same_device(x, a, b, logits)
+    in_dim, batch = x.shape
+    lib = _lib.load()
+    y = torch.empty((batch, k), dtype=x.dtype, device=dev)
+    probs = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
+    ws = torch.empty(max(1, lib.dl_group_sum_workspace_bytes(out_dim, batch, k, code)), dtype=torch.uint8, device=dev)
+    with _on(dev):
+        st = lib.dl_logic_forward_group_sum(_p(x), _p(a), _p(b), _p(logits), _p(probs), _p(y), _p(ws), in_dim, out_dim,
+                                            batch, int(k), float(tau), code, _stream(dev))
+    if st:
+        _raise(st, "logic_layer_cuda_forward_group_sum")
+    return y, probs
+
+
+def backward_group_sum(x, a, b, probs, grad_cls, start, idx, schedule, scale, want_x, want_w):
+    """Gradients of forward_group_sum: ``grad_cls`` [k, B] is the gradient of the sums, transposed
+    and already divided by tau; every neuron of class c sees row c as its grad_y (the broadcast
+    matrix is never built).  Returns (grad_logits or None, grad_x or None)."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (probs, "probs"), (grad_cls, "grad_cls")):
+        _check_input(t, n)
+    code = _float_code(x, "logic_layer_cuda_backward")
+    in_dim, batch = x.shape
+    out_dim = probs.shape[0]
+    k = grad_cls.shape[0]
+    if grad_cls.shape != (k, batch) or grad_cls.dtype != x.dtype or probs.shape != (out_dim, 16) or out_dim % k:
+        raise RuntimeError(f"expected grad_cls [k,B] and probs [out,16] of x's dtype, got {tuple(grad_cls.shape)}, "
+                           f"{tuple(probs.shape)}")
+    dev = _same_device(x, a, b, probs, grad_cls)
+    lib = _lib.load()
+    if want_x and want_w and schedule is not None:
+        _check_schedule(schedule, in_dim, out_dim, dev)
+        dst, fix_vertex, fix_start, n_fix, rows = schedule.backward_plan()
+        if rows <= in_dim * BACKWARD_CHAIN_MAX_OVERFLOW:
+            grad_w = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
+            grad_x = torch.empty_like(x)
+            ws_bytes = lib.dl_logic_backward_chained_workspace_bytes(rows, out_dim, batch, code)
+            if ws_bytes < 0:
+                _raise(-ws_bytes, "logic_layer_cuda_backward_chained")
+            workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+            with _on(dev):
+                st = lib.dl_logic_backward_chained_grouped(
+                    _p(x), _p(schedule.verts), _p(schedule.neuron), _p(schedule.flip), _p(dst), schedule.steps, _p(probs),
+                    _p(grad_cls), 1, _p(fix_vertex) if n_fix else None, _p(fix_start) if n_fix else None, n_fix, rows,
+                    _p(grad_w), _p(grad_x), _p(workspace) if ws_bytes else None, in_dim, out_dim, batch, k, float(scale),
+                    code, _stream(dev))
+            if st == _lib.DL_OK:
+                return grad_w, grad_x
+            if st != _lib.DL_ERR_TOO_LARGE:
+                _raise(st, "logic_layer_cuda_backward_chained_grouped")
+    grad_w = grad_x = None
+    with _on(dev):
+        if want_x:
+            _check_index(start, "given_x_indices_of_y_start", in_dim + 1)
+            _check_index(idx, "given_x_indices_of_y", 2 * out_dim)
+            grad_x = torch.empty_like(x)
+            st = lib.dl_logic_backward_x_grouped(_p(x), _p(a), _p(b), _p(probs), _p(grad_cls), _p(start), _p(idx),
+                                                 _p(grad_x), in_dim, out_dim, batch, k, float(scale), code, _stream(dev))
+            if st:
+                _raise(st, "logic_layer_cuda_backward_x_grouped")
+        if want_w:
+            grad_w = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
+            st = lib.dl_logic_backward_logits_grouped(_p(x), _p(a), _p(b), _p(grad_cls), _p(probs), _p(grad_w), in_dim,
+                                                      out_dim, batch, k, code, _stream(dev))
+            if st:
+                _raise(st, "logic_layer_cuda_backward_logits_grouped")
+    return grad_w, grad_x
+
+
 def group_sum_forward(x, k, tau):
     """Feature-major GroupSum: x [out,B] -> [B,k] = per-class sums over neurons / tau
     (difflogic/difflogic.py:195-196 on the layout the layer kernels produce)."""

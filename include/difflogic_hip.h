@@ -161,6 +161,37 @@ int dl_group_sum_forward(const void *x, void *y, void *workspace, int64_t out_di
 int dl_group_sum_backward(const void *grad_y, void *grad_x, int64_t out_dim, int64_t batch, int64_t k,
                           double tau, int dtype, void *stream);
 
+/* The last LogicLayer of a model and the GroupSum that follows it as ONE step (the pair
+ * difflogic/difflogic.py:123-126 then :195-196, and their backward passes): the layer's output
+ * [out_dim, batch] and the broadcast gradient GroupSum's backward would hand back are never
+ * materialised.  No counterpart in the reference.
+ *   dl_logic_forward_group_sum : y[r, c] = (1/tau) * sum over the neurons n of class c of
+ *       forward(x, a, b, w)[n, r];  y [batch, k].  probs != NULL: w holds logits and probs
+ *       receives softmax(w) (as dl_logic_forward_logits); NULL: w holds probabilities.
+ *       workspace: dl_group_sum_workspace_bytes(out_dim, batch, k, dtype) bytes.  Deterministic.
+ *   dl_logic_backward_*_grouped : as dl_logic_backward_logits (probs == NULL: as
+ *       dl_logic_backward_w), dl_logic_backward_x and dl_logic_backward_chained, with
+ *       grad_y[n, r] = grad_cls[class(n), r]:  grad_cls [k, batch] is GroupSum's incoming gradient,
+ *       transposed and already divided by tau; class(n) = n / (out_dim / k). */
+int dl_logic_forward_group_sum(const void *x, const int64_t *a, const int64_t *b, const void *w,
+                               void *probs, void *y, void *workspace, int64_t in_dim, int64_t out_dim,
+                               int64_t batch, int64_t k, double tau, int dtype, void *stream);
+int dl_logic_backward_logits_grouped(const void *x, const int64_t *a, const int64_t *b,
+                                     const void *grad_cls, const void *probs, void *grad_w,
+                                     int64_t in_dim, int64_t out_dim, int64_t batch, int64_t k,
+                                     int dtype, void *stream);
+int dl_logic_backward_x_grouped(const void *x, const int64_t *a, const int64_t *b, const void *w,
+                                const void *grad_cls, const int64_t *start, const int64_t *idx,
+                                void *grad_x, int64_t in_dim, int64_t out_dim, int64_t batch,
+                                int64_t k, double scale, int dtype, void *stream);
+int dl_logic_backward_chained_grouped(const void *x, const int32_t *verts, const int32_t *neuron,
+                                      const uint8_t *flip, const int32_t *dst, int64_t steps,
+                                      const void *w, const void *grad_cls, int softmax_backward,
+                                      const int32_t *fix_vertex, const int32_t *fix_start,
+                                      int64_t n_fix, int64_t overflow_rows, void *grad_w,
+                                      void *grad_x, void *workspace, int64_t in_dim, int64_t out_dim,
+                                      int64_t batch, int64_t k, double scale, int dtype, void *stream);
+
 /* ---- packed inference mode ------------------------------------------------------------ */
 
 /* Replaces `eval` = logic_layer_cuda_eval (difflogic.cpp:63-68, difflogic_kernel.cu:503-541).

@@ -502,3 +502,115 @@ def test_layer_module_with_half_and_double_activations(dtype, rtol):
     assert ok, err
     ok, err = close(layer.weights.grad, w32.grad, rtol)
     assert ok, err
+
+
+@pytest.mark.parametrize("in_dim,out_dim,batch,k", [(12, 30, 7, 3), (33, 100, 256, 10), (50, 77, 513, 7), (16, 40, 2048, 2),
+                                                    (64, 1300, 260, 10), (20, 64, 64, 1)])
+def test_forward_and_backward_fused_with_group_sum(ext, in_dim, out_dim, batch, k):
+    """dl_logic_forward_group_sum / dl_logic_backward_*_grouped against the separate kernels (same
+    terms, the class sums in another order) and the fp64 python formulation."""
+    g = torch.Generator().manual_seed(in_dim + batch)
+    x = torch.rand(in_dim, batch, generator=g)
+    a = torch.randint(0, in_dim, (out_dim,), generator=g)
+    b = torch.randint(0, in_dim, (out_dim,), generator=g)
+    b[1] = a[1]
+    logits = 2 * torch.randn(out_dim, 16, generator=g)
+    gs = torch.randn(batch, k, generator=g)
+    tau = 3.5
+    xd, ad, bd, ld = x.cuda(), a.cuda(), b.cuda(), logits.cuda()
+    start, idx = (t.cuda() for t in _csr(a, b, in_dim))
+
+    sums, probs = ext.forward_group_sum(xd, ad, bd, ld, k, tau)
+    y0, p0 = ext.forward_logits(xd, ad, bd, ld)
+    assert torch.equal(probs, p0) and sums.shape == (batch, k)
+    assert close(sums, ext.group_sum_forward(y0, k, tau))[0]
+    lw = logits.double().requires_grad_()
+    xr = x.double().t().contiguous().requires_grad_()
+    want = fo.group_sum(fo.layer_forward_sequential(xr, a, b, torch.softmax(lw, -1)), k, tau)
+    assert close(sums, want)[0]
+    assert torch.equal(sums, ext.forward_group_sum(xd, ad, bd, ld, k, tau)[0])           # deterministic
+
+    (want * gs.double()).sum().backward()
+    grad_cls = (gs.cuda() / tau).t().contiguous()
+    gw, gx = ext.backward_group_sum(xd, ad, bd, probs, grad_cls, start, idx, None, 1.5, True, True)
+    gy_full = ext.group_sum_backward(gs.cuda(), out_dim, tau)
+    assert close(gw, ext.backward_logits(xd, ad, bd, gy_full, probs))[0]
+    assert close(gx, ext.backward_x(xd, ad, bd, probs, gy_full, start, idx, 1.5))[0]
+    l32 = logits.clone().requires_grad_()
+    x32 = x.t().contiguous().requires_grad_()
+    (fo.group_sum(fo.layer_forward_sequential(x32, a, b, torch.softmax(l32, -1)), k, tau) * gs).sum().backward()
+    ok, rep = within_budget(gw, lw.grad, l32.grad)
+    assert ok, rep
+    ok, rep = within_budget(gx, 1.5 * xr.grad.t(), 1.5 * x32.grad.t())
+    assert ok, rep
+    # along the schedule (one pass): the same gradients
+    sched = ext.schedule_for(ad, bd, in_dim)
+    if batch % 4 == 0:
+        gw2, gx2 = ext.backward_group_sum(xd, ad, bd, probs, grad_cls, start, idx, sched, 1.5, True, True)
+        assert close(gw2, gw)[0] and close(gx2, gx)[0]
+    only_w, none_x = ext.backward_group_sum(xd, ad, bd, probs, grad_cls, start, idx, sched, 1.5, False, True)
+    assert none_x is None and torch.equal(only_w, gw)
+
+
+@pytest.mark.parametrize("widths,batch,conn,grad_factor,wide", [([400, 400, 300], 128, "random", 1.0, False),
+                                                                ([300, 600, 600], 100, "unique", 2.0, False),
+                                                                ([500, 500], 64, "random", 1.0, True)])
+def test_fuse_group_sum_trains_like_the_unfused_model(widths, batch, conn, grad_factor, wide, monkeypatch):
+    """fuse_group_sum(model): same positions, parameters and state_dict keys; in training the same
+    class scores, loss and gradients as the unfused model (up to summation order) and as the CPU
+    python implementation; eval mode and packed inference unchanged."""
+    import difflogic_amd as dl
+    if wide:          # the last layer takes the kernels that walk the schedule
+        monkeypatch.setattr(dl.LogicLayer, "_CHAIN_MIN_IN_DIM", 0)
+        monkeypatch.setattr(dl.LogicLayer, "_CHAIN_MIN_OUT_DIM", 0)
+    torch.manual_seed(3)
+    F, k, tau = 60, 10, 10.0
+    mods, d = [torch.nn.Flatten()], F
+    for wd in widths:
+        mods.append(dl.LogicLayer(d, wd, grad_factor=grad_factor, connections=conn))
+        d = wd
+    model = torch.nn.Sequential(*mods, dl.GroupSum(k, tau)).train()
+    fused = dl.fuse_group_sum(model).train()
+    assert list(fused.state_dict()) == list(model.state_dict()) and len(fused) == len(model)
+    assert isinstance(fused[-2], dl.FusedLogicLayerGroupSum) and fused[-2].weights is model[-2].weights
+    layers = [m for m in model if isinstance(m, dl.LogicLayer)]
+    x = (torch.rand(batch, F) < 0.3).float()
+    labels = torch.randint(0, k, (batch,))
+
+    def run(net):
+        net.zero_grad(set_to_none=True)
+        xg = x.cuda().requires_grad_()
+        out = net(xg)
+        loss = torch.nn.functional.cross_entropy(out, labels.cuda())
+        loss.backward()
+        return out.detach(), loss.detach(), [l.weights.grad.clone() for l in layers], xg.grad.clone()
+
+    out0, loss0, gw0, gx0 = run(model)
+    out1, loss1, gw1, gx1 = run(fused)
+    assert close(out1, out0)[0] and abs(float(loss1) - float(loss0)) <= RTOL * abs(float(loss0))
+
+    def python_impl(dtype):
+        lg = [l.weights.detach().cpu().to(dtype).requires_grad_() for l in layers]
+        net = fo.PythonNet([(l.indices[0].cpu(), l.indices[1].cpu(), w) for l, w in zip(layers, lg)], k, tau, grad_factor)
+        xo = x.detach().clone().to(dtype).requires_grad_()
+        o = net(xo)
+        torch.nn.functional.cross_entropy(o, labels).backward()
+        return o.detach(), [w.grad for w in lg], xo.grad
+
+    o64, w64, x64 = python_impl(torch.float64)
+    o32, w32, x32 = python_impl(torch.float32)
+    assert close(out1, o64)[0]
+    for got, r64, r32 in zip(gw1, w64, w32):
+        ok, rep = within_budget(got, r64, r32)
+        assert ok, rep
+    ok, rep = within_budget(gx1, x64, x32)
+    assert ok, rep
+    out2, loss2, gw2, gx2 = run(fused)
+    assert torch.equal(out1, out2) and all(torch.equal(u, v) for u, v in zip(gw1, gw2)) and torch.equal(gx1, gx2)
+
+    # eval mode: float and packed inference go through the two original modules
+    model.eval(), fused.eval()
+    with torch.no_grad():
+        assert torch.equal(fused(x.cuda()), model(x.cuda()))
+        assert torch.equal(fused(dl.PackBitsTensor(x.bool().cuda(), bit_count=64)),
+                           model(dl.PackBitsTensor(x.bool().cuda(), bit_count=64)))
