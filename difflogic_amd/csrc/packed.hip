@@ -972,19 +972,21 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
 
 #pragma unroll 1
     for (int b = 0; b < blocks; ++b) {
-        // phase A: walk DL_CC_WAVE_STEPS steps, four at a time (their rows are requested together)
+        // phase A: walk DL_CC_WAVE_STEPS steps, BATCH at a time (their rows are requested together)
+        constexpr int BATCH = DL_CC_WAVE_STEPS % 4 == 0 ? 4 : 3;
+        static_assert(DL_CC_WAVE_STEPS % BATCH == 0, "whole batches of steps");
 #pragma unroll
-        for (int h = 0; h < DL_CC_WAVE_STEPS; h += 4) {
-            dl_u32x4 r[4];
-            V ra[4], rb[4];
+        for (int h = 0; h < DL_CC_WAVE_STEPS; h += BATCH) {
+            dl_u32x4 r[BATCH];
+            V ra[BATCH], rb[BATCH];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < BATCH; ++j) {
                 r[j] = wrec[1 + b * DL_CC_WAVE_STEPS + h + j];
                 ra[j] = xcol[(int64_t) r[j].x * ncols];
                 if (DS == 1) rb[j] = xcol[(int64_t) r[j].y * ncols];
             }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < BATCH; ++j) {
                 const V cur = vertex(ra[j], DS == 1 ? rb[j] : ra[j], r[j].z);
                 const uint32_t where = (r[j].z >> 8) & 255u;
                 if (where != 255u) stage[where][lane] = gate_apply<V>(prev, cur, gate_masks((r[j].z >> 4) & 15u));

@@ -218,19 +218,21 @@ extern "C" int dl_count_order_build(const int64_t *a_top, const int64_t *b_top, 
 
 // Plan for dl_logic_eval_chained_groupbitsum: the count kernel walks the top layer along the
 // evaluation schedule, so consecutive outputs belong to arbitrary classes.  A workgroup of
-// DL_CC_WAVES waves owns 64 * blocks consecutive steps (a contiguous range per wave) and proceeds
+// DL_CC_WAVES waves owns DL_CC_BLOCK * blocks consecutive steps (a contiguous range per wave) and proceeds
 // in `blocks` blocks of DL_CC_BLOCK outputs (DL_CC_WAVE_STEPS per wave): every wave parks its
 // outputs of the block in LDS at a slot that sorts the block by class, and the wave that owns a
 // class then reads that class's run of slots and adds it to its bit-sliced counters.
 //   slot [padded]           LDS slot of step s within its block, 255 = the step has no output
-//   runs [padded / 64 * k]  per block and class: first slot | number of slots << 8
+//   runs [padded / dl_count_chain_block() * k]  per block and class: first slot | number of slots << 8
 //   *blocks                 blocks per workgroup: the largest of 16, 8, 4, 2, 1 for which no
 //                           workgroup counts more than 255 neurons of one class (its counters have
 //                           DL_CC_PLANES planes); fewer blocks mean more partial counters
 // where step s of workgroup g, wave w, block b, position j is
-// g*64*blocks + w*8*blocks + b*DL_CC_WAVE_STEPS + j.  Returns the padded step count (a multiple of
+// (g*DL_CC_WAVES + w)*DL_CC_WAVE_STEPS*blocks + b*DL_CC_WAVE_STEPS + j.  Returns the padded step count (a multiple of
 // DL_CC_MAX_WG_STEPS; steps past `steps` have no output), or -DL_ERR_TOO_LARGE for more classes
 // than the kernel's waves can own.
+extern "C" int dl_count_chain_block(void) { return DL_CC_BLOCK; }
+
 extern "C" int64_t dl_count_chain_padded_steps(int64_t steps) {
     if (steps < 0) return -DL_ERR_INVALID_ARGUMENT;
     return (steps + DL_CC_MAX_WG_STEPS - 1) / DL_CC_MAX_WG_STEPS * DL_CC_MAX_WG_STEPS;
@@ -279,7 +281,7 @@ extern "C" int64_t dl_count_chain_plan_build(const int32_t *neuron, int64_t step
     for (int64_t s = 0; s < steps; ++s)
         if (neuron[s] >= out_dim) return -DL_ERR_INVALID_ARGUMENT;
     const int64_t padded = dl_count_chain_padded_steps(steps);
-    for (int nb = DL_CC_MAX_BLOCKS; nb >= 1; nb /= 2)       // one block holds 64 outputs: always fits
+    for (int nb = DL_CC_MAX_BLOCKS; nb >= 1; nb /= 2)       // one block holds at most DL_CC_BLOCK outputs: always fits
         if (count_chain_plan(neuron, steps, out_dim / k, k, nb, padded, slot, runs)) {
             *blocks = nb;
             return padded;

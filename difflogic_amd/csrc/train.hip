@@ -866,13 +866,14 @@ int forward_t(const void *x, const int64_t *a, const int64_t *b, const void *w, 
 template <typename T>
 int backward_w_t(const void *x, const int64_t *a, const int64_t *b, const void *gy, const void *probs, void *gw,
                  int64_t out_dim, int64_t batch, hipStream_t s, int64_t gdiv = 0) {
-    constexpr int NPW = 2;
+    constexpr int NPW = 2;       // neurons per wave when the workgroup's waves split a neuron's batch
+    constexpr int NPW1 = 2;      // ... when a wave owns whole rows: short rows, more neurons' loads in flight per wave
     constexpr int V = Vec16<T>::n;
     const bool vec = batch % V == 0 && dl_aligned(x, 16) && dl_aligned(gy, 16);
     const int64_t ncols = vec ? batch / V : batch;
     // Split one neuron's batch over the four waves once every wave still gets whole segments.
     const bool split = ncols >= 8 * DL_WAVE;
-    const int64_t blocks = split ? dl_ceil_div(out_dim, NPW) : dl_ceil_div(out_dim, 4 * NPW);
+    const int64_t blocks = split ? dl_ceil_div(out_dim, NPW) : dl_ceil_div(out_dim, 4 * NPW1);
     if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     const dim3 grid((unsigned) blocks), block(DL_BLOCK);
     const T *xp = (const T *) x, *gp = (const T *) gy, *pp = (const T *) probs;
@@ -880,11 +881,11 @@ int backward_w_t(const void *x, const int64_t *a, const int64_t *b, const void *
     if (vec && split)
         DL_LAUNCH((backward_w_kernel<T, V, NPW, 4>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv);
     else if (vec)
-        DL_LAUNCH((backward_w_kernel<T, V, NPW, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv);
+        DL_LAUNCH((backward_w_kernel<T, V, NPW1, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv);
     else if (split)
         DL_LAUNCH((backward_w_kernel<T, 1, NPW, 4>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv);
     else
-        DL_LAUNCH((backward_w_kernel<T, 1, NPW, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv);
+        DL_LAUNCH((backward_w_kernel<T, 1, NPW1, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv);
     return dl_launch_status();
 }
 

@@ -473,7 +473,7 @@ class EvalSchedule:
             _, neuron = self._host
             padded = lib.dl_count_chain_padded_steps(self.steps)
             slot = np.empty(max(1, padded), dtype=np.uint8)
-            runs = np.empty(max(1, padded // 64 * k), dtype=np.uint16)
+            runs = np.empty(max(1, padded // lib.dl_count_chain_block() * k), dtype=np.uint16)
             blocks = ctypes.c_int(0)
             got = lib.dl_count_chain_plan_build(neuron.ctypes.data, self.steps, self.out_dim, int(k), slot.ctypes.data,
                                                 runs.ctypes.data, ctypes.byref(blocks))

@@ -295,11 +295,12 @@ int dl_logic_eval_fused_groupbitsum(const void *x, int depth, const int64_t *con
  * one instead of two).  Same result as dl_logic_eval_fused_groupbitsum.  No counterpart in the
  * reference.
  *   verts, neuron, flip, steps   DEVICE copies of the top layer's schedule (dl_eval_schedule_build)
+ *   dl_count_chain_block()         outputs a workgroup parks in LDS per block
  *   dl_count_chain_padded_steps()  HOST: steps rounded up to whole workgroups
  *   dl_count_chain_plan_build()    HOST pointers.  From the schedule's neuron [steps], out_dim and k
- *       writes slot [padded] and runs [padded / 64 * k]: where every workgroup parks the outputs
+ *       writes slot [padded] and runs [padded / dl_count_chain_block() * k]: where every workgroup parks the outputs
  *       of a block so that they are sorted by class, and each class's run of slots; and *blocks:
- *       how many blocks of 64 steps a workgroup walks (16 at most; fewer where a workgroup would
+ *       how many blocks of steps a workgroup walks (16 at most; fewer where a workgroup would
  *       otherwise count more than 255 neurons of one class).  Returns padded, or a negated
  *       dl_status: -DL_ERR_TOO_LARGE for k > 16 (the caller then uses
  *       dl_logic_eval_fused_groupbitsum).
@@ -309,6 +310,7 @@ int dl_logic_eval_fused_groupbitsum(const void *x, int depth, const int64_t *con
  *             and the current gate ids) and the bit-sliced partial counters.
  * depth is 1 or 2; a, b are read for the layer below the top one only (a[0], b[0] at depth 2).
  * DL_ERR_TOO_LARGE: rows are not whole 64-bit words or k > 16. */
+int dl_count_chain_block(void);
 int64_t dl_count_chain_padded_steps(int64_t steps);
 int64_t dl_count_chain_plan_build(const int32_t *neuron, int64_t steps, int64_t out_dim, int64_t k,
                                   uint8_t *slot, uint16_t *runs, int *blocks);
