@@ -502,7 +502,7 @@ def test_chained_groupbitsum_declines_where_it_does_not_apply(ext):
     layers, dev_layers = _chain(rng, 30, [60, 170])
     x = _dev(rng.integers(0, 1 << 62, (30, 2), dtype=np.int64))
     assert ext.eval_chained_groupbitsum(x, dev_layers, 0, 34) is None                 # more classes than the waves own
-    assert ext.eval_chained_groupbitsum(x, dev_layers, 0, 17) is not None
+    assert ext.eval_chained_groupbitsum(x, dev_layers, 0, 10) is not None
     # 3000 neurons on one trail: with 12 classes (250 each) a workgroup walks 16 blocks, with one class only 2
     a = torch.arange(3000) % 2999
     b = (torch.arange(3000) + 1) % 2999
