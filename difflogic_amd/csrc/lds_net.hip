@@ -11,10 +11,25 @@
 // is evaluated class by class (one wave per class): every lane adds its neurons' output words
 // into bit-sliced counters, and the 64 lanes' counters are summed by a butterfly that halves
 // the sample range a lane is responsible for at every exchange, so after six exchanges lane s
-// holds the count of sample s.
+// holds the counts of samples COLS * s .. COLS * s + COLS - 1 of the workgroup.
 //
 // The wiring is read from a compact table built per call (one 32-bit record per gate: two
 // 14-bit row ids and the 4-bit gate id), which every workgroup streams from L2.
+//
+// A hidden layer whose evaluation schedule is given (schedule.cpp: its neurons ordered along
+// trails, consecutive ones sharing an input) is walked along it instead: a thread takes one chunk
+// of 8 steps, reads 9 rows instead of 16, and its records hold one row id and the gate (inputs
+// swapped where the schedule says so); the records are stored transposed (a thread's j-th entry at
+// [j][thread]) so that a wave's loads are lane-consecutive.  A schedule of more than 1024 chunks
+// has its remaining steps (at most 1024) evaluated one per thread from records of the
+// neuron-by-neuron form.  Such a layer stores its outputs in SCHEDULE order, step s at row
+// (s % 8) * stride + s / 8, so that a wave's stores are lane-consecutive; the records of the
+// layer above are composed with its inputs renamed accordingly (the order of a hidden layer's rows
+// is nobody else's business).
+//
+// One workgroup of 1024 threads fills a CU (its LDS), so nothing else runs there to hide a
+// latency that all of its threads wait out together: every layer's records are requested one
+// layer ahead, and the class phase's an iteration ahead.
 #include "dl_common.h"
 
 #define DL_NET_MAX_DEPTH 16
@@ -28,23 +43,74 @@ struct NetWiring {
     const int64_t *a[DL_NET_MAX_DEPTH];
     const int64_t *b[DL_NET_MAX_DEPTH];
     const uint8_t *w[DL_NET_MAX_DEPTH];
-    int32_t width[DL_NET_MAX_DEPTH];    // neurons of layer l
-    int32_t offset[DL_NET_MAX_DEPTH];   // first record of layer l
+    const int32_t *verts[DL_NET_MAX_DEPTH];     // schedule of layer l, or null: evaluated neuron by neuron
+    const int32_t *neuron[DL_NET_MAX_DEPTH];
+    const uint8_t *flip[DL_NET_MAX_DEPTH];
+    int32_t *pos[DL_NET_MAX_DEPTH];             // scheduled layers: row at which neuron n's output is stored
+    int32_t width[DL_NET_MAX_DEPTH];            // neurons of layer l
+    int32_t offset[DL_NET_MAX_DEPTH];           // first record of layer l
+    int32_t steps[DL_NET_MAX_DEPTH];            // scheduled layers: steps (a multiple of 8); else 0
+    int32_t stride[DL_NET_MAX_DEPTH];           // scheduled layers: row stride between a chunk's steps
 };
 
 struct NetShape {
     int32_t depth, in_dim;
     int32_t width[DL_NET_MAX_DEPTH];
     int32_t offset[DL_NET_MAX_DEPTH];
+    int32_t steps[DL_NET_MAX_DEPTH];
+    int32_t stride[DL_NET_MAX_DEPTH];
 };
 
-// record of neuron n of layer blockIdx.y: a | b << 14 | gate << 28
+#define DL_NET_CHUNK 8                           // steps per thread of a scheduled layer (the schedule's chunk)
+
+__device__ __forceinline__ uint32_t swap_gate(uint32_t op) {   // f'(a, b) = f(b, a)
+    return (op & 9u) | ((op & 4u) >> 1) | ((op & 2u) << 1);
+}
+
+// rows of scheduled layers: neuron n of layer blockIdx.y -> (s % 8) * stride + s / 8 for its step s
+__global__ __launch_bounds__(DL_BLOCK) void compose_net_pos_kernel(NetWiring t) {
+    const int l = blockIdx.y;
+    const int s = (int) (blockIdx.x * DL_BLOCK + threadIdx.x);
+    if (s >= t.steps[l]) return;
+    const int32_t n = t.neuron[l][s];
+    if (n >= 0) t.pos[l][n] = (s % DL_NET_CHUNK) * t.stride[l] + s / DL_NET_CHUNK;
+}
+
+// Records of layer blockIdx.y.  Evaluated neuron by neuron: a | b << 14 | gate << 28 for neuron n.
+// Scheduled: entry i = row of vertex verts[i] | gate of step i - 1 << 28 (the gate with its inputs
+// swapped where the schedule walks the neuron from b to a; steps without a neuron keep gate 0 and
+// their output row is never read).  Row ids are those of the layer below: its pos[] if scheduled.
 __global__ __launch_bounds__(DL_BLOCK) void compose_net_kernel(NetWiring t, uint32_t *__restrict__ rec) {
     const int l = blockIdx.y;
-    const int n = (int) (blockIdx.x * DL_BLOCK + threadIdx.x);
-    if (n >= t.width[l]) return;
-    const uint32_t a = (uint32_t) t.a[l][n], b = (uint32_t) t.b[l][n], op = t.w[l][n] & 15u;
-    rec[t.offset[l] + n] = a | (b << DL_NET_ID_BITS) | (op << (2 * DL_NET_ID_BITS));
+    const int i = (int) (blockIdx.x * DL_BLOCK + threadIdx.x);
+    const int32_t *below = (l > 0 && t.steps[l - 1] > 0) ? t.pos[l - 1] : nullptr;
+    auto row = [&](int64_t v) -> uint32_t { return (uint32_t) (below ? below[v] : v); };
+    if (t.steps[l] > 0) {
+        if (i > t.steps[l]) return;
+        uint32_t gate = 0;
+        if (i >= 1) {
+            const int32_t n = t.neuron[l][i - 1];
+            if (n >= 0) {
+                gate = t.w[l][n] & 15u;
+                if (t.flip[l][i - 1]) gate = swap_gate(gate);
+            }
+        }
+        // entry 8 c + j is read by thread c as its j-th: stored at [j][c]; a chunk's ninth is the next one's first
+        const uint32_t entry = row(t.verts[l][i]) | (gate << (2 * DL_NET_ID_BITS));
+        uint32_t *tab = rec + t.offset[l];
+        const int stride = t.stride[l];
+        if (i < t.steps[l]) tab[(i % DL_NET_CHUNK) * stride + i / DL_NET_CHUNK] = entry;
+        if (i % DL_NET_CHUNK == 0 && i > 0) tab[DL_NET_CHUNK * stride + i / DL_NET_CHUNK - 1] = entry;
+        // steps past the chunks the workgroup's threads take (one each) are evaluated one per thread, from a record
+        // of the neuron-by-neuron form; `gate` is that of step i - 1, which reads entries i - 1 and i
+        const int first = DL_NET_CHUNK * DL_NET_THREADS;
+        if (i > first)
+            tab[(DL_NET_CHUNK + 1) * stride + i - 1 - first] =
+                row(t.verts[l][i - 1]) | (row(t.verts[l][i]) << DL_NET_ID_BITS) | (gate << (2 * DL_NET_ID_BITS));
+        return;
+    }
+    if (i >= t.width[l]) return;
+    rec[t.offset[l] + i] = row(t.a[l][i]) | (row(t.b[l][i]) << DL_NET_ID_BITS) | ((t.w[l][i] & 15u) << (2 * DL_NET_ID_BITS));
 }
 
 // COLS 64-bit words as 2 * COLS dwords
@@ -78,13 +144,12 @@ template <int COLS> __device__ __forceinline__ void lds_store(void *act, uint32_
     }
 }
 
-// gate id = truth table (f(0,0) f(0,1) f(1,0) f(1,1)), MSB first; masks are per lane here
+// gate id = truth table (f(0,0) f(0,1) f(1,0) f(1,1)), MSB first, in bits 28..31 of the record;
+// masks are per lane here
 template <int COLS>
-__device__ __forceinline__ Row<COLS> gate_rows(const void *act, uint32_t rec) {
-    const uint32_t ia = rec & ((1u << DL_NET_ID_BITS) - 1), ib = (rec >> DL_NET_ID_BITS) & ((1u << DL_NET_ID_BITS) - 1);
+__device__ __forceinline__ Row<COLS> gate_mix(const Row<COLS> &a, const Row<COLS> &b, uint32_t rec) {
     const uint32_t m00 = 0u - ((rec >> 31) & 1u), m01 = 0u - ((rec >> 30) & 1u);
     const uint32_t m10 = 0u - ((rec >> 29) & 1u), m11 = 0u - ((rec >> 28) & 1u);
-    const Row<COLS> a = lds_row<COLS>(act, ia), b = lds_row<COLS>(act, ib);
     Row<COLS> y;
 #pragma unroll
     for (int i = 0; i < 2 * COLS; ++i) {
@@ -93,6 +158,12 @@ __device__ __forceinline__ Row<COLS> gate_rows(const void *act, uint32_t rec) {
         y.d[i] = (a.d[i] & hi) | (~a.d[i] & lo);
     }
     return y;
+}
+
+template <int COLS>
+__device__ __forceinline__ Row<COLS> gate_rows(const void *act, uint32_t rec) {
+    const uint32_t ia = rec & ((1u << DL_NET_ID_BITS) - 1), ib = (rec >> DL_NET_ID_BITS) & ((1u << DL_NET_ID_BITS) - 1);
+    return gate_mix<COLS>(lds_row<COLS>(act, ia), lds_row<COLS>(act, ib), rec);
 }
 
 // carry-save adder on dwords: a + b + c = 2 * carry + sum, bit by bit
@@ -115,114 +186,234 @@ template <int NP> __device__ __forceinline__ void planes_add(uint32_t *a, const 
     a[NP] = carry;
 }
 
-// One exchange of the butterfly: lanes l and l ^ (1 << J) each hold counters for the same set of
-// sample bits (those selected by the earlier exchanges); the lane whose bit J is set keeps the
-// samples whose index has bit J set (dword positions `upper`), its partner the others, and each
-// adds the partner's counters for the samples it keeps.
-template <int NP, int J> __device__ __forceinline__ void butterfly(uint32_t *q, int lane) {
+// ---- summing the 64 lanes' bit-sliced counters ---------------------------------------------------
+// A lane enters with NP0 planes for each of the 2 * COLS dwords of its row (dword d = samples
+// 32 d .. 32 d + 31 of the workgroup's COLS * 64).  Every exchange pairs each lane with one whose
+// lane id differs in bit BIT, halves the set of samples a lane is responsible for, and adds the
+// partner's counters for the half it keeps (one more plane).  After six exchanges lane s is left
+// with the totals of samples COLS * s .. COLS * s + COLS - 1.  Any pairing that flips bit BIT
+// will do (the other bits it flips have not been used yet), which lets the four low exchanges be
+// DPP moves (mirrors and quad permutations) instead of trips through the LDS crossbar.
+
+template <int BIT> __device__ __forceinline__ uint32_t lane_partner(uint32_t v) {
+    if constexpr (BIT == 3)
+        return (uint32_t) __builtin_amdgcn_update_dpp(0, (int) v, 0x140, 0xf, 0xf, false);   // row_mirror: lane ^ 15
+    else if constexpr (BIT == 2)
+        return (uint32_t) __builtin_amdgcn_update_dpp(0, (int) v, 0x141, 0xf, 0xf, false);   // row_half_mirror: lane ^ 7
+    else if constexpr (BIT == 1)
+        return (uint32_t) __builtin_amdgcn_update_dpp(0, (int) v, 0x4e, 0xf, 0xf, false);    // quad_perm [2,3,0,1]: lane ^ 2
+    else if constexpr (BIT == 0)
+        return (uint32_t) __builtin_amdgcn_update_dpp(0, (int) v, 0xb1, 0xf, 0xf, false);    // quad_perm [1,0,3,2]: lane ^ 1
+    else
+        return (uint32_t) __shfl_xor((int) v, 1 << BIT, DL_WAVE);
+}
+
+// D dwords per lane -> D / 2: the lane whose bit BIT is set keeps the upper half of the dwords
+template <int D, int NP, int BIT, int NPMAX> __device__ __forceinline__ void fold_dwords(uint32_t (*q)[NPMAX], int lane) {
+    const bool up = ((lane >> BIT) & 1) != 0;
+#pragma unroll
+    for (int i = 0; i < D / 2; ++i) {
+        uint32_t other[NP];
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const uint32_t lo = q[i][p], hi = q[D / 2 + i][p];
+            other[p] = lane_partner<BIT>(up ? lo : hi);
+            q[i][p] = up ? hi : lo;
+        }
+        planes_add<NP>(q[i], other);
+    }
+}
+
+// one dword per lane: the lane whose bit BIT is set keeps the bit positions whose index has bit J set
+template <int NP, int J, int BIT> __device__ __forceinline__ void fold_bits(uint32_t *q, int lane) {
     constexpr uint32_t upper = J == 4 ? 0xffff0000u : J == 3 ? 0xff00ff00u : J == 2 ? 0xf0f0f0f0u
                              : J == 1 ? 0xccccccccu : 0xaaaaaaaau;
-    const uint32_t keep = ((lane >> J) & 1) ? upper : ~upper;
+    const uint32_t keep = ((lane >> BIT) & 1) ? upper : ~upper;
     uint32_t other[NP];
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
-        other[p] = (uint32_t) __shfl_xor((int) q[p], 1 << J, DL_WAVE) & keep;
+        other[p] = lane_partner<BIT>(q[p]) & keep;
         q[p] &= keep;
     }
     planes_add<NP>(q, other);
 }
 
-// Sums the 64 lanes' bit-sliced counters (NP0 planes of 64 sample bits: lo = samples 0..31,
-// hi = samples 32..63) and returns, in lane s, the count of sample s.
-template <int NP0> __device__ __forceinline__ int32_t lanes_count(const uint32_t *lo, const uint32_t *hi, int lane) {
-    uint32_t q[NP0 + 6], other[NP0];
-    const bool upper_half = (lane & 32) != 0;          // this lane keeps samples 32..63
-#pragma unroll
-    for (int p = 0; p < NP0; ++p) {
-        q[p] = upper_half ? hi[p] : lo[p];
-        other[p] = (uint32_t) __shfl_xor((int) (upper_half ? lo[p] : hi[p]), 32, DL_WAVE);
+// q[d][p]: plane p of dword d.  Returns in count[t] the total of sample COLS * lane + t.
+template <int COLS, int NP0>
+__device__ __forceinline__ void lanes_count(uint32_t (*q)[NP0 + 6], int lane, int32_t *count) {
+    static_assert(COLS == 1 || COLS == 2 || COLS == 4, "columns per workgroup");
+    if constexpr (COLS == 4) {
+        fold_dwords<8, NP0, 5, NP0 + 6>(q, lane);
+        fold_dwords<4, NP0 + 1, 4, NP0 + 6>(q, lane);
+        fold_dwords<2, NP0 + 2, 3, NP0 + 6>(q, lane);
+        fold_bits<NP0 + 3, 4, 2>(q[0], lane);
+        fold_bits<NP0 + 4, 3, 1>(q[0], lane);
+        fold_bits<NP0 + 5, 2, 0>(q[0], lane);
+    } else if constexpr (COLS == 2) {
+        fold_dwords<4, NP0, 5, NP0 + 6>(q, lane);
+        fold_dwords<2, NP0 + 1, 4, NP0 + 6>(q, lane);
+        fold_bits<NP0 + 2, 4, 3>(q[0], lane);
+        fold_bits<NP0 + 3, 3, 2>(q[0], lane);
+        fold_bits<NP0 + 4, 2, 1>(q[0], lane);
+        fold_bits<NP0 + 5, 1, 0>(q[0], lane);
+    } else {
+        fold_dwords<2, NP0, 5, NP0 + 6>(q, lane);
+        fold_bits<NP0 + 1, 4, 4>(q[0], lane);
+        fold_bits<NP0 + 2, 3, 3>(q[0], lane);
+        fold_bits<NP0 + 3, 2, 2>(q[0], lane);
+        fold_bits<NP0 + 4, 1, 1>(q[0], lane);
+        fold_bits<NP0 + 5, 0, 0>(q[0], lane);
     }
-    planes_add<NP0>(q, other);
-    butterfly<NP0 + 1, 4>(q, lane);
-    butterfly<NP0 + 2, 3>(q, lane);
-    butterfly<NP0 + 3, 2>(q, lane);
-    butterfly<NP0 + 4, 1>(q, lane);
-    butterfly<NP0 + 5, 0>(q, lane);
-    int32_t count = 0;
+    const int first = (lane * COLS) & 31;                      // bit position of sample COLS * lane in its dword
 #pragma unroll
-    for (int p = 0; p < NP0 + 6; ++p) count |= (int32_t) ((q[p] >> (lane & 31)) & 1u) << p;
-    return count;
+    for (int t = 0; t < COLS; ++t) {
+        count[t] = 0;
+#pragma unroll
+        for (int p = 0; p < NP0 + 6; ++p) count[t] |= (int32_t) ((q[0][p] >> (first + t)) & 1u) << p;
+    }
+}
+
+// records of the class phase: four neurons of a lane at a time, past the end of the class -> the class's last
+__device__ __forceinline__ void load_class_records(uint32_t *r4, const uint32_t *ctab, int64_t i0, int64_t per_class) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int64_t i = i0 + u * DL_WAVE;
+        r4[u] = ctab[i < per_class ? i : per_class - 1];
+    }
 }
 
 template <int COLS, int GPT, int NP0>
 __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint64_t *__restrict__ x,
                                                                       const uint32_t *__restrict__ rec, NetShape net,
                                                                       int32_t *__restrict__ out, int64_t ncols,
-                                                                      int64_t per_class, int64_t k, int64_t batch) {
+                                                                      int64_t per_class, int64_t k, int64_t batch,
+                                                                      uint32_t grouped_blocks) {
     extern __shared__ __align__(16) uint8_t act[];             // [rows][COLS] 64-bit words
     const int tid = (int) threadIdx.x;
-    const int64_t col0 = (int64_t) blockIdx.x * COLS;
+    const int wave = dl_wave_in_block(), lane = dl_lane();
+
+    // Workgroups are dealt round-robin to the 8 XCDs, each with an L2 of its own.  The 16 / COLS workgroups
+    // whose columns share a 128-byte line of every input row are given to ONE XCD, so a line is fetched
+    // into one L2 instead of eight (the blocks past the last whole group of 8 * 16 / COLS keep their index).
+    constexpr uint32_t SHARE = 16 / COLS;
+    uint32_t cb = blockIdx.x;
+    if (cb < grouped_blocks) {
+        const uint32_t xcd = cb % 8, j = cb / 8;
+        cb = ((j / SHARE) * 8 + xcd) * SHARE + j % SHARE;
+    }
+    const int64_t col0 = (int64_t) cb * COLS;
+
+    // records a thread needs for layer l, requested one layer ahead of their use
+    constexpr int NR = GPT > DL_NET_CHUNK + 2 ? GPT : DL_NET_CHUNK + 2;
+    auto load_records = [&](int l, uint32_t *r) __attribute__((always_inline)) {
+        const uint32_t *tab = rec + net.offset[l];
+        // scheduled: entry 8 tid + i sits at tab[i * stride + tid], i = 0..8, and the record of step 8192 + tid at
+        // tab[9 * stride + tid]; else neuron tid + 1024 i at tab[tid + 1024 i]
+        const bool sched = net.steps[l] > 0;
+        const int chunks = net.steps[l] / DL_NET_CHUNK;
+        const int limit = sched ? (chunks < DL_NET_THREADS ? chunks : DL_NET_THREADS) : net.width[l];
+        const int extra = net.steps[l] - DL_NET_CHUNK * limit;
+        const int step = sched ? net.stride[l] : DL_NET_THREADS;
+        const int entries = sched ? DL_NET_CHUNK + 2 : GPT;
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            // (threads and entries without work read entry 0 and compute on it; only their stores are skipped)
+            const bool live = i < entries && (!sched ? tid + i * DL_NET_THREADS < limit
+                                              : i <= DL_NET_CHUNK ? tid < limit : tid < extra);
+            r[i] = tab[live ? tid + i * step : 0];
+        }
+    };
+    uint32_t r[NR];
+    if (net.depth > 1) load_records(0, r);
+    // the class phase's first records (wave = class)
+    const uint32_t *ltab = rec + net.offset[net.depth - 1];
+    uint32_t rc[4] = {0, 0, 0, 0};
+    if (wave < k) load_class_records(rc, ltab + wave * per_class, lane, per_class);
 
     // the workgroup's word columns of the packed input; columns past the end read as zero
     for (int f = tid; f < net.in_dim; f += DL_NET_THREADS) {
-        Row<COLS> r;
+        Row<COLS> v;
+        if (COLS > 1 && col0 + COLS <= ncols && ncols % 2 == 0 && ((uintptr_t) x & 15) == 0) {   // whole, 16-byte aligned
+            const dl_u32x4 *src = reinterpret_cast<const dl_u32x4 *>(x + (int64_t) f * ncols + col0);
 #pragma unroll
-        for (int j = 0; j < COLS; ++j) {
-            const uint64_t v = col0 + j < ncols ? x[(int64_t) f * ncols + col0 + j] : 0;
-            r.d[2 * j] = (uint32_t) v, r.d[2 * j + 1] = (uint32_t) (v >> 32);
+            for (int q = 0; q < COLS / 2; ++q) {
+                const dl_u32x4 t = src[q];
+                v.d[4 * q] = t.x, v.d[4 * q + 1] = t.y, v.d[4 * q + 2] = t.z, v.d[4 * q + 3] = t.w;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < COLS; ++j) {
+                const uint64_t t = col0 + j < ncols ? x[(int64_t) f * ncols + col0 + j] : 0;
+                v.d[2 * j] = (uint32_t) t, v.d[2 * j + 1] = (uint32_t) (t >> 32);
+            }
         }
-        lds_store<COLS>(act, (uint32_t) f, r);
+        lds_store<COLS>(act, (uint32_t) f, v);
     }
     __syncthreads();
 
-    // every layer but the last: act <- layer(act).  The records of the next layer are requested
-    // before this layer's barrier, so their latency overlaps the exchange through LDS.
-    // every layer but the last: act <- layer(act).  (Measured: the hidden layers are bound by LDS
-    // throughput, bank conflicts of the random row reads included, not by its latency: putting all
-    // of a thread's reads in flight together is no faster than this gate-by-gate form.)
+    // Every layer but the last: act <- layer(act).  The hidden layers are bound by LDS throughput (bank
+    // conflicts of the random row reads included) and, run in lock step between barriers by the one
+    // workgroup a CU holds, by every latency that all threads wait out together: the next layer's
+    // records are therefore requested before this layer's rows are read.
     for (int l = 0; l + 1 < net.depth; ++l) {
-        const uint32_t *tab = rec + net.offset[l];
-        const int width = net.width[l];
-        uint32_t r[GPT];
+        uint32_t rn[NR];
+        if (l + 2 < net.depth) load_records(l + 1, rn);
+        if (net.steps[l] > 0) {
+            // along the schedule: this thread's chunk of 8 steps, 9 rows read, outputs in schedule order
+            // (and, of a schedule of more than 1024 chunks, one of the remaining steps)
+            const int stride = net.stride[l];
+            const int nchunks = net.steps[l] / DL_NET_CHUNK < DL_NET_THREADS ? net.steps[l] / DL_NET_CHUNK : DL_NET_THREADS;
+            const int extra = net.steps[l] - DL_NET_CHUNK * nchunks;
+            Row<COLS> y[DL_NET_CHUNK], ye;
+            if (extra > 0) ye = gate_rows<COLS>(act, r[DL_NET_CHUNK + 1]);
+            Row<COLS> prev = lds_row<COLS>(act, r[0] & ((1u << DL_NET_ID_BITS) - 1));
 #pragma unroll
-        for (int g = 0; g < GPT; ++g) {
-            const int n = tid + g * DL_NET_THREADS;
-            r[g] = n < width ? tab[n] : 0u;
-        }
-        Row<COLS> y[GPT];
+            for (int j = 0; j < DL_NET_CHUNK; ++j) {
+                const Row<COLS> cur = lds_row<COLS>(act, r[j + 1] & ((1u << DL_NET_ID_BITS) - 1));
+                y[j] = gate_mix<COLS>(prev, cur, r[j + 1]);
+                prev = cur;
+            }
+            __syncthreads();                                    // every thread has read its inputs
+            if (tid < nchunks) {
 #pragma unroll
-        for (int g = 0; g < GPT; ++g)
-            if (tid + g * DL_NET_THREADS < width) y[g] = gate_rows<COLS>(act, r[g]);
-        __syncthreads();                                        // every thread has read its inputs
+                for (int j = 0; j < DL_NET_CHUNK; ++j) lds_store<COLS>(act, (uint32_t) (j * stride + tid), y[j]);
+            }
+            if (tid < extra)                                    // step 8192 + tid
+                lds_store<COLS>(act, (uint32_t) ((tid % DL_NET_CHUNK) * stride + DL_NET_THREADS + tid / DL_NET_CHUNK), ye);
+        } else {
+            const int width = net.width[l];
+            Row<COLS> y[GPT];
 #pragma unroll
-        for (int g = 0; g < GPT; ++g) {
-            const int n = tid + g * DL_NET_THREADS;
-            if (n < width) lds_store<COLS>(act, (uint32_t) n, y[g]);
+            for (int g = 0; g < GPT; ++g) y[g] = gate_rows<COLS>(act, r[g]);
+            __syncthreads();                                    // every thread has read its inputs
+#pragma unroll
+            for (int g = 0; g < GPT; ++g) {
+                const int n = tid + g * DL_NET_THREADS;
+                if (n < width) lds_store<COLS>(act, (uint32_t) n, y[g]);
+            }
         }
         __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NR; ++i) r[i] = rn[i];
     }
 
     // last layer, one wave per class: evaluate, count bit-sliced per lane, sum the lanes
-    const int wave = dl_wave_in_block(), lane = dl_lane();
-    const uint32_t *tab = rec + net.offset[net.depth - 1];
     for (int64_t cls = wave; cls < k; cls += DL_NET_THREADS / DL_WAVE) {
-        uint32_t pl[2 * COLS][NP0];                              // [dword of the row][plane]
+        uint32_t pl[2 * COLS][NP0 + 6];                          // [dword of the row][plane]
 #pragma unroll
         for (int i = 0; i < 2 * COLS; ++i)
 #pragma unroll
             for (int p = 0; p < NP0; ++p) pl[i][p] = 0;
-        // four neurons at a time: their records are requested together, their output words are
+        // four neurons at a time: their records are requested an iteration ahead, their output words are
         // compressed by a carry-save tree into one word of weight 4 that ripples into the planes
         // above; neurons past the end of the class contribute zero words
-        const uint32_t *ctab = tab + cls * per_class;
+        const uint32_t *ctab = ltab + cls * per_class;
+        if (cls != wave) load_class_records(rc, ctab, lane, per_class);
         for (int64_t i0 = lane; i0 < per_class; i0 += 4 * DL_WAVE) {
             uint32_t r4[4], live[4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int64_t i = i0 + u * DL_WAVE;
-                live[u] = i < per_class ? ~0u : 0u;
-                r4[u] = ctab[i < per_class ? i : per_class - 1];
-            }
+            for (int u = 0; u < 4; ++u) r4[u] = rc[u], live[u] = i0 + u * DL_WAVE < per_class ? ~0u : 0u;
+            if (i0 - lane + 4 * DL_WAVE < per_class) load_class_records(rc, ctab, i0 + 4 * DL_WAVE, per_class);
             Row<COLS> y[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
@@ -244,11 +435,12 @@ __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint
                 }
             }
         }
+        int32_t count[COLS];
+        lanes_count<COLS, NP0>(pl, lane, count);
 #pragma unroll
-        for (int j = 0; j < COLS; ++j) {
-            const int32_t count = lanes_count<NP0>(pl[2 * j], pl[2 * j + 1], lane);
-            const int64_t sample = (col0 + j) * 64 + lane;
-            if (col0 + j < ncols && sample < batch) out[sample * k + cls] = count;
+        for (int t = 0; t < COLS; ++t) {
+            const int64_t sample = col0 * 64 + lane * COLS + t;
+            if (sample < batch && sample < ncols * 64) out[sample * k + cls] = count[t];
         }
     }
 }
@@ -260,13 +452,15 @@ int launch_net(const void *x, const uint32_t *rec, const NetShape &net, int32_t 
     if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     const size_t lds = (size_t) rows * 8 * COLS;
     const dim3 grid((unsigned) blocks), block(DL_NET_THREADS);
+    const uint32_t group = 8 * (16 / COLS);                    // workgroups sharing input lines, one set per XCD
+    const uint32_t grouped = (uint32_t) blocks / group * group;
     // a lane counts ceil(per_class / 64) neurons: NP0 planes hold up to 2^NP0 - 1
     if (dl_ceil_div(per_class, DL_WAVE) < 16)
         DL_LAUNCH((eval_net_lds_kernel<COLS, GPT, 4>), grid, block, lds, s, (const uint64_t *) x, rec, net, out, ncols,
-                  per_class, k, batch);
+                  per_class, k, batch, grouped);
     else
         DL_LAUNCH((eval_net_lds_kernel<COLS, GPT, 8>), grid, block, lds, s, (const uint64_t *) x, rec, net, out, ncols,
-                  per_class, k, batch);
+                  per_class, k, batch, grouped);
     return dl_launch_status();
 }
 
@@ -283,14 +477,20 @@ extern "C" int64_t dl_logic_net_lds_max_width(void) { return DL_NET_MAX_WIDTH; }
 
 extern "C" int64_t dl_logic_net_lds_workspace_bytes(int depth, const int64_t *dims) {
     if (depth < 1 || depth > DL_NET_MAX_DEPTH || !dims) return 0;
-    int64_t gates = 0;
-    for (int l = 1; l <= depth; ++l) gates += dims[l] > 0 ? dims[l] : 0;
-    return 4 * gates;
+    // per layer: the records (9 per chunk of a schedule of at most width + width / 4 + 32 steps, chunks
+    // rounded up to whole waves) and width row ids
+    int64_t bytes = 0;
+    for (int l = 1; l <= depth; ++l) {
+        const int64_t w = dims[l] > 0 ? dims[l] : 0;
+        bytes += 4 * (w + w / 2 + 640 + DL_NET_THREADS) + 4 * w;
+    }
+    return bytes;
 }
 
-extern "C" int dl_logic_net_lds_groupbitsum(const void *x, int depth, const int64_t *const *a, const int64_t *const *b,
-                                            const uint8_t *const *w, const int64_t *dims, int32_t *out, int64_t words,
-                                            int bit_count, int64_t pad_len, int64_t k, void *workspace, void *stream) {
+static int net_lds_run(const void *x, int depth, const int64_t *const *a, const int64_t *const *b, const uint8_t *const *w,
+                       const int64_t *dims, const int32_t *const *verts, const int32_t *const *neuron,
+                       const uint8_t *const *flip, const int64_t *steps, int32_t *out, int64_t words, int bit_count,
+                       int64_t pad_len, int64_t k, void *workspace, void *stream) {
     if (bit_count != 8 && bit_count != 16 && bit_count != 32 && bit_count != 64) return DL_ERR_BIT_COUNT;
     if (depth < 1 || !dims || !a || !b || !w || words < 0 || k <= 0 || pad_len < 0) return DL_ERR_INVALID_ARGUMENT;
     if (depth > DL_NET_MAX_DEPTH) return DL_ERR_TOO_LARGE;
@@ -307,38 +507,93 @@ extern "C" int dl_logic_net_lds_groupbitsum(const void *x, int depth, const int6
         return DL_ERR_TOO_LARGE;
     hipStream_t s = (hipStream_t) stream;
 
+    // The widest hidden layer (or the input) decides the columns per workgroup: rows * 8 * COLS bytes of LDS, and a
+    // thread holds the outputs of ceil(width / 1024) neurons in registers.
+    int64_t rows = dims[0], hidden = 0;
+    for (int l = 0; l + 1 < depth; ++l) {
+        if (dims[l + 1] > hidden) hidden = dims[l + 1];
+        if (dims[l + 1] > rows) rows = dims[l + 1];              // the last layer's output is never stored
+    }
+    const bool four = rows <= DL_NET_MAX_WIDTH / 2 && hidden <= 5 * DL_NET_THREADS;
+    const int64_t capacity = four ? DL_NET_MAX_WIDTH / 2 : DL_NET_MAX_WIDTH;        // rows of act[]
+
     NetWiring wiring;
     NetShape net;
     net.depth = depth;
     net.in_dim = (int32_t) dims[0];
-    int64_t rows = dims[0], widest = 0, offset = 0;
+    int64_t entries = 0, offset = 0, most_steps = 0;
+    char *pos_base = nullptr;
+    for (int l = 0; l < DL_NET_MAX_DEPTH; ++l) {
+        wiring.a[l] = wiring.b[l] = nullptr, wiring.w[l] = nullptr;
+        wiring.verts[l] = wiring.neuron[l] = nullptr, wiring.flip[l] = nullptr, wiring.pos[l] = nullptr;
+        wiring.width[l] = wiring.offset[l] = wiring.steps[l] = wiring.stride[l] = 0;
+        net.width[l] = net.offset[l] = net.steps[l] = net.stride[l] = 0;
+    }
     for (int l = 0; l < depth; ++l) {
         if (!a[l] || !b[l] || !w[l]) return DL_ERR_INVALID_ARGUMENT;
         wiring.a[l] = a[l], wiring.b[l] = b[l], wiring.w[l] = w[l];
         wiring.width[l] = net.width[l] = (int32_t) dims[l + 1];
         wiring.offset[l] = net.offset[l] = (int32_t) offset;
-        offset += dims[l + 1];
-        if (dims[l + 1] > widest) widest = dims[l + 1];
-        if (l + 1 < depth && dims[l + 1] > rows) rows = dims[l + 1];     // the last layer's output is never stored
-    }
-    for (int l = depth; l < DL_NET_MAX_DEPTH; ++l) {
-        wiring.a[l] = wiring.b[l] = nullptr, wiring.w[l] = nullptr;
-        wiring.width[l] = wiring.offset[l] = net.width[l] = net.offset[l] = 0;
+        int64_t count = dims[l + 1];
+        // A hidden layer is walked along its schedule when one is given, every chunk finds a thread, its outputs in
+        // schedule order fit the buffer, and the schedule is not much longer than the layer (few, long trails).
+        if (l + 1 < depth && steps && verts && neuron && flip && verts[l] && neuron[l] && flip[l] && steps[l] >= dims[l + 1] &&
+            steps[l] % DL_NET_CHUNK == 0) {
+            const int64_t nchunks = steps[l] / DL_NET_CHUNK;
+            const int64_t stride = dl_ceil_div(nchunks, DL_WAVE) * DL_WAVE;
+            const int64_t extra = steps[l] > DL_NET_CHUNK * DL_NET_THREADS ? steps[l] - DL_NET_CHUNK * DL_NET_THREADS : 0;
+            if (extra <= DL_NET_THREADS && DL_NET_CHUNK * stride <= capacity && steps[l] <= dims[l + 1] + dims[l + 1] / 4 + 32) {
+                wiring.verts[l] = verts[l], wiring.neuron[l] = neuron[l], wiring.flip[l] = flip[l];
+                wiring.steps[l] = net.steps[l] = (int32_t) steps[l];
+                wiring.stride[l] = net.stride[l] = (int32_t) stride;
+                count = (DL_NET_CHUNK + 1) * stride + extra;
+                if (DL_NET_CHUNK * stride > rows) rows = DL_NET_CHUNK * stride;
+                if (steps[l] > most_steps) most_steps = steps[l];
+            }
+        }
+        offset += count;
+        if (count > entries) entries = count;
     }
     uint32_t *rec = (uint32_t *) workspace;
-    DL_LAUNCH(compose_net_kernel, dim3((unsigned) dl_ceil_div(widest, DL_BLOCK), (unsigned) depth), dim3(DL_BLOCK), 0, s,
+    int32_t *pos = (int32_t *) workspace + offset;               // row ids of the scheduled layers follow the records
+    for (int l = 0; l + 1 < depth; ++l) {
+        if (wiring.steps[l] > 0) {
+            wiring.pos[l] = pos;
+            pos += dims[l + 1];
+        }
+    }
+    (void) pos_base;
+    if ((char *) pos - (char *) workspace > dl_logic_net_lds_workspace_bytes(depth, dims)) return DL_ERR_INVALID_ARGUMENT;
+    if (most_steps > 0) {
+        DL_LAUNCH(compose_net_pos_kernel, dim3((unsigned) dl_ceil_div(most_steps, DL_BLOCK), (unsigned) (depth - 1)),
+                  dim3(DL_BLOCK), 0, s, wiring);
+        const int st = dl_launch_status();
+        if (st != DL_OK) return st;
+    }
+    DL_LAUNCH(compose_net_kernel, dim3((unsigned) dl_ceil_div(entries, DL_BLOCK), (unsigned) depth), dim3(DL_BLOCK), 0, s,
               wiring, rec);
     int st = dl_launch_status();
     if (st != DL_OK) return st;
 
     const int64_t ncols = row_bytes / 8;
     const int64_t per_class = dims[depth] / k;
-    // widest hidden layer (or input) decides the columns per workgroup: rows * 8 * COLS bytes of LDS, and a thread
-    // holds the outputs of ceil(width / 1024) neurons in registers
-    int64_t hidden = 0;
-    for (int l = 0; l + 1 < depth; ++l)
-        if (dims[l + 1] > hidden) hidden = dims[l + 1];
-    if (rows <= DL_NET_MAX_WIDTH / 2 && hidden <= 5 * DL_NET_THREADS)
-        return launch_net<4, 5>(x, rec, net, out, ncols, per_class, k, batch, rows, s);
+    if (four) return launch_net<4, 5>(x, rec, net, out, ncols, per_class, k, batch, rows, s);
     return launch_net<2, 10>(x, rec, net, out, ncols, per_class, k, batch, rows, s);
+}
+
+extern "C" int dl_logic_net_lds_groupbitsum(const void *x, int depth, const int64_t *const *a, const int64_t *const *b,
+                                            const uint8_t *const *w, const int64_t *dims, int32_t *out, int64_t words,
+                                            int bit_count, int64_t pad_len, int64_t k, void *workspace, void *stream) {
+    return net_lds_run(x, depth, a, b, w, dims, nullptr, nullptr, nullptr, nullptr, out, words, bit_count, pad_len, k,
+                       workspace, stream);
+}
+
+extern "C" int dl_logic_net_lds_groupbitsum_scheduled(const void *x, int depth, const int64_t *const *a,
+                                                      const int64_t *const *b, const uint8_t *const *w,
+                                                      const int64_t *dims, const int32_t *const *verts,
+                                                      const int32_t *const *neuron, const uint8_t *const *flip,
+                                                      const int64_t *steps, int32_t *out, int64_t words, int bit_count,
+                                                      int64_t pad_len, int64_t k, void *workspace, void *stream) {
+    return net_lds_run(x, depth, a, b, w, dims, verts, neuron, flip, steps, out, words, bit_count, pad_len, k, workspace,
+                       stream);
 }

@@ -708,11 +708,13 @@ def net_lds_max_width():
     return int(_lib.load().dl_logic_net_lds_max_width())
 
 
-def eval_net_lds(x, layers, pad_len, k):
+def eval_net_lds(x, layers, pad_len, k, scheduled=True):
     """groupbitsum(eval(... eval(x, layer 0) ..., last layer), pad_len, k) for a whole narrow net
     (every layer and the input at most net_lds_max_width() wide, at most MAX_NET_DEPTH layers) in
-    one kernel that keeps the activations in LDS.  Returns None where it does not apply (the
-    caller then uses the streaming kernels).  Not part of the reference's extension."""
+    one kernel that keeps the activations in LDS.  ``scheduled``: hidden layers are walked along
+    their (cached) evaluation schedules where that fits, which nearly halves their LDS reads; the
+    result is the same.  Returns None where the kernel does not apply (the caller then uses the
+    streaming kernels).  Not part of the reference's extension."""
     dev, bits, depth, pa, pb, pw, pdims, dims = _fused_args(x, layers)
     out_dim, words = dims[-1], x.shape[1]
     if k <= 0 or out_dim % k != 0:
@@ -725,9 +727,19 @@ def eval_net_lds(x, layers, pad_len, k):
     lib = _lib.load()
     out = torch.empty((batch, k), dtype=torch.int32, device=dev)
     ws = torch.empty(max(1, lib.dl_logic_net_lds_workspace_bytes(depth, pdims) // 4), dtype=torch.int32, device=dev)
+    scheds = [schedule_for(a, b, dims[i]) for i, (a, b, _) in enumerate(layers[:-1])] if scheduled else []
     with _on(dev):
-        st = lib.dl_logic_net_lds_groupbitsum(_p(x), depth, pa, pb, pw, pdims, _p(out), words, bits, int(pad_len),
-                                              int(k), _p(ws), _stream(dev))
+        if scheds:
+            n = len(scheds)
+            pv = (ctypes.c_void_p * n)(*[sc.verts.data_ptr() for sc in scheds])
+            pn = (ctypes.c_void_p * n)(*[sc.neuron.data_ptr() for sc in scheds])
+            pf = (ctypes.c_void_p * n)(*[sc.flip.data_ptr() for sc in scheds])
+            ps = (ctypes.c_int64 * n)(*[sc.steps for sc in scheds])
+            st = lib.dl_logic_net_lds_groupbitsum_scheduled(_p(x), depth, pa, pb, pw, pdims, pv, pn, pf, ps, _p(out), words,
+                                                            bits, int(pad_len), int(k), _p(ws), _stream(dev))
+        else:
+            st = lib.dl_logic_net_lds_groupbitsum(_p(x), depth, pa, pb, pw, pdims, _p(out), words, bits, int(pad_len),
+                                                  int(k), _p(ws), _stream(dev))
     if st == _lib.DL_ERR_TOO_LARGE:
         return None
     if st:

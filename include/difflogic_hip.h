@@ -336,13 +336,25 @@ int dl_logic_eval_chained_groupbitsum(const void *x, int depth, const int64_t *c
  *   (8-byte aligned x); otherwise DL_ERR_TOO_LARGE is returned and the caller uses the streaming
  *   entry points.
  *   workspace DEVICE scratch of dl_logic_net_lds_workspace_bytes(depth, dims) bytes, 4-byte
- *             aligned: one 32-bit record per gate, rebuilt by every call. */
+ *             aligned: the per-gate records and row ids, rebuilt by every call.
+ *   dl_logic_net_lds_groupbitsum_scheduled() additionally takes, per hidden layer l < depth - 1, the
+ *   DEVICE copies of that layer's evaluation schedule (HOST arrays verts, neuron, flip of depth - 1
+ *   DEVICE pointers and HOST steps [depth - 1]; a NULL entry leaves the layer as it is): such a
+ *   layer is walked along its trails inside the kernel, which nearly halves its LDS row reads.
+ *   Same result; same workspace size. */
 int64_t dl_logic_net_lds_max_width(void);
 int64_t dl_logic_net_lds_workspace_bytes(int depth, const int64_t *dims);
 int dl_logic_net_lds_groupbitsum(const void *x, int depth, const int64_t *const *a,
                                  const int64_t *const *b, const uint8_t *const *w,
                                  const int64_t *dims, int32_t *out, int64_t words, int bit_count,
                                  int64_t pad_len, int64_t k, void *workspace, void *stream);
+int dl_logic_net_lds_groupbitsum_scheduled(const void *x, int depth, const int64_t *const *a,
+                                           const int64_t *const *b, const uint8_t *const *w,
+                                           const int64_t *dims, const int32_t *const *verts,
+                                           const int32_t *const *neuron, const uint8_t *const *flip,
+                                           const int64_t *steps, int32_t *out, int64_t words,
+                                           int bit_count, int64_t pad_len, int64_t k, void *workspace,
+                                           void *stream);
 
 /* dl_logic_eval_fused_groupbitsum without a workspace argument, for callers that cannot allocate
  * device memory: code under HIP graph capture, tight serving loops, harnesses that forbid

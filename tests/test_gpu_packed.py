@@ -387,6 +387,9 @@ def test_packed_inference_follows_weight_writes_through_data():
     (64, 64, [128, 2048], 2, 2, 11),                      # 1024 per class: 16 per lane, needs the fifth plane
     (64, 40, [80, 400], 4, 40, 9),                        # more classes than waves
     (64, 5, [3, 3, 3, 3, 3, 3, 3, 3, 3, 3, 3, 3, 3, 3, 3, 4], 2, 2, 0),     # 16 layers
+    (64, 200, [8100, 8100, 300], 2, 10, 0),               # more than 1024 chunks: the steps past them go one per thread
+    (64, 4000, [2000, 5000, 5000, 40], 5, 4, 0),          # 4 columns: some schedules fit its buffer, some do not
+    (64, 3000, [8190, 8250, 9000, 20], 3, 4, 0),          # schedules around 8192 steps and over 9216
 ])
 def test_net_lds_groupbitsum(ext, bits, in_dim, widths, W, k, pad):
     """The LDS-resident whole-net kernel against the oracle (eval per layer, then groupbitsum) and
@@ -405,6 +408,8 @@ def test_net_lds_groupbitsum(ext, bits, in_dim, widths, W, k, pad):
         return
     assert got is not None and got.dtype == torch.int32 and tuple(got.shape) == want.shape
     assert np.array_equal(got.cpu().numpy(), want)
+    # hidden layers evaluated neuron by neuron instead of along their schedules: the same counts
+    assert torch.equal(got, ext.eval_net_lds(_dev(x), dev_layers, pad, k, scheduled=False))
     t = _dev(x)
     for lay in dev_layers:
         t = ext.eval(t, *lay)
