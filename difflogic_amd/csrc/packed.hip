@@ -555,70 +555,83 @@ __global__ __launch_bounds__(DL_BLOCK) void packbits_batch_major_kernel(const ui
     }
 }
 
-// Variant for features % 16 == 0: the workgroup copies the 64 sample rows of one word column
-// (a slice of `slice` features of them when the rows are too long for LDS; consecutive workgroups
-// take the `nslices` slices of the same rows, so that the chip reads a contiguous region) into LDS with coalesced 16-byte loads, so no partial cache lines are fetched however
-// the rows fall, then every thread folds one group of four features from LDS exactly as above.
-// WC word columns per workgroup, so that a feature row is written in runs of 8 * WC bytes.
-template <int WC>
-__global__ __launch_bounds__(DL_BLOCK) void packbits_batch_major_lds_kernel(const uint8_t *__restrict__ x,
-                                                                            uint8_t *__restrict__ out, int64_t batch,
-                                                                            int64_t features, int slice, int nslices,
-                                                                            int64_t out_row_bytes) {
-    extern __shared__ __align__(16) uint8_t lds_raw[];
-    dl_u32x4 *stage = reinterpret_cast<dl_u32x4 *>(lds_raw);                        // 64 * slice bytes
-    uint64_t *words = reinterpret_cast<uint64_t *>(lds_raw + 64 * slice);            // [slice][WC]
-    const int64_t w0 = (int64_t) (blockIdx.x / (unsigned) nslices) * WC;
-    const int64_t f0 = (int64_t) (blockIdx.x % (unsigned) nslices) * slice;
-    const int fs = (int) (features - f0 < slice ? features - f0 : slice);           // this slice's features
-    const int groups = fs / 4;                                                       // dword columns
-    const int per_row = fs / 16;                                                     // 16-byte chunks per sample
-    const int chunks = 64 * per_row;
+// Variant for features % 16 == 0 that stages nothing on the way in: a workgroup owns WC word columns
+// (64 * WC consecutive samples, i.e. one contiguous region of the input) and a slice of the features.
+// A thread takes 16 features x 8 samples at a time: eight 16-byte loads (a wave's loads of one sample
+// row are contiguous), folded in registers into the 16 features' bytes for those 8 samples, which it
+// drops into an LDS tile of output words; the workgroup then writes 8 * WC contiguous bytes per feature
+// row.  The tile is laid out [feature % 16][feature / 16][WC words + 4 bytes] so that the lanes of a
+// wave (consecutive 16-feature chunks) fall 17 dwords apart, on distinct banks.
+#define DL_PACK_WC 8
+#define DL_PACK_PITCH (DL_PACK_WC * 8 + 4)
+#define DL_PACK_MAX_SLICE 2352                   // features per workgroup: 2352 * 68 bytes of LDS
 
-    for (int wc = 0; wc < WC; ++wc) {
-        const int64_t s0 = (w0 + wc) * 64;
-        if (s0 >= batch) break;                                                      // uniform
-        const int rows = (int) (batch - s0 < 64 ? batch - s0 : 64);                  // real samples
-        const uint8_t *src = x + s0 * features + f0;
-        __syncthreads();                                                             // previous column's readers are done
-        for (int i = threadIdx.x; i < chunks; i += DL_BLOCK) {
-            const int r = i / per_row, c = i - r * per_row;
-            stage[i] = r < rows ? __builtin_nontemporal_load(reinterpret_cast<const dl_u32x4 *>(src + r * features) + c)
-                                : dl_u32x4{0, 0, 0, 0};
+__global__ __launch_bounds__(DL_BLOCK) void packbits_batch_major_rows_kernel(const uint8_t *__restrict__ x,
+                                                                             uint8_t *__restrict__ out, int64_t batch,
+                                                                             int64_t features, int slice, int nslices,
+                                                                             int64_t out_row_bytes, uint32_t paired_blocks) {
+    extern __shared__ __align__(16) uint8_t tile[];                                  // [16][per_row][PITCH]
+    // Two workgroups share every 128-byte line of the output (64 bytes each): pairs stay on one of the 8
+    // XCDs, whose L2 merges the halves (workgroups are dealt to the XCDs round-robin by index).
+    uint32_t blk = blockIdx.x;
+    if (blk < paired_blocks) {
+        const uint32_t per = 2 * (uint32_t) nslices, xcd = blk % 8, j = blk / 8;
+        blk = ((j / per) * 8 + xcd) * per + j % per;
+    }
+    const int64_t w0 = (int64_t) (blk / (unsigned) nslices) * DL_PACK_WC;
+    const int64_t f0 = (int64_t) (blk % (unsigned) nslices) * slice;
+    const int fs = (int) (features - f0 < slice ? features - f0 : slice);           // this slice's features
+    const int per_row = fs / 16;                                                     // 16-byte chunks per sample
+    const int items = DL_PACK_WC * 8 * per_row;
+    const int64_t s0 = w0 * 64;
+
+    // item = 16 features x 8 samples: (oct, c), oct = wc * 8 + j the byte of the output row, c the 16-byte chunk
+    auto request = [&](int it, dl_u32x4 *v) __attribute__((always_inline)) {
+        const int oct = it / per_row, c = it - oct * per_row;
+        const int64_t row0 = s0 + 8 * oct;
+        const uint8_t *src = x + row0 * features + f0 + 16 * c;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            v[i] = row0 + i < batch ? __builtin_nontemporal_load(reinterpret_cast<const dl_u32x4 *>(src + i * features))
+                                    : dl_u32x4{0, 0, 0, 0};
+    };
+    auto fold = [&](int it, const dl_u32x4 *v) __attribute__((always_inline)) {
+        const int oct = it / per_row, c = it - oct * per_row;
+        uint8_t *dst = tile + (size_t) c * DL_PACK_PITCH + oct;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            uint32_t acc = 0;                                                        // byte k: feature 4 d + k, 8 samples
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t u = v[i][d];
+                acc |= (((((u & 0x7f7f7f7fu) + 0x7f7f7f7fu) | u) >> 7) & 0x01010101u) << i;
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                dst[(size_t) (4 * d + k) * per_row * DL_PACK_PITCH] = (uint8_t) (acc >> (8 * k));
         }
-        __syncthreads();
-        const uint32_t *flags = reinterpret_cast<const uint32_t *>(lds_raw);
-        for (int g = threadIdx.x; g < groups; g += DL_BLOCK) {
-            uint32_t oct[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                uint32_t acc = 0;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const uint32_t v = flags[(8 * j + i) * groups + g];
-                    acc |= (((((v & 0x7f7f7f7fu) + 0x7f7f7f7fu) | v) >> 7) & 0x01010101u) << i;
-                }
-                oct[j] = acc;
-            }
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                uint32_t lo = 0, hi = 0;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    lo |= ((oct[j] >> (8 * k)) & 0xffu) << (8 * j);
-                    hi |= ((oct[4 + j] >> (8 * k)) & 0xffu) << (8 * j);
-                }
-                words[(4 * g + k) * WC + wc] = ((uint64_t) hi << 32) | lo;
-            }
+    };
+    // a thread's next item is requested before the current one is folded, so its loads never stop
+    dl_u32x4 va[8], vb[8];
+    int it = threadIdx.x;
+    if (it < items) request(it, va);
+    for (; it < items; it += 2 * DL_BLOCK) {
+        const bool second = it + DL_BLOCK < items;
+        if (second) request(it + DL_BLOCK, vb);
+        fold(it, va);
+        if (second) {
+            if (it + 2 * DL_BLOCK < items) request(it + 2 * DL_BLOCK, va);
+            fold(it + DL_BLOCK, vb);
         }
     }
     __syncthreads();
-    // WC consecutive threads write the WC words of one feature row (out_row_bytes % 8 == 0 here)
+    // DL_PACK_WC consecutive threads write the words of one feature row (out_row_bytes % 8 == 0 here)
     const int64_t total_words = out_row_bytes / 8;
-    for (int i = threadIdx.x; i < fs * WC; i += DL_BLOCK) {
-        const int f = i / WC, wc = i - f * WC;
+    for (int i = threadIdx.x; i < fs * DL_PACK_WC; i += DL_BLOCK) {
+        const int f = i / DL_PACK_WC, wc = i - f * DL_PACK_WC;
+        const uint32_t *w = reinterpret_cast<const uint32_t *>(tile + ((size_t) (f % 16) * per_row + f / 16) * DL_PACK_PITCH) + 2 * wc;
         if (w0 + wc < total_words)
-            *reinterpret_cast<uint64_t *>(out + (f0 + f) * out_row_bytes + (w0 + wc) * 8) = words[f * WC + wc];
+            *reinterpret_cast<uint64_t *>(out + (f0 + f) * out_row_bytes + (w0 + wc) * 8) = ((uint64_t) w[1] << 32) | w[0];
     }
 }
 
@@ -1273,26 +1286,19 @@ extern "C" int dl_tensor_packbits_batch_major(const uint8_t *x, void *out, int64
     const int64_t gx = dl_ceil_div(dl_ceil_div(batch, 64), 16);
     if (gx > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     if (features % 16 == 0 && dl_aligned(x, 16) && out_row_bytes % 8 == 0) {
-        // A workgroup stages a slice of the features: 64 bytes of LDS per feature + 8 * WC for the result tile.
-        // Small footprints (several workgroups per CU overlap their load, fold and store phases) measured
-        // fastest: slices of 128 features with 8 word columns where rows are whole 128-byte lines (every
-        // request is then a full cache line, and feature rows are written in 64-byte runs), otherwise slices
-        // of up to 400 features with 2 word columns.
-        const bool lines = features % 128 == 0;
-        const int wc = lines ? 8 : 2;
-        const int64_t max_slice = lines ? 128 : 400;
-        const int64_t want = dl_ceil_div(features, max_slice);
-        const int64_t slice = dl_ceil_div(dl_ceil_div(features, want), 16) * 16;
+        // A workgroup takes 8 word columns and a slice of the features, 68 bytes of LDS per feature.  Measured:
+        // the longer the contiguous piece of a sample row a workgroup reads the better, down to one workgroup
+        // per CU (2352 features); slices are whole 128-byte lines where the rows are.
+        const int64_t unit = features % 128 == 0 ? 128 : 16;
+        const int64_t want = dl_ceil_div(features, DL_PACK_MAX_SLICE / unit * unit);
+        const int64_t slice = dl_ceil_div(dl_ceil_div(features, want), unit) * unit;
         const int64_t nslices = dl_ceil_div(features, slice);
-        const int64_t blocks = dl_ceil_div(dl_ceil_div(batch, 64), wc) * nslices;
-        if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
-        const size_t lds = (size_t) (64 * slice + slice * wc * 8);
-        if (wc == 2)
-            DL_LAUNCH(packbits_batch_major_lds_kernel<2>, dim3((unsigned) blocks), dim3(DL_BLOCK), lds, s, x,
-                      (uint8_t *) out, batch, features, (int) slice, (int) nslices, out_row_bytes);
-        else
-            DL_LAUNCH(packbits_batch_major_lds_kernel<8>, dim3((unsigned) blocks), dim3(DL_BLOCK), lds, s, x,
-                      (uint8_t *) out, batch, features, (int) slice, (int) nslices, out_row_bytes);
+        const int64_t blocks = dl_ceil_div(dl_ceil_div(batch, 64), DL_PACK_WC) * nslices;
+        if (blocks > 0x3fffffffLL) return DL_ERR_TOO_LARGE;
+        const size_t lds = (size_t) slice * DL_PACK_PITCH;
+        const int64_t group = 8 * 2 * nslices;                   // pairs of column groups, one set per XCD
+        DL_LAUNCH(packbits_batch_major_rows_kernel, dim3((unsigned) blocks), dim3(DL_BLOCK), lds, s, x, (uint8_t *) out,
+                  batch, features, (int) slice, (int) nslices, out_row_bytes, (uint32_t) (blocks / group * group));
     } else if (features % 4 == 0 && dl_aligned(x, 4)) {
         const int64_t gy = dl_ceil_div(features, 256);
         if (gy > 65535) return DL_ERR_TOO_LARGE;

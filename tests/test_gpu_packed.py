@@ -46,7 +46,8 @@ def test_packbits_nonzero_bytes_count_as_true(ext):
 
 @pytest.mark.parametrize("bits", [8, 16, 32, 64])
 @pytest.mark.parametrize("B,F", [(1, 1), (7, 3), (64, 8), (65, 12), (1000, 7), (1024, 256), (4112, 260), (70000, 2),
-                                 (3000, 784), (130, 1028), (200, 816), (333, 832), (129, 1648), (700, 9216)])
+                                 (3000, 784), (130, 1028), (200, 816), (333, 832), (129, 1648), (700, 9216),
+                                 (513, 16), (8200, 48), (1100, 2368), (600, 2352), (9000, 128)])
 def test_packbits_batch_major(ext, bits, B, F):
     rng = np.random.default_rng(F * 131 + B + bits)
     x = rng.random((B, F)) < 0.3
@@ -63,6 +64,12 @@ def test_packbits_batch_major_nonzero_bytes(ext):
     raw = torch.tensor([[0, 1, 2, 128], [255, 0, 7, 0], [3, 3, 0, 0]], dtype=torch.uint8).cuda()
     got, _ = ext.tensor_packbits_batch_major(raw.view(torch.bool), 8)
     want, _ = po.packbits((raw.cpu().numpy() != 0).T, 8)
+    assert np.array_equal(got.cpu().numpy(), want)
+    # rows of whole 16-byte chunks take the kernel that folds in registers: every byte value, every position
+    rng = np.random.default_rng(5)
+    raw = torch.as_tensor(rng.integers(0, 256, (777, 32), dtype=np.uint8) * (rng.random((777, 32)) < 0.5)).cuda()
+    got, _ = ext.tensor_packbits_batch_major(raw.view(torch.bool), 64)
+    want, _ = po.packbits((raw.cpu().numpy() != 0).T, 64)
     assert np.array_equal(got.cpu().numpy(), want)
 
 
