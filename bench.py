@@ -48,8 +48,8 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 TRAFFIC_JSON = os.path.join(ROOT, "profiles", "packed_kernel_traffic.json")
 # what the measured traffic of the packed launches depends on: the kernels and the launch plan
-TRAFFIC_SOURCES = ("difflogic_amd/csrc/packed.hip", "difflogic_amd/csrc/schedule.cpp", "difflogic_amd/csrc/dl_common.h",
-                   "difflogic_amd/packbitstensor.py")
+TRAFFIC_SOURCES = ("difflogic_amd/csrc/packed.hip", "difflogic_amd/csrc/count_chain.h", "difflogic_amd/csrc/schedule.cpp",
+                   "difflogic_amd/csrc/dl_common.h", "difflogic_amd/packbitstensor.py")
 
 
 def parse():
