@@ -333,8 +333,9 @@ def train_alg_bytes(dims, B):
 
 def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor, x, steps, warmup):
     """fp32 training step of one configuration with CrossEntropy: forward+backward and
-    forward+backward+Adam(lr 0.01, torch's fused multi-tensor kernel), each eager and replayed as
-    one HIP graph."""
+    forward+backward+Adam(lr 0.01), each eager and replayed as one HIP graph; once for the model as
+    the reference's user writes it (torch's fused Adam) and once with the training epilogue of this
+    package (last layer fused with GroupSum, difflogic_amd.FusedAdam)."""
     from difflogic_amd.graphs import GraphedTrainStep
     torch.manual_seed(0)
     mods, d = [torch.nn.Flatten()], F
@@ -365,7 +366,7 @@ def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor
 
     res = {"workload": name, "dtype": "f32", "algorithmic_GB_per_step": round(alg / 1e9, 3)}
 
-    def measure(net, out):
+    def measure(net, out, make_opt):
         """forward+backward and forward+backward+Adam of `net`, eager and as a replayed HIP graph."""
         def fwd_bwd():
             net.zero_grad(set_to_none=True)
@@ -389,7 +390,7 @@ def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor
         gc.collect()
 
         # with the optimizer step (experiments/main.py:169,174-181).  The weights move, so the loss differs per step.
-        opt = torch.optim.Adam(net.parameters(), lr=0.01, fused=True, capturable=True)
+        opt = make_opt(net.parameters())
 
         def full_step():
             opt.zero_grad(set_to_none=True)
@@ -412,9 +413,10 @@ def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor
 
     # the model as a user of the reference writes it, then with the last LogicLayer and GroupSum merged
     # (difflogic_amd.fuse_group_sum: same parameters; the Adam steps above moved them, so the losses differ)
-    measure(model, res)
-    res["fused_group_sum"] = {}
-    measure(dl.fuse_group_sum(model).train(), res["fused_group_sum"])
+    measure(model, res, lambda ps: torch.optim.Adam(ps, lr=0.01, fused=True, capturable=True))
+    res["optimizer"] = "torch.optim.Adam(fused=True, capturable=True)"
+    res["fused_group_sum"] = {"optimizer": "difflogic_amd.FusedAdam (one launch over all weight tensors)"}
+    measure(dl.fuse_group_sum(model).train(), res["fused_group_sum"], lambda ps: dl.FusedAdam(ps, lr=0.01))
     return res, model
 
 

@@ -1593,3 +1593,112 @@ extern "C" const char *dl_status_string(int status) {
     default: return "unknown status";
     }
 }
+
+// ---- Adam over all of a model's weight tensors in one launch ---------------------------------
+// Elementwise and bound by its 7 float streams (p, g, m, v read; p, m, v written).  The tensors'
+// pointers and sizes travel in the kernel arguments; a block takes DL_ADAM_BLOCK_ELEMS consecutive
+// elements of one tensor, found through the running block counts.  The step count lives on the
+// device so that a captured launch advances it on every replay; a one-thread kernel advances it and
+// derives the two bias-correction factors before the update runs.
+#define DL_ADAM_MAX_TENSORS 48
+#define DL_ADAM_BLOCK_ELEMS 4096
+
+namespace {
+
+struct AdamTensors {
+    float *p[DL_ADAM_MAX_TENSORS];
+    const float *g[DL_ADAM_MAX_TENSORS];
+    float *m[DL_ADAM_MAX_TENSORS];
+    float *v[DL_ADAM_MAX_TENSORS];
+    int64_t numel[DL_ADAM_MAX_TENSORS];
+    uint32_t first_block[DL_ADAM_MAX_TENSORS + 1];       // running sum of ceil(numel / DL_ADAM_BLOCK_ELEMS)
+    int count;
+};
+
+// state[0]: updates done; state[1], state[2]: lr / (1 - beta1^step) and 1 / sqrt(1 - beta2^step) of the update
+// under way, in double arithmetic (1 - 0.999^s cancels badly in float for small s)
+__global__ void adam_advance_kernel(float *state, double lr, double beta1, double beta2) {
+    const double s = (double) state[0] + 1.0;
+    state[0] = (float) s;
+    state[1] = (float) (lr / (1.0 - pow(beta1, s)));
+    state[2] = (float) (1.0 / sqrt(1.0 - pow(beta2, s)));
+}
+
+__global__ __launch_bounds__(DL_BLOCK) void adam_kernel(AdamTensors t, const float *__restrict__ state, float beta2,
+                                                        float one_minus_beta1, float one_minus_beta2, float eps,
+                                                        float weight_decay) {
+    // which tensor: scalar search over at most 48 entries
+    int ti = 0;
+    while (ti + 1 < t.count && blockIdx.x >= t.first_block[ti + 1]) ++ti;
+    const int64_t base = (int64_t) (blockIdx.x - t.first_block[ti]) * DL_ADAM_BLOCK_ELEMS;
+    const int64_t n = t.numel[ti];
+    float *__restrict__ p = t.p[ti];
+    const float *__restrict__ g = t.g[ti];
+    float *__restrict__ m = t.m[ti];
+    float *__restrict__ v = t.v[ti];
+
+    const float step_size = state[1], inv_bc2_sqrt = state[2];
+
+    auto update = [&](float &pi, float gi, float &mi, float &vi) {
+        if (weight_decay != 0.0f) gi = fmaf(weight_decay, pi, gi);
+        mi = fmaf(gi - mi, one_minus_beta1, mi);
+        vi = fmaf(beta2, vi, one_minus_beta2 * gi * gi);
+        pi -= step_size * mi / (sqrtf(vi) * inv_bc2_sqrt + eps);
+    };
+    const bool vec = ((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(m) |
+                       reinterpret_cast<uintptr_t>(v)) & 15) == 0;
+#pragma unroll
+    for (int r = 0; r < DL_ADAM_BLOCK_ELEMS / (4 * DL_BLOCK); ++r) {
+        const int64_t i = base + ((int64_t) r * DL_BLOCK + threadIdx.x) * 4;
+        if (i >= n) break;
+        if (vec && i + 4 <= n) {
+            float4 pv = *reinterpret_cast<const float4 *>(p + i), gv = *reinterpret_cast<const float4 *>(g + i);
+            float4 mv = *reinterpret_cast<const float4 *>(m + i), vv = *reinterpret_cast<const float4 *>(v + i);
+            update(pv.x, gv.x, mv.x, vv.x);
+            update(pv.y, gv.y, mv.y, vv.y);
+            update(pv.z, gv.z, mv.z, vv.z);
+            update(pv.w, gv.w, mv.w, vv.w);
+            *reinterpret_cast<float4 *>(p + i) = pv;
+            *reinterpret_cast<float4 *>(m + i) = mv;
+            *reinterpret_cast<float4 *>(v + i) = vv;
+        } else {
+            for (int64_t j = i; j < i + 4 && j < n; ++j) update(p[j], g[j], m[j], v[j]);
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int dl_adam_max_tensors(void) { return DL_ADAM_MAX_TENSORS; }
+
+extern "C" int dl_adam_step(int count, float *const *p, const float *const *g, float *const *m, float *const *v,
+                            const int64_t *numel, float *state, double lr, double beta1, double beta2, double eps,
+                            double weight_decay, void *stream) {
+    if (count < 0 || !(lr >= 0.0) || !(beta1 >= 0.0 && beta1 < 1.0) || !(beta2 >= 0.0 && beta2 < 1.0) || !(eps >= 0.0) ||
+        !(weight_decay >= 0.0))
+        return DL_ERR_INVALID_ARGUMENT;
+    if (count > DL_ADAM_MAX_TENSORS) return DL_ERR_TOO_LARGE;
+    if (count == 0) return DL_OK;
+    if (!p || !g || !m || !v || !numel || !state) return DL_ERR_INVALID_ARGUMENT;
+    AdamTensors t;
+    uint64_t blocks = 0;
+    t.count = 0;
+    for (int i = 0; i < count; ++i) {
+        if (numel[i] < 0) return DL_ERR_INVALID_ARGUMENT;
+        if (numel[i] == 0) continue;
+        if (!p[i] || !g[i] || !m[i] || !v[i]) return DL_ERR_INVALID_ARGUMENT;
+        const int k = t.count++;
+        t.p[k] = p[i], t.g[k] = g[i], t.m[k] = m[i], t.v[k] = v[i], t.numel[k] = numel[i];
+        t.first_block[k] = (uint32_t) blocks;
+        blocks += (uint64_t) dl_ceil_div(numel[i], DL_ADAM_BLOCK_ELEMS);
+        if (blocks > 0x7fffffffULL) return DL_ERR_TOO_LARGE;
+    }
+    hipStream_t s = (hipStream_t) stream;
+    DL_LAUNCH(adam_advance_kernel, dim3(1), dim3(1), 0, s, state, lr, beta1, beta2);
+    if (t.count > 0) {
+        t.first_block[t.count] = (uint32_t) blocks;
+        DL_LAUNCH(adam_kernel, dim3((unsigned) blocks), dim3(DL_BLOCK), 0, s, t, (const float *) state, (float) beta2,
+                  (float) (1.0 - beta1), (float) (1.0 - beta2), (float) eps, (float) weight_decay);
+    }
+    return dl_launch_status();
+}

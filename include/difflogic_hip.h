@@ -192,6 +192,22 @@ int dl_logic_backward_chained_grouped(const void *x, const int32_t *verts, const
                                       void *grad_x, void *workspace, int64_t in_dim, int64_t out_dim,
                                       int64_t batch, int64_t k, double scale, int dtype, void *stream);
 
+/* The optimizer step of the reference's training loop (torch.optim.Adam(lr=...).step(),
+ * experiments/main.py:169,179) for all of a model's fp32 weight tensors in one launch.  No counterpart
+ * in the reference's extension.  Semantics of torch.optim.Adam (amsgrad and maximize off):
+ *   step += 1;  g += weight_decay * p;  m += (1 - beta1) * (g - m);  v = beta2 * v + (1 - beta2) * g * g;
+ *   p -= lr / (1 - beta1^step) * m / (sqrt(v) / sqrt(1 - beta2^step) + eps)
+ *   p, g, m, v : HOST arrays of `count` (<= dl_adam_max_tensors()) DEVICE pointers to contiguous
+ *                fp32 tensors of numel[i] elements (numel: HOST array); m, v start as zeros.
+ *   state      : DEVICE fp32 [4]; state[0] holds the number of updates done so far (starts at 0) and
+ *                is advanced on the device, so a launch captured into a HIP graph stays correct on
+ *                replay; state[1..2] are scratch (the bias-correction factors of the update under
+ *                way, computed in double); state[3] is unused. */
+int dl_adam_max_tensors(void);
+int dl_adam_step(int count, float *const *p, const float *const *g, float *const *m, float *const *v,
+                 const int64_t *numel, float *state, double lr, double beta1, double beta2, double eps,
+                 double weight_decay, void *stream);
+
 /* ---- packed inference mode ------------------------------------------------------------ */
 
 /* Replaces `eval` = logic_layer_cuda_eval (difflogic.cpp:63-68, difflogic_kernel.cu:503-541).
