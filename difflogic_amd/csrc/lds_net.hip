@@ -404,23 +404,21 @@ __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint
         for (int i = 0; i < 2 * COLS; ++i)
 #pragma unroll
             for (int p = 0; p < NP0; ++p) pl[i][p] = 0;
-        // four neurons at a time: their records are requested an iteration ahead, their output words are
-        // compressed by a carry-save tree into one word of weight 4 that ripples into the planes
-        // above; neurons past the end of the class contribute zero words
+        // Four neurons at a time: their records are requested an iteration ahead, their output words are
+        // compressed by a carry-save tree into one word of weight 4 that ripples into the planes above.
+        // What is left of the class after the whole quads (fewer than 256 neurons) goes row by row: 64 neurons,
+        // lanes past the end of the class contributing zero words, rippled in with weight 1.
         const uint32_t *ctab = ltab + cls * per_class;
         if (cls != wave) load_class_records(rc, ctab, lane, per_class);
-        for (int64_t i0 = lane; i0 < per_class; i0 += 4 * DL_WAVE) {
-            uint32_t r4[4], live[4];
+        const int64_t quads = per_class / (4 * DL_WAVE);
+        for (int64_t q = 0; q < quads; ++q) {
+            uint32_t r4[4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) r4[u] = rc[u], live[u] = i0 + u * DL_WAVE < per_class ? ~0u : 0u;
-            if (i0 - lane + 4 * DL_WAVE < per_class) load_class_records(rc, ctab, i0 + 4 * DL_WAVE, per_class);
+            for (int u = 0; u < 4; ++u) r4[u] = rc[u];
+            load_class_records(rc, ctab, (q + 1) * 4 * DL_WAVE + lane, per_class);   // next quad, or the rest
             Row<COLS> y[4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                y[u] = gate_rows<COLS>(act, r4[u]);
-#pragma unroll
-                for (int i = 0; i < 2 * COLS; ++i) y[u].d[i] &= live[u];
-            }
+            for (int u = 0; u < 4; ++u) y[u] = gate_rows<COLS>(act, r4[u]);
 #pragma unroll
             for (int i = 0; i < 2 * COLS; ++i) {
                 uint32_t t2a, t2b, carry;
@@ -431,6 +429,23 @@ __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint
                 for (int p = 2; p < NP0; ++p) {                  // counter += carry * 4
                     const uint32_t old = pl[i][p];
                     pl[i][p] = old ^ carry;
+                    carry = old & carry;
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t i = (quads * 4 + u) * DL_WAVE;          // first neuron of this row
+            if (i >= per_class) break;                            // uniform
+            Row<COLS> y = gate_rows<COLS>(act, rc[u]);
+            const uint32_t live = i + lane < per_class ? ~0u : 0u;
+#pragma unroll
+            for (int d = 0; d < 2 * COLS; ++d) {
+                uint32_t carry = y.d[d] & live;
+#pragma unroll
+                for (int p = 0; p < NP0; ++p) {                  // counter += word
+                    const uint32_t old = pl[d][p];
+                    pl[d][p] = old ^ carry;
                     carry = old & carry;
                 }
             }
