@@ -412,11 +412,12 @@ def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor
         gc.collect()
 
     # the model as a user of the reference writes it, then with the last LogicLayer and GroupSum merged
-    # (difflogic_amd.fuse_group_sum: same parameters; the Adam steps above moved them, so the losses differ)
+    # and the first two layers merged (difflogic_amd.fuse_for_training: same parameters; the Adam steps above moved
+    # them, so the losses differ)
     measure(model, res, lambda ps: torch.optim.Adam(ps, lr=0.01, fused=True, capturable=True))
     res["optimizer"] = "torch.optim.Adam(fused=True, capturable=True)"
-    res["fused_group_sum"] = {"optimizer": "difflogic_amd.FusedAdam (one launch over all weight tensors)"}
-    measure(dl.fuse_group_sum(model).train(), res["fused_group_sum"], lambda ps: dl.FusedAdam(ps, lr=0.01))
+    res["fused_for_training"] = {"optimizer": "difflogic_amd.FusedAdam (one launch over all weight tensors)"}
+    measure(dl.fuse_for_training(model).train(), res["fused_for_training"], lambda ps: dl.FusedAdam(ps, lr=0.01))
     return res, model
 
 

@@ -626,13 +626,25 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_w_chain_kernel(const T *__r
 // owns `chunk` positions [s0, s0 + chunk); it recomputes the last neuron of the chunk before it to get
 // the carry into its first position, so chunks do not exchange partial rows.
 // ------------------------------------------------------------------------------------------
-template <typename T, int VEC, int CPL>
+// LOWER: the layer BELOW this one (whose output x is) needs no grad_x of its own and gets its grad_w
+// here: a vertex's finished grad_x row is the grad_y row of neuron `vertex` of the layer below, so its
+// four corner sums are taken on the spot from the row in registers and the two input rows of that
+// neuron (`low.x`, gathered through `low.a`, `low.b`), and the row is not stored at all.  Only the
+// vertices that finish in backward_fix_kernel still go through memory (backward_w_rows_kernel).
+template <typename T> struct LowerLayer {
+    const T *x;                 // [in_dim of the layer below, batch]
+    const int64_t *a, *b;       // its wiring, [in_dim]
+    const T *probs;             // its gate probabilities [in_dim, 16]: chain the softmax backward; null: plain grad_w
+    T *gw;                      // [in_dim, 16]
+};
+
+template <typename T, int VEC, int CPL, bool LOWER>
 __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
     const T *__restrict__ x, const int32_t *__restrict__ verts, const int32_t *__restrict__ neuron,
     const uint8_t *__restrict__ flip, const int32_t *__restrict__ dst, const T *__restrict__ w,
     const T *__restrict__ gy, const T *__restrict__ probs, T *__restrict__ gw,
     typename Acc<T>::type *__restrict__ partial, T *__restrict__ gx, T *__restrict__ overflow, int64_t steps, int chunk,
-    int64_t in_dim, int64_t out_dim, int64_t ncols, typename Acc<T>::type scale, int64_t gdiv) {
+    int64_t in_dim, int64_t out_dim, int64_t ncols, typename Acc<T>::type scale, int64_t gdiv, LowerLayer<T> low) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
     const int wave = dl_wave_in_block();
@@ -654,8 +666,30 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
             out[q] = (valid && col < ncols) ? base[row * ncols + col] : zero;
         }
     };
-    auto store_row = [&](int32_t row, const C (&val)[CPL][VEC]) {
+    // la, lb: with LOWER, the two input rows of neuron `row` of the layer below (requested a step ahead)
+    auto store_row = [&](int32_t row, const C (&val)[CPL][VEC], const P *la, const P *lb) {
         if (row < 0) return;
+        if (LOWER && row < in_dim) {
+            // as backward_w_kernel on the row this would have stored: same values, same order of additions
+            C s00 = (C) 0, s01 = (C) 0, s10 = (C) 0, s11 = (C) 0;
+#pragma unroll
+            for (int q = 0; q < CPL; ++q) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const C g = up<T>(down<T, C>(val[q][e] * scale));
+                    const C av = up<T>(la[q].v[e]), bv = up<T>(lb[q].v[e]);
+                    const C ga = g * av, gna = g - ga;
+                    const C t11 = ga * bv, t01 = gna * bv;
+                    s11 += t11;
+                    s10 += ga - t11;
+                    s01 += t01;
+                    s00 += gna - t01;
+                }
+            }
+            wave_sum4(s00, s01, s10, s11, lane);
+            store_grad_w<T>(lane, true, row, s00, s01, s10, s11, low.probs, low.gw);
+            return;
+        }
         P *base = row < in_dim ? reinterpret_cast<P *>(gx) + (int64_t) row * ncols
                                : reinterpret_cast<P *>(overflow) + ((int64_t) row - in_dim) * ncols;
 #pragma unroll
@@ -665,6 +699,15 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
 #pragma unroll
             for (int e = 0; e < VEC; ++e) r.v[e] = down<T, C>(val[q][e] * scale);
             if (col < ncols) base[col] = r;
+        }
+    };
+    auto lower_rows = [&](int32_t row, P *la, P *lb) {           // row: wave-uniform
+        if constexpr (LOWER) {
+            const bool valid = row >= 0 && row < in_dim;
+            const int64_t r = valid ? row : 0;
+            const P *lx = reinterpret_cast<const P *>(low.x);
+            load_row(lx, low.a[r], valid, la);
+            load_row(lx, low.b[r], valid, lb);
         }
     };
 
@@ -701,22 +744,24 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
     const int gate = lane & 15;
     // rows of step i: the new input row, the neuron's grad_y row (zero for a step without a neuron)
     // and, in every 16-lane row, the neuron's 16 gate probabilities
-    auto fetch = [&](int i, P *row, P *grad, C &prob) {
+    constexpr int LCPL = LOWER ? CPL : 1;
+    auto fetch = [&](int i, P *row, P *grad, C &prob, P *la, P *lb) {
         const int32_t n = __builtin_amdgcn_readlane(sch_n, i);
         const bool valid = n >= 0;
         const int64_t nn = valid ? n : 0;
         load_row(xv, __builtin_amdgcn_readlane(sch_v, i), true, row);
         load_row(gv, grad_row(nn, gdiv), valid, grad);
         prob = up<T>(w[nn * 16 + gate]);
+        lower_rows(__builtin_amdgcn_readlane(sch_d, i), la, lb);
     };
-    P cur[CPL], g[CPL];
+    P cur[CPL], g[CPL], la[LCPL], lb[LCPL];
     C pw;
-    fetch(0, cur, g, pw);
+    fetch(0, cur, g, pw, la, lb);
 #pragma unroll 1
     for (int i = 0; i < cnt; ++i) {
-        P ncur[CPL], ng[CPL];
+        P ncur[CPL], ng[CPL], nla[LCPL], nlb[LCPL];
         C npw = (C) 0;
-        if (i + 1 < cnt) fetch(i + 1, ncur, ng, npw);
+        if (i + 1 < cnt) fetch(i + 1, ncur, ng, npw, nla, nlb);
         const int32_t n = __builtin_amdgcn_readlane(sch_n, i);
         const bool valid = n >= 0;
         const int64_t nn = valid ? n : 0;
@@ -745,7 +790,6 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
                 carry[q][e] = gg * dl_fma(u0, dd, kv);
             }
         }
-        store_row(__builtin_amdgcn_readlane(sch_d, i), out);
         wave_sum4(s00, s01, s10, s11, lane);
         if (partial == nullptr) {
             // as store_grad_w, with the probabilities already at hand
@@ -764,32 +808,43 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
             const C mine = lane == 0 ? s00 : lane == 1 ? s01 : lane == 2 ? s10 : s11;
             partial[((int64_t) blockIdx.y * out_dim + nn) * 4 + lane] = mine;
         }
+        store_row(__builtin_amdgcn_readlane(sch_d, i), out, la, lb);
 #pragma unroll
         for (int q = 0; q < CPL; ++q) {
             prev[q] = cur[q];
             cur[q] = ncur[q];
             g[q] = ng[q];
         }
+        if (LOWER) {
+#pragma unroll
+            for (int q = 0; q < LCPL; ++q) la[q] = nla[q], lb[q] = nlb[q];
+        }
         pw = npw;
     }
-    if (s1 == steps) store_row(dst[steps], carry);   // the schedule's last position
+    if (s1 == steps) {                                // the schedule's last position
+        const int32_t last = dst[steps];
+        lower_rows(last, la, lb);
+        store_row(last, carry, la, lb);
+    }
 }
 
 // grad_x rows of the vertices that backward_chain_kernel could not finish in one write: vertex
 // fix_vertex[i] is the sum, in slot order, of overflow rows [fix_start[i], fix_start[i + 1])
 // (no rows: the input feeds no neuron and its gradient is zero).
+// compact: row i of gx instead of row fix_vertex[i] (gx then has n_fix rows only).
 template <typename T, int VEC>
 __global__ __launch_bounds__(DL_BLOCK) void backward_fix_kernel(const T *__restrict__ overflow,
                                                                 const int32_t *__restrict__ fix_vertex,
                                                                 const int32_t *__restrict__ fix_start,
-                                                                T *__restrict__ gx, int64_t n_fix, int64_t ncols) {
+                                                                T *__restrict__ gx, int64_t n_fix, int64_t ncols,
+                                                                bool compact) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
     const int wave = dl_wave_in_block();
     const int lane = dl_lane();
     const int64_t i = (int64_t) blockIdx.x * 4 + wave;
     if (i >= n_fix) return;
-    const int64_t v = fix_vertex[i];
+    const int64_t v = compact ? i : (int64_t) fix_vertex[i];
     const int32_t r0 = fix_start[i], r1 = fix_start[i + 1];
     const P *ov = reinterpret_cast<const P *>(overflow);
     P *out = reinterpret_cast<P *>(gx);
@@ -807,6 +862,40 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_fix_kernel(const T *__restr
         for (int e = 0; e < VEC; ++e) res.v[e] = down<T, C>(acc[e]);
         out[v * ncols + col] = res;
     }
+}
+
+// backward_w of the layer below for the few vertices whose grad_x row backward_fix_kernel finished:
+// neuron list[i] of that layer, its grad_y row = row i of `rows`.  One wave per neuron, the sums in
+// the order of backward_w_kernel.
+template <typename T, int VEC>
+__global__ __launch_bounds__(DL_BLOCK) void backward_w_rows_kernel(LowerLayer<T> low, const int32_t *__restrict__ list,
+                                                                   const T *__restrict__ rows, int64_t n_list,
+                                                                   int64_t ncols) {
+    typedef typename Acc<T>::type C;
+    typedef Pack<T, VEC> P;
+    const int lane = dl_lane();
+    const int64_t i = (int64_t) blockIdx.x * 4 + dl_wave_in_block();
+    if (i >= n_list) return;
+    const int64_t n = list[i];
+    const P *xv = reinterpret_cast<const P *>(low.x);
+    const P *gv = reinterpret_cast<const P *>(rows) + i * ncols;
+    const int64_t ia = low.a[n], ib = low.b[n];
+    C s00 = (C) 0, s01 = (C) 0, s10 = (C) 0, s11 = (C) 0;
+    for (int64_t col = lane; col < ncols; col += DL_WAVE) {
+        const P va = xv[ia * ncols + col], vb = xv[ib * ncols + col], vg = gv[col];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const C av = up<T>(va.v[e]), bv = up<T>(vb.v[e]), g = up<T>(vg.v[e]);
+            const C ga = g * av, gna = g - ga;
+            const C t11 = ga * bv, t01 = gna * bv;
+            s11 += t11;
+            s10 += ga - t11;
+            s01 += t01;
+            s00 += gna - t01;
+        }
+    }
+    wave_sum4(s00, s01, s10, s11, lane);
+    store_grad_w<T>(lane, true, n, s00, s01, s10, s11, low.probs, low.gw);
 }
 
 // grad_w from the per-segment corner sums of backward_chain_kernel, added in segment order.
@@ -1253,7 +1342,8 @@ template <typename T>
 int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, const uint8_t *flip, const int32_t *dst,
                      int64_t steps, const void *w, const void *gy, bool softmax_backward, const int32_t *fix_vertex,
                      const int32_t *fix_start, int64_t n_fix, int64_t overflow_rows, void *gw, void *gx, void *workspace,
-                     int64_t in_dim, int64_t out_dim, int64_t batch, double scale, hipStream_t s, int64_t gdiv = 0) {
+                     int64_t in_dim, int64_t out_dim, int64_t batch, double scale, hipStream_t s, int64_t gdiv = 0,
+                     const LowerLayer<T> *lower = nullptr) {
     typedef typename Acc<T>::type C;
     constexpr int V = Vec16<T>::n;
     if (batch % V != 0 || !dl_aligned(x, 16) || !dl_aligned(gy, 16) || !dl_aligned(gx, 16) || !dl_aligned(workspace, 16))
@@ -1261,6 +1351,9 @@ int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron,
     const int64_t ncols = batch / V;
     if (ncols > DL_ROWS_MAX_VECTORS) return DL_ERR_TOO_LARGE;
     const int segments = row_segments(ncols);
+    // with `lower`: whole rows per wave only, and gx holds the n_fix rows that finish after the pass
+    if (lower && (segments > 1 || !dl_aligned(lower->x, 16))) return DL_ERR_TOO_LARGE;
+    const LowerLayer<T> none = {nullptr, nullptr, nullptr, nullptr, nullptr};
     // workspace: [segments x out x 4 corner sums (only with several segments)] [overflow rows]
     const int64_t partial_bytes = backward_partial_bytes<T>(out_dim, batch);
     if ((partial_bytes > 0 || overflow_rows > 0) && workspace == nullptr) return DL_ERR_INVALID_ARGUMENT;
@@ -1272,9 +1365,15 @@ int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron,
     const dim3 grid((unsigned) blocks, (unsigned) segments), block(DL_BLOCK);
     const T *xp = (const T *) x, *wp = (const T *) w, *gp = (const T *) gy, *pp = softmax_backward ? wp : nullptr;
     constexpr int H = V >= 2 ? V / 2 : 1;
-#define DL_LAUNCH_BACKWARD_CHAIN(VV, CPL, NC)                                                                              \
-    DL_LAUNCH((backward_chain_kernel<T, VV, CPL>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp, pp, (T *) gw, \
-              partial, (T *) gx, overflow, steps, chunk, in_dim, out_dim, NC, (C) scale, gdiv)
+#define DL_LAUNCH_BACKWARD_CHAIN(VV, CPL, NC)                                                                               \
+    do {                                                                                                                    \
+        if (lower)                                                                                                          \
+            DL_LAUNCH((backward_chain_kernel<T, VV, CPL, true>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp,  \
+                      pp, (T *) gw, partial, (T *) gx, overflow, steps, chunk, in_dim, out_dim, NC, (C) scale, gdiv, *lower); \
+        else                                                                                                                \
+            DL_LAUNCH((backward_chain_kernel<T, VV, CPL, false>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp, \
+                      pp, (T *) gw, partial, (T *) gx, overflow, steps, chunk, in_dim, out_dim, NC, (C) scale, gdiv, none);  \
+    } while (0)
     if (V >= 2 && ncols <= DL_WAVE / 2)
         DL_LAUNCH_BACKWARD_CHAIN(H, 1, 2 * ncols);   // short rows: 8-byte vectors use all 64 lanes
     else if (ncols <= DL_WAVE)
@@ -1296,7 +1395,11 @@ int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron,
     }
     if (n_fix == 0) return DL_OK;
     DL_LAUNCH((backward_fix_kernel<T, V>), dim3((unsigned) fix_blocks, col_tiles(ncols)), block, 0, s,
-              (const T *) overflow, fix_vertex, fix_start, (T *) gx, n_fix, ncols);
+              (const T *) overflow, fix_vertex, fix_start, (T *) gx, n_fix, ncols, lower != nullptr);
+    st = dl_launch_status();
+    if (st != DL_OK || !lower) return st;
+    DL_LAUNCH((backward_w_rows_kernel<T, V>), dim3((unsigned) fix_blocks), block, 0, s, *lower, fix_vertex, (const T *) gx,
+              n_fix, ncols);
     return dl_launch_status();
 }
 
@@ -1336,6 +1439,45 @@ extern "C" int dl_logic_backward_chained(const void *x, const int32_t *verts, co
     default:
         return backward_chain_t<double>(x, verts, neuron, flip, dst, steps, w, grad_y, sb, fix_vertex, fix_start, n_fix,
                                         overflow_rows, grad_w, grad_x, workspace, in_dim, out_dim, batch, scale, s);
+    }
+}
+
+extern "C" int dl_logic_backward_chained_lower(const void *x, const int32_t *verts, const int32_t *neuron,
+                                               const uint8_t *flip, const int32_t *dst, int64_t steps, const void *w,
+                                               const void *grad_y, int softmax_backward, const int32_t *fix_vertex,
+                                               const int32_t *fix_start, int64_t n_fix, int64_t overflow_rows,
+                                               void *grad_w, void *fix_rows, void *workspace, const void *x_lower,
+                                               const int64_t *a_lower, const int64_t *b_lower, const void *probs_lower,
+                                               void *grad_w_lower, int64_t in_dim, int64_t out_dim, int64_t batch,
+                                               double scale, int dtype, void *stream) {
+    if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
+    if (in_dim <= 0 || out_dim <= 0 || batch <= 0 || steps < out_dim || n_fix < 0 || n_fix > in_dim || overflow_rows < 0)
+        return DL_ERR_INVALID_ARGUMENT;
+    if (!x || !verts || !neuron || !flip || !dst || !w || !grad_y || !grad_w || !x_lower || !a_lower || !b_lower ||
+        !grad_w_lower)
+        return DL_ERR_INVALID_ARGUMENT;
+    if (n_fix > 0 && (!fix_vertex || !fix_start || !fix_rows)) return DL_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t) stream;
+    const bool sb = softmax_backward != 0;
+    switch (dtype) {
+    case DL_F16: {
+        const LowerLayer<__half> low = {(const __half *) x_lower, a_lower, b_lower, (const __half *) probs_lower,
+                                        (__half *) grad_w_lower};
+        return backward_chain_t<__half>(x, verts, neuron, flip, dst, steps, w, grad_y, sb, fix_vertex, fix_start, n_fix,
+                                        overflow_rows, grad_w, fix_rows, workspace, in_dim, out_dim, batch, scale, s, 0, &low);
+    }
+    case DL_F32: {
+        const LowerLayer<float> low = {(const float *) x_lower, a_lower, b_lower, (const float *) probs_lower,
+                                       (float *) grad_w_lower};
+        return backward_chain_t<float>(x, verts, neuron, flip, dst, steps, w, grad_y, sb, fix_vertex, fix_start, n_fix,
+                                       overflow_rows, grad_w, fix_rows, workspace, in_dim, out_dim, batch, scale, s, 0, &low);
+    }
+    default: {
+        const LowerLayer<double> low = {(const double *) x_lower, a_lower, b_lower, (const double *) probs_lower,
+                                        (double *) grad_w_lower};
+        return backward_chain_t<double>(x, verts, neuron, flip, dst, steps, w, grad_y, sb, fix_vertex, fix_start, n_fix,
+                                        overflow_rows, grad_w, fix_rows, workspace, in_dim, out_dim, batch, scale, s, 0, &low);
+    }
     }
 }
 

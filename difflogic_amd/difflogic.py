@@ -314,6 +314,113 @@ class FusedLogicLayerGroupSum(torch.nn.Module):
         return "{}, {}".format(self.layer.extra_repr(), self.group_sum.extra_repr())
 
 
+class LogicLayerPairFunction(torch.autograd.Function):
+    """A model's first two LogicLayers as one autograd node: feature-major input [in, B] that
+    needs no gradient and both layers' gate logits -> the second layer's output [out2, B].  In the
+    backward pass the first layer's grad_y (= the second layer's grad_x) is consumed row by row
+    where the second layer's one-pass backward finishes it and never touches memory."""
+
+    @staticmethod
+    def forward(ctx, x, a1, b1, logits1, schedule1, a2, b2, logits2, start2, idx2, grad_factor2, schedule2):
+        y1, probs1 = difflogic_cuda.forward_logits(x, a1, b1, logits1.detach().contiguous(), schedule1)
+        y2, probs2 = difflogic_cuda.forward_logits(y1, a2, b2, logits2.detach().contiguous(), schedule2)
+        ctx.save_for_backward(x, a1, b1, probs1, y1, a2, b2, probs2, start2, idx2)
+        ctx.grad_factor2, ctx.schedule1, ctx.schedule2 = grad_factor2, schedule1, schedule2
+        return y2
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        x, a1, b1, probs1, y1, a2, b2, probs2, start2, idx2 = ctx.saved_tensors
+        grad_y = grad_y.contiguous()
+        want1, want2 = ctx.needs_input_grad[3], ctx.needs_input_grad[7]
+        g1 = g2 = None
+        if want1 and want2:
+            both = difflogic_cuda.backward_chained_lower(y1, probs2, grad_y, ctx.schedule2, x, a1, b1, probs1,
+                                                         ctx.grad_factor2, softmax_backward=True)
+            if both is not None:
+                g2, g1 = both
+                return None, None, None, g1, None, None, None, g2, None, None, None, None
+        # the separate kernels, as two LogicLayers in a row would run them
+        if want1:
+            both = difflogic_cuda.backward_chained(y1, probs2, grad_y, ctx.schedule2, ctx.grad_factor2,
+                                                   softmax_backward=True) if want2 else None
+            if both is not None:
+                g2, grad_y1 = both
+            else:
+                grad_y1 = difflogic_cuda.backward_x(y1, a2, b2, probs2, grad_y, start2, idx2, ctx.grad_factor2)
+            g1 = difflogic_cuda.backward_logits(x, a1, b1, grad_y1, probs1, ctx.schedule1)
+        if want2 and g2 is None:
+            g2 = difflogic_cuda.backward_logits(y1, a2, b2, grad_y, probs2, ctx.schedule2)
+        return None, None, None, g1, None, None, None, g2, None, None, None, None
+
+
+class FusedLogicLayerPair(torch.nn.Module):
+    """``layer2(layer1(x))`` for a model's first two LogicLayers as one module (see
+    fuse_first_layers).  Registered under the first layer's position with the first layer's
+    ``weights``; the second layer's ``weights`` stay registered at its own position (_LayerDone),
+    so the state_dict keys are those of the unfused model.  Takes the fused path in training mode
+    on float inputs that need no gradient when the second layer is wide enough to be walked along
+    its schedule; everything else runs the two layers one after the other."""
+
+    def __init__(self, layer1: LogicLayer, layer2: LogicLayer):
+        super().__init__()
+        assert isinstance(layer1, LogicLayer) and isinstance(layer2, LogicLayer)
+        assert layer1.out_dim == layer2.in_dim, (layer1.out_dim, layer2.in_dim)
+        self.weights = layer1.weights
+        object.__setattr__(self, "layer1", layer1)
+        object.__setattr__(self, "layer2", layer2)                      # trained / moved through _LayerDone
+
+    def train(self, mode=True):
+        self.layer1.train(mode)
+        return super().train(mode)
+
+    def _apply(self, fn, recurse=True):
+        self.layer1._apply(fn)
+        super()._apply(fn, recurse)
+        self.weights = self.layer1.weights
+        return self
+
+    def forward(self, x):
+        l1, l2 = self.layer1, self.layer2
+        if (isinstance(x, PackBitsTensor) or not self.training or not l2.training or l1.implementation != "cuda"
+                or l2.implementation != "cuda" or not x.is_cuda or x.ndim != 2 or x.requires_grad
+                or x.dtype != l1.weights.dtype or x.dtype != l2.weights.dtype or x.shape[0] == 0
+                or l2._train_schedule() is None):
+            return l2(l1(x))
+        xt = x.transpose(0, 1).contiguous()
+        assert xt.shape[0] == l1.in_dim, (xt.shape, l1.in_dim)
+        return LogicLayerPairFunction.apply(xt, l1.indices[0], l1.indices[1], l1.weights, l1._train_schedule(),
+                                            l2.indices[0], l2.indices[1], l2.weights, l2.given_x_indices_of_y_start,
+                                            l2.given_x_indices_of_y, float(l2.grad_factor),
+                                            l2._train_schedule()).transpose(0, 1)
+
+    def extra_repr(self):
+        return "({}) -> ({})".format(self.layer1.extra_repr(), self.layer2.extra_repr())
+
+
+class _LayerDone(torch.nn.Module):
+    """Stands where the second layer stood after fuse_first_layers: the module before it already
+    evaluated that layer.  Keeps the layer's ``weights`` registered at this position."""
+
+    def __init__(self, layer: LogicLayer):
+        super().__init__()
+        self.weights = layer.weights
+        object.__setattr__(self, "layer", layer)
+
+    def train(self, mode=True):
+        self.layer.train(mode)
+        return super().train(mode)
+
+    def _apply(self, fn, recurse=True):
+        self.layer._apply(fn)
+        super()._apply(fn, recurse)
+        self.weights = self.layer.weights
+        return self
+
+    def forward(self, x):
+        return x
+
+
 class _GroupSumDone(torch.nn.Module):
     """Stands where the GroupSum stood after fuse_group_sum: the module before it already summed."""
 
@@ -332,3 +439,26 @@ def fuse_group_sum(model: torch.nn.Sequential) -> torch.nn.Sequential:
         if isinstance(mods[i], LogicLayer) and isinstance(mods[i + 1], GroupSum) and mods[i].implementation == "cuda":
             mods[i], mods[i + 1] = FusedLogicLayerGroupSum(mods[i], mods[i + 1]), _GroupSumDone()
     return torch.nn.Sequential(*mods)
+
+
+def fuse_first_layers(model: torch.nn.Sequential) -> torch.nn.Sequential:
+    """Returns a ``nn.Sequential`` in which the first two ``LogicLayer`` modules, when they follow
+    each other directly, are replaced by one fused module: in training the first layer's weight
+    gradient is then formed inside the second layer's backward pass, and the gradient between the
+    two layers (``[width, batch]``) is neither written nor read back.  Module positions, parameters
+    and state_dict keys are unchanged; the input model is not modified and shares its parameters
+    with the result."""
+    mods = list(model)
+    first = next((i for i, m in enumerate(mods) if isinstance(m, LogicLayer)), None)
+    if (first is not None and first + 1 < len(mods) and isinstance(mods[first + 1], LogicLayer)
+            and mods[first].implementation == "cuda" and mods[first + 1].implementation == "cuda"):
+        l1, l2 = mods[first], mods[first + 1]
+        mods[first], mods[first + 1] = FusedLogicLayerPair(l1, l2), _LayerDone(l2)
+    return torch.nn.Sequential(*mods)
+
+
+def fuse_for_training(model: torch.nn.Sequential) -> torch.nn.Sequential:
+    """fuse_first_layers and fuse_group_sum together (the last layer is left to fuse_group_sum
+    when a model has only two layers)."""
+    fused = fuse_group_sum(model)
+    return fuse_first_layers(fused)

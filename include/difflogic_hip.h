@@ -147,6 +147,33 @@ int dl_logic_backward_chained(const void *x, const int32_t *verts, const int32_t
 int64_t dl_logic_backward_chained_workspace_bytes(int64_t overflow_rows, int64_t out_dim,
                                                   int64_t batch, int dtype);
 
+/* dl_logic_backward_chained for a layer whose input x is the output of a layer that needs no
+ * grad_x itself (a model's first layer): that lower layer's backward_w (difflogic/difflogic.py:220
+ * of the layer below) is taken in the same pass.  A finished grad_x row IS the grad_y row of neuron
+ * `row` of the lower layer, so its corner sums are formed from the row in registers and the
+ * neuron's two input rows, and grad_x is never written or read back.  No counterpart in the
+ * reference.  Arguments as dl_logic_backward_chained, except:
+ *   fix_rows       DEVICE [n_fix, batch] scratch (NULL if n_fix == 0) in place of grad_x: the rows
+ *                  of the vertices on the fix-up list, the only ones that still pass through memory
+ *   x_lower        [in_dim_lower, batch] input of the lower layer; a_lower, b_lower [in_dim] its wiring
+ *   probs_lower    [in_dim, 16] its gate probabilities: grad_w_lower is then the gradient with respect
+ *                  to its logits (as dl_logic_backward_logits); NULL: with respect to the
+ *                  probabilities (as dl_logic_backward_w)
+ *   grad_w_lower   [in_dim, 16] out.  Same values as the separate calls (grad_x rounded to dtype in
+ *                  between, as when stored).
+ * Applies to rows of at most 4 KB; otherwise DL_ERR_TOO_LARGE and the caller uses the separate
+ * entry points. */
+int dl_logic_backward_chained_lower(const void *x, const int32_t *verts, const int32_t *neuron,
+                                    const uint8_t *flip, const int32_t *dst, int64_t steps,
+                                    const void *w, const void *grad_y, int softmax_backward,
+                                    const int32_t *fix_vertex, const int32_t *fix_start,
+                                    int64_t n_fix, int64_t overflow_rows, void *grad_w,
+                                    void *fix_rows, void *workspace, const void *x_lower,
+                                    const int64_t *a_lower, const int64_t *b_lower,
+                                    const void *probs_lower, void *grad_w_lower, int64_t in_dim,
+                                    int64_t out_dim, int64_t batch, double scale, int dtype,
+                                    void *stream);
+
 /* ---- GroupSum on the feature-major layout (training mode) ------------------------------- */
 
 /* Replaces the float branch of GroupSum.forward (difflogic/difflogic.py:195-196) for the

@@ -216,7 +216,7 @@ def test_full_size_training_step(name, F, width, L, B, tau, connections, grad_fa
         assert _close(u, v, 2 * RTOL), (name, i)
 
 
-@pytest.mark.parametrize("fused", [False, True], ids=["as written", "fuse_group_sum"])
+@pytest.mark.parametrize("fused", [False, True], ids=["as written", "fuse_for_training"])
 def test_c1_training_steps_with_adam(fused):
     """BASELINE config C1 in full on the HIP path: 784 -> 4 x 8000 -> GroupSum(10, tau 10), B = 128,
     'random' wiring, CrossEntropy, three Adam(lr 0.01) steps (experiments/main.py:169,174-181).
@@ -233,8 +233,8 @@ def test_c1_training_steps_with_adam(fused):
     model = torch.nn.Sequential(*mods, dl.GroupSum(k, tau)).train()
     layers = [m for m in model if isinstance(m, dl.LogicLayer)]
     assert all(m._train_schedule() is None for m in layers)
-    if fused:                     # the last layer and GroupSum as one step; same parameters
-        model = dl.fuse_group_sum(model).train()
+    if fused:                     # head and tail fused (the head only where layers walk their schedules); same parameters
+        model = dl.fuse_for_training(model).train()
     g = torch.Generator().manual_seed(1)
     x = (torch.rand(B, F, generator=g) < 0.2).float()
     labels = torch.randint(0, k, (B,), generator=g)
@@ -245,7 +245,7 @@ def test_c1_training_steps_with_adam(fused):
         return net, ws, torch.optim.Adam(ws, lr=0.01), x.to(dtype)
 
     refs = {dt: python_impl(dt) for dt in (torch.float64, torch.float32)}
-    opt = torch.optim.Adam(model.parameters(), lr=0.01)
+    opt = dl.FusedAdam(model.parameters(), lr=0.01) if fused else torch.optim.Adam(model.parameters(), lr=0.01)
     xd, ld = x.cuda(), labels.cuda()
     for step in range(3):
         res = {}

@@ -614,3 +614,152 @@ def test_fuse_group_sum_trains_like_the_unfused_model(widths, batch, conn, grad_
         assert torch.equal(fused(x.cuda()), model(x.cuda()))
         assert torch.equal(fused(dl.PackBitsTensor(x.bool().cuda(), bit_count=64)),
                            model(dl.PackBitsTensor(x.bool().cuda(), bit_count=64)))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16])
+@pytest.mark.parametrize("in0,in_dim,out_dim,batch,kind", [(40, 64, 64, 256, "random"), (100, 300, 300, 512, "random"),
+                                                           (30, 50, 60, 1024, "unique"), (150, 200, 200, 64, "unique"),
+                                                           (20, 30, 47, 260, "any"), (9, 5, 3, 64, "self"),
+                                                           (25, 40, 20, 16, "sparse"), (15, 20, 40, 8, "any"),
+                                                           (784, 1000, 1200, 128, "random")])
+@pytest.mark.parametrize("softmax_lower", [False, True])
+def test_chained_backward_with_the_lower_layers_backward_w(ext, monkeypatch, dtype, in0, in_dim, out_dim, batch, kind,
+                                                           softmax_lower):
+    """dl_logic_backward_chained_lower: grad_w of the layer as the plain one-pass backward gives it,
+    and grad_w of the layer below as backward_w / backward_logits give it on the grad_x rows the
+    plain pass stores (which this one never writes)."""
+    from oracle import connections as oc
+    monkeypatch.setattr(ext, "BACKWARD_CHAIN_MAX_OVERFLOW", 1e9)     # exercise the fix-up rows on any wiring
+    g = torch.Generator().manual_seed(in_dim + batch + in0)
+    torch.manual_seed(in_dim)
+    if kind == "random":
+        a, b = oc.random_connections(in_dim, out_dim)
+    elif kind == "unique":
+        a, b = oc.unique_connections(in_dim, out_dim)
+    elif kind == "self":
+        a, b = torch.tensor([1, 1, 2]), torch.tensor([1, 1, 2])
+    elif kind == "sparse":                                           # half of the inputs feed no neuron
+        a, b = torch.randint(0, in_dim // 2, (out_dim,), generator=g), torch.randint(0, in_dim // 2, (out_dim,),
+                                                                                    generator=g)
+    else:
+        a, b = torch.randint(0, in_dim, (out_dim,), generator=g), torch.randint(0, in_dim, (out_dim,), generator=g)
+    a0 = torch.randint(0, in0, (in_dim,), generator=g).cuda()
+    b0 = torch.randint(0, in0, (in_dim,), generator=g).cuda()
+    x0 = torch.rand(in0, batch, generator=g).to(dtype).cuda()
+    p0 = torch.softmax(torch.randn(in_dim, 16, generator=g), -1).to(dtype).cuda()
+    x = torch.rand(in_dim, batch, generator=g).to(dtype).cuda()
+    w = torch.softmax(torch.randn(out_dim, 16, generator=g), -1).to(dtype).cuda()
+    gy = torch.randn(out_dim, batch, generator=g).to(dtype).cuda()
+    a, b = a.cuda(), b.cuda()
+    sched = ext.schedule_for(a, b, in_dim)
+    scale = 1.5
+    got = ext.backward_chained_lower(x, w, gy, sched, x0, a0, b0, p0 if softmax_lower else None, scale,
+                                     softmax_backward=True)
+    plain = ext.backward_chained(x, w, gy, sched, scale, softmax_backward=True)
+    if batch * x.element_size() % 16 or batch * x.element_size() > 256 * 16:
+        assert got is None                                          # whole 16-byte vectors, rows of at most 4 KB
+        return
+    assert got is not None and plain is not None
+    gw, gw0 = got
+    assert torch.equal(gw, plain[0])
+    want0 = ext.backward_logits(x0, a0, b0, plain[1], p0) if softmax_lower else ext.backward_w(x0, a0, b0, plain[1])
+    # the same terms; the same order of additions too for rows of 33..256 vectors (shorter rows: 8-byte vectors)
+    if dtype != torch.float16 and 32 * 16 < batch * x.element_size():
+        assert torch.equal(gw0, want0)
+    else:
+        rtol = {torch.float16: 4e-3, torch.float32: 1e-5, torch.float64: 1e-12}[dtype]
+        ok, err = close(gw0, want0.double(), rtol)
+        assert ok, err
+    again = ext.backward_chained_lower(x, w, gy, sched, x0, a0, b0, p0 if softmax_lower else None, scale,
+                                       softmax_backward=True)
+    assert torch.equal(again[0], gw) and torch.equal(again[1], gw0)  # deterministic
+
+
+@pytest.mark.parametrize("widths,batch,conn,grad_factor", [([400, 400, 300], 128, "random", 1.0),
+                                                           ([300, 600, 600], 100, "unique", 2.0),
+                                                           ([500, 500, 500, 250], 64, "random", 1.5),
+                                                           ([200, 400], 32, "random", 1.0)])
+def test_fuse_first_layers_trains_like_the_unfused_model(widths, batch, conn, grad_factor, monkeypatch):
+    """fuse_first_layers / fuse_for_training: same positions, parameters and state_dict keys; in
+    training the same scores and gradients as the unfused model and as the CPU python
+    implementation; inputs that want a gradient, eval mode and packed inference take the two
+    original layers."""
+    import difflogic_amd as dl
+    monkeypatch.setattr(dl.LogicLayer, "_CHAIN_MIN_IN_DIM", 0)        # layers this narrow walk their schedules too
+    monkeypatch.setattr(dl.LogicLayer, "_CHAIN_MIN_OUT_DIM", 0)
+    monkeypatch.setattr(dl.difflogic_cuda, "BACKWARD_CHAIN_MAX_OVERFLOW", 1e9)
+    torch.manual_seed(5)
+    F, k, tau = 60, 10, 10.0
+    mods, d = [torch.nn.Flatten()], F
+    for wd in widths:
+        mods.append(dl.LogicLayer(d, wd, grad_factor=grad_factor, connections=conn))
+        d = wd
+    model = torch.nn.Sequential(*mods, dl.GroupSum(k, tau)).train()
+    fused = dl.fuse_for_training(model).train()
+    assert list(fused.state_dict()) == list(model.state_dict()) and len(fused) == len(model)
+    assert isinstance(fused[-2], dl.FusedLogicLayerGroupSum)
+    if len(widths) > 2:
+        assert isinstance(fused[1], dl.FusedLogicLayerPair) and fused[1].weights is model[1].weights
+        assert fused[2].weights is model[2].weights
+    else:
+        assert isinstance(fused[1], dl.LogicLayer)                  # two layers: the second belongs to the tail
+    layers = [m for m in model if isinstance(m, dl.LogicLayer)]
+    x = (torch.rand(batch, F) < 0.3).float()
+    labels = torch.randint(0, k, (batch,))
+
+    def run(net, want_gx=False):
+        net.zero_grad(set_to_none=True)
+        xg = x.cuda()
+        if want_gx:
+            xg.requires_grad_()
+        out = net(xg)
+        torch.nn.functional.cross_entropy(out, labels.cuda()).backward()
+        return out.detach(), [l.weights.grad.clone() for l in layers], xg.grad
+
+    calls = []
+    real = dl.difflogic_cuda.backward_chained_lower
+    monkeypatch.setattr(dl.difflogic_cuda, "backward_chained_lower", lambda *a, **kw: calls.append(1) or real(*a, **kw))
+    out0, gw0, _ = run(model)
+    assert not calls
+    out1, gw1, _ = run(fused)
+    assert len(calls) == (1 if len(widths) > 2 else 0)
+    assert close(out1, out0)[0]
+    for u, v in zip(gw1, gw0):
+        assert close(u, v.double())[0]
+
+    def python_impl(dtype):
+        lg = [l.weights.detach().cpu().to(dtype).requires_grad_() for l in layers]
+        net = fo.PythonNet([(l.indices[0].cpu(), l.indices[1].cpu(), w) for l, w in zip(layers, lg)], k, tau, grad_factor)
+        o = net(x.detach().clone().to(dtype))
+        torch.nn.functional.cross_entropy(o, labels).backward()
+        return o.detach(), [w.grad for w in lg]
+
+    o64, w64 = python_impl(torch.float64)
+    o32, w32 = python_impl(torch.float32)
+    assert close(out1, o64)[0]
+    for got, r64, r32 in zip(gw1, w64, w32):
+        ok, rep = within_budget(got, r64, r32)
+        assert ok, rep
+    out2, gw2, _ = run(fused)
+    assert torch.equal(out1, out2) and all(torch.equal(u, v) for u, v in zip(gw1, gw2))
+
+    # an input that wants its gradient: the two layers run one after the other
+    n = len(calls)
+    _, gw3, gx3 = run(fused, want_gx=True)
+    _, gw4, gx4 = run(model, want_gx=True)
+    assert len(calls) == n and gx3 is not None and close(gx3, gx4.double())[0]
+    for u, v in zip(gw3, gw4):
+        assert close(u, v.double())[0]
+
+    # a frozen first layer: only the second layer's gradient, by the separate kernels
+    model[1].weights.requires_grad_(False)
+    fused.zero_grad(set_to_none=True)
+    torch.nn.functional.cross_entropy(fused(x.cuda()), labels.cuda()).backward()
+    assert model[1].weights.grad is None and close(model[2].weights.grad, gw0[1].double())[0]
+    model[1].weights.requires_grad_(True)
+
+    model.eval(), fused.eval()
+    with torch.no_grad():
+        assert torch.equal(fused(x.cuda()), model(x.cuda()))
+        assert torch.equal(fused(dl.PackBitsTensor(x.bool().cuda(), bit_count=64)),
+                           model(dl.PackBitsTensor(x.bool().cuda(), bit_count=64)))
