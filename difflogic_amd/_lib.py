@@ -36,8 +36,10 @@ SIGNATURES = {
     "dl_backward_schedule_build": [_vp, _vp, _i64, _i64, _vp, _vp, _vp, ctypes.POINTER(_i64)],
     "dl_logic_backward_chained": [_vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _int, _vp, _vp, _i64, _i64, _vp, _vp, _vp,
                                   _i64, _i64, _i64, _dbl, _int, _vp],
+    "dl_logic_forward_chained_lower": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
+                                       _int, _vp],
     "dl_logic_backward_chained_lower": [_vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _int, _vp, _vp, _i64, _i64, _vp, _vp, _vp,
-                                        _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _dbl, _int, _vp],
+                                        _vp, _vp, _vp, _vp, _int, _vp, _i64, _i64, _i64, _dbl, _int, _vp],
     "dl_logic_backward_chained_workspace_bytes": [_i64, _i64, _i64, _int],
     "dl_group_sum_workspace_bytes": [_i64, _i64, _i64, _int],
     "dl_group_sum_forward": [_vp, _vp, _vp, _i64, _i64, _i64, _dbl, _int, _vp],

@@ -482,6 +482,78 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_chain_kernel(const T *__rest
     }
 }
 
+// forward_chain_kernel for a layer whose input is the output of the layer below, with that output
+// recomputed instead of read: input row v = forward of neuron v of the lower layer, from lower input
+// rows low_a[v], low_b[v] of `lx` (a small matrix that stays in the L2 caches) and its gate weights
+// (LOGITS: logits, whose softmax goes to `lprobs`).  Values and rounding are those of forward_kernel
+// on the lower layer, so the result equals running the two layers one after the other bit for bit,
+// but the activation between them is neither written nor read.
+template <typename T, int VEC, int CHUNK, bool LOGITS>
+__global__ __launch_bounds__(DL_BLOCK) void forward_chain_lower_kernel(
+    const T *__restrict__ lx, const int64_t *__restrict__ low_a, const int64_t *__restrict__ low_b,
+    const T *__restrict__ lw, T *__restrict__ lprobs, const int32_t *__restrict__ verts,
+    const int32_t *__restrict__ neuron, const uint8_t *__restrict__ flip, const T *__restrict__ w, T *__restrict__ y,
+    T *__restrict__ probs, int64_t nchunks, int64_t ncols) {
+    typedef typename Acc<T>::type C;
+    typedef Pack<T, VEC> P;
+    const int wave = dl_wave_in_block();
+    const int lane = dl_lane();
+    const int64_t c = (int64_t) blockIdx.x * 4 + wave;
+    if (c >= nchunks) return;
+    static_assert(CHUNK % 4 == 0, "neurons are served four at a time");
+    const int64_t s0 = c * CHUNK;
+    const P *xv = reinterpret_cast<const P *>(lx);
+    P *yv = reinterpret_cast<P *>(y);
+
+    for (int64_t ct = blockIdx.y; ct * DL_WAVE < ncols; ct += gridDim.y) {
+        const int64_t col = ct * DL_WAVE + lane;
+        const bool live = col < ncols;
+        const int64_t cl = live ? col : 0;
+        // the chunk's CHUNK + 1 input rows, four lower neurons at a time
+        P rows[CHUNK + 4];
+#pragma unroll
+        for (int j0 = 0; j0 <= CHUNK; j0 += 4) {
+            int32_t v[4];
+            P va[4], vb[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                v[i] = j0 + i <= CHUNK ? verts[s0 + j0 + i] : -1;
+                const int64_t r = v[i] >= 0 ? v[i] : 0;
+                va[i] = xv[low_a[r] * ncols + cl];
+                vb[i] = xv[low_b[r] * ncols + cl];
+            }
+            C p00[4], p10[4], d0[4], d1[4];
+            corners4<T, LOGITS>(lw, v, lane, ct == 0, lprobs, p00, p10, d0, d1);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e)
+                    rows[j0 + i].v[e] = down<T, C>(mix<C>(up<T>(va[i].v[e]), up<T>(vb[i].v[e]), p00[i], p10[i], d0[i], d1[i]));
+            }
+        }
+#pragma unroll
+        for (int j0 = 0; j0 < CHUNK; j0 += 4) {
+            int32_t n[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) n[i] = neuron[s0 + j0 + i];
+            C p00[4], p10[4], d0[4], d1[4];
+            corners4<T, LOGITS>(w, n, lane, ct == 0, probs, p00, p10, d0, d1);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int j = j0 + i;
+                const bool f = flip[s0 + j] != 0;
+                P r;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const C u0 = up<T>(rows[j].v[e]), u1 = up<T>(rows[j + 1].v[e]);
+                    r.v[e] = down<T, C>(mix<C>(f ? u1 : u0, f ? u0 : u1, p00[i], p10[i], d0[i], d1[i]));
+                }
+                if (live && n[i] >= 0) yv[(int64_t) n[i] * ncols + col] = r;
+            }
+        }
+    }
+}
+
 // Forward along the schedule for long rows: one wave owns `chunk` steps and a segment of
 // CPL * 64 consecutive vectors of the row (blockIdx.y picks the segment; lane l holds its vectors
 // l, l + 64, ...), so every gathered row is one contiguous request of up to 4 KB, and the next
@@ -626,19 +698,23 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_w_chain_kernel(const T *__r
 // owns `chunk` positions [s0, s0 + chunk); it recomputes the last neuron of the chunk before it to get
 // the carry into its first position, so chunks do not exchange partial rows.
 // ------------------------------------------------------------------------------------------
-// LOWER: the layer BELOW this one (whose output x is) needs no grad_x of its own and gets its grad_w
-// here: a vertex's finished grad_x row is the grad_y row of neuron `vertex` of the layer below, so its
-// four corner sums are taken on the spot from the row in registers and the two input rows of that
-// neuron (`low.x`, gathered through `low.a`, `low.b`), and the row is not stored at all.  Only the
+// LOWER >= 1: the layer BELOW this one (whose output x is) needs no grad_x of its own and gets its
+// grad_w here: a vertex's finished grad_x row is the grad_y row of neuron `vertex` of the layer below,
+// so its four corner sums are taken on the spot from the row in registers and the two input rows of
+// that neuron (`low.x`, gathered through `low.a`, `low.b`), and the row is not stored at all.  Only the
 // vertices that finish in backward_fix_kernel still go through memory (backward_w_rows_kernel).
+// LOWER == 2: x itself is not read either: row v of x is recomputed as the lower layer's forward pass
+// computed it (same arithmetic, same rounding) from the two lower input rows that the vertex's
+// backward_w needs anyway, so the activation between the two layers never exists in memory.
 template <typename T> struct LowerLayer {
     const T *x;                 // [in_dim of the layer below, batch]
     const int64_t *a, *b;       // its wiring, [in_dim]
-    const T *probs;             // its gate probabilities [in_dim, 16]: chain the softmax backward; null: plain grad_w
+    const T *w;                 // its gate probabilities [in_dim, 16]
+    const T *probs;             // == w: chain the softmax backward into gw; null: gw is the plain grad_w
     T *gw;                      // [in_dim, 16]
 };
 
-template <typename T, int VEC, int CPL, bool LOWER>
+template <typename T, int VEC, int CPL, int LOWER>
 __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
     const T *__restrict__ x, const int32_t *__restrict__ verts, const int32_t *__restrict__ neuron,
     const uint8_t *__restrict__ flip, const int32_t *__restrict__ dst, const T *__restrict__ w,
@@ -647,6 +723,8 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
     int64_t in_dim, int64_t out_dim, int64_t ncols, typename Acc<T>::type scale, int64_t gdiv, LowerLayer<T> low) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
+    constexpr bool RECOMPUTE = LOWER == 2;
+    constexpr int LCPL = LOWER ? CPL : 1;                       // registers for lower rows only where they are used
     const int wave = dl_wave_in_block();
     const int lane = dl_lane();
     const int64_t s0 = ((int64_t) blockIdx.x * 4 + wave) * chunk;
@@ -654,7 +732,9 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
     const int64_t s1 = s0 + chunk < steps ? s0 + chunk : steps;
     const P *xv = reinterpret_cast<const P *>(x);
     const P *gv = reinterpret_cast<const P *>(gy);
+    const P *lx = reinterpret_cast<const P *>(low.x);
     const int64_t col0 = (int64_t) blockIdx.y * (CPL * DL_WAVE);   // this wave's segment of the rows
+    const int gate = lane & 15;
     P zero;
 #pragma unroll
     for (int e = 0; e < VEC; ++e) zero.v[e] = down<T, C>((C) 0);
@@ -666,10 +746,32 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
             out[q] = (valid && col < ncols) ? base[row * ncols + col] : zero;
         }
     };
-    // la, lb: with LOWER, the two input rows of neuron `row` of the layer below (requested a step ahead)
+    // the two input rows of neuron v of the layer below (v wave-uniform)
+    auto lower_rows = [&](int64_t v, bool valid, P *la, P *lb) {
+        if constexpr (LOWER != 0) {
+            const int64_t r = valid ? v : 0;
+            load_row(lx, low.a[r], valid, la);
+            load_row(lx, low.b[r], valid, lb);
+        }
+    };
+    // row v of x as the lower layer's forward kernel stored it: lane `gate` of every 16-lane row holds the
+    // neuron's probability of that gate; corner sums and their order as corners4()
+    auto lower_forward = [&](const P *la, const P *lb, C lp, P *out) {
+        const C zc = (C) 0;
+        const C q00 = row16_sum((gate & 8) ? lp : zc), q01 = row16_sum((gate & 4) ? lp : zc);
+        const C q10 = row16_sum((gate & 2) ? lp : zc), q11 = row16_sum((gate & 1) ? lp : zc);
+        const C p00 = lane_value(q00, 0), p10 = lane_value(q10, 0);
+        const C d0 = lane_value(q01 - q00, 0), d1 = lane_value(q11 - q10, 0);
+#pragma unroll
+        for (int q = 0; q < CPL; ++q)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+                out[q].v[e] = down<T, C>(mix<C>(up<T>(la[q].v[e]), up<T>(lb[q].v[e]), p00, p10, d0, d1));
+    };
+    // la, lb: with LOWER, the two input rows of neuron `row` of the layer below
     auto store_row = [&](int32_t row, const C (&val)[CPL][VEC], const P *la, const P *lb) {
         if (row < 0) return;
-        if (LOWER && row < in_dim) {
+        if (LOWER != 0 && row < in_dim) {
             // as backward_w_kernel on the row this would have stored: same values, same order of additions
             C s00 = (C) 0, s01 = (C) 0, s10 = (C) 0, s11 = (C) 0;
 #pragma unroll
@@ -701,19 +803,18 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
             if (col < ncols) base[col] = r;
         }
     };
-    auto lower_rows = [&](int32_t row, P *la, P *lb) {           // row: wave-uniform
-        if constexpr (LOWER) {
-            const bool valid = row >= 0 && row < in_dim;
-            const int64_t r = valid ? row : 0;
-            const P *lx = reinterpret_cast<const P *>(low.x);
-            load_row(lx, low.a[r], valid, la);
-            load_row(lx, low.b[r], valid, lb);
-        }
-    };
 
-    P prev[CPL];
+    // prev: row of the vertex at the chunk's first position; pla, plb: (RECOMPUTE) the lower rows it came from,
+    // which also serve that vertex's backward_w at step 0
+    P prev[CPL], pla[LCPL], plb[LCPL];
     C carry[CPL][VEC];
-    load_row(xv, verts[s0], true, prev);
+    if constexpr (RECOMPUTE) {
+        const int64_t v0 = verts[s0];
+        lower_rows(v0, true, pla, plb);
+        lower_forward(pla, plb, up<T>(low.w[v0 * 16 + gate]), prev);
+    } else {
+        load_row(xv, verts[s0], true, prev);
+    }
 #pragma unroll
     for (int q = 0; q < CPL; ++q)
 #pragma unroll
@@ -722,7 +823,14 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
         const int32_t n = neuron[s0 - 1];
         const bool f = flip[s0 - 1] != 0;
         P before[CPL], g[CPL];
-        load_row(xv, verts[s0 - 1], true, before);
+        if constexpr (RECOMPUTE) {
+            const int64_t vb = verts[s0 - 1];
+            P ba[LCPL], bb[LCPL];
+            lower_rows(vb, true, ba, bb);
+            lower_forward(ba, bb, up<T>(low.w[vb * 16 + gate]), before);
+        } else {
+            load_row(xv, verts[s0 - 1], true, before);
+        }
         load_row(gv, grad_row(n, gdiv), true, g);
         const Corners<C> k = corners<T>(w, n);
         const C d0 = k.p01 - k.p00, dd = (k.p11 - k.p10) - d0, da = k.p10 - k.p00;
@@ -741,27 +849,37 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
     const int32_t sch_v = has ? verts[s0 + 1 + lane] : 0;
     const int32_t sch_d = has ? dst[s0 + lane] : -1;
     const int32_t sch_f = has ? (int32_t) flip[s0 + lane] : 0;
-    const int gate = lane & 15;
-    // rows of step i: the new input row, the neuron's grad_y row (zero for a step without a neuron)
-    // and, in every 16-lane row, the neuron's 16 gate probabilities
-    constexpr int LCPL = LOWER ? CPL : 1;
-    auto fetch = [&](int i, P *row, P *grad, C &prob, P *la, P *lb) {
+    // Rows of step i: the new input row (RECOMPUTE: the two lower rows and the lower probabilities it is
+    // recomputed from), the neuron's grad_y row (zero for a step without a neuron) and, in every 16-lane
+    // row, the neuron's 16 gate probabilities.  LOWER == 1: la, lb are the lower rows of the vertex that
+    // step i finishes (dst[i]); RECOMPUTE: of the vertex that step i brings in.
+    auto fetch = [&](int i, P *row, P *grad, C &prob, P *la, P *lb, C &lprob) {
         const int32_t n = __builtin_amdgcn_readlane(sch_n, i);
         const bool valid = n >= 0;
         const int64_t nn = valid ? n : 0;
-        load_row(xv, __builtin_amdgcn_readlane(sch_v, i), true, row);
+        const int32_t v = __builtin_amdgcn_readlane(sch_v, i);
+        if constexpr (RECOMPUTE) {
+            lower_rows(v, true, la, lb);
+            lprob = up<T>(low.w[(int64_t) v * 16 + gate]);
+        } else {
+            load_row(xv, v, true, row);
+            if constexpr (LOWER == 1) {
+                const int32_t d = __builtin_amdgcn_readlane(sch_d, i);
+                lower_rows(d, d >= 0 && d < in_dim, la, lb);
+            }
+        }
         load_row(gv, grad_row(nn, gdiv), valid, grad);
         prob = up<T>(w[nn * 16 + gate]);
-        lower_rows(__builtin_amdgcn_readlane(sch_d, i), la, lb);
     };
     P cur[CPL], g[CPL], la[LCPL], lb[LCPL];
-    C pw;
-    fetch(0, cur, g, pw, la, lb);
+    C pw, lpw = (C) 0;
+    fetch(0, cur, g, pw, la, lb, lpw);
 #pragma unroll 1
     for (int i = 0; i < cnt; ++i) {
         P ncur[CPL], ng[CPL], nla[LCPL], nlb[LCPL];
-        C npw = (C) 0;
-        if (i + 1 < cnt) fetch(i + 1, ncur, ng, npw, nla, nlb);
+        C npw = (C) 0, nlpw = (C) 0;
+        if (i + 1 < cnt) fetch(i + 1, ncur, ng, npw, nla, nlb, nlpw);
+        if constexpr (RECOMPUTE) lower_forward(la, lb, lpw, cur);
         const int32_t n = __builtin_amdgcn_readlane(sch_n, i);
         const bool valid = n >= 0;
         const int64_t nn = valid ? n : 0;
@@ -808,23 +926,28 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
             const C mine = lane == 0 ? s00 : lane == 1 ? s01 : lane == 2 ? s10 : s11;
             partial[((int64_t) blockIdx.y * out_dim + nn) * 4 + lane] = mine;
         }
-        store_row(__builtin_amdgcn_readlane(sch_d, i), out, la, lb);
+        // the vertex at position s0 + i is finished: RECOMPUTE keeps its lower rows from the step that brought it in
+        store_row(__builtin_amdgcn_readlane(sch_d, i), out, RECOMPUTE ? pla : la, RECOMPUTE ? plb : lb);
 #pragma unroll
         for (int q = 0; q < CPL; ++q) {
             prev[q] = cur[q];
             cur[q] = ncur[q];
             g[q] = ng[q];
         }
-        if (LOWER) {
+        if constexpr (LOWER != 0) {
 #pragma unroll
-            for (int q = 0; q < LCPL; ++q) la[q] = nla[q], lb[q] = nlb[q];
+            for (int q = 0; q < LCPL; ++q) {
+                if constexpr (RECOMPUTE) pla[q] = la[q], plb[q] = lb[q];
+                la[q] = nla[q], lb[q] = nlb[q];
+            }
         }
         pw = npw;
+        lpw = nlpw;
     }
     if (s1 == steps) {                                // the schedule's last position
         const int32_t last = dst[steps];
-        lower_rows(last, la, lb);
-        store_row(last, carry, la, lb);
+        if constexpr (LOWER == 1) lower_rows(last, last >= 0 && last < in_dim, la, lb);
+        store_row(last, carry, RECOMPUTE ? pla : la, RECOMPUTE ? plb : lb);
     }
 }
 
@@ -1310,6 +1433,22 @@ int forward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, 
     return dl_launch_status();
 }
 
+template <typename T, bool LOGITS>
+int forward_chain_lower_t(const void *lx, const int64_t *la, const int64_t *lb, const void *lw, void *lprobs,
+                          const int32_t *verts, const int32_t *neuron, const uint8_t *flip, int64_t steps, const void *w,
+                          void *y, void *probs, int64_t batch, hipStream_t s) {
+    constexpr int V = Vec16<T>::n;
+    if (batch % V != 0 || !dl_aligned(lx, 16) || !dl_aligned(y, 16)) return DL_ERR_TOO_LARGE;
+    const int64_t nchunks = steps / DL_TRAIN_CHUNK, ncols = batch / V;
+    if (ncols > DL_FWD_ROWS_MIN) return DL_ERR_TOO_LARGE;        // rows of at most 2 KB
+    const int64_t blocks = dl_ceil_div(nchunks, 4);
+    if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    DL_LAUNCH((forward_chain_lower_kernel<T, V, DL_TRAIN_CHUNK, LOGITS>), dim3((unsigned) blocks, col_tiles(ncols)),
+              dim3(DL_BLOCK), 0, s, (const T *) lx, la, lb, (const T *) lw, (T *) lprobs, verts, neuron, flip, (const T *) w,
+              (T *) y, (T *) probs, nchunks, ncols);
+    return dl_launch_status();
+}
+
 template <typename T>
 int backward_w_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, const uint8_t *flip, int64_t steps,
                        const void *gy, const void *probs, void *gw, int64_t batch, hipStream_t s, int64_t gdiv = 0) {
@@ -1348,12 +1487,13 @@ int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron,
     constexpr int V = Vec16<T>::n;
     if (batch % V != 0 || !dl_aligned(x, 16) || !dl_aligned(gy, 16) || !dl_aligned(gx, 16) || !dl_aligned(workspace, 16))
         return DL_ERR_TOO_LARGE;
+    if (!x && (!lower || !lower->w)) return DL_ERR_INVALID_ARGUMENT;     // x may only be left out for recomputation
     const int64_t ncols = batch / V;
     if (ncols > DL_ROWS_MAX_VECTORS) return DL_ERR_TOO_LARGE;
     const int segments = row_segments(ncols);
     // with `lower`: whole rows per wave only, and gx holds the n_fix rows that finish after the pass
     if (lower && (segments > 1 || !dl_aligned(lower->x, 16))) return DL_ERR_TOO_LARGE;
-    const LowerLayer<T> none = {nullptr, nullptr, nullptr, nullptr, nullptr};
+    const LowerLayer<T> none = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
     // workspace: [segments x out x 4 corner sums (only with several segments)] [overflow rows]
     const int64_t partial_bytes = backward_partial_bytes<T>(out_dim, batch);
     if ((partial_bytes > 0 || overflow_rows > 0) && workspace == nullptr) return DL_ERR_INVALID_ARGUMENT;
@@ -1367,11 +1507,14 @@ int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron,
     constexpr int H = V >= 2 ? V / 2 : 1;
 #define DL_LAUNCH_BACKWARD_CHAIN(VV, CPL, NC)                                                                               \
     do {                                                                                                                    \
-        if (lower)                                                                                                          \
-            DL_LAUNCH((backward_chain_kernel<T, VV, CPL, true>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp,  \
+        if (lower && !x)                                                                                                    \
+            DL_LAUNCH((backward_chain_kernel<T, VV, CPL, 2>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp,     \
+                      pp, (T *) gw, partial, (T *) gx, overflow, steps, chunk, in_dim, out_dim, NC, (C) scale, gdiv, *lower); \
+        else if (lower)                                                                                                     \
+            DL_LAUNCH((backward_chain_kernel<T, VV, CPL, 1>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp,     \
                       pp, (T *) gw, partial, (T *) gx, overflow, steps, chunk, in_dim, out_dim, NC, (C) scale, gdiv, *lower); \
         else                                                                                                                \
-            DL_LAUNCH((backward_chain_kernel<T, VV, CPL, false>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp, \
+            DL_LAUNCH((backward_chain_kernel<T, VV, CPL, 0>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp,     \
                       pp, (T *) gw, partial, (T *) gx, overflow, steps, chunk, in_dim, out_dim, NC, (C) scale, gdiv, none);  \
     } while (0)
     if (V >= 2 && ncols <= DL_WAVE / 2)
@@ -1447,34 +1590,37 @@ extern "C" int dl_logic_backward_chained_lower(const void *x, const int32_t *ver
                                                const void *grad_y, int softmax_backward, const int32_t *fix_vertex,
                                                const int32_t *fix_start, int64_t n_fix, int64_t overflow_rows,
                                                void *grad_w, void *fix_rows, void *workspace, const void *x_lower,
-                                               const int64_t *a_lower, const int64_t *b_lower, const void *probs_lower,
-                                               void *grad_w_lower, int64_t in_dim, int64_t out_dim, int64_t batch,
-                                               double scale, int dtype, void *stream) {
+                                               const int64_t *a_lower, const int64_t *b_lower, const void *w_lower,
+                                               int softmax_backward_lower, void *grad_w_lower, int64_t in_dim,
+                                               int64_t out_dim, int64_t batch, double scale, int dtype, void *stream) {
     if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
     if (in_dim <= 0 || out_dim <= 0 || batch <= 0 || steps < out_dim || n_fix < 0 || n_fix > in_dim || overflow_rows < 0)
         return DL_ERR_INVALID_ARGUMENT;
-    if (!x || !verts || !neuron || !flip || !dst || !w || !grad_y || !grad_w || !x_lower || !a_lower || !b_lower ||
-        !grad_w_lower)
+    if (!verts || !neuron || !flip || !dst || !w || !grad_y || !grad_w || !x_lower || !a_lower || !b_lower || !grad_w_lower)
         return DL_ERR_INVALID_ARGUMENT;
+    if ((softmax_backward_lower || !x) && !w_lower) return DL_ERR_INVALID_ARGUMENT;
     if (n_fix > 0 && (!fix_vertex || !fix_start || !fix_rows)) return DL_ERR_INVALID_ARGUMENT;
+    // recomputing x needs the lower layer's probabilities exactly as its forward pass used them; the fp16 kernels
+    // form them in fp32 and round only what they store
+    if (!x && dtype == DL_F16) return DL_ERR_TOO_LARGE;
     hipStream_t s = (hipStream_t) stream;
     const bool sb = softmax_backward != 0;
     switch (dtype) {
     case DL_F16: {
-        const LowerLayer<__half> low = {(const __half *) x_lower, a_lower, b_lower, (const __half *) probs_lower,
-                                        (__half *) grad_w_lower};
+        const LowerLayer<__half> low = {(const __half *) x_lower, a_lower, b_lower, (const __half *) w_lower,
+                                        softmax_backward_lower ? (const __half *) w_lower : nullptr, (__half *) grad_w_lower};
         return backward_chain_t<__half>(x, verts, neuron, flip, dst, steps, w, grad_y, sb, fix_vertex, fix_start, n_fix,
                                         overflow_rows, grad_w, fix_rows, workspace, in_dim, out_dim, batch, scale, s, 0, &low);
     }
     case DL_F32: {
-        const LowerLayer<float> low = {(const float *) x_lower, a_lower, b_lower, (const float *) probs_lower,
-                                       (float *) grad_w_lower};
+        const LowerLayer<float> low = {(const float *) x_lower, a_lower, b_lower, (const float *) w_lower,
+                                       softmax_backward_lower ? (const float *) w_lower : nullptr, (float *) grad_w_lower};
         return backward_chain_t<float>(x, verts, neuron, flip, dst, steps, w, grad_y, sb, fix_vertex, fix_start, n_fix,
                                        overflow_rows, grad_w, fix_rows, workspace, in_dim, out_dim, batch, scale, s, 0, &low);
     }
     default: {
-        const LowerLayer<double> low = {(const double *) x_lower, a_lower, b_lower, (const double *) probs_lower,
-                                        (double *) grad_w_lower};
+        const LowerLayer<double> low = {(const double *) x_lower, a_lower, b_lower, (const double *) w_lower,
+                                        softmax_backward_lower ? (const double *) w_lower : nullptr, (double *) grad_w_lower};
         return backward_chain_t<double>(x, verts, neuron, flip, dst, steps, w, grad_y, sb, fix_vertex, fix_start, n_fix,
                                         overflow_rows, grad_w, fix_rows, workspace, in_dim, out_dim, batch, scale, s, 0, &low);
     }
@@ -1502,6 +1648,36 @@ extern "C" int dl_logic_forward_chained(const void *x, const int32_t *verts, con
     case DL_F32: return forward_chain_t<float, false>(x, verts, neuron, flip, steps, w, y, nullptr, batch, s);
     default: return forward_chain_t<double, false>(x, verts, neuron, flip, steps, w, y, nullptr, batch, s);
     }
+}
+
+extern "C" int dl_logic_forward_chained_lower(const void *x_lower, const int64_t *a_lower, const int64_t *b_lower,
+                                              const void *w_lower, void *probs_lower, const int32_t *verts,
+                                              const int32_t *neuron, const uint8_t *flip, int64_t steps, const void *w,
+                                              void *y, void *probs, int64_t in_dim_lower, int64_t in_dim, int64_t out_dim,
+                                              int64_t batch, int dtype, void *stream) {
+    if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
+    if (in_dim_lower <= 0 || in_dim <= 0 || out_dim < 0 || batch <= 0 || steps < out_dim || steps % DL_TRAIN_CHUNK != 0)
+        return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim == 0) return DL_OK;
+    if (!x_lower || !a_lower || !b_lower || !w_lower || !verts || !neuron || !flip || !w || !y) return DL_ERR_INVALID_ARGUMENT;
+    if ((probs == nullptr) != (probs_lower == nullptr)) return DL_ERR_INVALID_ARGUMENT;    // both layers on logits, or neither
+    hipStream_t s = (hipStream_t) stream;
+#define DL_FCL(TT, LG)                                                                                                  \
+    forward_chain_lower_t<TT, LG>(x_lower, a_lower, b_lower, w_lower, probs_lower, verts, neuron, flip, steps, w, y, probs, \
+                                  batch, s)
+    if (probs) {
+        switch (dtype) {
+        case DL_F16: return DL_FCL(__half, true);
+        case DL_F32: return DL_FCL(float, true);
+        default: return DL_FCL(double, true);
+        }
+    }
+    switch (dtype) {
+    case DL_F16: return DL_FCL(__half, false);
+    case DL_F32: return DL_FCL(float, false);
+    default: return DL_FCL(double, false);
+    }
+#undef DL_FCL
 }
 
 extern "C" int dl_logic_backward_w_chained(const void *x, const int32_t *verts, const int32_t *neuron,

@@ -318,19 +318,38 @@ class LogicLayerPairFunction(torch.autograd.Function):
     """A model's first two LogicLayers as one autograd node: feature-major input [in, B] that
     needs no gradient and both layers' gate logits -> the second layer's output [out2, B].  In the
     backward pass the first layer's grad_y (= the second layer's grad_x) is consumed row by row
-    where the second layer's one-pass backward finishes it and never touches memory."""
+    where the second layer's one-pass backward finishes it and never touches memory.  When the
+    input is small enough to stay in the L2 caches (and the dtype is fp32 / fp64) the first layer's
+    output does not exist in memory either: forward and backward recompute its rows from the
+    input."""
+
+    # the input [in, B] stays cache-resident below this size: recomputing a row of the first layer's
+    # output (two gathered input rows) is then cheaper than storing and re-reading it
+    RECOMPUTE_MAX_INPUT_BYTES = 4 << 20
 
     @staticmethod
     def forward(ctx, x, a1, b1, logits1, schedule1, a2, b2, logits2, start2, idx2, grad_factor2, schedule2):
-        y1, probs1 = difflogic_cuda.forward_logits(x, a1, b1, logits1.detach().contiguous(), schedule1)
-        y2, probs2 = difflogic_cuda.forward_logits(y1, a2, b2, logits2.detach().contiguous(), schedule2)
-        ctx.save_for_backward(x, a1, b1, probs1, y1, a2, b2, probs2, start2, idx2)
+        l1, l2 = logits1.detach().contiguous(), logits2.detach().contiguous()
+        fused = None
+        if (x.dtype in (torch.float32, torch.float64)
+                and x.numel() * x.element_size() <= LogicLayerPairFunction.RECOMPUTE_MAX_INPUT_BYTES):
+            fused = difflogic_cuda.forward_logits_lower(x, a1, b1, l1, l2, schedule2)
+        if fused is not None:
+            y2, probs1, probs2 = fused
+            y1 = None
+            ctx.save_for_backward(x, a1, b1, probs1, a2, b2, probs2, start2, idx2)
+        else:
+            y1, probs1 = difflogic_cuda.forward_logits(x, a1, b1, l1, schedule1)
+            y2, probs2 = difflogic_cuda.forward_logits(y1, a2, b2, l2, schedule2)
+            ctx.save_for_backward(x, a1, b1, probs1, a2, b2, probs2, start2, idx2, y1)
+        ctx.recompute = y1 is None
         ctx.grad_factor2, ctx.schedule1, ctx.schedule2 = grad_factor2, schedule1, schedule2
         return y2
 
     @staticmethod
     def backward(ctx, grad_y):
-        x, a1, b1, probs1, y1, a2, b2, probs2, start2, idx2 = ctx.saved_tensors
+        x, a1, b1, probs1, a2, b2, probs2, start2, idx2 = ctx.saved_tensors[:9]
+        y1 = None if ctx.recompute else ctx.saved_tensors[9]
         grad_y = grad_y.contiguous()
         want1, want2 = ctx.needs_input_grad[3], ctx.needs_input_grad[7]
         g1 = g2 = None
@@ -341,6 +360,8 @@ class LogicLayerPairFunction(torch.autograd.Function):
                 g2, g1 = both
                 return None, None, None, g1, None, None, None, g2, None, None, None, None
         # the separate kernels, as two LogicLayers in a row would run them
+        if y1 is None:
+            y1 = difflogic_cuda.forward(x, a1, b1, probs1, ctx.schedule1)
         if want1:
             both = difflogic_cuda.backward_chained(y1, probs2, grad_y, ctx.schedule2, ctx.grad_factor2,
                                                    softmax_backward=True) if want2 else None

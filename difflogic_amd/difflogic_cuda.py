@@ -289,42 +289,87 @@ def backward_chained(x, w, grad_y, schedule, scale=1.0, softmax_backward=False):
     return grad_w, grad_x
 
 
-def backward_chained_lower(x, w, grad_y, schedule, x_lower, a_lower, b_lower, probs_lower, scale=1.0,
-                           softmax_backward=False):
+def forward_logits_lower(x_lower, a_lower, b_lower, logits_lower, logits, schedule):
+    """``forward_logits(forward_logits(x_lower, ...)[0], a, b, logits, schedule)`` in one kernel that
+    recomputes the rows of the intermediate activation instead of writing and reading them
+    (``schedule``: the EvalSchedule of the upper layer's (a, b)).  Returns (y [out,B],
+    probs_lower [in,16], probs [out,16]) with the values the two calls give, or None where the
+    kernel does not apply (rows longer than 2 KB or not whole 16-byte vectors).  Not part of the
+    reference's extension."""
+    for t, n in ((x_lower, "x_lower"), (a_lower, "a_lower"), (b_lower, "b_lower"), (logits_lower, "logits_lower"),
+                 (logits, "logits")):
+        _check_input(t, n)
+    code = _float_code(x_lower, "logic_layer_cuda_forward")
+    if (x_lower.dim() != 2 or logits_lower.dim() != 2 or logits_lower.shape[1] != 16 or logits.dim() != 2
+            or logits.shape[1] != 16 or logits_lower.dtype != x_lower.dtype or logits.dtype != x_lower.dtype
+            or x_lower.shape[1] == 0):
+        raise RuntimeError(f"expected x_lower [in0,B>0] and logits [*,16] of one dtype, got {tuple(x_lower.shape)} "
+                           f"{x_lower.dtype}, {tuple(logits_lower.shape)}, {tuple(logits.shape)}")
+    in_dim, out_dim = logits_lower.shape[0], logits.shape[0]
+    _check_index(a_lower, "a_lower", in_dim)
+    _check_index(b_lower, "b_lower", in_dim)
+    dev = _same_device(x_lower, a_lower, b_lower, logits_lower, logits)
+    in0, batch = x_lower.shape
+    if in0 == 0 or in_dim == 0 or out_dim == 0:
+        return None
+    _check_schedule(schedule, in_dim, out_dim, dev)
+    y = torch.empty((out_dim, batch), dtype=x_lower.dtype, device=dev)
+    probs = torch.empty((out_dim, 16), dtype=x_lower.dtype, device=dev)
+    # rows of lower neurons that feed nothing are never visited: zero probabilities give them a zero gradient
+    probs_lower = torch.zeros((in_dim, 16), dtype=x_lower.dtype, device=dev)
+    with _on(dev):
+        st = _lib.load().dl_logic_forward_chained_lower(
+            _p(x_lower), _p(a_lower), _p(b_lower), _p(logits_lower), _p(probs_lower), _p(schedule.verts),
+            _p(schedule.neuron), _p(schedule.flip), schedule.steps, _p(logits), _p(y), _p(probs), in0, in_dim, out_dim,
+            batch, code, _stream(dev))
+    if st == _lib.DL_ERR_TOO_LARGE:
+        return None
+    if st:
+        _raise(st, "logic_layer_cuda_forward_chained_lower")
+    return y, probs_lower, probs
+
+
+def backward_chained_lower(x, w, grad_y, schedule, x_lower, a_lower, b_lower, w_lower, scale=1.0,
+                           softmax_backward=False, softmax_backward_lower=True):
     """backward_chained for a layer whose input ``x`` is the output of a layer that needs no
     input gradient (a model's first layer), with that lower layer's backward_w in the same pass:
     the grad_x rows are consumed where they are finished instead of being written and read
-    back.  ``probs_lower`` [in,16]: the lower layer's probabilities from forward_logits (the
-    result is then the gradient of its logits), or None (gradient of its probabilities).
-    Returns (grad_w [out,16], grad_w_lower [in,16]), or None where the fused pass does not
-    apply.  Not part of the reference's extension."""
-    for t, n in ((x, "x"), (w, "w"), (grad_y, "grad_y"), (x_lower, "x_lower"), (a_lower, "a_lower"), (b_lower, "b_lower")):
+    back.  ``w_lower`` [in,16]: the lower layer's probabilities; with ``softmax_backward_lower``
+    the second result is the gradient of its logits, else of its probabilities.  ``x`` may be
+    None (fp32 / fp64): its rows are then recomputed from the lower layer (forward_logits_lower
+    never stored them).  Returns (grad_w [out,16], grad_w_lower [in,16]), or None where the fused
+    pass does not apply.  Not part of the reference's extension."""
+    for t, n in ((w, "w"), (grad_y, "grad_y"), (x_lower, "x_lower"), (a_lower, "a_lower"), (b_lower, "b_lower"),
+                 (w_lower, "w_lower")):
         _check_input(t, n)
-    code = _float_code(x, "logic_layer_cuda_backward")
-    if (x.dim() != 2 or grad_y.dim() != 2 or grad_y.shape[1] != x.shape[1] or grad_y.dtype != x.dtype
-            or w.shape != (grad_y.shape[0], 16) or w.dtype != x.dtype):
-        raise RuntimeError(f"expected x [in,B], w [out,16], grad_y [out,B] of one dtype, got {tuple(x.shape)}, "
-                           f"{tuple(w.shape)}, {tuple(grad_y.shape)}")
-    in_dim, batch = x.shape
-    out_dim = grad_y.shape[0]
-    if x_lower.dim() != 2 or x_lower.shape[1] != batch or x_lower.dtype != x.dtype:
-        raise RuntimeError(f"expected x_lower [in_lower,{batch}] {x.dtype}, got {tuple(x_lower.shape)} {x_lower.dtype}")
+    code = _float_code(grad_y, "logic_layer_cuda_backward")
+    dtype = grad_y.dtype
+    out_dim, batch = grad_y.shape if grad_y.dim() == 2 else (0, 0)
+    in_dim = w_lower.shape[0]
+    if x is not None:
+        _check_input(x, "x")
+        if x.dim() != 2 or tuple(x.shape) != (in_dim, batch) or x.dtype != dtype:
+            raise RuntimeError(f"expected x [{in_dim},{batch}] {dtype}, got {tuple(x.shape)} {x.dtype}")
+    if grad_y.dim() != 2 or w.shape != (out_dim, 16) or w.dtype != dtype:
+        raise RuntimeError(f"expected w [out,16], grad_y [out,B] of one dtype, got {tuple(w.shape)}, {tuple(grad_y.shape)}")
+    if x_lower.dim() != 2 or x_lower.shape[1] != batch or x_lower.dtype != dtype:
+        raise RuntimeError(f"expected x_lower [in_lower,{batch}] {dtype}, got {tuple(x_lower.shape)} {x_lower.dtype}")
+    if w_lower.shape != (in_dim, 16) or w_lower.dtype != dtype:
+        raise RuntimeError(f"expected w_lower [{in_dim},16] {dtype}, got {tuple(w_lower.shape)} {w_lower.dtype}")
     _check_index(a_lower, "a_lower", in_dim)
     _check_index(b_lower, "b_lower", in_dim)
-    if probs_lower is not None:
-        _check_input(probs_lower, "probs_lower")
-        if probs_lower.shape != (in_dim, 16) or probs_lower.dtype != x.dtype:
-            raise RuntimeError(f"expected probs_lower [{in_dim},16] {x.dtype}, got {tuple(probs_lower.shape)}")
-    dev = _same_device(x, w, grad_y, x_lower, a_lower, b_lower)
+    dev = _same_device(w, grad_y, x_lower, a_lower, b_lower, w_lower)
     if in_dim == 0 or out_dim == 0 or batch == 0 or x_lower.shape[0] == 0:
+        return None
+    if x is None and dtype == torch.float16:
         return None
     _check_schedule(schedule, in_dim, out_dim, dev)
     dst, fix_vertex, fix_start, n_fix, rows = schedule.backward_plan()
     if rows > in_dim * BACKWARD_CHAIN_MAX_OVERFLOW:
         return None
-    grad_w = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
-    grad_w_lower = torch.empty((in_dim, 16), dtype=x.dtype, device=dev)
-    fix_rows = torch.empty((n_fix, batch), dtype=x.dtype, device=dev) if n_fix else None
+    grad_w = torch.empty((out_dim, 16), dtype=dtype, device=dev)
+    grad_w_lower = torch.empty((in_dim, 16), dtype=dtype, device=dev)
+    fix_rows = torch.empty((n_fix, batch), dtype=dtype, device=dev) if n_fix else None
     lib = _lib.load()
     ws_bytes = lib.dl_logic_backward_chained_workspace_bytes(rows, out_dim, batch, code)
     if ws_bytes < 0:
@@ -332,12 +377,11 @@ def backward_chained_lower(x, w, grad_y, schedule, x_lower, a_lower, b_lower, pr
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
     with _on(dev):
         st = lib.dl_logic_backward_chained_lower(
-            _p(x), _p(schedule.verts), _p(schedule.neuron), _p(schedule.flip), _p(dst), schedule.steps, _p(w),
-            _p(grad_y), 1 if softmax_backward else 0, _p(fix_vertex) if n_fix else None,
+            _p(x) if x is not None else None, _p(schedule.verts), _p(schedule.neuron), _p(schedule.flip), _p(dst),
+            schedule.steps, _p(w), _p(grad_y), 1 if softmax_backward else 0, _p(fix_vertex) if n_fix else None,
             _p(fix_start) if n_fix else None, n_fix, rows, _p(grad_w), _p(fix_rows) if n_fix else None,
-            _p(workspace) if ws_bytes else None, _p(x_lower), _p(a_lower), _p(b_lower),
-            _p(probs_lower) if probs_lower is not None else None, _p(grad_w_lower), in_dim, out_dim, batch,
-            float(scale), code, _stream(dev))
+            _p(workspace) if ws_bytes else None, _p(x_lower), _p(a_lower), _p(b_lower), _p(w_lower),
+            1 if softmax_backward_lower else 0, _p(grad_w_lower), in_dim, out_dim, batch, float(scale), code, _stream(dev))
     if st == _lib.DL_ERR_TOO_LARGE:
         return None
     if st:

@@ -153,12 +153,17 @@ int64_t dl_logic_backward_chained_workspace_bytes(int64_t overflow_rows, int64_t
  * `row` of the lower layer, so its corner sums are formed from the row in registers and the
  * neuron's two input rows, and grad_x is never written or read back.  No counterpart in the
  * reference.  Arguments as dl_logic_backward_chained, except:
+ *   x              may be NULL (fp32 / fp64): row v of x is then recomputed as
+ *                  dl_logic_forward(x_lower, a_lower, b_lower, w_lower) produced it (bit for bit),
+ *                  from the two lower rows that vertex v's backward_w reads anyway, so the activation
+ *                  between the two layers need not exist in memory (see dl_logic_forward_chained_lower)
  *   fix_rows       DEVICE [n_fix, batch] scratch (NULL if n_fix == 0) in place of grad_x: the rows
  *                  of the vertices on the fix-up list, the only ones that still pass through memory
  *   x_lower        [in_dim_lower, batch] input of the lower layer; a_lower, b_lower [in_dim] its wiring
- *   probs_lower    [in_dim, 16] its gate probabilities: grad_w_lower is then the gradient with respect
- *                  to its logits (as dl_logic_backward_logits); NULL: with respect to the
- *                  probabilities (as dl_logic_backward_w)
+ *   w_lower        [in_dim, 16] the lower layer's gate probabilities (needed when x is NULL or
+ *                  softmax_backward_lower is set; else may be NULL)
+ *   softmax_backward_lower  0: grad_w_lower as dl_logic_backward_w; else with respect to the lower
+ *                  layer's logits, as dl_logic_backward_logits
  *   grad_w_lower   [in_dim, 16] out.  Same values as the separate calls (grad_x rounded to dtype in
  *                  between, as when stored).
  * Applies to rows of at most 4 KB; otherwise DL_ERR_TOO_LARGE and the caller uses the separate
@@ -170,9 +175,9 @@ int dl_logic_backward_chained_lower(const void *x, const int32_t *verts, const i
                                     int64_t n_fix, int64_t overflow_rows, void *grad_w,
                                     void *fix_rows, void *workspace, const void *x_lower,
                                     const int64_t *a_lower, const int64_t *b_lower,
-                                    const void *probs_lower, void *grad_w_lower, int64_t in_dim,
-                                    int64_t out_dim, int64_t batch, double scale, int dtype,
-                                    void *stream);
+                                    const void *w_lower, int softmax_backward_lower,
+                                    void *grad_w_lower, int64_t in_dim, int64_t out_dim,
+                                    int64_t batch, double scale, int dtype, void *stream);
 
 /* ---- GroupSum on the feature-major layout (training mode) ------------------------------- */
 
@@ -218,6 +223,23 @@ int dl_logic_backward_chained_grouped(const void *x, const int32_t *verts, const
                                       int64_t n_fix, int64_t overflow_rows, void *grad_w,
                                       void *grad_x, void *workspace, int64_t in_dim, int64_t out_dim,
                                       int64_t batch, int64_t k, double scale, int dtype, void *stream);
+
+/* dl_logic_forward_chained for a layer whose input is the output of the layer below, with that
+ * output recomputed row by row instead of read: y = forward(forward(x_lower, a_lower, b_lower,
+ * w_lower), a, b, w) bit for bit, but the activation between the two layers is neither written nor
+ * read (two calls of difflogic/difflogic.py:123-126 / :209).  Pays when x_lower is small enough to
+ * stay in the L2 caches (a model's 784-row input).  No counterpart in the reference.
+ *   probs != NULL (then probs_lower != NULL too): w and w_lower hold logits and the two receive
+ *   their softmax, as dl_logic_forward_logits; NULL (both): they hold probabilities.
+ *   verts, neuron, flip, steps: the evaluation schedule of (a, b) (dl_eval_schedule_build).
+ * Applies to rows of at most 2 KB; otherwise DL_ERR_TOO_LARGE.  Only the vertices the schedule
+ * visits get their probs_lower row: clear it first if the other rows are read later. */
+int dl_logic_forward_chained_lower(const void *x_lower, const int64_t *a_lower, const int64_t *b_lower,
+                                   const void *w_lower, void *probs_lower, const int32_t *verts,
+                                   const int32_t *neuron, const uint8_t *flip, int64_t steps,
+                                   const void *w, void *y, void *probs, int64_t in_dim_lower,
+                                   int64_t in_dim, int64_t out_dim, int64_t batch, int dtype,
+                                   void *stream);
 
 /* The optimizer step of the reference's training loop (torch.optim.Adam(lr=...).step(),
  * experiments/main.py:169,179) for all of a model's fp32 weight tensors in one launch.  No counterpart

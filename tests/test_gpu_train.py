@@ -653,8 +653,8 @@ def test_chained_backward_with_the_lower_layers_backward_w(ext, monkeypatch, dty
     a, b = a.cuda(), b.cuda()
     sched = ext.schedule_for(a, b, in_dim)
     scale = 1.5
-    got = ext.backward_chained_lower(x, w, gy, sched, x0, a0, b0, p0 if softmax_lower else None, scale,
-                                     softmax_backward=True)
+    got = ext.backward_chained_lower(x, w, gy, sched, x0, a0, b0, p0, scale, softmax_backward=True,
+                                     softmax_backward_lower=softmax_lower)
     plain = ext.backward_chained(x, w, gy, sched, scale, softmax_backward=True)
     if batch * x.element_size() % 16 or batch * x.element_size() > 256 * 16:
         assert got is None                                          # whole 16-byte vectors, rows of at most 4 KB
@@ -670,9 +670,20 @@ def test_chained_backward_with_the_lower_layers_backward_w(ext, monkeypatch, dty
         rtol = {torch.float16: 4e-3, torch.float32: 1e-5, torch.float64: 1e-12}[dtype]
         ok, err = close(gw0, want0.double(), rtol)
         assert ok, err
-    again = ext.backward_chained_lower(x, w, gy, sched, x0, a0, b0, p0 if softmax_lower else None, scale,
-                                       softmax_backward=True)
+    again = ext.backward_chained_lower(x, w, gy, sched, x0, a0, b0, p0, scale, softmax_backward=True,
+                                       softmax_backward_lower=softmax_lower)
     assert torch.equal(again[0], gw) and torch.equal(again[1], gw0)  # deterministic
+    # x left out: its rows are recomputed from the layer below (fp32 / fp64); the same gradients bit for bit when x
+    # is what that layer's forward pass gives
+    x1 = ext.forward(x0, a0, b0, p0)
+    ref = ext.backward_chained_lower(x1, w, gy, sched, x0, a0, b0, p0, scale, softmax_backward=True,
+                                     softmax_backward_lower=softmax_lower)
+    rec = ext.backward_chained_lower(None, w, gy, sched, x0, a0, b0, p0, scale, softmax_backward=True,
+                                     softmax_backward_lower=softmax_lower)
+    if dtype == torch.float16:
+        assert rec is None
+    else:
+        assert torch.equal(rec[0], ref[0]) and torch.equal(rec[1], ref[1])
 
 
 @pytest.mark.parametrize("widths,batch,conn,grad_factor", [([400, 400, 300], 128, "random", 1.0),
@@ -718,11 +729,12 @@ def test_fuse_first_layers_trains_like_the_unfused_model(widths, batch, conn, gr
 
     calls = []
     real = dl.difflogic_cuda.backward_chained_lower
-    monkeypatch.setattr(dl.difflogic_cuda, "backward_chained_lower", lambda *a, **kw: calls.append(1) or real(*a, **kw))
+    monkeypatch.setattr(dl.difflogic_cuda, "backward_chained_lower",
+                        lambda *a, **kw: calls.append(a[0] is None) or real(*a, **kw))
     out0, gw0, _ = run(model)
     assert not calls
     out1, gw1, _ = run(fused)
-    assert len(calls) == (1 if len(widths) > 2 else 0)
+    assert calls == ([True] if len(widths) > 2 else [])           # the pair recomputes its inner activation
     assert close(out1, out0)[0]
     for u, v in zip(gw1, gw0):
         assert close(u, v.double())[0]
@@ -763,3 +775,51 @@ def test_fuse_first_layers_trains_like_the_unfused_model(widths, batch, conn, gr
         assert torch.equal(fused(x.cuda()), model(x.cuda()))
         assert torch.equal(fused(dl.PackBitsTensor(x.bool().cuda(), bit_count=64)),
                            model(dl.PackBitsTensor(x.bool().cuda(), bit_count=64)))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16])
+@pytest.mark.parametrize("in0,in_dim,out_dim,batch,kind", [(40, 64, 64, 256, "random"), (100, 300, 300, 512, "random"),
+                                                           (30, 50, 60, 128, "unique"), (20, 30, 47, 260, "any"),
+                                                           (15, 20, 40, 8, "any"), (25, 40, 24, 16, "sparse"),
+                                                           (784, 1000, 1200, 128, "random"), (30, 50, 60, 1024, "unique")])
+def test_two_layer_forward_recomputes_the_inner_activation(ext, dtype, in0, in_dim, out_dim, batch, kind):
+    """dl_logic_forward_chained_lower: the output and both layers' probabilities of two forward_logits
+    calls in a row, bit for bit, without the activation between them."""
+    from oracle import connections as oc
+    g = torch.Generator().manual_seed(in_dim + batch + in0)
+    torch.manual_seed(in_dim)
+    if kind == "random":
+        a, b = oc.random_connections(in_dim, out_dim)
+    elif kind == "unique":
+        a, b = oc.unique_connections(in_dim, out_dim)
+    elif kind == "sparse":                                           # half of the lower neurons feed nothing
+        a, b = torch.randint(0, in_dim // 2, (out_dim,), generator=g), torch.randint(0, in_dim // 2, (out_dim,),
+                                                                                    generator=g)
+    else:
+        a, b = torch.randint(0, in_dim, (out_dim,), generator=g), torch.randint(0, in_dim, (out_dim,), generator=g)
+    a0 = torch.randint(0, in0, (in_dim,), generator=g).cuda()
+    b0 = torch.randint(0, in0, (in_dim,), generator=g).cuda()
+    x0 = torch.rand(in0, batch, generator=g).to(dtype).cuda()
+    l0 = torch.randn(in_dim, 16, generator=g).to(dtype).cuda()
+    l1 = torch.randn(out_dim, 16, generator=g).to(dtype).cuda()
+    a, b = a.cuda(), b.cuda()
+    sched = ext.schedule_for(a, b, in_dim)
+    got = ext.forward_logits_lower(x0, a0, b0, l0, l1, sched)
+    if batch * x0.element_size() % 16 or batch * x0.element_size() > 128 * 16:
+        assert got is None                                          # whole 16-byte vectors, rows of at most 2 KB
+        return
+    y1, p0 = ext.forward_logits(x0, a0, b0, l0)
+    y2, p1 = ext.forward_logits(y1, a, b, l1, sched)
+    used = torch.zeros(in_dim, dtype=torch.bool, device="cuda")
+    used[a] = True
+    used[b] = True
+    if dtype == torch.float16:
+        # same fp32 arithmetic; the compiler may fold the final fp32 -> fp16 rounding into a fused multiply-add in
+        # one kernel and not in the other: rare last-bit differences (which the second layer then carries on)
+        for u, v in ((got[0], y2), (got[2], p1), (got[1][used], p0[used])):
+            diff = (u.float() - v.float()).abs()
+            assert float((diff > 0).float().mean()) < 0.05
+            assert bool((diff <= 2.0 ** -9 * u.float().abs().clamp(min=2.0 ** -14)).all())
+    else:
+        assert torch.equal(got[0], y2) and torch.equal(got[2], p1) and torch.equal(got[1][used], p0[used])
+    assert bool((got[1][~used] == 0).all())
