@@ -505,51 +505,70 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_chain_lower_kernel(
     const P *xv = reinterpret_cast<const P *>(lx);
     P *yv = reinterpret_cast<P *>(y);
 
+    // corner coefficients of the chunk's CHUNK + 1 lower neurons and CHUNK neurons, once for all column tiles
+    constexpr int NV = CHUNK + 4;
+    int32_t v[NV], n[CHUNK];
+    C lp00[NV], lp10[NV], ld0[NV], ld1[NV], p00[CHUNK], p10[CHUNK], d0[CHUNK], d1[CHUNK];
+#pragma unroll
+    for (int j0 = 0; j0 <= CHUNK; j0 += 4) {
+        int32_t v4[4];
+        C q00[4], q10[4], e0[4], e1[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v4[i] = j0 + i <= CHUNK ? verts[s0 + j0 + i] : -1;
+        corners4<T, LOGITS>(lw, v4, lane, blockIdx.y == 0, lprobs, q00, q10, e0, e1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[j0 + i] = v4[i], lp00[j0 + i] = q00[i], lp10[j0 + i] = q10[i], ld0[j0 + i] = e0[i], ld1[j0 + i] = e1[i];
+    }
+#pragma unroll
+    for (int j0 = 0; j0 < CHUNK; j0 += 4) {
+        int32_t n4[4];
+        C q00[4], q10[4], e0[4], e1[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) n4[i] = neuron[s0 + j0 + i];
+        corners4<T, LOGITS>(w, n4, lane, blockIdx.y == 0, probs, q00, q10, e0, e1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) n[j0 + i] = n4[i], p00[j0 + i] = q00[i], p10[j0 + i] = q10[i], d0[j0 + i] = e0[i], d1[j0 + i] = e1[i];
+    }
+    int64_t ia[CHUNK + 1], ib[CHUNK + 1];
+#pragma unroll
+    for (int j = 0; j <= CHUNK; ++j) ia[j] = low_a[v[j]], ib[j] = low_b[v[j]];
+
     for (int64_t ct = blockIdx.y; ct * DL_WAVE < ncols; ct += gridDim.y) {
         const int64_t col = ct * DL_WAVE + lane;
         const bool live = col < ncols;
         const int64_t cl = live ? col : 0;
-        // the chunk's CHUNK + 1 input rows, four lower neurons at a time
-        P rows[CHUNK + 4];
+        // the chunk's CHUNK + 1 input rows, recomputed four at a time
+        P rows[CHUNK + 1];
 #pragma unroll
         for (int j0 = 0; j0 <= CHUNK; j0 += 4) {
-            int32_t v[4];
             P va[4], vb[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                v[i] = j0 + i <= CHUNK ? verts[s0 + j0 + i] : -1;
-                const int64_t r = v[i] >= 0 ? v[i] : 0;
-                va[i] = xv[low_a[r] * ncols + cl];
-                vb[i] = xv[low_b[r] * ncols + cl];
+                if (j0 + i <= CHUNK) {
+                    va[i] = xv[ia[j0 + i] * ncols + cl];
+                    vb[i] = xv[ib[j0 + i] * ncols + cl];
+                }
             }
-            C p00[4], p10[4], d0[4], d1[4];
-            corners4<T, LOGITS>(lw, v, lane, ct == 0, lprobs, p00, p10, d0, d1);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-#pragma unroll
-                for (int e = 0; e < VEC; ++e)
-                    rows[j0 + i].v[e] = down<T, C>(mix<C>(up<T>(va[i].v[e]), up<T>(vb[i].v[e]), p00[i], p10[i], d0[i], d1[i]));
-            }
-        }
-#pragma unroll
-        for (int j0 = 0; j0 < CHUNK; j0 += 4) {
-            int32_t n[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) n[i] = neuron[s0 + j0 + i];
-            C p00[4], p10[4], d0[4], d1[4];
-            corners4<T, LOGITS>(w, n, lane, ct == 0, probs, p00, p10, d0, d1);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int j = j0 + i;
-                const bool f = flip[s0 + j] != 0;
-                P r;
+                if (j <= CHUNK) {
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    const C u0 = up<T>(rows[j].v[e]), u1 = up<T>(rows[j + 1].v[e]);
-                    r.v[e] = down<T, C>(mix<C>(f ? u1 : u0, f ? u0 : u1, p00[i], p10[i], d0[i], d1[i]));
+                    for (int e = 0; e < VEC; ++e)
+                        rows[j].v[e] = down<T, C>(mix<C>(up<T>(va[i].v[e]), up<T>(vb[i].v[e]), lp00[j], lp10[j], ld0[j], ld1[j]));
                 }
-                if (live && n[i] >= 0) yv[(int64_t) n[i] * ncols + col] = r;
             }
+        }
+#pragma unroll
+        for (int j = 0; j < CHUNK; ++j) {
+            const bool f = flip[s0 + j] != 0;
+            P r;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const C u0 = up<T>(rows[j].v[e]), u1 = up<T>(rows[j + 1].v[e]);
+                r.v[e] = down<T, C>(mix<C>(f ? u1 : u0, f ? u0 : u1, p00[j], p10[j], d0[j], d1[j]));
+            }
+            if (live && n[j] >= 0) yv[(int64_t) n[j] * ncols + col] = r;
         }
     }
 }
@@ -1443,7 +1462,8 @@ int forward_chain_lower_t(const void *lx, const int64_t *la, const int64_t *lb, 
     if (ncols > DL_FWD_ROWS_MIN) return DL_ERR_TOO_LARGE;        // rows of at most 2 KB
     const int64_t blocks = dl_ceil_div(nchunks, 4);
     if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
-    DL_LAUNCH((forward_chain_lower_kernel<T, V, DL_TRAIN_CHUNK, LOGITS>), dim3((unsigned) blocks, col_tiles(ncols)),
+    // one wave takes every column tile of its chunk (at most two): the corner coefficients are formed once
+    DL_LAUNCH((forward_chain_lower_kernel<T, V, DL_TRAIN_CHUNK, LOGITS>), dim3((unsigned) blocks, 1),
               dim3(DL_BLOCK), 0, s, (const T *) lx, la, lb, (const T *) lw, (T *) lprobs, verts, neuron, flip, (const T *) w,
               (T *) y, (T *) probs, nchunks, ncols);
     return dl_launch_status();
