@@ -73,3 +73,36 @@ def test_graphed_step_with_optimizer_tracks_eager_training():
         torch.cuda.synchronize()
     assert losses_g == losses_e, (losses_g, losses_e)
     assert losses_g[-1] < losses_g[0]
+
+
+def test_graphed_step_of_the_fused_model_equals_its_eager_step(monkeypatch):
+    """fuse_for_training (first two layers with the inner activation recomputed, last layer with
+    GroupSum) captured and replayed: every replay reproduces the eager step of the same fused
+    model bit for bit, on changing inputs."""
+    import copy
+
+    import difflogic_amd as dl
+    from difflogic_amd.graphs import GraphedTrainStep
+    monkeypatch.setattr(dl.LogicLayer, "_CHAIN_MIN_IN_DIM", 0)        # layers this narrow walk their schedules too
+    monkeypatch.setattr(dl.LogicLayer, "_CHAIN_MIN_OUT_DIM", 0)
+    monkeypatch.setattr(dl.difflogic_cuda, "BACKWARD_CHAIN_MAX_OVERFLOW", 1e9)
+    base = _model(dl, 2)
+    model = dl.fuse_for_training(base).train()
+    eager = dl.fuse_for_training(copy.deepcopy(base)).train()
+    assert isinstance(model[1], dl.FusedLogicLayerPair) and isinstance(model[-2], dl.FusedLogicLayerGroupSum)
+    loss_fn = torch.nn.CrossEntropyLoss()
+    g = torch.Generator(device="cuda").manual_seed(0)
+    xs = [(torch.rand(64, 60, device="cuda", generator=g) < 0.3).float() for _ in range(3)]
+    ys = [torch.randint(0, 10, (64,), device="cuda", generator=g) for _ in range(3)]
+    graphed = GraphedTrainStep(model, loss_fn, xs[0], ys[0])
+    for rep in range(5):
+        x, y = xs[rep % 3], ys[rep % 3]
+        loss_g = graphed.step(x, y)
+        torch.cuda.synchronize()
+        eager.zero_grad(set_to_none=True)
+        loss_e = loss_fn(eager(x), y)
+        loss_e.backward()
+        torch.cuda.synchronize()
+        assert torch.equal(loss_g, loss_e.detach()), rep
+        for pg, pe in zip(model.parameters(), eager.parameters()):
+            assert pg.grad is not None and torch.equal(pg.grad, pe.grad), rep
