@@ -206,6 +206,20 @@ def test_full_size_training_step(name, F, width, L, B, tau, connections, grad_fa
     out2, loss2, grads2 = run(everything)
     assert torch.equal(out, out2) and torch.equal(loss, loss2), name
     assert all(torch.equal(u, v) for u, v in zip(grads, grads2)), name
+    # fuse_for_training: first two layers as one node (C3: the activation between them recomputed), last layer with
+    # GroupSum.  Same parameters; the same sums in another order (the fused tail hands a slightly different gradient
+    # down to every layer below it).
+    plain_model, model = model, dl.fuse_for_training(model).train()
+    assert isinstance(model[1], dl.FusedLogicLayerPair) and isinstance(model[-2], dl.FusedLogicLayerGroupSum)
+    check_against_python(*run(rows), "fused for training")
+    outf, lossf, gradsf = run(everything)
+    assert _close(outf, out), name
+    # (the gradients are not compared with the unfused run's: the fused tail adds 6400 / 12800 terms per class in
+    # another order, and that difference is carried through every layer below; each layer is held to the python
+    # formulation's error budget above instead)
+    out2f, loss2f, grads2f = run(everything)
+    assert torch.equal(outf, out2f) and all(torch.equal(u, v) for u, v in zip(gradsf, grads2f)), name
+    model = plain_model
     monkeypatch.setattr(dl.LogicLayer, "_CHAIN_MIN_OUT_DIM", 1 << 40)
     check_against_python(*run(rows), "plain kernels")
     out3, loss3, grads3 = run(everything)
