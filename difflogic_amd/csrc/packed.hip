@@ -4,6 +4,8 @@
 // All three treat a packed matrix as rows of BYTES: with little-endian words, sample s of a
 // row is bit (s % 8) of byte (s / 8) whatever the word width, so one code path serves the
 // 8/16/32/64-bit word types and the widest vector access the row length allows is used.
+#include <hip/hip_fp16.h>
+
 #include "dl_common.h"
 
 #include <mutex>
@@ -1269,6 +1271,64 @@ extern "C" int dl_tensor_packbits(const uint8_t *t, void *out, int64_t features,
         DL_LAUNCH(packbits_generic_kernel, dim3((unsigned) gx, gy), dim3(DL_BLOCK), 0, s, t,
                            (uint8_t *) out, features, batch, out_row_bytes);
     }
+    return dl_launch_status();
+}
+
+// Gate ids of a layer for packed inference: argmax over each neuron's 16 weights, as
+// weights.argmax(-1).to(uint8): the first maximal value wins, a NaN counts as maximal.
+template <typename T>
+__global__ __launch_bounds__(DL_BLOCK) void gate_ids_kernel(const T *__restrict__ w, uint8_t *__restrict__ ids,
+                                                            int64_t out_dim) {
+    const int64_t n = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x;
+    if (n >= out_dim) return;
+    float best = (float) w[n * 16];
+    int at = 0;
+    if (best == best) {                                   // not NaN: look on
+#pragma unroll
+        for (int i = 1; i < 16; ++i) {
+            const float v = (float) w[n * 16 + i];
+            if (v != v) {                                 // the first NaN
+                at = i;
+                break;
+            }
+            if (v > best) best = v, at = i;
+        }
+    }
+    ids[n] = (uint8_t) at;
+}
+
+__global__ __launch_bounds__(DL_BLOCK) void gate_ids_f64_kernel(const double *__restrict__ w, uint8_t *__restrict__ ids,
+                                                                int64_t out_dim) {
+    const int64_t n = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x;
+    if (n >= out_dim) return;
+    double best = w[n * 16];
+    int at = 0;
+    if (best == best) {
+#pragma unroll
+        for (int i = 1; i < 16; ++i) {
+            const double v = w[n * 16 + i];
+            if (v != v) {
+                at = i;
+                break;
+            }
+            if (v > best) best = v, at = i;
+        }
+    }
+    ids[n] = (uint8_t) at;
+}
+
+extern "C" int dl_gate_ids(const void *w, uint8_t *ids, int64_t out_dim, int dtype, void *stream) {
+    if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
+    if (out_dim < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim == 0) return DL_OK;
+    if (!w || !ids) return DL_ERR_INVALID_ARGUMENT;
+    const int64_t blocks = dl_ceil_div(out_dim, DL_BLOCK);
+    if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    hipStream_t s = (hipStream_t) stream;
+    const dim3 grid((unsigned) blocks), block(DL_BLOCK);
+    if (dtype == DL_F16) DL_LAUNCH(gate_ids_kernel<__half>, grid, block, 0, s, (const __half *) w, ids, out_dim);
+    else if (dtype == DL_F32) DL_LAUNCH(gate_ids_kernel<float>, grid, block, 0, s, (const float *) w, ids, out_dim);
+    else DL_LAUNCH(gate_ids_f64_kernel, grid, block, 0, s, (const double *) w, ids, out_dim);
     return dl_launch_status();
 }
 

@@ -133,7 +133,10 @@ class LogicLayer(torch.nn.Module):
     def _gate_ids(self):
         """uint8 [out_dim] argmax gate per neuron.  Recomputed on every call like the reference
         (difflogic/difflogic.py:146): a cache could not see writes through ``weights.data``."""
-        return self.weights.detach().argmax(-1).to(torch.uint8)
+        w = self.weights.detach()
+        if w.is_cuda and w.is_contiguous() and w.dtype in (torch.float16, torch.float32, torch.float64):
+            return difflogic_cuda.gate_ids(w)
+        return w.argmax(-1).to(torch.uint8)
 
     def extra_repr(self):
         return "{}, {}, {}".format(self.in_dim, self.out_dim, "train" if self.training else "eval")

@@ -416,6 +416,22 @@ def eval(x, a, b, w):  # noqa: A001  (the reference's name)
     return y
 
 
+def gate_ids(weights):
+    """uint8 [out] argmax gate per neuron of float weights / logits [out, 16]:
+    ``weights.argmax(-1).to(torch.uint8)`` (difflogic/difflogic.py:146) in one kernel.  Not part
+    of the reference's extension."""
+    _check_input(weights, "weights")
+    code = _float_code(weights, "gate_ids")
+    if weights.dim() != 2 or weights.shape[1] != 16:
+        raise RuntimeError(f"expected weights [out,16], got {tuple(weights.shape)}")
+    ids = torch.empty(weights.shape[0], dtype=torch.uint8, device=weights.device)
+    with _on(weights.device):
+        st = _lib.load().dl_gate_ids(_p(weights), _p(ids), weights.shape[0], code, _stream(weights.device))
+    if st:
+        _raise(st, "gate_ids")
+    return ids
+
+
 def tensor_packbits_cuda(t, bit_count):
     """bool [F,B] -> (int{bit_count} [F, ceil(B/bit_count)], pad_len)   (difflogic.cpp:69-74)."""
     _check_input(t, "t")

@@ -259,6 +259,11 @@ int dl_adam_step(int count, float *const *p, const float *const *g, float *const
 
 /* ---- packed inference mode ------------------------------------------------------------ */
 
+/* The gate ids packed inference evaluates: ids[n] = argmax_i w[n, i] as uint8, i.e.
+ * `self.weights.argmax(-1).to(torch.uint8)` of difflogic/difflogic.py:146 in one kernel (the first
+ * maximal value wins; a NaN counts as maximal, as in torch).  w [out_dim, 16] of `dtype`. */
+int dl_gate_ids(const void *w, uint8_t *ids, int64_t out_dim, int dtype, void *stream);
+
 /* Replaces `eval` = logic_layer_cuda_eval (difflogic.cpp:63-68, difflogic_kernel.cu:503-541).
  *   x [in_dim, words], y [out_dim, words] of signed integers of `bit_count` bits;
  *   w [out_dim] uint8 gate ids (4-bit truth tables, difflogic_kernel.cu:418-435).

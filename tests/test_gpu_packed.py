@@ -522,3 +522,24 @@ def test_chained_groupbitsum_declines_where_it_does_not_apply(ext):
     assert sched.count_plan(12)[3] == 16 and sched.count_plan(1)[3] in (2, 4) and sched.count_plan(24) is None
     x32 = torch.zeros((30, 3), dtype=torch.int32, device="cuda")
     assert ext.eval_chained_groupbitsum(x32, dev_layers, 0, 10) is None               # rows are not whole 64-bit words
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16])
+def test_gate_ids_match_torch_argmax(ext, dtype):
+    """dl_gate_ids against weights.argmax(-1).to(uint8) (difflogic/difflogic.py:146): ties go to the
+    first maximal value, a NaN counts as maximal."""
+    g = torch.Generator().manual_seed(3)
+    w = torch.randn(5000, 16, generator=g)
+    w[::7] = torch.randint(0, 3, (w[::7].shape[0], 16), generator=g).float()      # many ties
+    w[5, 3] = float("nan")
+    w[6, 0] = float("nan")
+    w[8, 15] = float("nan")
+    w[8, 9] = float("nan")
+    w[9] = float("-inf")
+    w[10, 4] = float("inf")
+    w = w.to(dtype).cuda()
+    got = ext.gate_ids(w)
+    assert got.dtype == torch.uint8 and torch.equal(got, w.argmax(-1).to(torch.uint8))
+    assert ext.gate_ids(w[:0]).shape == (0,)
+    with pytest.raises(RuntimeError):
+        ext.gate_ids(w[:, :8].contiguous())
