@@ -127,7 +127,7 @@ def packed_run(torch, dl, model, x, k, steps, warmup):
     W = B // 64
     ext = dl.difflogic_cuda
     names = ("tensor_packbits_batch_major", "eval", "eval_fused", "eval_chained", "eval_fused_groupbitsum",
-             "eval_chained_groupbitsum", "eval_net_lds", "groupbitsum")
+             "eval_chained_groupbitsum", "eval_net_lds", "eval_net_lds_bool", "groupbitsum")
     names = tuple(n for n in names if hasattr(ext, n))
     real = {n: getattr(ext, n) for n in names}
     launches = []          # (kernel label, algorithmic bytes, start_event, end_event)
@@ -142,11 +142,14 @@ def packed_run(torch, dl, model, x, k, steps, warmup):
             return "groupbitsum %d" % a[0].shape[0], 8 * W * a[0].shape[0] + 4 * k * B
         if name == "eval":
             return "eval %d->%d" % (a[0].shape[0], a[3].shape[0]), eval_layer_bytes(a[0].shape[0], a[3].shape[0], W)
-        dims = [a[0].shape[0]] + [l[2].shape[0] for l in a[1]]
-        by = sum(eval_layer_bytes(i, o, W) for i, o in zip(dims[:-1], dims[1:]))
-        counted = name in ("eval_fused_groupbitsum", "eval_chained_groupbitsum", "eval_net_lds")
+        from_bool = name == "eval_net_lds_bool"           # x [B, F] bool: the packing happens inside the launch
+        dims = [a[0].shape[1] if from_bool else a[0].shape[0]] + [l[2].shape[0] for l in a[1]]
+        by = sum(eval_layer_bytes(i, o, W) for i, o in zip(dims[:-1], dims[1:])) + (B * F + 8 * W * F if from_bool else 0)
+        counted = name in ("eval_fused_groupbitsum", "eval_chained_groupbitsum", "eval_net_lds", "eval_net_lds_bool")
         base = {"eval_fused_groupbitsum": "eval_fused", "eval_chained_groupbitsum": "eval_chained"}.get(name, name)
         label = "%s x%d %s" % (base, len(a[1]), "->".join(str(d) for d in dims))
+        if from_bool:
+            label = "packbits + " + label
         if counted:
             by += 8 * W * dims[-1] + 4 * k * B
             label += " +groupbitsum"

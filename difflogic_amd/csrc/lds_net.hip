@@ -51,10 +51,11 @@ struct NetWiring {
     int32_t offset[DL_NET_MAX_DEPTH];           // first record of layer l
     int32_t steps[DL_NET_MAX_DEPTH];            // scheduled layers: steps (a multiple of 8); else 0
     int32_t stride[DL_NET_MAX_DEPTH];           // scheduled layers: row stride between a chunk's steps
+    int32_t in_base;                            // row of act[] at which the net's input starts
 };
 
 struct NetShape {
-    int32_t depth, in_dim;
+    int32_t depth, in_dim, in_base;
     int32_t width[DL_NET_MAX_DEPTH];
     int32_t offset[DL_NET_MAX_DEPTH];
     int32_t steps[DL_NET_MAX_DEPTH];
@@ -84,7 +85,8 @@ __global__ __launch_bounds__(DL_BLOCK) void compose_net_kernel(NetWiring t, uint
     const int l = blockIdx.y;
     const int i = (int) (blockIdx.x * DL_BLOCK + threadIdx.x);
     const int32_t *below = (l > 0 && t.steps[l - 1] > 0) ? t.pos[l - 1] : nullptr;
-    auto row = [&](int64_t v) -> uint32_t { return (uint32_t) (below ? below[v] : v); };
+    const int64_t first_row = l == 0 ? t.in_base : 0;
+    auto row = [&](int64_t v) -> uint32_t { return (uint32_t) (below ? below[v] : v + first_row); };
     if (t.steps[l] > 0) {
         if (i > t.steps[l]) return;
         uint32_t gate = 0;
@@ -282,8 +284,12 @@ __device__ __forceinline__ void load_class_records(uint32_t *r4, const uint32_t 
     }
 }
 
-template <int COLS, int GPT, int NP0>
+// BOOLIN: the input is the bool matrix [batch, in_dim] itself (sample-major, as the user holds it) and is
+// packed on the way into LDS, so neither the pack kernel nor the packed input exist: the workgroup reads
+// the COLS * 64 sample rows of its columns (one contiguous region) and folds them into the input rows.
+template <int COLS, int GPT, int NP0, bool BOOLIN>
 __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint64_t *__restrict__ x,
+                                                                      const uint8_t *__restrict__ xb,
                                                                       const uint32_t *__restrict__ rec, NetShape net,
                                                                       int32_t *__restrict__ out, int64_t ncols,
                                                                       int64_t per_class, int64_t k, int64_t batch,
@@ -292,19 +298,21 @@ __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint
     const int tid = (int) threadIdx.x;
     const int wave = dl_wave_in_block(), lane = dl_lane();
 
-    // Workgroups are dealt round-robin to the 8 XCDs, each with an L2 of its own.  The 16 / COLS workgroups
-    // whose columns share a 128-byte line of every input row are given to ONE XCD, so a line is fetched
-    // into one L2 instead of eight (the blocks past the last whole group of 8 * 16 / COLS keep their index).
+    // Packed input: workgroups are dealt round-robin to the 8 XCDs, each with an L2 of its own.  The
+    // 16 / COLS workgroups whose columns share a 128-byte line of every input row are given to ONE XCD,
+    // so a line is fetched into one L2 instead of eight (the blocks past the last whole group of
+    // 8 * 16 / COLS keep their index).
     constexpr uint32_t SHARE = 16 / COLS;
-    uint32_t cb = blockIdx.x;
-    if (cb < grouped_blocks) {
-        const uint32_t xcd = cb % 8, j = cb / 8;
-        cb = ((j / SHARE) * 8 + xcd) * SHARE + j % SHARE;
+    int64_t group = blockIdx.x;
+    if (!BOOLIN && blockIdx.x < grouped_blocks) {
+        const uint32_t xcd = blockIdx.x % 8, j = blockIdx.x / 8;
+        group = ((j / SHARE) * 8 + xcd) * SHARE + j % SHARE;
     }
-    const int64_t col0 = (int64_t) cb * COLS;
+    const int64_t col0 = group * COLS;
 
     // records a thread needs for layer l, requested one layer ahead of their use
     constexpr int NR = GPT > DL_NET_CHUNK + 2 ? GPT : DL_NET_CHUNK + 2;
+    const int rt = tid;
     auto load_records = [&](int l, uint32_t *r) __attribute__((always_inline)) {
         const uint32_t *tab = rec + net.offset[l];
         // scheduled: entry 8 tid + i sits at tab[i * stride + tid], i = 0..8, and the record of step 8192 + tid at
@@ -318,36 +326,92 @@ __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
             // (threads and entries without work read entry 0 and compute on it; only their stores are skipped)
-            const bool live = i < entries && (!sched ? tid + i * DL_NET_THREADS < limit
-                                              : i <= DL_NET_CHUNK ? tid < limit : tid < extra);
-            r[i] = tab[live ? tid + i * step : 0];
+            const bool live = i < entries && (!sched ? rt + i * DL_NET_THREADS < limit
+                                              : i <= DL_NET_CHUNK ? rt < limit : rt < extra);
+            r[i] = tab[live ? rt + i * step : 0];
         }
     };
+    // BOOLIN: packs group g's COLS * 64 samples of the bool input into the input rows.  A thread takes 16 features
+    // x 8 samples at a time: eight 16-byte loads (a wave's loads of one sample row are contiguous), folded into one
+    // register per 4 features (byte = feature, bit = sample), whose 16 bytes go to byte `oct` of the 16 features'
+    // rows.  All of a workgroup's loads are in flight together.  Samples past the batch read as zero.
+    auto stage_bool = [&](int64_t g, int t, int nthreads) __attribute__((always_inline)) {
+        const int per_row = net.in_dim / 16;
+        const int items = 8 * COLS * per_row;
+        const int64_t s_base = g * (COLS * 64);
+        for (int it = t; it < items; it += nthreads) {
+            const int oct = it / per_row, c = it - oct * per_row;      // byte of the row, 16-feature chunk
+            const int64_t s0 = s_base + 8 * oct;
+            const uint8_t *src = xb + s0 * net.in_dim + 16 * c;
+            dl_u32x4 v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                v[i] = s0 + i < batch ? __builtin_nontemporal_load(reinterpret_cast<const dl_u32x4 *>(src + (int64_t) i * net.in_dim))
+                                      : dl_u32x4{0, 0, 0, 0};
+            // bytes of a bool tensor are 0 or 1: then a shift and an OR per dword do; any other non-zero byte (a
+            // uint8 tensor viewed as bool) counts as true as well and sends the item through the general form
+            uint32_t acc[4], seen = 0;
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                acc[d] = 0;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    acc[d] |= v[i][d] << i;
+                    seen |= v[i][d];
+                }
+            }
+            if (seen & 0xfefefefeu) {
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    acc[d] = 0;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const uint32_t u = v[i][d];
+                        acc[d] |= (((((u & 0x7f7f7f7fu) + 0x7f7f7f7fu) | u) >> 7) & 0x01010101u) << i;
+                    }
+                }
+            }
+            // byte 4 d + kk of acc[] belongs to feature 16 c + 4 d + kk.  A wave's lanes hold consecutive chunks, whose
+            // rows lie 256 bytes apart, i.e. on one bank: every lane therefore starts with another of its 16 features
+            uint8_t *dst = act + ((size_t) net.in_base + 16 * c) * (8 * COLS) + oct;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int idx = (j + t) & 15;
+                const uint32_t lo = (idx & 4) ? acc[1] : acc[0], hi = (idx & 4) ? acc[3] : acc[2];
+                const uint32_t word = (idx & 8) ? hi : lo;
+                dst[(size_t) idx * (8 * COLS)] = (uint8_t) (word >> (8 * (idx & 3)));
+            }
+        }
+    };
+    const uint32_t *ltab = rec + net.offset[net.depth - 1];
     uint32_t r[NR];
     if (net.depth > 1) load_records(0, r);
     // the class phase's first records (wave = class)
-    const uint32_t *ltab = rec + net.offset[net.depth - 1];
     uint32_t rc[4] = {0, 0, 0, 0};
     if (wave < k) load_class_records(rc, ltab + wave * per_class, lane, per_class);
 
-    // the workgroup's word columns of the packed input; columns past the end read as zero
-    for (int f = tid; f < net.in_dim; f += DL_NET_THREADS) {
-        Row<COLS> v;
-        if (COLS > 1 && col0 + COLS <= ncols && ncols % 2 == 0 && ((uintptr_t) x & 15) == 0) {   // whole, 16-byte aligned
-            const dl_u32x4 *src = reinterpret_cast<const dl_u32x4 *>(x + (int64_t) f * ncols + col0);
+    if (BOOLIN) {
+        stage_bool(group, tid, DL_NET_THREADS);
+    } else {
+        // the workgroup's word columns of the packed input; columns past the end read as zero
+        for (int f = tid; f < net.in_dim; f += DL_NET_THREADS) {
+            Row<COLS> v;
+            if (COLS > 1 && col0 + COLS <= ncols && ncols % 2 == 0 && ((uintptr_t) x & 15) == 0) {   // whole, 16-byte aligned
+                const dl_u32x4 *src = reinterpret_cast<const dl_u32x4 *>(x + (int64_t) f * ncols + col0);
 #pragma unroll
-            for (int q = 0; q < COLS / 2; ++q) {
-                const dl_u32x4 t = src[q];
-                v.d[4 * q] = t.x, v.d[4 * q + 1] = t.y, v.d[4 * q + 2] = t.z, v.d[4 * q + 3] = t.w;
-            }
-        } else {
+                for (int q = 0; q < COLS / 2; ++q) {
+                    const dl_u32x4 t = src[q];
+                    v.d[4 * q] = t.x, v.d[4 * q + 1] = t.y, v.d[4 * q + 2] = t.z, v.d[4 * q + 3] = t.w;
+                }
+            } else {
 #pragma unroll
-            for (int j = 0; j < COLS; ++j) {
-                const uint64_t t = col0 + j < ncols ? x[(int64_t) f * ncols + col0 + j] : 0;
-                v.d[2 * j] = (uint32_t) t, v.d[2 * j + 1] = (uint32_t) (t >> 32);
+                for (int j = 0; j < COLS; ++j) {
+                    const uint64_t t = col0 + j < ncols ? x[(int64_t) f * ncols + col0 + j] : 0;
+                    v.d[2 * j] = (uint32_t) t, v.d[2 * j + 1] = (uint32_t) (t >> 32);
+                }
             }
+            lds_store<COLS>(act, (uint32_t) f, v);
         }
-        lds_store<COLS>(act, (uint32_t) f, v);
     }
     __syncthreads();
 
@@ -461,21 +525,33 @@ __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint
 }
 
 template <int COLS, int GPT>
-int launch_net(const void *x, const uint32_t *rec, const NetShape &net, int32_t *out, int64_t ncols, int64_t per_class,
-               int64_t k, int64_t batch, int64_t rows, hipStream_t s) {
-    const int64_t blocks = dl_ceil_div(ncols, COLS);
-    if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+int launch_net(const void *x, bool bool_input, const uint32_t *rec, const NetShape &net, int32_t *out, int64_t ncols,
+               int64_t per_class, int64_t k, int64_t batch, int64_t rows, hipStream_t s) {
+    const int64_t groups = dl_ceil_div(ncols, COLS);
+    if (groups > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     const size_t lds = (size_t) rows * 8 * COLS;
-    const dim3 grid((unsigned) blocks), block(DL_NET_THREADS);
-    const uint32_t group = 8 * (16 / COLS);                    // workgroups sharing input lines, one set per XCD
-    const uint32_t grouped = (uint32_t) blocks / group * group;
+    const dim3 block(DL_NET_THREADS);
     // a lane counts ceil(per_class / 64) neurons: NP0 planes hold up to 2^NP0 - 1
-    if (dl_ceil_div(per_class, DL_WAVE) < 16)
-        DL_LAUNCH((eval_net_lds_kernel<COLS, GPT, 4>), grid, block, lds, s, (const uint64_t *) x, rec, net, out, ncols,
-                  per_class, k, batch, grouped);
+    const bool small = dl_ceil_div(per_class, DL_WAVE) < 16;
+    if (bool_input) {
+        const dim3 grid((unsigned) groups);
+        if (small)
+            DL_LAUNCH((eval_net_lds_kernel<COLS, GPT, 4, true>), grid, block, lds, s, (const uint64_t *) nullptr,
+                      (const uint8_t *) x, rec, net, out, ncols, per_class, k, batch, 0u);
+        else
+            DL_LAUNCH((eval_net_lds_kernel<COLS, GPT, 8, true>), grid, block, lds, s, (const uint64_t *) nullptr,
+                      (const uint8_t *) x, rec, net, out, ncols, per_class, k, batch, 0u);
+        return dl_launch_status();
+    }
+    const dim3 grid((unsigned) groups);
+    const uint32_t share = 8 * (16 / COLS);                    // workgroups sharing input lines, one set per XCD
+    const uint32_t grouped = (uint32_t) groups / share * share;
+    if (small)
+        DL_LAUNCH((eval_net_lds_kernel<COLS, GPT, 4, false>), grid, block, lds, s, (const uint64_t *) x,
+                  (const uint8_t *) nullptr, rec, net, out, ncols, per_class, k, batch, grouped);
     else
-        DL_LAUNCH((eval_net_lds_kernel<COLS, GPT, 8>), grid, block, lds, s, (const uint64_t *) x, rec, net, out, ncols,
-                  per_class, k, batch, grouped);
+        DL_LAUNCH((eval_net_lds_kernel<COLS, GPT, 8, false>), grid, block, lds, s, (const uint64_t *) x,
+                  (const uint8_t *) nullptr, rec, net, out, ncols, per_class, k, batch, grouped);
     return dl_launch_status();
 }
 
@@ -502,40 +578,48 @@ extern "C" int64_t dl_logic_net_lds_workspace_bytes(int depth, const int64_t *di
     return bytes;
 }
 
-static int net_lds_run(const void *x, int depth, const int64_t *const *a, const int64_t *const *b, const uint8_t *const *w,
-                       const int64_t *dims, const int32_t *const *verts, const int32_t *const *neuron,
-                       const uint8_t *const *flip, const int64_t *steps, int32_t *out, int64_t words, int bit_count,
-                       int64_t pad_len, int64_t k, void *workspace, void *stream) {
-    if (bit_count != 8 && bit_count != 16 && bit_count != 32 && bit_count != 64) return DL_ERR_BIT_COUNT;
+// bool_input: x is the bool matrix [batch, dims[0]] (sample-major); words, bit_count and pad_len are then unused.
+static int net_lds_run(const void *x, bool bool_input, int64_t batch, int depth, const int64_t *const *a,
+                       const int64_t *const *b, const uint8_t *const *w, const int64_t *dims, const int32_t *const *verts,
+                       const int32_t *const *neuron, const uint8_t *const *flip, const int64_t *steps, int32_t *out,
+                       int64_t words, int bit_count, int64_t pad_len, int64_t k, void *workspace, void *stream) {
+    if (!bool_input && bit_count != 8 && bit_count != 16 && bit_count != 32 && bit_count != 64) return DL_ERR_BIT_COUNT;
     if (depth < 1 || !dims || !a || !b || !w || words < 0 || k <= 0 || pad_len < 0) return DL_ERR_INVALID_ARGUMENT;
     if (depth > DL_NET_MAX_DEPTH) return DL_ERR_TOO_LARGE;
     for (int l = 0; l <= depth; ++l)
         if (dims[l] <= 0) return DL_ERR_INVALID_ARGUMENT;
     if (dims[depth] % k != 0) return DL_ERR_NOT_DIVISIBLE;
-    const int64_t batch = words * bit_count - pad_len;
+    if (!bool_input) batch = words * bit_count - pad_len;
     if (batch < 0) return DL_ERR_INVALID_ARGUMENT;
     if (batch == 0) return DL_OK;
     if (!x || !out || !workspace) return DL_ERR_INVALID_ARGUMENT;
-    const int64_t row_bytes = words * (bit_count / 8);
+    const int64_t row_bytes = bool_input ? dl_ceil_div(batch, 64) * 8 : words * (bit_count / 8);
     // rows of whole 64-bit words and layers that fit the LDS buffer; otherwise the caller runs the streaming kernels
     if (!net_shape_ok(depth, dims, k) || row_bytes % 8 != 0 || !dl_aligned(x, 8) || !dl_aligned(workspace, 4))
         return DL_ERR_TOO_LARGE;
+    // the bool input is read in 16-byte pieces of a sample row
+    if (bool_input && (dims[0] % 16 != 0 || !dl_aligned(x, 16))) return DL_ERR_TOO_LARGE;
     hipStream_t s = (hipStream_t) stream;
 
     // The widest hidden layer (or the input) decides the columns per workgroup: rows * 8 * COLS bytes of LDS, and a
-    // thread holds the outputs of ceil(width / 1024) neurons in registers.
-    int64_t rows = dims[0], hidden = 0;
+    // thread holds the outputs of ceil(width / 1024) neurons in registers.  A packed input occupies the rows the
+    // first layer then overwrites; a bool input has rows of its own behind those of the hidden layers, because it is
+    // filled for the next group of columns while this one is still being counted.
+    const int64_t input_rows = bool_input ? dims[0] : 0;
+    int64_t rows = bool_input ? 0 : dims[0], hidden = 0;
     for (int l = 0; l + 1 < depth; ++l) {
         if (dims[l + 1] > hidden) hidden = dims[l + 1];
         if (dims[l + 1] > rows) rows = dims[l + 1];              // the last layer's output is never stored
     }
-    const bool four = rows <= DL_NET_MAX_WIDTH / 2 && hidden <= 5 * DL_NET_THREADS;
-    const int64_t capacity = four ? DL_NET_MAX_WIDTH / 2 : DL_NET_MAX_WIDTH;        // rows of act[]
+    if (rows + input_rows > DL_NET_MAX_WIDTH) return DL_ERR_TOO_LARGE;
+    const bool four = rows + input_rows <= DL_NET_MAX_WIDTH / 2 && hidden <= 5 * DL_NET_THREADS;
+    const int64_t capacity = (four ? DL_NET_MAX_WIDTH / 2 : DL_NET_MAX_WIDTH) - input_rows;   // rows of the layers
 
     NetWiring wiring;
     NetShape net;
     net.depth = depth;
     net.in_dim = (int32_t) dims[0];
+    net.in_base = wiring.in_base = 0;
     int64_t entries = 0, offset = 0, most_steps = 0;
     char *pos_base = nullptr;
     for (int l = 0; l < DL_NET_MAX_DEPTH; ++l) {
@@ -585,6 +669,7 @@ static int net_lds_run(const void *x, int depth, const int64_t *const *a, const 
         const int st = dl_launch_status();
         if (st != DL_OK) return st;
     }
+    net.in_base = wiring.in_base = (int32_t) (bool_input ? rows : 0);      // the input's rows follow the layers'
     DL_LAUNCH(compose_net_kernel, dim3((unsigned) dl_ceil_div(entries, DL_BLOCK), (unsigned) depth), dim3(DL_BLOCK), 0, s,
               wiring, rec);
     int st = dl_launch_status();
@@ -592,15 +677,15 @@ static int net_lds_run(const void *x, int depth, const int64_t *const *a, const 
 
     const int64_t ncols = row_bytes / 8;
     const int64_t per_class = dims[depth] / k;
-    if (four) return launch_net<4, 5>(x, rec, net, out, ncols, per_class, k, batch, rows, s);
-    return launch_net<2, 10>(x, rec, net, out, ncols, per_class, k, batch, rows, s);
+    if (four) return launch_net<4, 5>(x, bool_input, rec, net, out, ncols, per_class, k, batch, rows + input_rows, s);
+    return launch_net<2, 10>(x, bool_input, rec, net, out, ncols, per_class, k, batch, rows + input_rows, s);
 }
 
 extern "C" int dl_logic_net_lds_groupbitsum(const void *x, int depth, const int64_t *const *a, const int64_t *const *b,
                                             const uint8_t *const *w, const int64_t *dims, int32_t *out, int64_t words,
                                             int bit_count, int64_t pad_len, int64_t k, void *workspace, void *stream) {
-    return net_lds_run(x, depth, a, b, w, dims, nullptr, nullptr, nullptr, nullptr, out, words, bit_count, pad_len, k,
-                       workspace, stream);
+    return net_lds_run(x, false, 0, depth, a, b, w, dims, nullptr, nullptr, nullptr, nullptr, out, words, bit_count, pad_len,
+                       k, workspace, stream);
 }
 
 extern "C" int dl_logic_net_lds_groupbitsum_scheduled(const void *x, int depth, const int64_t *const *a,
@@ -609,6 +694,16 @@ extern "C" int dl_logic_net_lds_groupbitsum_scheduled(const void *x, int depth, 
                                                       const int32_t *const *neuron, const uint8_t *const *flip,
                                                       const int64_t *steps, int32_t *out, int64_t words, int bit_count,
                                                       int64_t pad_len, int64_t k, void *workspace, void *stream) {
-    return net_lds_run(x, depth, a, b, w, dims, verts, neuron, flip, steps, out, words, bit_count, pad_len, k, workspace,
+    return net_lds_run(x, false, 0, depth, a, b, w, dims, verts, neuron, flip, steps, out, words, bit_count, pad_len, k,
+                       workspace, stream);
+}
+
+extern "C" int dl_logic_net_lds_groupbitsum_bool(const uint8_t *x, int64_t batch, int depth, const int64_t *const *a,
+                                                 const int64_t *const *b, const uint8_t *const *w, const int64_t *dims,
+                                                 const int32_t *const *verts, const int32_t *const *neuron,
+                                                 const uint8_t *const *flip, const int64_t *steps, int32_t *out,
+                                                 int64_t k, void *workspace, void *stream) {
+    if (batch < 0) return DL_ERR_INVALID_ARGUMENT;
+    return net_lds_run(x, true, batch, depth, a, b, w, dims, verts, neuron, flip, steps, out, 0, 64, 0, k, workspace,
                        stream);
 }

@@ -863,6 +863,55 @@ def eval_net_lds(x, layers, pad_len, k, scheduled=True):
     return out
 
 
+def eval_net_lds_bool(x, layers, k, scheduled=True):
+    """eval_net_lds on the bool input itself: ``x`` [B, in] bool (sample-major, as PackBitsTensor
+    receives it) -> int32 [B, k], the result of packing x with 64-bit words, evaluating every layer
+    and groupbitsum, in one kernel that packs the input on its way into LDS (no pack kernel, no
+    packed input in memory).  Returns None where the kernel does not apply (in not a multiple of
+    16, input and widest hidden layer together beyond net_lds_max_width(), unaligned x).  Not part
+    of the reference's extension."""
+    _check_input(x, "x")
+    if x.dtype != torch.bool or x.dim() != 2 or not layers:
+        raise RuntimeError(f"expected x [B,in] bool and at least one layer, got {x.dtype} {tuple(x.shape)}")
+    batch, in_dim = x.shape
+    dims, tensors = [in_dim], [x]
+    for a, b, w in layers:
+        _check_input(w, "w")
+        if w.dim() != 1 or w.dtype != torch.uint8:
+            raise RuntimeError(f"expected w [out] uint8, got {tuple(w.shape)} {w.dtype}")
+        _check_index(a, "a", w.shape[0])
+        _check_index(b, "b", w.shape[0])
+        dims.append(w.shape[0])
+        tensors += [a, b, w]
+    dev = _same_device(*tensors)
+    depth, out_dim = len(layers), dims[-1]
+    if k <= 0 or out_dim % k != 0:
+        raise ValueError(f"in_dim ({out_dim}) has to be divisible by k ({k}) but it is not")
+    if depth > MAX_NET_DEPTH or 0 in dims or max(dims) > net_lds_max_width() or in_dim % 16 != 0:
+        return None
+    ptrs = lambda i: (ctypes.c_void_p * depth)(*[l[i].data_ptr() for l in layers])  # noqa: E731
+    pdims = (ctypes.c_int64 * (depth + 1))(*dims)
+    lib = _lib.load()
+    out = torch.empty((batch, k), dtype=torch.int32, device=dev)
+    if batch == 0:
+        return out
+    ws = torch.empty(max(1, lib.dl_logic_net_lds_workspace_bytes(depth, pdims) // 4), dtype=torch.int32, device=dev)
+    scheds = [schedule_for(a, b, dims[i]) for i, (a, b, _) in enumerate(layers[:-1])] if scheduled else []
+    n = len(scheds)
+    pv = (ctypes.c_void_p * n)(*[sc.verts.data_ptr() for sc in scheds]) if n else None
+    pn = (ctypes.c_void_p * n)(*[sc.neuron.data_ptr() for sc in scheds]) if n else None
+    pf = (ctypes.c_void_p * n)(*[sc.flip.data_ptr() for sc in scheds]) if n else None
+    ps = (ctypes.c_int64 * n)(*[sc.steps for sc in scheds]) if n else None
+    with _on(dev):
+        st = lib.dl_logic_net_lds_groupbitsum_bool(_p(x), batch, depth, ptrs(0), ptrs(1), ptrs(2), pdims, pv, pn, pf, ps,
+                                                   _p(out), int(k), _p(ws), _stream(dev))
+    if st == _lib.DL_ERR_TOO_LARGE:
+        return None
+    if st:
+        _raise(st, "logic_net_lds_groupbitsum_bool")
+    return out
+
+
 def eval_fused_groupbitsum_noalloc(x, layers, pad_len, k, out, order=None):
     """eval_fused_groupbitsum into the caller's ``out`` (int32 [batch, k], contiguous) through the
     entry point that allocates no device memory: its workspace is a static device array of

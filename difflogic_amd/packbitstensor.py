@@ -120,30 +120,48 @@ class PackBitsTensor:
         self.bit_count = bit_count
         self.device = device
         self._t = None
+        self._src = None              # the bool input [B, F] while it has not been packed yet
         self._pending = []            # [(a, b, w)] applied to _t but not yet evaluated
         if device == "cuda":
+            if bit_count not in (8, 16, 32, 64):
+                raise ValueError("`bit_count` has to be in { 8, 16, 32, 64 }")
             t = t.to(device)
+            self.pad_len = (bit_count - t.shape[0] % bit_count) % bit_count
             if t.dtype == torch.bool and t.is_contiguous():
-                # transpose + pack in one kernel
-                self.t, self.pad_len = difflogic_cuda.tensor_packbits_batch_major(t, self.bit_count)
+                # packed (transpose + pack in one kernel) when the words are first needed: a narrow net
+                # that runs resident in LDS reads the bool input itself
+                self._src = t
             else:
-                self.t, self.pad_len = difflogic_cuda.tensor_packbits_cuda(t.T.contiguous(), self.bit_count)
+                self._t, self.pad_len = difflogic_cuda.tensor_packbits_cuda(t.T.contiguous(), self.bit_count)
         else:
             raise NotImplementedError(device)
+
+    def _words(self):
+        """The packed input words, packing the bool input now if that has not happened yet."""
+        if self._t is None:
+            self._t, self.pad_len = difflogic_cuda.tensor_packbits_batch_major(self._src, self.bit_count)
+            self._src = None
+        return self._t
+
+    def _in_features(self):
+        return self._src.shape[1] if self._t is None else self._t.shape[0]
 
     @property
     def features(self):
         """Number of rows ``.t`` has (after the deferred layers)."""
-        return self._pending[-1][2].shape[0] if self._pending else self._t.shape[0]
+        return self._pending[-1][2].shape[0] if self._pending else self._in_features()
 
     def _words64(self):
         """Row length in 64-bit words (what the planner's byte counts are based on)."""
+        if self._t is None:
+            return max(1, -(-self._src.shape[0] // 64))
         return max(1, self._t.shape[1] * self.bit_count // 64)
 
     def _dims(self):
-        return [self._t.shape[0]] + [w.shape[0] for _, _, w in self._pending]
+        return [self._in_features()] + [w.shape[0] for _, _, w in self._pending]
 
     def _run_groups(self, groups):
+        self._words()
         pos = 0
         for depth in groups:
             run = difflogic_cuda.eval_chained if _chained(depth) else difflogic_cuda.eval_fused
@@ -155,11 +173,12 @@ class PackBitsTensor:
     def t(self):
         if self._pending:
             self._run_groups(plan_groups(self._dims(), False, self._words64()))
-        return self._t
+        return self._words()
 
     @t.setter
     def t(self, value):
         self._pending = []
+        self._src = None
         self._t = value
 
     def defer_layer(self, a, b, w):
@@ -177,20 +196,25 @@ class PackBitsTensor:
             if tail:
                 # the narrow end of the net runs resident in LDS; what lies before it streams
                 head = len(self._pending) - tail
+                if head == 0 and self._t is None:
+                    # the whole net, straight from the bool input: packing happens on the way into LDS
+                    out = difflogic_cuda.eval_net_lds_bool(self._src, self._pending, k)
+                    if out is not None:
+                        return out
                 if head:
                     self._run_groups(plan_groups(dims[:head + 1], False, self._words64()))
-                out = difflogic_cuda.eval_net_lds(self._t, self._pending, self.pad_len, k)
+                out = difflogic_cuda.eval_net_lds(self._words(), self._pending, self.pad_len, k)
                 if out is not None:
                     return out
             groups = plan_groups(self._dims(), True, self._words64())
             self._run_groups(groups[:-1])
             # the last group stays pending: the object's state does not change by counting
-            out = difflogic_cuda.eval_chained_groupbitsum(self._t, self._pending, self.pad_len, k)
+            out = difflogic_cuda.eval_chained_groupbitsum(self._words(), self._pending, self.pad_len, k)
             if out is not None:
                 return out
             order = difflogic_cuda.count_order_for(self._pending, self._t.shape[0], k)
             return difflogic_cuda.eval_fused_groupbitsum(self._t, self._pending, self.pad_len, k, order)
-        return difflogic_cuda.groupbitsum(self._t, self.pad_len, k)
+        return difflogic_cuda.groupbitsum(self._words(), self.pad_len, k)
 
     def flatten(self, start_dim=0, end_dim=-1, **kwargs):
         """Returns the object itself; the arguments are ignored."""

@@ -411,7 +411,13 @@ int dl_logic_eval_chained_groupbitsum(const void *x, int depth, const int64_t *c
  *   DEVICE copies of that layer's evaluation schedule (HOST arrays verts, neuron, flip of depth - 1
  *   DEVICE pointers and HOST steps [depth - 1]; a NULL entry leaves the layer as it is): such a
  *   layer is walked along its trails inside the kernel, which nearly halves its LDS row reads.
- *   Same result; same workspace size. */
+ *   Same result; same workspace size.
+ *   dl_logic_net_lds_groupbitsum_bool() takes the bool matrix x [batch, dims[0]] itself (sample-major,
+ *   one byte per value, any non-zero byte true: what PackBitsTensor.__init__ receives,
+ *   difflogic/packbitstensor.py:6-16) and packs it on the way into LDS, so the pack kernel and the packed
+ *   input do not exist; out [batch, k].  Applies when dims[0] is a multiple of 16, x is 16-byte aligned
+ *   and the input fits the LDS buffer next to the widest hidden layer (dims[0] + max hidden width <=
+ *   dl_logic_net_lds_max_width()); otherwise DL_ERR_TOO_LARGE. */
 int64_t dl_logic_net_lds_max_width(void);
 int64_t dl_logic_net_lds_workspace_bytes(int depth, const int64_t *dims);
 int dl_logic_net_lds_groupbitsum(const void *x, int depth, const int64_t *const *a,
@@ -425,6 +431,12 @@ int dl_logic_net_lds_groupbitsum_scheduled(const void *x, int depth, const int64
                                            const int64_t *steps, int32_t *out, int64_t words,
                                            int bit_count, int64_t pad_len, int64_t k, void *workspace,
                                            void *stream);
+int dl_logic_net_lds_groupbitsum_bool(const uint8_t *x, int64_t batch, int depth,
+                                      const int64_t *const *a, const int64_t *const *b,
+                                      const uint8_t *const *w, const int64_t *dims,
+                                      const int32_t *const *verts, const int32_t *const *neuron,
+                                      const uint8_t *const *flip, const int64_t *steps, int32_t *out,
+                                      int64_t k, void *workspace, void *stream);
 
 /* dl_logic_eval_fused_groupbitsum without a workspace argument, for callers that cannot allocate
  * device memory: code under HIP graph capture, tight serving loops, harnesses that forbid

@@ -543,3 +543,44 @@ def test_gate_ids_match_torch_argmax(ext, dtype):
     assert ext.gate_ids(w[:0]).shape == (0,)
     with pytest.raises(RuntimeError):
         ext.gate_ids(w[:, :8].contiguous())
+
+
+@pytest.mark.parametrize("in_dim,widths,B,k", [
+    (32, [60], 100, 3),                                   # a single layer: the class phase reads the input rows
+    (48, [100, 640], 7 * 64 + 1, 10), (16, [33, 130, 77, 130], 129 * 64 - 5, 2),
+    (784, [8000] * 6, 9 * 64 + 3, 10),                    # C2's net: 2 columns per workgroup, odd column count, ragged
+    (784, [4000] * 3, 11 * 64, 10),                       # 4 columns per workgroup, 3 columns left over
+    (2048, [3000, 8000, 3000], 200, 3),                   # input + widest hidden layer just fit next to each other
+    (96, [300, 4096], 5 * 64, 2),                         # 2048 neurons per class: 8 counter planes per lane
+    (64, [80, 400], 300, 40),                             # more classes than waves
+    (1024, [8190, 8250, 20], 130, 4),                     # schedules around 8192 steps
+])
+def test_net_lds_from_the_bool_input(ext, in_dim, widths, B, k):
+    """dl_logic_net_lds_groupbitsum_bool: packing on the way into LDS gives the counts of packing
+    first (any non-zero byte is true), for ragged batches too."""
+    rng = np.random.default_rng(in_dim + B + k + widths[-1] + len(widths))
+    raw = (rng.integers(0, 256, (B, in_dim), dtype=np.uint8) * (rng.random((B, in_dim)) < 0.4)).astype(np.uint8)
+    layers, dev_layers = _chain(rng, in_dim, widths)
+    xb = torch.as_tensor(raw).cuda().view(torch.bool)
+    got = ext.eval_net_lds_bool(xb, dev_layers, k)
+    assert got is not None and got.dtype == torch.int32 and tuple(got.shape) == (B, k)
+    words, pad = po.packbits((raw != 0).T, 64)
+    y = words
+    for a, b, op in layers:
+        y = po.eval_layer(y, a, b, op)
+    assert np.array_equal(got.cpu().numpy(), po.groupbitsum(y, pad, k))
+    packed, pad2 = ext.tensor_packbits_batch_major(xb, 64)
+    assert torch.equal(got, ext.eval_net_lds(packed, dev_layers, pad2, k))
+    assert torch.equal(got, ext.eval_net_lds_bool(xb, dev_layers, k, scheduled=False))
+
+
+def test_net_lds_from_the_bool_input_declines_what_does_not_fit(ext):
+    rng = np.random.default_rng(4)
+    _, dev_layers = _chain(rng, 40, [60, 30])
+    assert ext.eval_net_lds_bool(torch.zeros(10, 40, dtype=torch.bool, device="cuda"), dev_layers, 3) is None   # 40 % 16
+    _, dev_layers = _chain(rng, 4096, [8000, 30])
+    assert ext.eval_net_lds_bool(torch.zeros(10, 4096, dtype=torch.bool, device="cuda"), dev_layers, 3) is None  # no room
+    _, dev_layers = _chain(rng, 48, [60, 30])
+    assert ext.eval_net_lds_bool(torch.zeros(0, 48, dtype=torch.bool, device="cuda"), dev_layers, 3).shape == (0, 3)
+    with pytest.raises(ValueError):
+        ext.eval_net_lds_bool(torch.zeros(10, 48, dtype=torch.bool, device="cuda"), dev_layers, 7)
