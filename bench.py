@@ -126,7 +126,7 @@ def packed_run(torch, dl, model, x, k, steps, warmup):
     B, F = x.shape
     W = B // 64
     ext = dl.difflogic_cuda
-    names = ("tensor_packbits_batch_major", "eval", "eval_fused", "eval_chained", "eval_fused_groupbitsum",
+    names = ("tensor_packbits_batch_major", "tensor_packbits_batch_major_rows", "eval", "eval_fused", "eval_chained", "eval_fused_groupbitsum",
              "eval_chained_groupbitsum", "eval_net_lds", "eval_net_lds_bool", "groupbitsum")
     names = tuple(n for n in names if hasattr(ext, n))
     real = {n: getattr(ext, n) for n in names}
@@ -136,7 +136,7 @@ def packed_run(torch, dl, model, x, k, steps, warmup):
     def describe(name, a):
         """(label, algorithmic bytes): per layer 8*W*(in+out) + 17*out, the count 8*W*out + 4*k*B, the
         packing B*F + F*W*8; a fused launch is charged the sum over the layers it replaces."""
-        if name == "tensor_packbits_batch_major":
+        if name in ("tensor_packbits_batch_major", "tensor_packbits_batch_major_rows"):
             return "packbits_batch_major %dx%d" % tuple(a[0].shape), B * F + 8 * W * F
         if name == "groupbitsum":
             return "groupbitsum %d" % a[0].shape[0], 8 * W * a[0].shape[0] + 4 * k * B
@@ -269,8 +269,31 @@ def packed_headline(args, torch, dl):
         "path_alg_GBps": round(total_alg / (ms_per_step * 1e-3) / 1e9, 1),
         "first_call_ms": round(first_ms, 1),
         "checksum": int(out.sum().item()),
+        "other_word_widths": word_width_variants(torch, dl, model, x, out),
     }
     return value, ms_per_step, roofline, info, model, x, out
+
+
+def word_width_variants(torch, dl, model, x, want):
+    """The same step with PackBitsTensor's other word widths (32 is the reference's default) and with a
+    batch that fills neither the last word nor the last 16 bytes of a row: ms per step, and whether the
+    counts equal the int64 run's."""
+    res = {}
+    ragged = x[:x.shape[0] - 37].contiguous()
+    for name, inp, bits in (("int32", x, 32), ("int16", x, 16), ("int8", x, 8), ("int32, batch - 37", ragged, 32),
+                            ("int64, batch - 37", ragged, 64)):
+        def step():
+            with torch.no_grad():
+                return model(dl.PackBitsTensor(inp, bit_count=bits))
+        step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(3):
+            got = step()
+        torch.cuda.synchronize()
+        res[name] = {"ms_per_step": round((time.perf_counter() - t0) / 3 * 1e3, 4),
+                     "equal_to_int64_run": bool(torch.equal(got, want[:inp.shape[0]]))}
+    return res
 
 
 def net_tables(model, dl):
@@ -334,7 +357,7 @@ def train_alg_bytes(dims, B):
     return alg + sum(4 * B * (2 * i + o) + 64 * o for i, o in zip(dims[1:-1], dims[2:]))
 
 
-def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor, x, steps, warmup):
+def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor, x, steps, warmup, other_dtypes=False):
     """fp32 training step of one configuration with CrossEntropy: forward+backward and
     forward+backward+Adam(lr 0.01), each eager and replayed as one HIP graph; once for the model as
     the reference's user writes it (torch's fused Adam) and once with the training epilogue of this
@@ -421,6 +444,37 @@ def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor
     res["optimizer"] = "torch.optim.Adam(fused=True, capturable=True)"
     res["fused_for_training"] = {"optimizer": "difflogic_amd.FusedAdam (one launch over all weight tensors)"}
     measure(dl.fuse_for_training(model).train(), res["fused_for_training"], lambda ps: dl.FusedAdam(ps, lr=0.01))
+
+    if other_dtypes:
+        # experiments/main.py:19-23,286 (--training-bit-count 16 / 64): the input is cast, the weights stay fp32
+        res["other_input_dtypes"] = {}
+        for key, dtype, size in (("f16", torch.float16, 2), ("f64", torch.float64, 8)):
+            xd = x.to(dtype)
+
+            def fwd_bwd():
+                model.zero_grad(set_to_none=True)
+                loss = loss_fn(model(xd), labels)
+                loss.backward()
+                return loss
+
+            def report_dtype(sec, loss):
+                r = report(sec, loss)
+                r["alg_GBps"] = round(r["alg_GBps"] * size / 4, 1)
+                r["frac_hbm_algorithmic"] = round(r["frac_hbm_algorithmic"] * size / 4, 4)
+                return r
+
+            out = res["other_input_dtypes"][key] = {}
+            sec, loss = timeit(fwd_bwd)
+            out["fwd_bwd_eager"] = report_dtype(sec, loss.item())
+            del loss
+            model.zero_grad(set_to_none=True)
+            gc.collect()
+            torch.cuda.synchronize()
+            graphed = GraphedTrainStep(model, loss_fn, xd, labels)
+            sec, loss = timeit(graphed.step)
+            out["fwd_bwd_graph"] = report_dtype(sec, loss.item())
+            del graphed, loss, xd
+            gc.collect()
     return res, model
 
 
@@ -592,7 +646,7 @@ def extra_configs(args, torch, dl):
         x = bernoulli_input(torch, B, 784, 2).float()
         configs["C3"], model = train_config(
             torch, dl, "fp32 train 784->6x64000->GroupSum(10,tau=30), B=512, connections=unique, CrossEntropy",
-            784, [64000] * 6, 10, 30.0, B, "unique", 1.0, x, steps, warmup)
+            784, [64000] * 6, 10, 30.0, B, "unique", 1.0, x, steps, warmup, other_dtypes=True)
         configs["C3"]["kernels_alone_64000x64000"] = train_kernels_alone(torch, dl, model, B, 64000)
         del model, x
         gc.collect()

@@ -55,6 +55,7 @@ SIGNATURES = {
     "dl_logic_eval": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "dl_tensor_packbits": [_vp, _vp, _i64, _i64, _int, ctypes.POINTER(_i64), _vp],
     "dl_tensor_packbits_batch_major": [_vp, _vp, _i64, _i64, _int, ctypes.POINTER(_i64), _vp],
+    "dl_tensor_packbits_batch_major_rows": [_vp, _vp, _i64, _i64, _i64, _vp],
     "dl_groupbitsum": [_vp, _vp, _i64, _i64, _int, _i64, _i64, _vp],
     "dl_logic_eval_fused_workspace_bytes": [_int, _i64],
     "dl_logic_eval_fused": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _vp, _vp],

@@ -1332,18 +1332,13 @@ extern "C" int dl_gate_ids(const void *w, uint8_t *ids, int64_t out_dim, int dty
     return dl_launch_status();
 }
 
-extern "C" int dl_tensor_packbits_batch_major(const uint8_t *x, void *out, int64_t batch, int64_t features,
-                                              int bit_count, int64_t *pad_len, void *stream) {
-    if (!valid_bit_count(bit_count)) return DL_ERR_BIT_COUNT;
-    if (features < 0 || batch < 0) return DL_ERR_INVALID_ARGUMENT;
-    if (pad_len) *pad_len = (bit_count - batch % bit_count) % bit_count;
-    if (features == 0 || batch == 0) return DL_OK;
-    if (!x || !out) return DL_ERR_INVALID_ARGUMENT;
-    hipStream_t s = (hipStream_t) stream;
-    const int64_t words = dl_ceil_div(batch, bit_count);
-    const int64_t out_row_bytes = words * (bit_count / 8);
+// Sample-major bool bytes -> feature rows of `out_row_bytes` bytes each (a little-endian bit stream: sample s is
+// bit s % 8 of byte s / 8, whatever the word width); bits past the batch are zero.
+static int pack_batch_major_rows(const uint8_t *x, void *out, int64_t batch, int64_t features, int64_t out_row_bytes,
+                                 hipStream_t s) {
     if (out_row_bytes % 8 == 0 && !dl_aligned(out, 8)) return DL_ERR_INVALID_ARGUMENT;
-    const int64_t gx = dl_ceil_div(dl_ceil_div(batch, 64), 16);
+    const int64_t cols = dl_ceil_div(out_row_bytes, 8);          // 64-sample columns of the output
+    const int64_t gx = dl_ceil_div(cols, 16);
     if (gx > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     if (features % 16 == 0 && dl_aligned(x, 16) && out_row_bytes % 8 == 0) {
         // A workgroup takes 8 word columns and a slice of the features, 68 bytes of LDS per feature.  Measured:
@@ -1353,7 +1348,7 @@ extern "C" int dl_tensor_packbits_batch_major(const uint8_t *x, void *out, int64
         const int64_t want = dl_ceil_div(features, DL_PACK_MAX_SLICE / unit * unit);
         const int64_t slice = dl_ceil_div(dl_ceil_div(features, want), unit) * unit;
         const int64_t nslices = dl_ceil_div(features, slice);
-        const int64_t blocks = dl_ceil_div(dl_ceil_div(batch, 64), DL_PACK_WC) * nslices;
+        const int64_t blocks = dl_ceil_div(cols, DL_PACK_WC) * nslices;
         if (blocks > 0x3fffffffLL) return DL_ERR_TOO_LARGE;
         const size_t lds = (size_t) slice * DL_PACK_PITCH;
         const int64_t group = 8 * 2 * nslices;                   // pairs of column groups, one set per XCD
@@ -1371,6 +1366,25 @@ extern "C" int dl_tensor_packbits_batch_major(const uint8_t *x, void *out, int64
                            (uint8_t *) out, batch, features, out_row_bytes);
     }
     return dl_launch_status();
+}
+
+extern "C" int dl_tensor_packbits_batch_major(const uint8_t *x, void *out, int64_t batch, int64_t features,
+                                              int bit_count, int64_t *pad_len, void *stream) {
+    if (!valid_bit_count(bit_count)) return DL_ERR_BIT_COUNT;
+    if (features < 0 || batch < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (pad_len) *pad_len = (bit_count - batch % bit_count) % bit_count;
+    if (features == 0 || batch == 0) return DL_OK;
+    if (!x || !out) return DL_ERR_INVALID_ARGUMENT;
+    return pack_batch_major_rows(x, out, batch, features, dl_ceil_div(batch, bit_count) * (bit_count / 8),
+                                 (hipStream_t) stream);
+}
+
+extern "C" int dl_tensor_packbits_batch_major_rows(const uint8_t *x, void *out, int64_t batch, int64_t features,
+                                                   int64_t out_row_bytes, void *stream) {
+    if (features < 0 || batch < 0 || out_row_bytes < 0 || batch > 8 * out_row_bytes) return DL_ERR_INVALID_ARGUMENT;
+    if (features == 0 || out_row_bytes == 0) return DL_OK;
+    if (!out || (!x && batch > 0)) return DL_ERR_INVALID_ARGUMENT;
+    return pack_batch_major_rows(x, out, batch, features, out_row_bytes, (hipStream_t) stream);
 }
 
 extern "C" int dl_groupbitsum(const void *b, int32_t *out, int64_t in_dim, int64_t words, int bit_count,

@@ -101,7 +101,7 @@ class LogicLayer(torch.nn.Module):
                 return LogicLayerLogitsFunction.apply(x, a, b, self.weights, *tail,
                                                       self._train_schedule()).transpose(0, 1)
             w = torch.nn.functional.softmax(self.weights, dim=-1).to(x.dtype)
-            return LogicLayerCudaFunction.apply(x, a, b, w, *tail).transpose(0, 1)
+            return LogicLayerCudaFunction.apply(x, a, b, w, *tail, self._train_schedule()).transpose(0, 1)
         # eval mode: the discretised net on float inputs (no gradients)
         w = torch.nn.functional.one_hot(self.weights.argmax(-1), 16).to(x.dtype)
         with torch.no_grad():
@@ -185,25 +185,32 @@ class GroupSum(torch.nn.Module):
 class LogicLayerCudaFunction(torch.autograd.Function):
     """Feature-major forward/backward of one layer (difflogic/difflogic.py:205-221).  The
     optional trailing ``grad_factor`` is folded into backward_x instead of a separate
-    elementwise pass over the input gradient."""
+    elementwise pass over the input gradient; ``schedule`` (the layer's evaluation schedule) selects
+    the kernels that walk the wiring along its trails."""
 
     @staticmethod
-    def forward(ctx, x, a, b, w, given_x_indices_of_y_start, given_x_indices_of_y, grad_factor=1.0):
+    def forward(ctx, x, a, b, w, given_x_indices_of_y_start, given_x_indices_of_y, grad_factor=1.0, schedule=None):
         ctx.save_for_backward(x, a, b, w, given_x_indices_of_y_start, given_x_indices_of_y)
         ctx.grad_factor = grad_factor
-        return difflogic_cuda.forward(x, a, b, w)
+        ctx.schedule = schedule
+        return difflogic_cuda.forward(x, a, b, w, schedule)
 
     @staticmethod
     def backward(ctx, grad_y):
         x, a, b, w, given_x_indices_of_y_start, given_x_indices_of_y = ctx.saved_tensors
         grad_y = grad_y.contiguous()
         grad_w = grad_x = None
+        if ctx.needs_input_grad[0] and ctx.needs_input_grad[3] and ctx.schedule is not None:
+            # one pass along the schedule yields both gradients
+            both = difflogic_cuda.backward_chained(x, w, grad_y, ctx.schedule, ctx.grad_factor)
+            if both is not None:
+                return both[1], None, None, both[0], None, None, None, None
         if ctx.needs_input_grad[0]:
             grad_x = difflogic_cuda.backward_x(x, a, b, w, grad_y, given_x_indices_of_y_start,
                                                given_x_indices_of_y, ctx.grad_factor)
         if ctx.needs_input_grad[3]:
-            grad_w = difflogic_cuda.backward_w(x, a, b, grad_y)
-        return grad_x, None, None, grad_w, None, None, None
+            grad_w = difflogic_cuda.backward_w(x, a, b, grad_y, ctx.schedule)
+        return grad_x, None, None, grad_w, None, None, None, None
 
 
 class LogicLayerLogitsFunction(torch.autograd.Function):

@@ -123,8 +123,9 @@ def forward(x, a, b, w, schedule=None):
     return y
 
 
-def backward_w(x, a, b, grad_y):
-    """-> grad_w [out,16]   (difflogic.cpp:52-56)."""
+def backward_w(x, a, b, grad_y, schedule=None):
+    """-> grad_w [out,16]   (difflogic.cpp:52-56).  ``schedule`` selects the chained kernel
+    (bit-identical result in fp32 / fp64)."""
     for t, n in ((x, "x"), (a, "a"), (b, "b"), (grad_y, "grad_y")):
         _check_input(t, n)
     code = _float_code(x, "logic_layer_cuda_backward_w")
@@ -137,9 +138,17 @@ def backward_w(x, a, b, grad_y):
     dev = _same_device(x, a, b, grad_y)
     in_dim, batch = x.shape
     grad_w = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
+    lib = _lib.load()
     with _on(dev):
-        st = _lib.load().dl_logic_backward_w(_p(x), _p(a), _p(b), _p(grad_y), _p(grad_w), in_dim, out_dim, batch, code,
-                                             _stream(dev))
+        st = _lib.DL_ERR_TOO_LARGE
+        if schedule is not None and out_dim > 0 and batch > 0:
+            _check_schedule(schedule, in_dim, out_dim, dev)
+            st = lib.dl_logic_backward_w_chained(_p(x), _p(schedule.verts), _p(schedule.neuron), _p(schedule.flip),
+                                                 schedule.steps, _p(grad_y), None, _p(grad_w), in_dim, out_dim, batch,
+                                                 code, _stream(dev))
+        if st == _lib.DL_ERR_TOO_LARGE:
+            st = lib.dl_logic_backward_w(_p(x), _p(a), _p(b), _p(grad_y), _p(grad_w), in_dim, out_dim, batch, code,
+                                         _stream(dev))
     if st:
         _raise(st, "logic_layer_cuda_backward_w")
     return grad_w
@@ -470,6 +479,26 @@ def tensor_packbits_batch_major(x, bit_count):
     if st:
         _raise(st, "tensor_packbits_batch_major")
     return out, int(pad.value)
+
+
+def tensor_packbits_batch_major_rows(x, row_bytes):
+    """bool [B,F] (sample-major) -> int64 [F, row_bytes / 8]: the packing of
+    difflogic/packbitstensor.py:15-16 into rows of ``row_bytes`` bytes (a multiple of 8, at least
+    B bits); sample s is bit s % 64 of word s / 64, bits past the batch are zero.  The bytes are
+    those of int{8,16,32} words as well.  Not part of the reference's extension; PackBitsTensor
+    uses it."""
+    _check_input(x, "x")
+    if x.dtype != torch.bool or x.dim() != 2:
+        raise RuntimeError(f"expected x to be a 2-D bool tensor, got {x.dtype} with {x.dim()} dims")
+    batch, features = x.shape
+    if row_bytes % 8 or row_bytes * 8 < batch:
+        raise RuntimeError(f"row_bytes ({row_bytes}) has to be a multiple of 8 that holds {batch} bits")
+    out = torch.empty((features, row_bytes // 8), dtype=torch.int64, device=x.device)
+    with _on(x.device):
+        st = _lib.load().dl_tensor_packbits_batch_major_rows(_p(x), _p(out), batch, features, row_bytes, _stream(x.device))
+    if st:
+        _raise(st, "tensor_packbits_batch_major_rows")
+    return out
 
 
 def groupbitsum(b, pad_len, k):

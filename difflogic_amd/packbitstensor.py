@@ -113,38 +113,75 @@ class PackBitsTensor:
     Layers applied to the object are held back (``defer_layer``) until ``.t`` is read or
     ``group_sum`` is called; consecutive layers are then evaluated in fused groups (and the last
     group together with the bit count), so most intermediate activations never reach memory.
-    Reading ``.t`` always returns the up-to-date words, as in the reference."""
+    Reading ``.t`` always returns the up-to-date words, as in the reference.
+
+    Inside, a row is a little-endian bit stream padded with zeros to a multiple of 16 bytes and held
+    as int64 words: the same bytes as words of any of the four widths, so every batch size and word
+    width runs the same vector kernels.  ``.t`` is a view of those rows where their length allows
+    it and a copy cut to ``ceil(B / bit_count)`` words otherwise."""
 
     def __init__(self, t: torch.BoolTensor, bit_count=32, device="cuda"):
         assert len(t.shape) == 2, t.shape
         self.bit_count = bit_count
         self.device = device
-        self._t = None
         self._src = None              # the bool input [B, F] while it has not been packed yet
-        self._pending = []            # [(a, b, w)] applied to _t but not yet evaluated
+        self._rows = None             # int64 [features, 2 * ceil(B / 128)]: the padded rows
+        self._public = None           # what `.t` handed out or was set to, while it is current
+        self._pending = []            # [(a, b, w)] applied to the rows but not yet evaluated
         if device == "cuda":
             if bit_count not in (8, 16, 32, 64):
                 raise ValueError("`bit_count` has to be in { 8, 16, 32, 64 }")
             t = t.to(device)
+            self._batch = t.shape[0]
             self.pad_len = (bit_count - t.shape[0] % bit_count) % bit_count
             if t.dtype == torch.bool and t.is_contiguous():
                 # packed (transpose + pack in one kernel) when the words are first needed: a narrow net
                 # that runs resident in LDS reads the bool input itself
                 self._src = t
             else:
-                self._t, self.pad_len = difflogic_cuda.tensor_packbits_cuda(t.T.contiguous(), self.bit_count)
+                self._public, self.pad_len = difflogic_cuda.tensor_packbits_cuda(t.T.contiguous(), self.bit_count)
         else:
             raise NotImplementedError(device)
 
+    @staticmethod
+    def _row_bytes(batch):
+        return 16 * -(-batch // 128)
+
+    def _adopt(self, value):
+        """(rows, shared): ``value`` (words as `.t` shows them) as padded int64 rows; ``shared`` says
+        whether the rows are the same memory."""
+        bits = difflogic_cuda._WORD_BITS.get(value.dtype)
+        if bits is None or value.dim() != 2:
+            raise RuntimeError(f"expected 2-D integer words, got {value.dtype} with {value.dim()} dims")
+        row_bytes = value.shape[1] * bits // 8
+        if row_bytes % 16 == 0 and value.is_contiguous() and value.data_ptr() % 16 == 0:
+            return value.view(torch.int64), True
+        rows = torch.zeros((value.shape[0], 2 * -(-row_bytes // 16)), dtype=torch.int64, device=value.device)
+        rows.view(torch.uint8)[:, :row_bytes] = value.contiguous().view(torch.uint8)
+        return rows, False
+
     def _words(self):
-        """The packed input words, packing the bool input now if that has not happened yet."""
-        if self._t is None:
-            self._t, self.pad_len = difflogic_cuda.tensor_packbits_batch_major(self._src, self.bit_count)
-            self._src = None
-        return self._t
+        """The padded rows, packing the bool input now if that has not happened yet."""
+        if self._rows is not None:
+            return self._rows
+        if self._public is not None:
+            rows, shared = self._adopt(self._public)
+            if shared:
+                self._rows = rows
+            return rows               # a copy is not kept: writes into `.t` have to stay visible
+        self._rows = difflogic_cuda.tensor_packbits_batch_major_rows(self._src, self._row_bytes(self._batch))
+        self._src = None
+        return self._rows
+
+    def _pad(self, rows):
+        """Padding bits at the end of a padded row."""
+        return rows.shape[1] * 64 - self._batch
 
     def _in_features(self):
-        return self._src.shape[1] if self._t is None else self._t.shape[0]
+        for held in (self._rows, self._public):
+            if held is not None:
+                return held.shape[0]
+        return self._src.shape[1]
 
     @property
     def features(self):
@@ -153,33 +190,45 @@ class PackBitsTensor:
 
     def _words64(self):
         """Row length in 64-bit words (what the planner's byte counts are based on)."""
-        if self._t is None:
-            return max(1, -(-self._src.shape[0] // 64))
-        return max(1, self._t.shape[1] * self.bit_count // 64)
+        return max(1, self._row_bytes(self._batch) // 8)
 
     def _dims(self):
         return [self._in_features()] + [w.shape[0] for _, _, w in self._pending]
 
     def _run_groups(self, groups):
-        self._words()
+        rows = self._words()
         pos = 0
         for depth in groups:
             run = difflogic_cuda.eval_chained if _chained(depth) else difflogic_cuda.eval_fused
-            self._t = run(self._t, self._pending[pos:pos + depth])
+            rows = run(rows, self._pending[pos:pos + depth])
             pos += depth
+        if pos:
+            self._rows, self._public = rows, None
         self._pending = self._pending[pos:]
 
     @property
     def t(self):
         if self._pending:
             self._run_groups(plan_groups(self._dims(), False, self._words64()))
-        return self._words()
+        if self._public is None:
+            rows = self._words()
+            dtype = difflogic_cuda._BITS_TO_DTYPE[self.bit_count]
+            row_bytes = -(-self._batch // self.bit_count) * (self.bit_count // 8)
+            if row_bytes == rows.shape[1] * 8:
+                self._public = rows.view(dtype)
+            else:
+                self._public = rows.view(torch.uint8)[:, :row_bytes].contiguous().view(dtype)
+                self._rows = None     # the copy the caller holds is the state from here on
+        return self._public
 
     @t.setter
     def t(self, value):
         self._pending = []
         self._src = None
-        self._t = value
+        self._rows = None
+        self._public = value
+        bits = difflogic_cuda._WORD_BITS.get(value.dtype, self.bit_count)
+        self._batch = max(0, value.shape[1] * bits - self.pad_len)
 
     def defer_layer(self, a, b, w):
         """Applies the gate layer (a, b, w) lazily."""
@@ -196,25 +245,28 @@ class PackBitsTensor:
             if tail:
                 # the narrow end of the net runs resident in LDS; what lies before it streams
                 head = len(self._pending) - tail
-                if head == 0 and self._t is None:
+                if head == 0 and self._src is not None:
                     # the whole net, straight from the bool input: packing happens on the way into LDS
                     out = difflogic_cuda.eval_net_lds_bool(self._src, self._pending, k)
                     if out is not None:
                         return out
                 if head:
                     self._run_groups(plan_groups(dims[:head + 1], False, self._words64()))
-                out = difflogic_cuda.eval_net_lds(self._words(), self._pending, self.pad_len, k)
+                rows = self._words()
+                out = difflogic_cuda.eval_net_lds(rows, self._pending, self._pad(rows), k)
                 if out is not None:
                     return out
             groups = plan_groups(self._dims(), True, self._words64())
             self._run_groups(groups[:-1])
             # the last group stays pending: the object's state does not change by counting
-            out = difflogic_cuda.eval_chained_groupbitsum(self._words(), self._pending, self.pad_len, k)
+            rows = self._words()
+            out = difflogic_cuda.eval_chained_groupbitsum(rows, self._pending, self._pad(rows), k)
             if out is not None:
                 return out
-            order = difflogic_cuda.count_order_for(self._pending, self._t.shape[0], k)
-            return difflogic_cuda.eval_fused_groupbitsum(self._t, self._pending, self.pad_len, k, order)
-        return difflogic_cuda.groupbitsum(self._words(), self.pad_len, k)
+            order = difflogic_cuda.count_order_for(self._pending, rows.shape[0], k)
+            return difflogic_cuda.eval_fused_groupbitsum(rows, self._pending, self._pad(rows), k, order)
+        rows = self._words()
+        return difflogic_cuda.groupbitsum(rows, self._pad(rows), k)
 
     def flatten(self, start_dim=0, end_dim=-1, **kwargs):
         """Returns the object itself; the arguments are ignored."""

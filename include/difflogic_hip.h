@@ -285,6 +285,14 @@ int dl_tensor_packbits(const uint8_t *t, void *out, int64_t features, int64_t ba
 int dl_tensor_packbits_batch_major(const uint8_t *x, void *out, int64_t batch, int64_t features,
                                    int bit_count, int64_t *pad_len, void *stream);
 
+/* The same packing (difflogic/packbitstensor.py:15-16) into rows of a length the caller chooses:
+ *   out [features, out_row_bytes] bytes, 8 * out_row_bytes >= batch; sample s is bit s % 8 of byte
+ *   s / 8 of its feature's row (the memory image of little-endian words of any of the four widths),
+ *   every bit past the batch is zero.  PackBitsTensor uses it to keep rows a multiple of 16 bytes
+ *   whatever the batch size and word width, so that the gate kernels always run on whole vectors. */
+int dl_tensor_packbits_batch_major_rows(const uint8_t *x, void *out, int64_t batch, int64_t features,
+                                        int64_t out_row_bytes, void *stream);
+
 /* Replaces `groupbitsum` (difflogic.cpp:75-83, difflogic_kernel.cu:666-700), including the
  * final transpose.
  *   b [in_dim, words] words -> out [words*bit_count - pad_len, k] int32 (sample-major):

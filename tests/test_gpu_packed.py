@@ -60,6 +60,62 @@ def test_packbits_batch_major(ext, bits, B, F):
     assert torch.equal(got, two)
 
 
+@pytest.mark.parametrize("B,F,row_bytes", [(1, 1, 16), (7, 3, 8), (64, 8, 16), (65, 12, 16), (1000, 7, 128), (1000, 16, 144),
+                                            (1000, 784, 128), (4112, 260, 528), (130, 1028, 32), (700, 9216, 96),
+                                            (513, 16, 80), (0, 5, 16), (8200, 48, 1040), (129, 1648, 2064)])
+def test_packbits_batch_major_rows(ext, B, F, row_bytes):
+    """Rows longer than the batch needs: the bits are where tensor_packbits_cuda puts them, the rest is zero
+    (the output buffer starts out as ones)."""
+    rng = np.random.default_rng(F * 131 + B + row_bytes)
+    x = rng.random((B, F)) < 0.3
+    want = np.zeros((F, row_bytes), np.uint8)
+    want[:, :-(-B // 8)] = np.packbits(x.T, axis=1, bitorder="little")
+    got = ext.tensor_packbits_batch_major_rows(_dev(x), row_bytes)
+    assert got.dtype == torch.int64 and tuple(got.shape) == (F, row_bytes // 8)
+    assert np.array_equal(got.cpu().numpy().view(np.uint8), want)
+    with pytest.raises(RuntimeError):
+        ext.tensor_packbits_batch_major_rows(_dev(x), 8 * ((B - 1) // 64))  # too short
+
+
+@pytest.mark.parametrize("bits", [8, 16, 32, 64])
+@pytest.mark.parametrize("B", [1, 37, 64, 100, 128, 200, 1000, 1024 + 96])
+def test_pack_tensor_every_width_and_batch(bits, B):
+    """PackBitsTensor keeps padded rows inside; `.t`, `.pad_len` and the counts are the reference's for every
+    word width and batch size, before, between and after layers, and writes into `.t` are seen."""
+    import difflogic_amd as dl
+    rng = np.random.default_rng(B * 4 + bits)
+    layers = random_layers(rng, 24, [48, 48, 30])
+    x = rng.random((B, 24)) < 0.5
+    model = build_model(24, layers, 3).eval()
+    logic = [m for m in model if isinstance(m, dl.LogicLayer)]
+    want_t, want_pad = po.packbits(x.T, bits)
+    p = dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=bits)
+    assert p.pad_len == want_pad and p.features == 24
+    assert p.t.dtype == torch.as_tensor(want_t).dtype and np.array_equal(p.t.cpu().numpy(), want_t)
+    assert p.t.is_contiguous() and p.t is p.t
+    assert np.array_equal(p.group_sum(3).cpu().numpy(), po.groupbitsum(want_t, want_pad, 3))
+    with torch.no_grad():
+        p = logic[0](p)
+    t1 = po.eval_layer(want_t, *layers[0])
+    assert np.array_equal(p.t.cpu().numpy(), t1)
+    with torch.no_grad():
+        p = logic[2](logic[1](p))
+    t3 = po.eval_layer(po.eval_layer(t1, *layers[1]), *layers[2])
+    assert np.array_equal(p.group_sum(3).cpu().numpy(), po.groupbitsum(t3, want_pad, 3))     # last layers still deferred
+    assert np.array_equal(p.t.cpu().numpy(), t3) and p.features == 30
+    assert np.array_equal(p.group_sum(3).cpu().numpy(), po.groupbitsum(t3, want_pad, 3))
+    p.t.zero_()                                                                              # in place, through `.t`
+    assert int(p.group_sum(3).sum()) == 0
+    p.t = torch.as_tensor(t1).cuda()                                                         # assigned
+    with torch.no_grad():
+        got = logic[2](logic[1](p)).group_sum(3)
+    assert np.array_equal(got.cpu().numpy(), po.groupbitsum(t3, want_pad, 3))
+    # the whole model at once (no `.t` read in between) against the bitwise oracle
+    with torch.no_grad():
+        got = model(dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=bits))
+    assert np.array_equal(got.cpu().numpy(), po.net_eval_bitwise(x, layers, 3))
+
+
 def test_packbits_batch_major_nonzero_bytes(ext):
     raw = torch.tensor([[0, 1, 2, 128], [255, 0, 7, 0], [3, 3, 0, 0]], dtype=torch.uint8).cuda()
     got, _ = ext.tensor_packbits_batch_major(raw.view(torch.bool), 8)

@@ -470,17 +470,24 @@ def test_chained_layer_matches_the_python_formulation_on_random_wirings(monkeypa
         assert ok, (tag, rep)
 
 
+@pytest.mark.parametrize("along_schedule", [False, True])
 @pytest.mark.parametrize("dtype,rtol", [(torch.float16, 4e-3), (torch.float64, 1e-5)])
-def test_layer_module_with_half_and_double_activations(dtype, rtol):
+def test_layer_module_with_half_and_double_activations(dtype, rtol, along_schedule, monkeypatch):
     """The reference's --training-bit-count 16 / 64 (experiments/main.py:19-23,286): the input is
     cast to half / double while the weights stay fp32, so LogicLayer takes the
     softmax-in-torch + LogicLayerCudaFunction route (difflogic/difflogic.py:123-126,205-221).
     Outputs and both gradients against the same formulation on CPU (fp64 arithmetic on the
-    values as rounded to ``dtype``, the fp32 softmax and the casts as autograd sees them)."""
+    values as rounded to ``dtype``, the fp32 softmax and the casts as autograd sees them).
+    ``along_schedule``: the layer counts as wide, so the same route runs the kernels that walk the
+    wiring along its trails (forward, and both gradients in one pass)."""
     import difflogic_amd as dl
+    if along_schedule:
+        monkeypatch.setattr(dl.LogicLayer, "_CHAIN_MIN_IN_DIM", 0)
+        monkeypatch.setattr(dl.LogicLayer, "_CHAIN_MIN_OUT_DIM", 0)
     torch.manual_seed(5)
     in_dim, out_dim, batch = 48, 120, 264
     layer = dl.LogicLayer(in_dim, out_dim, grad_factor=1.5).train()
+    assert (layer._train_schedule() is not None) == along_schedule
     a, b = layer.indices[0].cpu(), layer.indices[1].cpu()
     g = torch.Generator().manual_seed(6)
     x = torch.rand(batch, in_dim, generator=g).to(dtype)
