@@ -63,7 +63,7 @@ def parse():
     ap.add_argument("--features", type=int, default=784)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-train", action="store_true", help="skip the training configurations (C1, C3, C5)")
-    ap.add_argument("--no-configs", action="store_true", help="skip the other packed configurations (C2, C4)")
+    ap.add_argument("--no-configs", action="store_true", help="skip the other packed configurations (C2, C4, other word widths)")
     ap.add_argument("--only", default="", help="comma list out of c1,c2,c3,c4,c5: run only these extra configurations")
     ap.add_argument("--skip-headline", action="store_true",
                     help="profiling aid: run only the configurations selected with --only and print their results")
@@ -269,8 +269,9 @@ def packed_headline(args, torch, dl):
         "path_alg_GBps": round(total_alg / (ms_per_step * 1e-3) / 1e9, 1),
         "first_call_ms": round(first_ms, 1),
         "checksum": int(out.sum().item()),
-        "other_word_widths": word_width_variants(torch, dl, model, x, out),
     }
+    if not args.no_configs:
+        info["other_word_widths"] = word_width_variants(torch, dl, model, x, out)
     return value, ms_per_step, roofline, info, model, x, out
 
 
