@@ -70,6 +70,9 @@ def parse():
     ap.add_argument("--cpu-sample-log2", type=int, default=18)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 4 plain device copies of 1 GiB (for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE)")
+    ap.add_argument("--cpu-generated-c", action="store_true",
+                    help="also time the reference's own CPU inference path on the host: the generated C of the headline "
+                         "net and of C2, gcc-compiled as experiments/main.py:362 does (minutes of compile time)")
     ap.add_argument("--ceilings", action="store_true",
                     help="measure streaming read/write/copy and row-gather ceilings instead of the benchmark")
     return ap.parse_args()
@@ -317,11 +320,54 @@ def cpu_baseline(args, model, x, out, dl):
     dt = time.perf_counter() - t0
     got = out[:n].cpu().numpy()
     return {"value": round(n / dt, 1), "unit": "samples/s", "cores": 1, "kind": "port",
-            "sample": "first %d of %d samples, same net; oracle/c/packed_interp.c, 1 thread, %.1f s" % (n, x.shape[0], dt),
+            "sample": "first %d of %d samples, same net; oracle/c/packed_interp.c, 1 thread, %.1f s (the reference's "
+                      "generated C itself: --cpu-generated-c, minutes of gcc)" % (n, x.shape[0], dt),
             "gpu_matches_cpu_on_sample": bool((got == want).all())}
 
 
-def packed_config(torch, dl, name, F, widths, B, x, check_cpu):
+def cpu_generated_c(model, x, out, dl, sample_log2=16):
+    """The reference's CPU inference path for `model` on this host: the C text CompiledLogicNet generates
+    (difflogic/compiled_model.py:159-239, restated by oracle/cgen.py), compiled the way the reference's
+    driver does (experiments/main.py:362: gcc -O1 below 50 000 gates, else -O0), 64-bit words, one thread,
+    the whole apply_logic_gate_net call (bool packing, gates, adders) on the first 2^sample_log2 samples."""
+    import subprocess
+    import tempfile
+    from oracle import cgen
+    layers = net_tables(model, dl)
+    gates = sum(len(l[2]) for l in layers)
+    opt = 1 if gates < 50000 else 0
+    work = tempfile.mkdtemp(prefix="dl_bench_cgen_")
+    c_path, so_path = os.path.join(work, "net.c"), os.path.join(work, "net.so")
+    with open(c_path, "w") as f:
+        f.write(cgen.generate_c(layers, x.shape[1], 10, 64))
+    t0 = time.perf_counter()
+    proc = subprocess.Popen(["gcc", "-shared", "-fPIC", "-O%d" % opt, "-o", so_path, c_path])
+    while proc.poll() is None:
+        try:
+            proc.wait(timeout=30)
+        except subprocess.TimeoutExpired:
+            print("bench.py: gcc -O%d on %d gates, %.0f s so far" % (opt, gates, time.perf_counter() - t0),
+                  file=sys.stderr, flush=True)
+    if proc.returncode:
+        return {"error": "gcc exited with %d" % proc.returncode}
+    compile_s = time.perf_counter() - t0
+    fn = cgen.load_apply_fn(so_path)
+    n = min(1 << sample_log2, x.shape[0])
+    xs = x[:n].cpu().numpy()
+    cgen.call_apply_fn(fn, xs[:64], 10, 64)
+    t0 = time.perf_counter()
+    want = cgen.call_apply_fn(fn, xs, 10, 64)
+    dt = time.perf_counter() - t0
+    for path in (c_path, so_path):
+        os.remove(path)
+    os.rmdir(work)
+    return {"value": round(n / dt, 1), "unit": "samples/s", "cores": 1, "kind": "reference's generated C (restated text)",
+            "gates": gates, "compiler": "gcc -shared -fPIC -O%d" % opt, "compile_s": round(compile_s, 1),
+            "sample": "first %d samples, %.1f s" % (n, dt),
+            "gpu_matches_cpu_on_sample": bool((out[:n].cpu().numpy() == want).all())}
+
+
+def packed_config(torch, dl, name, F, widths, B, x, check_cpu, generated_c=False):
     """One of the other packed configurations: samples/s, per-launch times, and the first 4096
     samples of the full-batch result compared with the CPU interpreter."""
     k = 10
@@ -343,6 +389,8 @@ def packed_config(torch, dl, name, F, widths, B, x, check_cpu):
         dt = time.perf_counter() - t0
         res["bit_exact_vs_cpu_interpreter"] = {"samples": n, "equal": bool((out[:n].cpu().numpy() == want).all()),
                                                "cpu_samples_per_s": round(n / dt, 1)}
+    if generated_c:
+        res["cpu_generated_c"] = cpu_generated_c(model, x, out, dl)
     del model, out
     return res
 
@@ -633,7 +681,8 @@ def extra_configs(args, torch, dl):
     if want("c2", args.no_configs):
         B = 1 << 20
         configs["C2"] = packed_config(torch, dl, "packed inference 784->6x8000->GroupSum(10), batch 2^20, int64 words",
-                                      784, [8000] * 6, B, bernoulli_input(torch, B, 784, 1), check)
+                                      784, [8000] * 6, B, bernoulli_input(torch, B, 784, 1), check,
+                                      generated_c=args.cpu_generated_c)
         torch.cuda.empty_cache()
     if want("c4", args.no_configs):
         B = 1 << 18
@@ -712,6 +761,8 @@ def main():
     }
     result["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(args, model, x, out, dl)
     extra = dict(info)
+    if args.cpu_generated_c:
+        extra["cpu_generated_c"] = cpu_generated_c(model, x, out, dl)
     del model, x, out
     gc.collect()
     torch.cuda.empty_cache()
