@@ -196,12 +196,27 @@ def packed_run(torch, dl, model, x, k, steps, warmup):
             setattr(ext, n, real[n])
         record["on"] = False
 
+    # the same step captured once into a HIP graph and replayed (difflogic_amd.graphs.GraphedPackedInference;
+    # the batch sits in the graph's static input buffer, as the eager step's sits in x)
+    from difflogic_amd.graphs import GraphedPackedInference
+    graphed = GraphedPackedInference(model, x, bit_count=64)
+    graphed()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        replayed = graphed()
+    torch.cuda.synchronize()
+    graph_ms = (time.perf_counter() - t0) / steps * 1e3
+    graph_info = {"ms_per_step": round(graph_ms, 4), "samples_per_s": round(B / graph_ms * 1e3, 1),
+                  "equal_to_eager": bool(torch.equal(replayed, out))}
+    del graphed, replayed
+
     per_kernel = {}
     for label, by, s, e in launches:
         d = per_kernel.setdefault(label, {"n": 0, "ms": 0.0, "bytes": by})
         d["n"] += 1
         d["ms"] += s.elapsed_time(e)
-    return B * steps / elapsed, elapsed / steps * 1e3, per_kernel, out, first_call_ms
+    return B * steps / elapsed, elapsed / steps * 1e3, per_kernel, out, first_call_ms, graph_info
 
 
 def kernel_table(per_kernel, steps):
@@ -232,7 +247,7 @@ def packed_headline(args, torch, dl):
     B = 1 << args.batch_log2
     model = packed_model(torch, dl, F, [width] * L, k)
     x = bernoulli_input(torch, B, F, 1)
-    value, ms_per_step, per_kernel, out, first_ms = packed_run(torch, dl, model, x, k, args.steps, args.warmup)
+    value, ms_per_step, per_kernel, out, first_ms, graph_info = packed_run(torch, dl, model, x, k, args.steps, args.warmup)
 
     # dominant kernel = the launch kind that takes the most time in a step
     dom = max(per_kernel, key=lambda kk: per_kernel[kk]["ms"])
@@ -271,6 +286,7 @@ def packed_headline(args, torch, dl):
         "path_algorithmic_GB_per_step": round(total_alg / 1e9, 2),
         "path_alg_GBps": round(total_alg / (ms_per_step * 1e-3) / 1e9, 1),
         "first_call_ms": round(first_ms, 1),
+        "hip_graph_replay": graph_info,
         "checksum": int(out.sum().item()),
     }
     if not args.no_configs:
@@ -372,14 +388,14 @@ def packed_config(torch, dl, name, F, widths, B, x, check_cpu, generated_c=False
     samples of the full-batch result compared with the CPU interpreter."""
     k = 10
     model = packed_model(torch, dl, F, widths, k)
-    value, ms, per_kernel, out, first_ms = packed_run(torch, dl, model, x, k, steps=5, warmup=2)
+    value, ms, per_kernel, out, first_ms, graph_info = packed_run(torch, dl, model, x, k, steps=5, warmup=2)
     W = B // 64
     dims = [F] + list(widths)
     alg = sum(eval_layer_bytes(i, o, W) for i, o in zip(dims[:-1], dims[1:])) + 8 * W * dims[-1] + 4 * k * B
     res = {"workload": name, "dtype": "int64", "samples_per_s": round(value, 1), "ms_per_step": round(ms, 4),
            "algorithmic_GB_per_step_without_pack": round(alg / 1e9, 2),
            "alg_over_peak": round(alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-           "first_call_ms": round(first_ms, 1), "kernels": kernel_table(per_kernel, 5),
+           "first_call_ms": round(first_ms, 1), "hip_graph_replay": graph_info, "kernels": kernel_table(per_kernel, 5),
            "checksum": int(out.sum().item())}
     if check_cpu:
         from oracle import interp

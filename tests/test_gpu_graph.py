@@ -106,3 +106,37 @@ def test_graphed_step_of_the_fused_model_equals_its_eager_step(monkeypatch):
         assert torch.equal(loss_g, loss_e.detach()), rep
         for pg, pe in zip(model.parameters(), eager.parameters()):
             assert pg.grad is not None and torch.equal(pg.grad, pe.grad), rep
+
+
+@pytest.mark.parametrize("F,widths,k,B", [(64, [512, 512, 320], 10, 1000), (784, [12000, 12000, 12000], 10, 4096),
+                                          (48, [96, 48], 4, 77), (784, [40000, 40000], 10, 1024)])
+def test_graphed_packed_inference_equals_eager_on_every_replay(F, widths, k, B):
+    """Packing, gate layers and count captured once (the narrow nets run resident in LDS, the wide ones
+    stream) and replayed on new batches, with eager work and synchronisation between the replays; every
+    replay equals the eager result and the bitwise oracle.  Gate weights changed in place are picked up."""
+    import numpy as np
+    import difflogic_amd as dl
+    from difflogic_amd.graphs import GraphedPackedInference
+    from oracle import interp
+    from tests.helpers import build_model, random_layers
+    rng = np.random.default_rng(F + B)
+    layers = random_layers(rng, F, widths)
+    model = build_model(F, layers, k).eval()
+    xs = [torch.as_tensor(rng.random((B, F)) < p).cuda() for p in (0.2, 0.5, 0.8, 0.35)]
+    graphed = GraphedPackedInference(model, xs[0], bit_count=32)
+    for i, x in enumerate(xs):
+        got = graphed(x).clone()
+        with torch.no_grad():
+            eager = model(dl.PackBitsTensor(x, bit_count=32))
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), i
+        if B <= 1024 or i == 0:
+            assert np.array_equal(got.cpu().numpy(), interp.net_eval(x.cpu().numpy(), layers, k)), i
+    # another gate table in the same storage: the graph reads the weights at replay time
+    last = [m for m in model if isinstance(m, dl.LogicLayer)][-1]
+    with torch.no_grad():
+        last.weights.copy_(torch.randn_like(last.weights))
+    got = graphed(xs[1]).clone()
+    with torch.no_grad():
+        eager = model(dl.PackBitsTensor(xs[1], bit_count=32))
+    assert torch.equal(got, eager)
