@@ -315,6 +315,33 @@ __global__ __launch_bounds__(DL_BLOCK) void eval_chain_kernel(const V *__restric
 // subtree tables, neuron -> gate id, flip), and every gather is a scalar row base plus the lane's
 // constant 32-bit offset.  Applies when rows * row length and out_dim * row length fit 32 bits.
 // ------------------------------------------------------------------------------------------
+// Inputs a gate does not look at.  A gate id is the truth table (f(0,0) f(0,1) f(1,0) f(1,1)), MSB first; six of
+// the sixteen ignore an input (constants, a, b, not a, not b).  Whatever feeds an ignored input cannot change the
+// result, so the kernels that evaluate trees of gates per output do not fetch it: with uniformly drawn gates a
+// leaf three gates below its root is needed with probability 0.75^3.
+__host__ __device__ __forceinline__ bool gate_uses_a(uint32_t op) {
+    return (((op >> 3) ^ (op >> 1)) & 1u) || (((op >> 2) ^ op) & 1u);
+}
+__host__ __device__ __forceinline__ bool gate_uses_b(uint32_t op) {
+    return (((op >> 3) ^ (op >> 2)) & 1u) || (((op >> 1) ^ op) & 1u);
+}
+
+// Bit g set: leaf g of a depth-D subtree reaches its root (gates packed as TreeFold reads them).
+template <int D> struct LiveLeaves {
+    static __host__ __device__ __forceinline__ uint32_t of(uint64_t gates) {
+        constexpr int half = 1 << (D - 1);
+        const uint32_t top = (uint32_t) (gates >> (4 * (2 * half - 2))) & 15u;
+        const uint32_t left = gate_uses_a(top) ? LiveLeaves<D - 1>::of(gates) : 0u;
+        const uint32_t right = gate_uses_b(top) ? LiveLeaves<D - 1>::of(gates >> (4 * (half - 1))) : 0u;
+        return left | (right << half);
+    }
+};
+template <> struct LiveLeaves<0> {
+    static __host__ __device__ __forceinline__ uint32_t of(uint64_t) { return 1u; }
+};
+
+#define DL_STEP_DEAD 0xffffffffu        // leaf of a step record that no gate looks at: not fetched
+
 template <int DS> struct alignas(DS == 3 ? 64 : DS == 2 ? 32 : 16) StepRec {
     uint32_t leaf[1 << DS];
     uint32_t gates;
@@ -336,20 +363,31 @@ __global__ __launch_bounds__(DL_BLOCK) void compose_steps_kernel(const int32_t *
     const int64_t v = verts[i];
     StepRec<DS> r;
     uint32_t gates = 0;
-    if (DS == 0) {
-        r.leaf[0] = (uint32_t) v * ncols;
-    } else {
-        gates = (uint32_t) sub_gates[v];
-#pragma unroll
-        for (int g = 0; g < (1 << DS); ++g) r.leaf[g] = (uint32_t) sub_leaves[v * (1 << DS) + g] * ncols;
-    }
     r.out = 0xffffffffu;
+    // the vertex is the second input of step i - 1's neuron and the first input of step i's
+    bool needed = false;
     if (i >= 1 && neuron[i - 1] >= 0) {
         const int32_t n = neuron[i - 1];
         uint32_t top = w_top[n] & 15u;
         if (flip[i - 1]) top = swap_gate_inputs(top);
         gates |= top << 28;
         r.out = (uint32_t) n * ncols;
+        needed = gate_uses_b(top);
+    }
+    if (i < steps && neuron[i] >= 0) {
+        uint32_t next = w_top[neuron[i]] & 15u;
+        if (flip[i]) next = swap_gate_inputs(next);
+        needed = needed || gate_uses_a(next);
+    }
+    if (DS == 0) {
+        r.leaf[0] = needed ? (uint32_t) v * ncols : DL_STEP_DEAD;
+    } else {
+        const uint64_t sub = sub_gates[v];
+        gates |= (uint32_t) sub;
+        const uint32_t live = needed ? LiveLeaves<DS>::of(sub) : 0u;
+#pragma unroll
+        for (int g = 0; g < (1 << DS); ++g)
+            r.leaf[g] = (live >> g) & 1u ? (uint32_t) sub_leaves[v * (1 << DS) + g] * ncols : DL_STEP_DEAD;
     }
     r.gates = gates;
     rec[i] = r;
@@ -374,6 +412,7 @@ __global__ __launch_bounds__(DL_BLOCK) void eval_steps_kernel(const V *__restric
         const uint32_t col = (uint32_t) (ct * DL_WAVE) + (uint32_t) lane;
         if (col >= ncols) continue;
         auto row = [&](uint32_t start) -> V {                                  // scalar row base + the lane's offset
+            if (start == DL_STEP_DEAD) return V{};                             // (wave-uniform) no gate looks at this row
             if constexpr (BUF && sizeof(V) == 16) {
                 const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *) x, 0, (int) x_bytes, 0x00027000);
                 return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int) (col * 16u), (int) (start * 16u), 0));
@@ -940,6 +979,9 @@ __global__ __launch_bounds__(DL_BLOCK) void compose_count_chain_kernel(TreeTable
         la = (uint32_t) v;
     }
     uint32_t where = 255;
+    // the vertex is the second input of step i - 1's neuron and the first input of step i's; rows that no gate
+    // looks at are not fetched (.w: bit 0 = skip la, bit 1 = skip lb)
+    bool needed = false;
     if (i >= 1) {
         const int64_t s = i - 1;
         where = slot[s];
@@ -947,9 +989,18 @@ __global__ __launch_bounds__(DL_BLOCK) void compose_count_chain_kernel(TreeTable
             uint32_t top = t.w[DS][neuron[s]] & 15u;
             if (flip[s]) top = swap_gate_inputs(top);
             bits |= top << 4;
+            needed = gate_uses_b(top);
         }
     }
-    rec[i] = dl_u32x4{la, lb, bits | (where << 8), 0u};
+    if (i < steps && neuron[i] >= 0) {
+        uint32_t next = t.w[DS][neuron[i]] & 15u;
+        if (flip[i]) next = swap_gate_inputs(next);
+        needed = needed || gate_uses_a(next);
+    }
+    uint32_t skip = 0;
+    if (!needed || (DS == 1 && !gate_uses_a(bits & 15u))) skip |= 1u;
+    if (DS == 1 && (!needed || !gate_uses_b(bits & 15u))) skip |= 2u;
+    rec[i] = dl_u32x4{la, lb, bits | (where << 8), skip};
 }
 
 template <typename V, int DS, int CPW>
@@ -975,8 +1026,8 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
     V prev;
     {
         const dl_u32x4 r = wrec[0];
-        const V ra = xcol[(int64_t) r.x * ncols];
-        const V rb = DS == 1 ? xcol[(int64_t) r.y * ncols] : ra;
+        const V ra = (r.w & 1u) ? Words<V>::zero() : xcol[(int64_t) r.x * ncols];
+        const V rb = DS != 1 ? ra : (r.w & 2u) ? Words<V>::zero() : xcol[(int64_t) r.y * ncols];
         prev = vertex(ra, rb, r.z);
     }
     V cnt[CPW][DL_CC_PLANES];
@@ -997,8 +1048,9 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
 #pragma unroll
             for (int j = 0; j < BATCH; ++j) {
                 r[j] = wrec[1 + b * DL_CC_WAVE_STEPS + h + j];
-                ra[j] = xcol[(int64_t) r[j].x * ncols];
-                if (DS == 1) rb[j] = xcol[(int64_t) r[j].y * ncols];
+                // (wave-uniform flags: rows that no gate looks at are not fetched)
+                ra[j] = (r[j].w & 1u) ? Words<V>::zero() : xcol[(int64_t) r[j].x * ncols];
+                if (DS == 1) rb[j] = (r[j].w & 2u) ? Words<V>::zero() : xcol[(int64_t) r[j].y * ncols];
             }
 #pragma unroll
             for (int j = 0; j < BATCH; ++j) {
