@@ -110,6 +110,32 @@ __global__ __launch_bounds__(DL_BLOCK) void eval_kernel(const V *__restrict__ x,
 // ------------------------------------------------------------------------------------------
 #define DL_MAX_FUSE_DEPTH 4
 
+// Inputs a gate does not look at.  A gate id is the truth table (f(0,0) f(0,1) f(1,0) f(1,1)), MSB first; six of
+// the sixteen ignore an input (constants, a, b, not a, not b).  Whatever feeds an ignored input cannot change the
+// result, so the kernels that evaluate trees of gates per output do not fetch it: with uniformly drawn gates a
+// leaf three gates below its root is needed with probability 0.75^3.
+__host__ __device__ __forceinline__ bool gate_uses_a(uint32_t op) {
+    return (((op >> 3) ^ (op >> 1)) & 1u) || (((op >> 2) ^ op) & 1u);
+}
+__host__ __device__ __forceinline__ bool gate_uses_b(uint32_t op) {
+    return (((op >> 3) ^ (op >> 2)) & 1u) || (((op >> 1) ^ op) & 1u);
+}
+
+// Bit g set: leaf g of a depth-D subtree reaches its root (gates packed as TreeFold reads them).
+template <int D> struct LiveLeaves {
+    static __host__ __device__ __forceinline__ uint32_t of(uint64_t gates) {
+        constexpr int half = 1 << (D - 1);
+        const uint32_t top = (uint32_t) (gates >> (4 * (2 * half - 2))) & 15u;
+        const uint32_t left = gate_uses_a(top) ? LiveLeaves<D - 1>::of(gates) : 0u;
+        const uint32_t right = gate_uses_b(top) ? LiveLeaves<D - 1>::of(gates >> (4 * (half - 1))) : 0u;
+        return left | (right << half);
+    }
+};
+template <> struct LiveLeaves<0> {
+    static __host__ __device__ __forceinline__ uint32_t of(uint64_t) { return 1u; }
+};
+
+
 struct TreeTables {
     const int64_t *a[DL_MAX_FUSE_DEPTH];   // [0] = first (lowest) layer of the group
     const int64_t *b[DL_MAX_FUSE_DEPTH];
@@ -146,8 +172,9 @@ __global__ __launch_bounds__(DL_BLOCK) void compose_tree_kernel(TreeTables t, co
 #pragma unroll
         for (int i = 0; i < (2 << r); ++i) nodes[i] = next[i];
     }
+    const uint32_t live = LiveLeaves<D>::of(packed);   // a row that no gate looks at is not fetched: id -1
 #pragma unroll
-    for (int i = 0; i < (1 << D); ++i) leaves[n * (1 << D) + i] = (int32_t) nodes[i];
+    for (int i = 0; i < (1 << D); ++i) leaves[n * (1 << D) + i] = (live >> i) & 1u ? (int32_t) nodes[i] : -1;
     gates[n] = packed;
 }
 
@@ -195,7 +222,7 @@ __global__ __launch_bounds__(DL_BLOCK) void eval_tree_kernel(const V *__restrict
 #pragma unroll
                 for (int j = 0; j < NPW; ++j) {
 #pragma unroll
-                    for (int g = 0; g < G; ++g) v[j][g] = x[(int64_t) id[j][g] * ncols + col];
+                    for (int g = 0; g < G; ++g) v[j][g] = id[j][g] < 0 ? V{} : x[(int64_t) id[j][g] * ncols + col];
                 }
 #pragma unroll
                 for (int j = 0; j < NPW; ++j) {
@@ -229,7 +256,7 @@ template <typename V, int DS> struct Subtree {
     }
     __device__ __forceinline__ void gather(const V *__restrict__ xcol, int64_t ncols, V *v) const {
 #pragma unroll
-        for (int g = 0; g < (1 << DS); ++g) v[g] = xcol[(int64_t) leaf[g] * ncols];
+        for (int g = 0; g < (1 << DS); ++g) v[g] = leaf[g] < 0 ? V{} : xcol[(int64_t) leaf[g] * ncols];
     }
 };
 template <typename V> struct Subtree<V, 0> {
@@ -315,38 +342,52 @@ __global__ __launch_bounds__(DL_BLOCK) void eval_chain_kernel(const V *__restric
 // subtree tables, neuron -> gate id, flip), and every gather is a scalar row base plus the lane's
 // constant 32-bit offset.  Applies when rows * row length and out_dim * row length fit 32 bits.
 // ------------------------------------------------------------------------------------------
-// Inputs a gate does not look at.  A gate id is the truth table (f(0,0) f(0,1) f(1,0) f(1,1)), MSB first; six of
-// the sixteen ignore an input (constants, a, b, not a, not b).  Whatever feeds an ignored input cannot change the
-// result, so the kernels that evaluate trees of gates per output do not fetch it: with uniformly drawn gates a
-// leaf three gates below its root is needed with probability 0.75^3.
-__host__ __device__ __forceinline__ bool gate_uses_a(uint32_t op) {
-    return (((op >> 3) ^ (op >> 1)) & 1u) || (((op >> 2) ^ op) & 1u);
-}
-__host__ __device__ __forceinline__ bool gate_uses_b(uint32_t op) {
-    return (((op >> 3) ^ (op >> 2)) & 1u) || (((op >> 1) ^ op) & 1u);
-}
-
-// Bit g set: leaf g of a depth-D subtree reaches its root (gates packed as TreeFold reads them).
-template <int D> struct LiveLeaves {
-    static __host__ __device__ __forceinline__ uint32_t of(uint64_t gates) {
+// Bit j set: the gate in nibble j of a depth-D subtree's packed gates feeds its root (`alive`: the root does).
+template <int D> struct LiveGates {
+    static __host__ __device__ __forceinline__ uint32_t of(uint64_t gates, bool alive) {
+        if (!alive) return 0u;
         constexpr int half = 1 << (D - 1);
         const uint32_t top = (uint32_t) (gates >> (4 * (2 * half - 2))) & 15u;
-        const uint32_t left = gate_uses_a(top) ? LiveLeaves<D - 1>::of(gates) : 0u;
-        const uint32_t right = gate_uses_b(top) ? LiveLeaves<D - 1>::of(gates >> (4 * (half - 1))) : 0u;
-        return left | (right << half);
+        return (1u << (2 * half - 2)) | LiveGates<D - 1>::of(gates, gate_uses_a(top)) |
+               (LiveGates<D - 1>::of(gates >> (4 * (half - 1)), gate_uses_b(top)) << (half - 1));
     }
 };
-template <> struct LiveLeaves<0> {
-    static __host__ __device__ __forceinline__ uint32_t of(uint64_t) { return 1u; }
+template <> struct LiveGates<0> {
+    static __host__ __device__ __forceinline__ uint32_t of(uint64_t, bool) { return 0u; }
 };
 
 #define DL_STEP_DEAD 0xffffffffu        // leaf of a step record that no gate looks at: not fetched
 
-template <int DS> struct alignas(DS == 3 ? 64 : DS == 2 ? 32 : 16) StepRec {
+// records of subtrees with more than one gate also say which gates are worth evaluating (LiveGates)
+template <int DS> struct StepLive {};
+template <> struct StepLive<2> { uint32_t live; };
+template <> struct StepLive<3> { uint32_t live; };
+
+template <int DS> struct alignas(DS == 3 ? 64 : DS == 2 ? 32 : 16) StepRec : StepLive<DS> {
     uint32_t leaf[1 << DS];
     uint32_t gates;
     uint32_t out;
 };
+
+// TreeFold that leaves out the gates nobody looks at (`live` as LiveGates numbers them; wave-uniform branches)
+template <typename V, int D> struct TreeFoldLive {
+    static __device__ __forceinline__ V run(const V *leaf, uint32_t gates, uint32_t live) {
+        constexpr int half = 1 << (D - 1);
+        if (!((live >> (2 * half - 2)) & 1u)) return V{};
+        const V l = TreeFoldLive<V, D - 1>::run(leaf, gates, live);
+        const V r = TreeFoldLive<V, D - 1>::run(leaf + half, gates >> (4 * (half - 1)), live >> (half - 1));
+        return gate_apply<V>(l, r, gate_masks((gates >> (4 * (2 * half - 2))) & 15u));
+    }
+};
+template <typename V> struct TreeFoldLive<V, 0> {
+    static __device__ __forceinline__ V run(const V *leaf, uint32_t, uint32_t) { return leaf[0]; }
+};
+
+// the subtree value of a step record
+template <typename V, int DS> __device__ __forceinline__ V fold_record(const V *leaf, const StepRec<DS> &r) {
+    if constexpr (DS >= 2) return TreeFoldLive<V, DS>::run(leaf, r.gates, r.live);
+    else return TreeFold<V, DS>::run(leaf, r.gates);
+}
 static_assert(sizeof(StepRec<3>) == 64 && sizeof(StepRec<2>) == 32 && sizeof(StepRec<1>) == 16 && sizeof(StepRec<0>) == 16,
               "records are whole scalar-load units");
 
@@ -385,6 +426,7 @@ __global__ __launch_bounds__(DL_BLOCK) void compose_steps_kernel(const int32_t *
         const uint64_t sub = sub_gates[v];
         gates |= (uint32_t) sub;
         const uint32_t live = needed ? LiveLeaves<DS>::of(sub) : 0u;
+        if constexpr (DS >= 2) r.live = LiveGates<DS>::of(sub, needed);
 #pragma unroll
         for (int g = 0; g < (1 << DS); ++g)
             r.leaf[g] = (live >> g) & 1u ? (uint32_t) sub_leaves[v * (1 << DS) + g] * ncols : DL_STEP_DEAD;
@@ -426,7 +468,7 @@ __global__ __launch_bounds__(DL_BLOCK) void eval_steps_kernel(const V *__restric
             V leaves0[G];
 #pragma unroll
             for (int g = 0; g < G; ++g) leaves0[g] = row(r.leaf[g]);
-            prev = TreeFold<V, DS>::run(leaves0, r.gates);
+            prev = fold_record<V, DS>(leaves0, r);
         }
 #pragma unroll 1
         for (int j = 0; j < STEPS; j += 2) {
@@ -437,8 +479,8 @@ __global__ __launch_bounds__(DL_BLOCK) void eval_steps_kernel(const V *__restric
             for (int g = 0; g < G; ++g) la[g] = row(ra.leaf[g]);
 #pragma unroll
             for (int g = 0; g < G; ++g) lb[g] = row(rb.leaf[g]);
-            const V va = TreeFold<V, DS>::run(la, ra.gates);
-            const V vb = TreeFold<V, DS>::run(lb, rb.gates);
+            const V va = fold_record<V, DS>(la, ra);
+            const V vb = fold_record<V, DS>(lb, rb);
             if (ra.out != 0xffffffffu)
                 __builtin_nontemporal_store(gate_apply<V>(prev, va, gate_masks(ra.gates >> 28)), (y + ra.out) + col);
             if (rb.out != 0xffffffffu)
@@ -887,8 +929,10 @@ __global__ __launch_bounds__(DL_BLOCK) void count_partial_kernel(const V *__rest
             const int64_t nn = cls * per_class + r;
             gt[j] = gates[nn];
 #pragma unroll
-            for (int g = 0; g < G; ++g)
-                leaf[j][g] = live ? xcol[(int64_t) leaves[nn * G + g] * ncols] : Words<V>::zero();
+            for (int g = 0; g < G; ++g) {
+                const int32_t id = leaves[nn * G + g];           // wave-uniform; -1: no gate looks at this row
+                leaf[j][g] = live && id >= 0 ? xcol[(int64_t) id * ncols] : Words<V>::zero();
+            }
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
