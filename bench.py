@@ -291,7 +291,35 @@ def packed_headline(args, torch, dl):
     }
     if not args.no_configs:
         info["other_word_widths"] = word_width_variants(torch, dl, model, x, out)
+        info["two_input_gates_only"] = two_input_gates_variant(torch, dl, model, x)
     return value, ms_per_step, roofline, info, model, x, out
+
+
+def two_input_gates_variant(torch, dl, model, x):
+    """The same net with every gate drawn from the ten that look at both of their inputs.  The packed kernels do
+    not fetch rows that no gate looks at (six of the sixteen gates ignore an input), so the headline, whose gate
+    ids are uniform over all sixteen, moves fewer bytes than a net without such gates: this is that net."""
+    import copy
+    two_input = torch.tensor([1, 2, 4, 6, 7, 8, 9, 11, 13, 14], device="cuda")
+    net = copy.deepcopy(model)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    with torch.no_grad():
+        for m in net:
+            if isinstance(m, dl.LogicLayer):
+                ids = two_input[torch.randint(0, 10, (m.out_dim,), device="cuda", generator=g)]
+                m.weights.copy_(torch.nn.functional.one_hot(ids, 16).float())
+
+    def step():
+        with torch.no_grad():
+            return net(dl.PackBitsTensor(x, bit_count=64))
+    step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / 5 * 1e3
+    return {"ms_per_step": round(ms, 4), "samples_per_s": round(x.shape[0] / ms * 1e3, 1)}
 
 
 def word_width_variants(torch, dl, model, x, want):

@@ -47,6 +47,32 @@ template <typename V> __device__ __forceinline__ V gate_apply(V a, V b, const Ga
     return (V) ((a & hi) | (~a & lo));
 }
 
+// Inputs a gate does not look at.  A gate id is the truth table (f(0,0) f(0,1) f(1,0) f(1,1)), MSB first; six of
+// the sixteen ignore an input (constants, a, b, not a, not b).  Whatever feeds an ignored input cannot change the
+// result, so the kernels that evaluate trees of gates per output do not fetch it: with uniformly drawn gates a
+// leaf three gates below its root is needed with probability 0.75^3.
+__host__ __device__ __forceinline__ bool gate_uses_a(uint32_t op) {
+    return (((op >> 3) ^ (op >> 1)) & 1u) || (((op >> 2) ^ op) & 1u);
+}
+__host__ __device__ __forceinline__ bool gate_uses_b(uint32_t op) {
+    return (((op >> 3) ^ (op >> 2)) & 1u) || (((op >> 1) ^ op) & 1u);
+}
+
+// Bit g set: leaf g of a depth-D subtree reaches its root (gates packed as TreeFold reads them).
+template <int D> struct LiveLeaves {
+    static __host__ __device__ __forceinline__ uint32_t of(uint64_t gates) {
+        constexpr int half = 1 << (D - 1);
+        const uint32_t top = (uint32_t) (gates >> (4 * (2 * half - 2))) & 15u;
+        const uint32_t left = gate_uses_a(top) ? LiveLeaves<D - 1>::of(gates) : 0u;
+        const uint32_t right = gate_uses_b(top) ? LiveLeaves<D - 1>::of(gates >> (4 * (half - 1))) : 0u;
+        return left | (right << half);
+    }
+};
+template <> struct LiveLeaves<0> {
+    static __host__ __device__ __forceinline__ uint32_t of(uint64_t) { return 1u; }
+};
+
+
 // One wave owns NPW neurons x 64 consecutive vectors of the row; a workgroup owns
 // 4 * NPW * ITERS consecutive neurons.  blockIdx.x walks neuron tiles, blockIdx.y column
 // tiles: workgroups are dispatched x-fastest, so the chip sweeps all neurons of one column
@@ -80,9 +106,9 @@ __global__ __launch_bounds__(DL_BLOCK) void eval_kernel(const V *__restrict__ x,
             if (live) {
                 V va[NPW], vb[NPW];
 #pragma unroll
-                for (int j = 0; j < NPW; ++j) {
-                    va[j] = x[ia[j] * ncols + col];
-                    vb[j] = x[ib[j] * ncols + col];
+                for (int j = 0; j < NPW; ++j) {                  // (wave-uniform) a row the gate does not look at is not fetched
+                    va[j] = gate_uses_a(op[j]) ? x[ia[j] * ncols + col] : V{};
+                    vb[j] = gate_uses_b(op[j]) ? x[ib[j] * ncols + col] : V{};
                 }
 #pragma unroll
                 for (int j = 0; j < NPW; ++j) {
@@ -109,32 +135,6 @@ __global__ __launch_bounds__(DL_BLOCK) void eval_kernel(const V *__restrict__ x,
 // subtree's own gate at off + 4*(2^d - 2).  Leaves are in left-to-right order (`a` before `b`).
 // ------------------------------------------------------------------------------------------
 #define DL_MAX_FUSE_DEPTH 4
-
-// Inputs a gate does not look at.  A gate id is the truth table (f(0,0) f(0,1) f(1,0) f(1,1)), MSB first; six of
-// the sixteen ignore an input (constants, a, b, not a, not b).  Whatever feeds an ignored input cannot change the
-// result, so the kernels that evaluate trees of gates per output do not fetch it: with uniformly drawn gates a
-// leaf three gates below its root is needed with probability 0.75^3.
-__host__ __device__ __forceinline__ bool gate_uses_a(uint32_t op) {
-    return (((op >> 3) ^ (op >> 1)) & 1u) || (((op >> 2) ^ op) & 1u);
-}
-__host__ __device__ __forceinline__ bool gate_uses_b(uint32_t op) {
-    return (((op >> 3) ^ (op >> 2)) & 1u) || (((op >> 1) ^ op) & 1u);
-}
-
-// Bit g set: leaf g of a depth-D subtree reaches its root (gates packed as TreeFold reads them).
-template <int D> struct LiveLeaves {
-    static __host__ __device__ __forceinline__ uint32_t of(uint64_t gates) {
-        constexpr int half = 1 << (D - 1);
-        const uint32_t top = (uint32_t) (gates >> (4 * (2 * half - 2))) & 15u;
-        const uint32_t left = gate_uses_a(top) ? LiveLeaves<D - 1>::of(gates) : 0u;
-        const uint32_t right = gate_uses_b(top) ? LiveLeaves<D - 1>::of(gates >> (4 * (half - 1))) : 0u;
-        return left | (right << half);
-    }
-};
-template <> struct LiveLeaves<0> {
-    static __host__ __device__ __forceinline__ uint32_t of(uint64_t) { return 1u; }
-};
-
 
 struct TreeTables {
     const int64_t *a[DL_MAX_FUSE_DEPTH];   // [0] = first (lowest) layer of the group

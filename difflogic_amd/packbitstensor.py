@@ -14,7 +14,9 @@ from . import difflogic_cuda
 _L2_GATHER_RATE = 31e12      # B/s: row gathers + stores through the L2s when the input tile stays L2-resident
 _FABRIC_RATE = 7.5e12        # B/s: row gathers + stores between the L2s and Infinity Cache / HBM
 _WRITE_RATE = 6.1e12         # B/s: streaming stores to HBM
-_COUNT_EFFICIENCY = 0.87     # the count kernels reach this fraction of the fabric rate (barriers between phases)
+_COUNT_RATE = 5.2e12         # B/s of counted rows: what the chained count kernel parks in LDS, sorts by class and adds up
+_LIVE_INPUT = 0.75           # share of gate inputs a gate looks at when the gate ids are uniform (10 of 16 gates use both
+                             # inputs, 4 one, 2 none); rows that no gate looks at are not fetched
 _TILE_BYTES = 1024           # one wave covers 64 lanes x 16 bytes of a row
 _L2_RESIDENT_BYTES = 4 << 20     # input tiles (rows x 1 KB each) in flight up to this size are re-read from L2 (4 MB per XCD)
 _LDS_GATE_WORD_SECONDS = 9.4e-13     # LDS-resident whole-net kernel: seconds per gate and 64-sample word
@@ -30,12 +32,15 @@ def group_cost(rows_in, out, depth, words, counted):
     """Modelled seconds of one fused group: `depth` layers from `rows_in` input rows to `out` output
     rows of `words` 64-bit words, ending in the per-class count when `counted`."""
     row_bytes = 8.0 * words
+    # rows gathered per output row: the leaves of a tree of gates that are looked at.  Along a schedule the tree is
+    # the subtree under the vertex two consecutive neurons share (needed unless both ignore it).
+    shared_needed = 1 - (1 - _LIVE_INPUT) ** 2
     if counted:                                    # walked along the schedule: one seed per 128 steps
-        gathers = (1 << (depth - 1)) * (1 + 1 / 128) * out
+        gathers = (2 * _LIVE_INPUT) ** (depth - 1) * shared_needed * (1 + 1 / 128) * out
     elif _chained(depth):                          # one seed per 16 steps
-        gathers = (1 << (depth - 1)) * (1 + 1 / 16) * out
+        gathers = (2 * _LIVE_INPUT) ** (depth - 1) * shared_needed * (1 + 1 / 16) * out
     else:
-        gathers = (1 << depth) * out
+        gathers = (2 * _LIVE_INPUT) ** depth * out
     gathered = gathers * row_bytes
     written = 0.0 if counted else out * row_bytes
     # The chip sweeps all output rows of one 1 KB column tile before the next, but a narrow layer
@@ -48,7 +53,8 @@ def group_cost(rows_in, out, depth, words, counted):
     beyond_l2 = ((1 - hit) * gathered + written) / (_WRITE_RATE if hit == 1.0 else _FABRIC_RATE)
     t = max(through_l2, beyond_l2) + 0.3 * min(through_l2, beyond_l2)                  # the two overlap only in part
     if counted:
-        t /= _COUNT_EFFICIENCY
+        counting = out * row_bytes / _COUNT_RATE                         # overlaps with the gathers only in part, too
+        t = max(t, counting) + 0.3 * min(t, counting)
         t += 2 * (out / 128.0) * row_bytes / _FABRIC_RATE                # partial counters: written, then read once
     # kernels on the stream: the per-call table builders, the group's kernel, the count's second pass
     return t + _LAUNCH_SECONDS * (3 if counted or _chained(depth) else 1)

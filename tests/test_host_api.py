@@ -118,9 +118,11 @@ def test_group_planner():
         if count:
             assert groups[-1] <= 2
     assert plan_groups([7], True) == []
-    # a wide net over few inputs: deep first group (its gathers hit in L2), pairs afterwards
+    # a wide net over few inputs: deep first group (its gathers hit in L2); square layers beyond the caches fuse deep as
+    # well, since a quarter of the inputs of uniformly drawn gates is never fetched (measured on MI355X, 64000-wide,
+    # 16384 words: four layers in one group 4.6 ms, as two pairs 6.5 ms)
     assert plan_groups([784] + [64000] * 6, True)[0] >= 3
-    assert plan_groups([64000] * 5, False) == [2, 2]
+    assert plan_groups([64000] * 5, False) == [4]
 
 
 def test_gate_ids_follow_writes_through_data():
