@@ -52,6 +52,7 @@ SIGNATURES = {
     "dl_adam_max_tensors": [],
     "dl_adam_step": [_int, _vp, _vp, _vp, _vp, _vp, _vp, _dbl, _dbl, _dbl, _dbl, _dbl, _vp],
     "dl_gate_ids": [_vp, _vp, _i64, _int, _vp],
+    "dl_fold_gate_constants": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp],
     "dl_logic_eval": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "dl_tensor_packbits": [_vp, _vp, _i64, _i64, _int, ctypes.POINTER(_i64), _vp],
     "dl_tensor_packbits_batch_major": [_vp, _vp, _i64, _i64, _int, ctypes.POINTER(_i64), _vp],

@@ -1428,6 +1428,46 @@ extern "C" int dl_gate_ids(const void *w, uint8_t *ids, int64_t out_dim, int dty
     return dl_launch_status();
 }
 
+// Constants folded into the gates above them.  A neuron whose gate is constant (ids 0 and 15), or becomes so
+// because its inputs are, has the same output word for every sample; the gate that reads it can be replaced by the
+// one-input gate it amounts to: f'(a, b) = f(c, b) for every a.  The replaced gate ignores that input, so nothing is
+// fetched for it.  Layer by layer: `state_in` says which input rows are constant (0 varies, 1 all zeros, 2 all ones;
+// NULL: all vary), `w_out` receives the gate ids to evaluate (the same function of the varying inputs, bit for bit),
+// `state_out` the constants among this layer's outputs.
+__global__ __launch_bounds__(DL_BLOCK) void fold_gate_constants_kernel(const int64_t *__restrict__ a,
+                                                                       const int64_t *__restrict__ b,
+                                                                       const uint8_t *__restrict__ w,
+                                                                       const uint8_t *__restrict__ state_in,
+                                                                       uint8_t *__restrict__ w_out,
+                                                                       uint8_t *__restrict__ state_out, int64_t out_dim) {
+    const int64_t n = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x;
+    if (n >= out_dim) return;
+    uint32_t op = w[n] & 15u;                                   // (f(0,0) f(0,1) f(1,0) f(1,1)), MSB first
+    const uint32_t sa = state_in ? state_in[a[n]] : 0u, sb = state_in ? state_in[b[n]] : 0u;
+    if (sa) {                                                   // a is the constant sa - 1
+        const uint32_t f0 = sa == 2 ? (op >> 1) & 1u : (op >> 3) & 1u, f1 = sa == 2 ? op & 1u : (op >> 2) & 1u;
+        op = f0 << 3 | f1 << 2 | f0 << 1 | f1;
+    }
+    if (sb) {
+        const uint32_t f0 = sb == 2 ? (op >> 2) & 1u : (op >> 3) & 1u, f1 = sb == 2 ? op & 1u : (op >> 1) & 1u;
+        op = f0 << 3 | f0 << 2 | f1 << 1 | f1;
+    }
+    w_out[n] = (uint8_t) op;
+    state_out[n] = op == 0u ? 1 : op == 15u ? 2 : 0;
+}
+
+extern "C" int dl_fold_gate_constants(const int64_t *a, const int64_t *b, const uint8_t *w, const uint8_t *state_in,
+                                      uint8_t *w_out, uint8_t *state_out, int64_t out_dim, void *stream) {
+    if (out_dim < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim == 0) return DL_OK;
+    if (!a || !b || !w || !w_out || !state_out) return DL_ERR_INVALID_ARGUMENT;
+    const int64_t blocks = dl_ceil_div(out_dim, DL_BLOCK);
+    if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    DL_LAUNCH(fold_gate_constants_kernel, dim3((unsigned) blocks), dim3(DL_BLOCK), 0, (hipStream_t) stream, a, b, w, state_in,
+              w_out, state_out, out_dim);
+    return dl_launch_status();
+}
+
 // Sample-major bool bytes -> feature rows of `out_row_bytes` bytes each (a little-endian bit stream: sample s is
 // bit s % 8 of byte s / 8, whatever the word width); bits past the batch are zero.
 static int pack_batch_major_rows(const uint8_t *x, void *out, int64_t batch, int64_t features, int64_t out_row_bytes,

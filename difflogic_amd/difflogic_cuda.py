@@ -441,6 +441,33 @@ def gate_ids(weights):
     return ids
 
 
+def fold_gate_constants(layers):
+    """``layers`` = [(a, b, w), ...] applied one after the other to rows that vary -> the same list
+    with gate ids in which constants are folded: a neuron that reads a constant neuron (gate id 0 or
+    15, or constant through its own inputs) gets the one-input gate it amounts to.  Same function,
+    bit for bit; the packed kernels then fetch nothing for the ignored inputs.  Not part of the
+    reference's extension."""
+    out, state = [], None
+    lib = _lib.load()
+    for a, b, w in layers:
+        _check_input(w, "w")
+        if w.dim() != 1 or w.dtype != torch.uint8:
+            raise RuntimeError(f"expected w [out] uint8, got {tuple(w.shape)} {w.dtype}")
+        _check_index(a, "a", w.shape[0])
+        _check_index(b, "b", w.shape[0])
+        dev = _same_device(a, b, w)
+        folded = torch.empty_like(w)
+        consts = torch.empty_like(w)
+        with _on(dev):
+            st = lib.dl_fold_gate_constants(_p(a), _p(b), _p(w), _p(state) if state is not None else None, _p(folded),
+                                            _p(consts), w.shape[0], _stream(dev))
+        if st:
+            _raise(st, "fold_gate_constants")
+        out.append((a, b, folded))
+        state = consts
+    return out
+
+
 def tensor_packbits_cuda(t, bit_count):
     """bool [F,B] -> (int{bit_count} [F, ceil(B/bit_count)], pad_len)   (difflogic.cpp:69-74)."""
     _check_input(t, "t")

@@ -134,6 +134,7 @@ class PackBitsTensor:
         self._rows = None             # int64 [features, 2 * ceil(B / 128)]: the padded rows
         self._public = None           # what `.t` handed out or was set to, while it is current
         self._pending = []            # [(a, b, w)] applied to the rows but not yet evaluated
+        self._folded = True           # constants folded through the pending layers' gate ids (_fold_pending)
         if device == "cuda":
             if bit_count not in (8, 16, 32, 64):
                 raise ValueError("`bit_count` has to be in { 8, 16, 32, 64 }")
@@ -201,7 +202,15 @@ class PackBitsTensor:
     def _dims(self):
         return [self._in_features()] + [w.shape[0] for _, _, w in self._pending]
 
+    def _fold_pending(self):
+        """Before the streaming kernels run: constants folded through the deferred layers' gate ids, so that the
+        kernels fetch nothing for inputs that are constant (same words, bit for bit)."""
+        if not self._folded and self._pending:
+            self._pending = difflogic_cuda.fold_gate_constants(self._pending)
+        self._folded = True
+
     def _run_groups(self, groups):
+        self._fold_pending()
         rows = self._words()
         pos = 0
         for depth in groups:
@@ -230,6 +239,7 @@ class PackBitsTensor:
     @t.setter
     def t(self, value):
         self._pending = []
+        self._folded = True
         self._src = None
         self._rows = None
         self._public = value
@@ -239,6 +249,7 @@ class PackBitsTensor:
     def defer_layer(self, a, b, w):
         """Applies the gate layer (a, b, w) lazily."""
         self._pending.append((a, b, w))
+        self._folded = False
         return self
 
     def group_sum(self, k):
@@ -262,6 +273,7 @@ class PackBitsTensor:
                 out = difflogic_cuda.eval_net_lds(rows, self._pending, self._pad(rows), k)
                 if out is not None:
                     return out
+            self._fold_pending()
             groups = plan_groups(self._dims(), True, self._words64())
             self._run_groups(groups[:-1])
             # the last group stays pending: the object's state does not change by counting

@@ -264,6 +264,18 @@ int dl_adam_step(int count, float *const *p, const float *const *g, float *const
  * maximal value wins; a NaN counts as maximal, as in torch).  w [out_dim, 16] of `dtype`. */
 int dl_gate_ids(const void *w, uint8_t *ids, int64_t out_dim, int dtype, void *stream);
 
+/* Constant folding over the gate ids of one layer, for packed inference (no counterpart in the
+ * reference, whose generated C leaves it to the compiler: difflogic/compiled_model.py:97-128 emits
+ * one statement per gate).  A neuron with a constant gate (ids 0, 15), or one whose inputs make it
+ * constant, outputs the same word for every sample; a gate reading it is replaced by the gate it
+ * amounts to with that input fixed, which ignores the input (so the packed kernels fetch nothing
+ * for it).  The evaluated function is unchanged, bit for bit.
+ *   a, b [out_dim] the layer's wiring; w [out_dim] its gate ids;
+ *   state_in [in_dim] or NULL: 0 = the input row varies, 1 = all zeros, 2 = all ones;
+ *   w_out [out_dim]: the gate ids to evaluate; state_out [out_dim]: the constants among the outputs. */
+int dl_fold_gate_constants(const int64_t *a, const int64_t *b, const uint8_t *w, const uint8_t *state_in,
+                           uint8_t *w_out, uint8_t *state_out, int64_t out_dim, void *stream);
+
 /* Replaces `eval` = logic_layer_cuda_eval (difflogic.cpp:63-68, difflogic_kernel.cu:503-541).
  *   x [in_dim, words], y [out_dim, words] of signed integers of `bit_count` bits;
  *   w [out_dim] uint8 gate ids (4-bit truth tables, difflogic_kernel.cu:418-435).

@@ -391,6 +391,39 @@ def test_eval_chained_equals_eval_fused(ext, bits, in_dim, widths, W, kind):
     assert ext.schedule_for(dev_layers[-1][0], dev_layers[-1][1], sched.in_dim) is sched         # cached
 
 
+def test_fold_gate_constants(ext):
+    """Constants folded through the gate ids: the folded net is the same function of the rows that vary (checked
+    against the per-layer oracle on the ORIGINAL gate ids), constant neurons are found (their folded id is 0 or
+    15), and a gate that reads one ignores that input afterwards."""
+    rng = np.random.default_rng(11)
+    in_dim, widths, W = 40, [300, 300, 300, 200], 5
+    layers = random_layers(rng, in_dim, widths)
+    for l in layers:                                         # plenty of constant and one-input gates
+        l[2][rng.random(len(l[2])) < 0.3] = rng.choice([0, 15, 3, 5, 10, 12])
+    dev_layers = [tuple(_dev(t) for t in l) for l in layers]
+    folded = ext.fold_gate_constants(dev_layers)
+    x = rng.integers(np.iinfo(np.int64).min, np.iinfo(np.int64).max, (in_dim, W), dtype=np.int64, endpoint=True)
+    want, got = x, x
+    consts = np.zeros(in_dim, bool)
+    for (a, b, op), (_, _, fop) in zip(layers, folded):
+        fop = fop.cpu().numpy()
+        want = po.eval_layer(want, a, b, op)
+        got = po.eval_layer(got, a, b, fop)
+        assert np.array_equal(got, want)
+        is_const = (fop == 0) | (fop == 15)
+        # every row that is constant for ALL inputs it can see is found when it follows from the gates alone:
+        # a folded constant really is one, and a gate reading a constant row no longer looks at it
+        assert np.all((want[is_const] == 0) | (want[is_const] == -1))
+        uses_a = (((fop >> 3) ^ (fop >> 1)) & 1) | (((fop >> 2) ^ fop) & 1)
+        uses_b = (((fop >> 3) ^ (fop >> 2)) & 1) | (((fop >> 1) ^ fop) & 1)
+        assert not np.any(uses_a.astype(bool) & consts[a]) and not np.any(uses_b.astype(bool) & consts[b])
+        consts = is_const
+    assert consts.sum() > 20
+    # folding is idempotent
+    again = ext.fold_gate_constants(folded)
+    assert all(torch.equal(u[2], v[2]) for u, v in zip(folded, again))
+
+
 def test_eval_schedule_rejects_bad_wiring(ext):
     with pytest.raises(RuntimeError):
         ext.EvalSchedule(torch.tensor([0, 5]).cuda(), torch.tensor([1, 1]).cuda(), 3)
