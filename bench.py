@@ -182,6 +182,12 @@ def packed_run(torch, dl, model, x, k, steps, warmup):
         out = step()
         torch.cuda.synchronize()
         first_call_ms = (time.perf_counter() - t_first) * 1e3       # includes the host-side schedule / order builds
+        # untimed: a third of a second of the same steps ahead of the warm-up proper, so that clocks and caches have
+        # settled however few warm-up steps were asked for (the first launches of a process run up to 1.5x slower)
+        t_settle = time.perf_counter() + 0.3
+        while time.perf_counter() < t_settle:
+            out = step()
+            torch.cuda.synchronize()
         for _ in range(max(0, warmup - 1)):
             out = step()
         torch.cuda.synchronize()

@@ -53,6 +53,7 @@ SIGNATURES = {
     "dl_adam_step": [_int, _vp, _vp, _vp, _vp, _vp, _vp, _dbl, _dbl, _dbl, _dbl, _dbl, _vp],
     "dl_gate_ids": [_vp, _vp, _i64, _int, _vp],
     "dl_fold_gate_constants": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp],
+    "dl_mark_live_inputs": [_vp, _vp, _vp, _vp, _vp, _i64, _vp],
     "dl_logic_eval": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "dl_tensor_packbits": [_vp, _vp, _i64, _i64, _int, ctypes.POINTER(_i64), _vp],
     "dl_tensor_packbits_batch_major": [_vp, _vp, _i64, _i64, _int, ctypes.POINTER(_i64), _vp],
@@ -64,7 +65,7 @@ SIGNATURES = {
     "dl_eval_schedule_capacity": [_i64, _int],
     "dl_eval_schedule_build": [_vp, _vp, _i64, _i64, _int, _vp, _vp, _vp],
     "dl_logic_eval_chained_workspace_bytes": [_int, _i64, _i64],
-    "dl_logic_eval_chained": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _int, _vp, _vp],
+    "dl_logic_eval_chained": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _int, _vp, _vp],
     "dl_logic_eval_fused_groupbitsum_workspace_bytes": [_int, _i64, _i64, _int, _i64],
     "dl_logic_eval_fused_groupbitsum": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _i64, _vp, _vp, _vp],
     "dl_logic_eval_fused_groupbitsum_noalloc": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _i64, _vp, _vp],

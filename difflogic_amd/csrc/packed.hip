@@ -397,7 +397,8 @@ __global__ __launch_bounds__(DL_BLOCK) void compose_steps_kernel(const int32_t *
                                                                  const int32_t *__restrict__ verts,
                                                                  const int32_t *__restrict__ neuron,
                                                                  const uint8_t *__restrict__ flip,
-                                                                 const uint8_t *__restrict__ w_top, int64_t steps,
+                                                                 const uint8_t *__restrict__ w_top,
+                                                                 const uint8_t *__restrict__ out_live, int64_t steps,
                                                                  uint32_t ncols, StepRec<DS> *__restrict__ rec) {
     const int64_t i = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x;      // record index: step i - 1
     if (i > steps) return;
@@ -406,8 +407,9 @@ __global__ __launch_bounds__(DL_BLOCK) void compose_steps_kernel(const int32_t *
     uint32_t gates = 0;
     r.out = 0xffffffffu;
     // the vertex is the second input of step i - 1's neuron and the first input of step i's
+    // (out_live: output rows nobody will read are neither computed nor written)
     bool needed = false;
-    if (i >= 1 && neuron[i - 1] >= 0) {
+    if (i >= 1 && neuron[i - 1] >= 0 && (!out_live || out_live[neuron[i - 1]])) {
         const int32_t n = neuron[i - 1];
         uint32_t top = w_top[n] & 15u;
         if (flip[i - 1]) top = swap_gate_inputs(top);
@@ -415,7 +417,7 @@ __global__ __launch_bounds__(DL_BLOCK) void compose_steps_kernel(const int32_t *
         r.out = (uint32_t) n * ncols;
         needed = gate_uses_b(top);
     }
-    if (i < steps && neuron[i] >= 0) {
+    if (i < steps && neuron[i] >= 0 && (!out_live || out_live[neuron[i]])) {
         uint32_t next = w_top[neuron[i]] & 15u;
         if (flip[i]) next = swap_gate_inputs(next);
         needed = needed || gate_uses_a(next);
@@ -1468,6 +1470,32 @@ extern "C" int dl_fold_gate_constants(const int64_t *a, const int64_t *b, const 
     return dl_launch_status();
 }
 
+// Input rows that a layer looks at: live_in[r] = 1 where some neuron n with live_out[n] (NULL: every neuron) reads
+// row r through an input its gate does not ignore.  live_in is cleared by the caller; the stores all write 1.
+__global__ __launch_bounds__(DL_BLOCK) void mark_live_inputs_kernel(const int64_t *__restrict__ a,
+                                                                    const int64_t *__restrict__ b,
+                                                                    const uint8_t *__restrict__ w,
+                                                                    const uint8_t *__restrict__ live_out,
+                                                                    uint8_t *__restrict__ live_in, int64_t out_dim) {
+    const int64_t n = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x;
+    if (n >= out_dim || (live_out && !live_out[n])) return;
+    const uint32_t op = w[n] & 15u;
+    if (gate_uses_a(op)) live_in[a[n]] = 1;
+    if (gate_uses_b(op)) live_in[b[n]] = 1;
+}
+
+extern "C" int dl_mark_live_inputs(const int64_t *a, const int64_t *b, const uint8_t *w, const uint8_t *live_out,
+                                   uint8_t *live_in, int64_t out_dim, void *stream) {
+    if (out_dim < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim == 0) return DL_OK;
+    if (!a || !b || !w || !live_in) return DL_ERR_INVALID_ARGUMENT;
+    const int64_t blocks = dl_ceil_div(out_dim, DL_BLOCK);
+    if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    DL_LAUNCH(mark_live_inputs_kernel, dim3((unsigned) blocks), dim3(DL_BLOCK), 0, (hipStream_t) stream, a, b, w, live_out,
+              live_in, out_dim);
+    return dl_launch_status();
+}
+
 // Sample-major bool bytes -> feature rows of `out_row_bytes` bytes each (a little-endian bit stream: sample s is
 // bit s % 8 of byte s / 8, whatever the word width); bits past the batch are zero.
 static int pack_batch_major_rows(const uint8_t *x, void *out, int64_t batch, int64_t features, int64_t out_row_bytes,
@@ -1712,13 +1740,13 @@ int launch_eval_chain(int sub_depth, const void *x, const int32_t *sub_leaves, c
 
 template <typename V, int DS>
 int launch_eval_steps(const void *x, const int32_t *sub_leaves, const uint64_t *sub_gates, const int32_t *verts,
-                      const int32_t *neuron, const uint8_t *flip, const uint8_t *w_top, void *y, void *records,
-                      int64_t steps, int64_t row_bytes, int64_t x_bytes, hipStream_t s) {
+                      const int32_t *neuron, const uint8_t *flip, const uint8_t *w_top, const uint8_t *out_live, void *y,
+                      void *records, int64_t steps, int64_t row_bytes, int64_t x_bytes, hipStream_t s) {
     constexpr int STEPS = 16;
     const int64_t ncols = row_bytes / (int64_t) sizeof(V);
     StepRec<DS> *rec = (StepRec<DS> *) records;
     DL_LAUNCH(compose_steps_kernel<DS>, dim3((unsigned) dl_ceil_div(steps + 1, DL_BLOCK)), dim3(DL_BLOCK), 0, s, sub_leaves,
-              sub_gates, verts, neuron, flip, w_top, steps, (uint32_t) ncols, rec);
+              sub_gates, verts, neuron, flip, w_top, out_live, steps, (uint32_t) ncols, rec);
     const int st = dl_launch_status();
     if (st != DL_OK) return st;
     int64_t ctiles = dl_ceil_div(ncols, DL_WAVE);
@@ -1745,8 +1773,8 @@ extern "C" int64_t dl_logic_eval_chained_workspace_bytes(int depth, int64_t sub_
 
 extern "C" int dl_logic_eval_chained(const void *x, int depth, const int64_t *const *a, const int64_t *const *b,
                                      const uint8_t *const *w, const int64_t *dims, const int32_t *verts,
-                                     const int32_t *neuron, const uint8_t *flip, int64_t steps, void *y, int64_t words,
-                                     int bit_count, void *workspace, void *stream) {
+                                     const int32_t *neuron, const uint8_t *flip, int64_t steps, const uint8_t *out_live,
+                                     void *y, int64_t words, int bit_count, void *workspace, void *stream) {
     if (!valid_bit_count(bit_count)) return DL_ERR_BIT_COUNT;
     if (depth < 1 || depth > DL_MAX_FUSE_DEPTH || !dims || !w || words < 0 || steps < 0 ||
         steps % DL_EVAL_SCHEDULE_CHUNK != 0)
@@ -1770,10 +1798,10 @@ extern "C" int dl_logic_eval_chained(const void *x, int depth, const int64_t *co
         void *records = (char *) workspace + ((tables + 63) / 64) * 64;
         const uint8_t *w_top = w[depth - 1];
         switch (depth - 1) {
-        case 0: return launch_eval_steps<dl_u32x4, 0>(x, sub_leaves, sub_gates, verts, neuron, flip, w_top, y, records, steps, row_bytes, dims[0] * row_bytes, s);
-        case 1: return launch_eval_steps<dl_u32x4, 1>(x, sub_leaves, sub_gates, verts, neuron, flip, w_top, y, records, steps, row_bytes, dims[0] * row_bytes, s);
-        case 2: return launch_eval_steps<dl_u32x4, 2>(x, sub_leaves, sub_gates, verts, neuron, flip, w_top, y, records, steps, row_bytes, dims[0] * row_bytes, s);
-        default: return launch_eval_steps<dl_u32x4, 3>(x, sub_leaves, sub_gates, verts, neuron, flip, w_top, y, records, steps, row_bytes, dims[0] * row_bytes, s);
+        case 0: return launch_eval_steps<dl_u32x4, 0>(x, sub_leaves, sub_gates, verts, neuron, flip, w_top, out_live, y, records, steps, row_bytes, dims[0] * row_bytes, s);
+        case 1: return launch_eval_steps<dl_u32x4, 1>(x, sub_leaves, sub_gates, verts, neuron, flip, w_top, out_live, y, records, steps, row_bytes, dims[0] * row_bytes, s);
+        case 2: return launch_eval_steps<dl_u32x4, 2>(x, sub_leaves, sub_gates, verts, neuron, flip, w_top, out_live, y, records, steps, row_bytes, dims[0] * row_bytes, s);
+        default: return launch_eval_steps<dl_u32x4, 3>(x, sub_leaves, sub_gates, verts, neuron, flip, w_top, out_live, y, records, steps, row_bytes, dims[0] * row_bytes, s);
         }
     }
     const int64_t nchunks = steps / DL_EVAL_SCHEDULE_CHUNK;

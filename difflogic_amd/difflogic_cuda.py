@@ -736,11 +736,39 @@ def schedule_for(a, b, in_dim):
     return _SCHEDULES.get((a, b), (int(in_dim),), lambda: EvalSchedule(a, b, in_dim))
 
 
-def eval_chained(x, layers, schedule=None):
+def live_inputs(layers, live_out=None):
+    """For consecutive layers [(a, b, w), ...] (``w`` uint8 gate ids) whose last one's output rows
+    are needed where ``live_out`` [out] is non-zero (None: all of them): a list with, per layer,
+    the uint8 vector of its INPUT rows that some needed neuron looks at (an input its gate ignores
+    does not count).  ``result[i]`` is what ``eval_chained(..., out_live=)`` takes for the group that
+    produces the input of ``layers[i]``.  Not part of the reference's extension."""
+    lib = _lib.load()
+    res = [None] * len(layers)
+    for i in range(len(layers) - 1, -1, -1):
+        a, b, w = layers[i]
+        _check_input(w, "w")
+        _check_index(a, "a", w.shape[0])
+        _check_index(b, "b", w.shape[0])
+        dev = _same_device(a, b, w)
+        in_dim = int(layers[i - 1][2].shape[0]) if i > 0 else None
+        if in_dim is None:
+            break                                     # the first layer's input rows are the caller's data
+        live_in = torch.zeros(in_dim, dtype=torch.uint8, device=dev)
+        with _on(dev):
+            st = lib.dl_mark_live_inputs(_p(a), _p(b), _p(w), _p(live_out) if live_out is not None else None, _p(live_in),
+                                         w.shape[0], _stream(dev))
+        if st:
+            _raise(st, "mark_live_inputs")
+        res[i] = live_out = live_in
+    return res
+
+
+def eval_chained(x, layers, schedule=None, out_live=None):
     """Same result as ``eval_fused(x, layers)``; the group's top layer is walked along
     ``schedule`` (default: the cached schedule of its wiring), which halves the rows gathered per
-    neuron.  Not part of the reference's extension.  Falls back to eval_fused where it does not
-    apply."""
+    neuron.  ``out_live`` (uint8 [out], see live_inputs): output rows marked 0 will not be read and
+    may be left unwritten.  Not part of the reference's extension.  Falls back to eval_fused where
+    it does not apply."""
     dev, bits, depth, pa, pb, pw, pdims, dims = _fused_args(x, layers)
     if depth > MAX_FUSE_DEPTH:
         raise RuntimeError(f"at most {MAX_FUSE_DEPTH} layers can be fused, got {depth}")
@@ -752,12 +780,16 @@ def eval_chained(x, layers, schedule=None):
     if schedule.in_dim != dims[-2] or schedule.out_dim != dims[-1]:
         raise RuntimeError(f"schedule is for a {schedule.in_dim}->{schedule.out_dim} layer, the group ends in "
                            f"{dims[-2]}->{dims[-1]}")
+    if out_live is not None and (out_live.dtype != torch.uint8 or out_live.shape != (dims[-1],) or out_live.device != dev
+                                 or not out_live.is_contiguous()):
+        raise RuntimeError(f"expected out_live to be a contiguous uint8 [{dims[-1]}] tensor on {dev}")
     y = torch.empty((dims[-1], words), dtype=x.dtype, device=dev)
     nbytes = _lib.load().dl_logic_eval_chained_workspace_bytes(depth, dims[-2], schedule.steps)
     ws = torch.empty(max(1, -(-nbytes // 8)), dtype=torch.int64, device=dev)      # torch aligns allocations to 512 bytes
     with _on(dev):
         st = _lib.load().dl_logic_eval_chained(_p(x), depth, pa, pb, pw, pdims, _p(schedule.verts), _p(schedule.neuron),
-                                               _p(schedule.flip), schedule.steps, _p(y), words, bits,
+                                               _p(schedule.flip), schedule.steps,
+                                               _p(out_live) if out_live is not None else None, _p(y), words, bits,
                                                _p(ws) if ws is not None else None, _stream(dev))
     if st == _lib.DL_ERR_TOO_LARGE:
         return eval_fused(x, layers)

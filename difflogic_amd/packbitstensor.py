@@ -209,14 +209,20 @@ class PackBitsTensor:
             self._pending = difflogic_cuda.fold_gate_constants(self._pending)
         self._folded = True
 
-    def _run_groups(self, groups):
+    def _run_groups(self, groups, live=None):
+        """Evaluates the first sum(groups) pending layers group by group.  ``live`` (difflogic_cuda.live_inputs of
+        the pending layers): rows that the layers still pending afterwards do not look at need not be written; the
+        rows then kept are for those layers only (`.t` of them is never handed out: reading `.t` evaluates the rest)."""
         self._fold_pending()
         rows = self._words()
         pos = 0
         for depth in groups:
-            run = difflogic_cuda.eval_chained if _chained(depth) else difflogic_cuda.eval_fused
-            rows = run(rows, self._pending[pos:pos + depth])
+            group = self._pending[pos:pos + depth]
             pos += depth
+            if _chained(depth):
+                rows = difflogic_cuda.eval_chained(rows, group, out_live=live[pos] if live and pos < len(live) else None)
+            else:
+                rows = difflogic_cuda.eval_fused(rows, group)
         if pos:
             self._rows, self._public = rows, None
         self._pending = self._pending[pos:]
@@ -275,7 +281,9 @@ class PackBitsTensor:
                     return out
             self._fold_pending()
             groups = plan_groups(self._dims(), True, self._words64())
-            self._run_groups(groups[:-1])
+            # output rows of the groups before the last that no gate above them looks at are not computed
+            live = difflogic_cuda.live_inputs(self._pending) if len(groups) > 1 else None
+            self._run_groups(groups[:-1], live)
             # the last group stays pending: the object's state does not change by counting
             rows = self._words()
             out = difflogic_cuda.eval_chained_groupbitsum(rows, self._pending, self._pad(rows), k)

@@ -276,6 +276,14 @@ int dl_gate_ids(const void *w, uint8_t *ids, int64_t out_dim, int dtype, void *s
 int dl_fold_gate_constants(const int64_t *a, const int64_t *b, const uint8_t *w, const uint8_t *state_in,
                            uint8_t *w_out, uint8_t *state_out, int64_t out_dim, void *stream);
 
+/* Which input rows a layer looks at, for packed inference across fused groups (no counterpart in the
+ * reference): live_in[r] is set to 1 where some neuron n with live_out[n] != 0 (live_out NULL: every
+ * neuron) reads row r through an input its gate does not ignore.  live_in [in_dim] is cleared by the
+ * caller beforehand.  Applied from the last layer downwards it yields, per layer, the output rows
+ * that have to exist; dl_logic_eval_chained takes that vector as out_live. */
+int dl_mark_live_inputs(const int64_t *a, const int64_t *b, const uint8_t *w, const uint8_t *live_out,
+                        uint8_t *live_in, int64_t out_dim, void *stream);
+
 /* Replaces `eval` = logic_layer_cuda_eval (difflogic.cpp:63-68, difflogic_kernel.cu:503-541).
  *   x [in_dim, words], y [out_dim, words] of signed integers of `bit_count` bits;
  *   w [out_dim] uint8 gate ids (4-bit truth tables, difflogic_kernel.cu:418-435).
@@ -342,7 +350,10 @@ int dl_logic_eval_fused(const void *x, int depth, const int64_t *const *a, const
  *   dl_logic_eval_chained()       as dl_logic_eval_fused plus the DEVICE schedule arrays; workspace
  *                                 of dl_logic_eval_chained_workspace_bytes(depth, dims[depth-1],
  *                                 steps) bytes, 64-byte aligned: the flattened subtrees and one
- *                                 record per step, both rebuilt by every call. */
+ *                                 record per step, both rebuilt by every call.
+ *                                 out_live [dims[depth]] or NULL: output rows with out_live[n] == 0
+ *                                 will not be read by the caller and MAY be left unwritten (see
+ *                                 dl_mark_live_inputs); NULL: every row is written. */
 int dl_eval_schedule_chunk(void);
 int64_t dl_eval_schedule_capacity(int64_t out_dim, int chunk);
 int64_t dl_eval_schedule_build(const int64_t *a, const int64_t *b, int64_t in_dim, int64_t out_dim,
@@ -350,8 +361,9 @@ int64_t dl_eval_schedule_build(const int64_t *a, const int64_t *b, int64_t in_di
 int64_t dl_logic_eval_chained_workspace_bytes(int depth, int64_t sub_dim, int64_t steps);
 int dl_logic_eval_chained(const void *x, int depth, const int64_t *const *a, const int64_t *const *b,
                           const uint8_t *const *w, const int64_t *dims, const int32_t *verts,
-                          const int32_t *neuron, const uint8_t *flip, int64_t steps, void *y,
-                          int64_t words, int bit_count, void *workspace, void *stream);
+                          const int32_t *neuron, const uint8_t *flip, int64_t steps,
+                          const uint8_t *out_live, void *y, int64_t words, int bit_count, void *workspace,
+                          void *stream);
 
 /* The net's last `depth` (1 or 2) layers fused with `groupbitsum` (the sequence
  * difflogic/difflogic.py:147 then difflogic/packbitstensor.py:22): the last layer's output words

@@ -424,6 +424,45 @@ def test_fold_gate_constants(ext):
     assert all(torch.equal(u[2], v[2]) for u, v in zip(folded, again))
 
 
+def test_live_inputs_and_rows_left_unwritten(ext):
+    """live_inputs marks exactly the rows some needed neuron looks at (numpy restatement); eval_chained with that
+    vector writes every marked row as the oracle has it, and the layers above give the same result whatever the
+    other rows hold."""
+    rng = np.random.default_rng(12)
+    in_dim, widths, W = 60, [500, 480, 520, 400, 300], 6
+    layers = random_layers(rng, in_dim, widths)
+    dev_layers = ext.fold_gate_constants([tuple(_dev(t) for t in l) for l in layers])
+    host = [(a, b, w.cpu().numpy()) for (a, b, _), (_, _, w) in zip(layers, dev_layers)]
+    live = ext.live_inputs(dev_layers)
+    assert live[0] is None
+    need = np.ones(widths[-1], bool)
+    for i in range(len(layers) - 1, 0, -1):
+        a, b, w = host[i]
+        uses_a = ((((w >> 3) ^ (w >> 1)) & 1) | (((w >> 2) ^ w) & 1)).astype(bool)
+        uses_b = ((((w >> 3) ^ (w >> 2)) & 1) | (((w >> 1) ^ w) & 1)).astype(bool)
+        want = np.zeros(widths[i - 1], bool)
+        want[a[need & uses_a]] = True
+        want[b[need & uses_b]] = True
+        assert np.array_equal(live[i].cpu().numpy().astype(bool), want), i
+        need = want
+    assert 0.2 < live[3].float().mean().item() < 0.95          # something to skip, something to keep
+    # the first three layers as one group whose output feeds layers 4 and 5
+    x = rng.integers(np.iinfo(np.int64).min, np.iinfo(np.int64).max, (in_dim, W), dtype=np.int64, endpoint=True)
+    want = x
+    for a, b, op in layers[:3]:
+        want = po.eval_layer(want, a, b, op)
+    got = ext.eval_chained(_dev(x), dev_layers[:3], out_live=live[3])
+    keep = live[3].cpu().numpy().astype(bool)
+    assert np.array_equal(got.cpu().numpy()[keep], want[keep])
+    full = want
+    for a, b, op in layers[3:]:
+        full = po.eval_layer(full, a, b, op)
+    rest = ext.eval_chained(got, dev_layers[3:])
+    assert np.array_equal(rest.cpu().numpy(), full)
+    with pytest.raises(RuntimeError):
+        ext.eval_chained(_dev(x), dev_layers[:3], out_live=live[2])
+
+
 def test_eval_schedule_rejects_bad_wiring(ext):
     with pytest.raises(RuntimeError):
         ext.EvalSchedule(torch.tensor([0, 5]).cuda(), torch.tensor([1, 1]).cuda(), 3)
