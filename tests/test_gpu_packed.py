@@ -424,6 +424,40 @@ def test_fold_gate_constants(ext):
     assert all(torch.equal(u[2], v[2]) for u, v in zip(folded, again))
 
 
+def test_pack_tensor_after_counting_with_rows_left_unwritten():
+    """A net too wide for the LDS kernel streams in several groups; group_sum leaves rows of the inner groups unwritten
+    that no gate above looks at.  The object stays usable: counting again, reading `.t` (every row of the last layer)
+    and applying one more layer give what the oracle gives."""
+    import difflogic_amd as dl
+    from difflogic_amd import packbitstensor as pbt
+    rng = np.random.default_rng(17)
+    F, widths, k, B = 100, [12000, 11000, 12000, 10500], 10, 200
+    layers = random_layers(rng, F, widths)
+    x = rng.random((B, F)) < 0.5
+    assert len(pbt.plan_groups([F] + widths, True, 4)) >= 2 and pbt.lds_tail([F] + widths, 4) == 0
+    model = build_model(F, layers, k).eval()
+    logic = [m for m in model if isinstance(m, dl.LogicLayer)]
+    want = po.net_eval_bitwise(x, layers, k)
+    p = dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=32)
+    with torch.no_grad():
+        for m in logic:
+            p = m(p)
+    assert np.array_equal(p.group_sum(k).cpu().numpy(), want)
+    assert np.array_equal(p.group_sum(k).cpu().numpy(), want)                   # again, from the rows kept
+    t = po.packbits(x.T, 32)[0]
+    for a, b, op in layers:
+        t = po.eval_layer(t, a, b, op)
+    assert np.array_equal(p.t.cpu().numpy(), t)                                 # every row of the last layer
+    assert np.array_equal(p.group_sum(k).cpu().numpy(), want)
+    extra = random_layers(rng, widths[-1], [6000])[0]
+    more = dl.LogicLayer(widths[-1], 6000)
+    more.set_connections(torch.as_tensor(extra[0]), torch.as_tensor(extra[1]))
+    with torch.no_grad():
+        more.weights.copy_(torch.nn.functional.one_hot(torch.as_tensor(extra[2]).long(), 16).float())
+        p = more.eval()(p)
+    assert np.array_equal(p.group_sum(k).cpu().numpy(), po.groupbitsum(po.eval_layer(t, *extra), p.pad_len, k))
+
+
 def test_live_inputs_and_rows_left_unwritten(ext):
     """live_inputs marks exactly the rows some needed neuron looks at (numpy restatement); eval_chained with that
     vector writes every marked row as the oracle has it, and the layers above give the same result whatever the
