@@ -746,3 +746,32 @@ def test_net_lds_from_the_bool_input_declines_what_does_not_fit(ext):
     assert ext.eval_net_lds_bool(torch.zeros(0, 48, dtype=torch.bool, device="cuda"), dev_layers, 3).shape == (0, 3)
     with pytest.raises(ValueError):
         ext.eval_net_lds_bool(torch.zeros(10, 48, dtype=torch.bool, device="cuda"), dev_layers, 7)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_nets_end_to_end(seed):
+    """Nets of random depth, widths (narrow ones for the LDS kernel, wide ones for the streaming groups), class
+    count, word width and batch, through PackBitsTensor and GroupSum as a user runs them, against the oracle."""
+    import difflogic_amd as dl
+    rng = np.random.default_rng(1000 + seed)
+    for case in range(10):
+        F = int(rng.integers(1, 70)) if case % 3 else int(rng.integers(1, 9)) * 16
+        L = int(rng.integers(1, 8)) if case % 4 else int(rng.integers(1, 5))
+        k = int(rng.choice([1, 2, 3, 5, 10, 16]))
+        widths, d = [], F
+        for i in range(L):
+            lo = max(1, (d + 1) // 2)
+            w = int(rng.integers(lo, lo + 200)) if case % 4 else int(rng.integers(max(lo, 2000), max(lo, 2000) + 11000))
+            if i == L - 1:
+                w = -(-w // k) * k
+            widths.append(w)
+            d = w
+        bits = int(rng.choice([8, 16, 32, 64]))
+        B = int(rng.choice([1, 7, 63, 64, 65, 200, 1000, 4096, 5000]))
+        layers = random_layers(rng, F, widths)
+        x = rng.random((B, F)) < 0.5
+        want = po.net_eval_bitwise(x, layers, k)
+        model = build_model(F, layers, k).eval()
+        with torch.no_grad():
+            got = model(dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=bits)).cpu().numpy()
+        assert got.shape == want.shape and np.array_equal(got, want), (seed, case, F, widths, k, bits, B)
