@@ -47,6 +47,14 @@ template <typename V> __device__ __forceinline__ V gate_apply(V a, V b, const Ga
     return (V) ((a & hi) | (~a & lo));
 }
 
+// What stands in for an operand that no gate looks at: whatever the registers hold (an empty statement that the
+// compiler takes to define them), so that nothing is executed to make a value up.
+template <typename V> __device__ __forceinline__ V any_value() {
+    V v;
+    asm volatile("" : "=v"(v));
+    return v;
+}
+
 // Inputs a gate does not look at.  A gate id is the truth table (f(0,0) f(0,1) f(1,0) f(1,1)), MSB first; six of
 // the sixteen ignore an input (constants, a, b, not a, not b).  Whatever feeds an ignored input cannot change the
 // result, so the kernels that evaluate trees of gates per output do not fetch it: with uniformly drawn gates a
@@ -736,10 +744,41 @@ __global__ __launch_bounds__(DL_BLOCK) void packbits_batch_major_rows_kernel(con
 // compose_tree_kernel writes; the output of the last layer never exists in memory.
 // ------------------------------------------------------------------------------------------
 
+// A full adder per bit: two three-input bit operations per dword (truth tables 0xe8 = majority, 0x96 = parity),
+// stated as such because the compiler otherwise rearranges a chain of adders into half as many again.
+template <typename V> struct FullAdd;
+template <> struct FullAdd<uint32_t> {
+    static __device__ __forceinline__ void run(uint32_t &carry, uint32_t &sum, uint32_t a, uint32_t b, uint32_t c) {
+        carry = __builtin_amdgcn_bitop3_b32(a, b, c, 0xe8);
+        sum = __builtin_amdgcn_bitop3_b32(a, b, c, 0x96);
+    }
+};
+template <> struct FullAdd<uint64_t> {
+    static __device__ __forceinline__ void run(uint64_t &carry, uint64_t &sum, uint64_t a, uint64_t b, uint64_t c) {
+        uint32_t cl, sl, ch, sh;
+        FullAdd<uint32_t>::run(cl, sl, (uint32_t) a, (uint32_t) b, (uint32_t) c);
+        FullAdd<uint32_t>::run(ch, sh, (uint32_t) (a >> 32), (uint32_t) (b >> 32), (uint32_t) (c >> 32));
+        carry = ((uint64_t) ch << 32) | cl;
+        sum = ((uint64_t) sh << 32) | sl;
+    }
+};
+template <> struct FullAdd<dl_u32x4> {
+    static __device__ __forceinline__ void run(dl_u32x4 &carry, dl_u32x4 &sum, dl_u32x4 a, dl_u32x4 b, dl_u32x4 c) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t cy, sm;
+            FullAdd<uint32_t>::run(cy, sm, a[i], b[i], c[i]);
+            carry[i] = cy;
+            sum[i] = sm;
+        }
+    }
+};
+
 template <typename V> __device__ __forceinline__ void csa(V &carry, V &sum, V a, V b, V c) {
-    const V u = a ^ b;
-    carry = (a & b) | (u & c);
-    sum = u ^ c;
+    V cy, sm;
+    FullAdd<V>::run(cy, sm, a, b, c);
+    carry = cy;
+    sum = sm;
 }
 
 template <typename V> struct Words;        // access to the 32-bit components of a vector
@@ -1055,9 +1094,10 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
                                                                             const uint16_t *__restrict__ runs,
                                                                             V *__restrict__ partial, int64_t ncols,
                                                                             int64_t k, int64_t nwg, int blocks) {
-    __shared__ V stage[DL_CC_BLOCK][DL_WAVE];
+    __shared__ V stage[DL_CC_BLOCK + 1][DL_WAVE];        // the last slot stays zero: what a run's padding reads
     const int wave = dl_wave_in_block();
     const int lane = dl_lane();
+    if (wave == 0) stage[DL_CC_BLOCK][lane] = Words<V>::zero();   // (visible after the first block's barrier)
     const int64_t g = blockIdx.x;
     const int64_t col = (int64_t) blockIdx.y * DL_WAVE + lane;
     const bool live = col < ncols;
@@ -1072,8 +1112,8 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
     V prev;
     {
         const dl_u32x4 r = wrec[0];
-        const V ra = (r.w & 1u) ? Words<V>::zero() : xcol[(int64_t) r.x * ncols];
-        const V rb = DS != 1 ? ra : (r.w & 2u) ? Words<V>::zero() : xcol[(int64_t) r.y * ncols];
+        const V ra = (r.w & 1u) ? any_value<V>() : xcol[(int64_t) r.x * ncols];
+        const V rb = DS != 1 ? ra : (r.w & 2u) ? any_value<V>() : xcol[(int64_t) r.y * ncols];
         prev = vertex(ra, rb, r.z);
     }
     V cnt[CPW][DL_CC_PLANES];
@@ -1095,8 +1135,8 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
             for (int j = 0; j < BATCH; ++j) {
                 r[j] = wrec[1 + b * DL_CC_WAVE_STEPS + h + j];
                 // (wave-uniform flags: rows that no gate looks at are not fetched)
-                ra[j] = (r[j].w & 1u) ? Words<V>::zero() : xcol[(int64_t) r[j].x * ncols];
-                if (DS == 1) rb[j] = (r[j].w & 2u) ? Words<V>::zero() : xcol[(int64_t) r[j].y * ncols];
+                ra[j] = (r[j].w & 1u) ? any_value<V>() : xcol[(int64_t) r[j].x * ncols];
+                if (DS == 1) rb[j] = (r[j].w & 2u) ? any_value<V>() : xcol[(int64_t) r[j].y * ncols];
             }
 #pragma unroll
             for (int j = 0; j < BATCH; ++j) {
@@ -1118,11 +1158,7 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
                 for (int q = 0; q < n; q += 4) {
                     V v[4];
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) {
-                        const int at = start + q + u;
-                        const V parked = stage[at < DL_CC_BLOCK ? at : DL_CC_BLOCK - 1][lane];
-                        v[u] = q + u < n ? parked : Words<V>::zero();
-                    }
+                    for (int u = 0; u < 4; ++u) v[u] = stage[q + u < n ? start + q + u : DL_CC_BLOCK][lane];
                     V carry = csa_quad(cnt[i][0], cnt[i][1], v);          // weight 4
 #pragma unroll
                     for (int p = 2; p < DL_CC_PLANES; ++p) {
