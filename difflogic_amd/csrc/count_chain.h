@@ -2,7 +2,7 @@
 // and the host-side plan builder.
 #pragma once
 
-#define DL_CC_WAVES 8                                   // waves per workgroup
+#define DL_CC_WAVES 16                                  // waves per workgroup (one workgroup per CU)
 #define DL_CC_WAVE_STEPS 8                              // steps a wave walks per block
 #define DL_CC_MAX_BLOCKS 16                             // blocks per workgroup: 16, 8, 4, 2 or 1 (chosen by the plan)
 #define DL_CC_BLOCK (DL_CC_WAVES * DL_CC_WAVE_STEPS)    // outputs parked in LDS per block

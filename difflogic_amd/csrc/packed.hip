@@ -774,6 +774,38 @@ template <> struct FullAdd<dl_u32x4> {
     }
 };
 
+// A half adder in place (plane += carry, carry = what leaves the plane), also stated as two bit operations so that
+// a ripple through the planes stays a chain of them: rearranged into wider operations on the planes' old values it
+// needs every plane twice in registers.
+template <typename V> struct HalfAdd;
+template <> struct HalfAdd<uint32_t> {
+    static __device__ __forceinline__ void run(uint32_t &plane, uint32_t &carry) {
+        const uint32_t out = __builtin_amdgcn_bitop3_b32(plane, carry, carry, 0xc0);     // plane & carry
+        plane = __builtin_amdgcn_bitop3_b32(plane, carry, carry, 0x3c);                  // plane ^ carry
+        carry = out;
+    }
+};
+template <> struct HalfAdd<uint64_t> {
+    static __device__ __forceinline__ void run(uint64_t &plane, uint64_t &carry) {
+        uint32_t pl = (uint32_t) plane, ph = (uint32_t) (plane >> 32), cl = (uint32_t) carry, ch = (uint32_t) (carry >> 32);
+        HalfAdd<uint32_t>::run(pl, cl);
+        HalfAdd<uint32_t>::run(ph, ch);
+        plane = ((uint64_t) ph << 32) | pl;
+        carry = ((uint64_t) ch << 32) | cl;
+    }
+};
+template <> struct HalfAdd<dl_u32x4> {
+    static __device__ __forceinline__ void run(dl_u32x4 &plane, dl_u32x4 &carry) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t p = plane[i], c = carry[i];
+            HalfAdd<uint32_t>::run(p, c);
+            plane[i] = p;
+            carry[i] = c;
+        }
+    }
+};
+
 template <typename V> __device__ __forceinline__ void csa(V &carry, V &sum, V a, V b, V c) {
     V cy, sm;
     FullAdd<V>::run(cy, sm, a, b, c);
@@ -1122,37 +1154,60 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
 #pragma unroll
         for (int p = 0; p < DL_CC_PLANES; ++p) cnt[i][p] = Words<V>::zero();
 
+    // Phase A walks the wave's DL_CC_WAVE_STEPS steps of the block.  With one class per wave the registers hold the
+    // rows of all of them, and they are requested before the block before is counted, so that the counting phase
+    // hides most of their latency; with two sets of counters the rows are requested in two batches as the walk
+    // needs them.  (Rows that no gate looks at are not fetched: wave-uniform flags.  Loads return in order and a
+    // wait cannot tell how many of the conditional ones were issued since, so it covers all of them: nothing in the
+    // counting phase may wait on a load.)
+    constexpr int FIRST = CPW == 1 ? DL_CC_WAVE_STEPS : DL_CC_WAVE_STEPS / 2, REST = DL_CC_WAVE_STEPS - FIRST;
+    constexpr bool AHEAD = CPW == 1;
+    dl_u32x4 r0[FIRST];
+    V ra0[FIRST], rb0[FIRST];
+    auto request = [&](auto count, int first, dl_u32x4 *r, V *ra, V *rb) {
+#pragma unroll
+        for (int j = 0; j < decltype(count)::value; ++j) {
+            r[j] = wrec[1 + first + j];
+            ra[j] = (r[j].w & 1u) ? any_value<V>() : xcol[(int64_t) r[j].x * ncols];
+            if (DS == 1) rb[j] = (r[j].w & 2u) ? any_value<V>() : xcol[(int64_t) r[j].y * ncols];
+        }
+    };
+    auto walk = [&](auto count, const dl_u32x4 *r, const V *ra, const V *rb) {
+#pragma unroll
+        for (int j = 0; j < decltype(count)::value; ++j) {
+            const V cur = vertex(ra[j], DS == 1 ? rb[j] : ra[j], r[j].z);
+            const uint32_t where = (r[j].z >> 8) & 255u;
+            if (where != 255u) stage[where][lane] = gate_apply<V>(prev, cur, gate_masks((r[j].z >> 4) & 15u));
+            prev = cur;
+        }
+    };
+    const std::integral_constant<int, FIRST> first_batch;
+    const std::integral_constant<int, REST> second_batch;
+    if constexpr (AHEAD) request(first_batch, 0, r0, ra0, rb0);
 #pragma unroll 1
     for (int b = 0; b < blocks; ++b) {
-        // phase A: walk DL_CC_WAVE_STEPS steps, BATCH at a time (their rows are requested together)
-        constexpr int BATCH = DL_CC_WAVE_STEPS % 4 == 0 ? 4 : 3;
-        static_assert(DL_CC_WAVE_STEPS % BATCH == 0, "whole batches of steps");
-#pragma unroll
-        for (int h = 0; h < DL_CC_WAVE_STEPS; h += BATCH) {
-            dl_u32x4 r[BATCH];
-            V ra[BATCH], rb[BATCH];
-#pragma unroll
-            for (int j = 0; j < BATCH; ++j) {
-                r[j] = wrec[1 + b * DL_CC_WAVE_STEPS + h + j];
-                // (wave-uniform flags: rows that no gate looks at are not fetched)
-                ra[j] = (r[j].w & 1u) ? any_value<V>() : xcol[(int64_t) r[j].x * ncols];
-                if (DS == 1) rb[j] = (r[j].w & 2u) ? any_value<V>() : xcol[(int64_t) r[j].y * ncols];
-            }
-#pragma unroll
-            for (int j = 0; j < BATCH; ++j) {
-                const V cur = vertex(ra[j], DS == 1 ? rb[j] : ra[j], r[j].z);
-                const uint32_t where = (r[j].z >> 8) & 255u;
-                if (where != 255u) stage[where][lane] = gate_apply<V>(prev, cur, gate_masks((r[j].z >> 4) & 15u));
-                prev = cur;
-            }
+        if constexpr (!AHEAD) request(first_batch, b * DL_CC_WAVE_STEPS, r0, ra0, rb0);
+        walk(first_batch, r0, ra0, rb0);
+        if constexpr (REST > 0) {
+            dl_u32x4 r[REST > 0 ? REST : 1];
+            V ra[REST > 0 ? REST : 1], rb[REST > 0 ? REST : 1];
+            request(second_batch, b * DL_CC_WAVE_STEPS + FIRST, r, ra, rb);
+            walk(second_batch, r, ra, rb);
         }
+        __builtin_amdgcn_sched_barrier(0);          // (requests moved up into the walk would not fit the registers)
+        if constexpr (AHEAD)
+            if (b + 1 < blocks) request(first_batch, (b + 1) * DL_CC_WAVE_STEPS, r0, ra0, rb0);
         __syncthreads();
         // phase B: the owner of a class adds that class's run of parked outputs to its counters
 #pragma unroll
         for (int i = 0; i < CPW; ++i) {
             const int64_t cls = wave + i * DL_CC_WAVES;
             if (cls < k) {
-                const uint32_t run = runs[(g * blocks + b) * k + cls];
+                // (a scalar load of the pair of entries that holds this one: a vector load here would have to wait
+                // for the rows requested above, which return in order)
+                const int64_t at = (g * blocks + b) * k + cls;
+                const uint32_t pair = reinterpret_cast<const uint32_t *>(runs)[at >> 1];
+                const uint32_t run = (at & 1) ? pair >> 16 : pair & 0xffffu;
                 const int start = (int) (run & 255u), n = (int) (run >> 8);
 #pragma unroll 1
                 for (int q = 0; q < n; q += 4) {
@@ -1161,11 +1216,7 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
                     for (int u = 0; u < 4; ++u) v[u] = stage[q + u < n ? start + q + u : DL_CC_BLOCK][lane];
                     V carry = csa_quad(cnt[i][0], cnt[i][1], v);          // weight 4
 #pragma unroll
-                    for (int p = 2; p < DL_CC_PLANES; ++p) {
-                        const V old = cnt[i][p];
-                        cnt[i][p] = old ^ carry;
-                        carry = old & carry;
-                    }
+                    for (int p = 2; p < DL_CC_PLANES; ++p) HalfAdd<V>::run(cnt[i][p], carry);
                 }
             }
         }
@@ -1918,6 +1969,7 @@ extern "C" int dl_logic_eval_chained_groupbitsum(const void *x, int depth, const
     if (batch < 0) return DL_ERR_INVALID_ARGUMENT;
     if (batch == 0) return DL_OK;
     if (!out || !x || !verts || !neuron || !flip || !slot || !runs || !workspace) return DL_ERR_INVALID_ARGUMENT;
+    if (!dl_aligned(runs, 4)) return DL_ERR_INVALID_ARGUMENT;       // read two entries at a time (their number is even)
     for (int l = 0; l < depth; ++l)
         if (!w[l] || (l + 1 < depth && (!a || !b || !a[l] || !b[l])) || dims[l] <= 0) return DL_ERR_INVALID_ARGUMENT;
     const int64_t per_class = out_dim / k;
