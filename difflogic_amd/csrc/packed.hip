@@ -31,6 +31,21 @@ __device__ __forceinline__ GateMasks gate_masks(uint32_t op) {
     return m;
 }
 
+// What stands in for an operand that no gate looks at: whatever the registers hold (an empty statement that the
+// compiler takes to define them), so that nothing is executed to make a value up.  Not for a place where loads
+// into the same registers may still be in flight: the compiler then waits for them before the statement.
+template <typename V> __device__ __forceinline__ V any_value() {
+    if constexpr (sizeof(V) < 4) {
+        uint32_t v;
+        asm volatile("" : "=v"(v));
+        return (V) v;
+    } else {
+        V v;
+        asm volatile("" : "=v"(v));
+        return v;
+    }
+}
+
 template <typename V> struct Splat;
 template <> struct Splat<dl_u32x4> { static __device__ __forceinline__ dl_u32x4 of(uint32_t v) { return dl_u32x4{v, v, v, v}; } };
 template <> struct Splat<dl_u32x2> { static __device__ __forceinline__ dl_u32x2 of(uint32_t v) { return dl_u32x2{v, v}; } };
@@ -45,14 +60,6 @@ template <typename V> __device__ __forceinline__ V gate_apply(V a, V b, const Ga
     const V hi = (b & Splat<V>::of(m.m11)) | (~b & Splat<V>::of(m.m10));  // value if a = 1
     const V lo = (b & Splat<V>::of(m.m01)) | (~b & Splat<V>::of(m.m00));  // value if a = 0
     return (V) ((a & hi) | (~a & lo));
-}
-
-// What stands in for an operand that no gate looks at: whatever the registers hold (an empty statement that the
-// compiler takes to define them), so that nothing is executed to make a value up.
-template <typename V> __device__ __forceinline__ V any_value() {
-    V v;
-    asm volatile("" : "=v"(v));
-    return v;
 }
 
 // Inputs a gate does not look at.  A gate id is the truth table (f(0,0) f(0,1) f(1,0) f(1,1)), MSB first; six of
@@ -381,7 +388,7 @@ template <int DS> struct alignas(DS == 3 ? 64 : DS == 2 ? 32 : 16) StepRec : Ste
 template <typename V, int D> struct TreeFoldLive {
     static __device__ __forceinline__ V run(const V *leaf, uint32_t gates, uint32_t live) {
         constexpr int half = 1 << (D - 1);
-        if (!((live >> (2 * half - 2)) & 1u)) return V{};
+        if (!((live >> (2 * half - 2)) & 1u)) return leaf[0];        // nobody looks at the result: any value does
         const V l = TreeFoldLive<V, D - 1>::run(leaf, gates, live);
         const V r = TreeFoldLive<V, D - 1>::run(leaf + half, gates >> (4 * (half - 1)), live >> (half - 1));
         return gate_apply<V>(l, r, gate_masks((gates >> (4 * (2 * half - 2))) & 15u));
@@ -464,7 +471,6 @@ __global__ __launch_bounds__(DL_BLOCK) void eval_steps_kernel(const V *__restric
         const uint32_t col = (uint32_t) (ct * DL_WAVE) + (uint32_t) lane;
         if (col >= ncols) continue;
         auto row = [&](uint32_t start) -> V {                                  // scalar row base + the lane's offset
-            if (start == DL_STEP_DEAD) return V{};                             // (wave-uniform) no gate looks at this row
             if constexpr (BUF && sizeof(V) == 16) {
                 const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *) x, 0, (int) x_bytes, 0x00027000);
                 return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int) (col * 16u), (int) (start * 16u), 0));
@@ -477,18 +483,30 @@ __global__ __launch_bounds__(DL_BLOCK) void eval_steps_kernel(const V *__restric
             const StepRec<DS> r = wrec[0];
             V leaves0[G];
 #pragma unroll
-            for (int g = 0; g < G; ++g) leaves0[g] = row(r.leaf[g]);
+            for (int g = 0; g < G; ++g) leaves0[g] = any_value<V>();
+#pragma unroll
+            for (int g = 0; g < G; ++g)
+                if (r.leaf[g] != DL_STEP_DEAD) leaves0[g] = row(r.leaf[g]);
             prev = fold_record<V, DS>(leaves0, r);
         }
 #pragma unroll 1
         for (int j = 0; j < STEPS; j += 2) {
             if (first + j >= nsteps) break;                // the schedule is a whole number of step pairs
             const StepRec<DS> ra = wrec[1 + j], rb = wrec[2 + j];
+            // a row that no gate looks at (wave-uniform marker) is not fetched, and nothing is executed in its place:
+            // the registers are "defined" here, before any request of this pair of steps is in flight
             V la[G], lb[G];
 #pragma unroll
-            for (int g = 0; g < G; ++g) la[g] = row(ra.leaf[g]);
+            for (int g = 0; g < G; ++g) {
+                la[g] = any_value<V>();
+                lb[g] = any_value<V>();
+            }
 #pragma unroll
-            for (int g = 0; g < G; ++g) lb[g] = row(rb.leaf[g]);
+            for (int g = 0; g < G; ++g)
+                if (ra.leaf[g] != DL_STEP_DEAD) la[g] = row(ra.leaf[g]);
+#pragma unroll
+            for (int g = 0; g < G; ++g)
+                if (rb.leaf[g] != DL_STEP_DEAD) lb[g] = row(rb.leaf[g]);
             const V va = fold_record<V, DS>(la, ra);
             const V vb = fold_record<V, DS>(lb, rb);
             if (ra.out != 0xffffffffu)
