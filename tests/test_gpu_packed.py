@@ -640,6 +640,9 @@ def test_pack_tensor_runs_narrow_tail_in_lds(monkeypatch):
     (784, [8000, 8000], 33, 10, 5, "random"), (784, [8000, 8000], 32, 10, 0, "unique"),
     (300, [3000, 3000], 16, 1, 0, "random"),               # one class: every output lands in one counter
     (20, [40, 64], 4, 16, 3, "self"), (40, [80, 2400], 2, 12, 0, "any"),
+    # more classes than a workgroup has waves: two sets of counters per wave
+    (50, [100, 640], 70, 20, 63, "any"), (784, [8000, 8000], 32, 32, 0, "random"), (40, [96], 5, 24, 7, "any"),
+    (30, [60, 3200], 3, 25, 0, "any"), (300, [6800], 16, 17, 0, "random"),
 ])
 def test_chained_groupbitsum(ext, in_dim, widths, W, k, pad, kind):
     """The count walked along the evaluation schedule against the oracle and the unchained
