@@ -169,10 +169,19 @@ __device__ __forceinline__ Row<COLS> gate_rows(const void *act, uint32_t rec) {
 }
 
 // carry-save adder on dwords: a + b + c = 2 * carry + sum, bit by bit
+// (two three-input bit operations, truth tables 0xe8 = majority and 0x96 = parity, stated as such: the compiler
+// otherwise rearranges a chain of adders into half as many instructions again)
 __device__ __forceinline__ void csa32(uint32_t &carry, uint32_t &sum, uint32_t a, uint32_t b, uint32_t c) {
-    const uint32_t u = a ^ b;
-    carry = (a & b) | (u & c);
-    sum = u ^ c;
+    const uint32_t cy = __builtin_amdgcn_bitop3_b32(a, b, c, 0xe8);
+    sum = __builtin_amdgcn_bitop3_b32(a, b, c, 0x96);
+    carry = cy;
+}
+
+// plane += carry in place, carry = what leaves the plane (also two stated bit operations, so that a ripple stays a chain)
+__device__ __forceinline__ void half_add32(uint32_t &plane, uint32_t &carry) {
+    const uint32_t out = __builtin_amdgcn_bitop3_b32(plane, carry, carry, 0xc0);
+    plane = __builtin_amdgcn_bitop3_b32(plane, carry, carry, 0x3c);
+    carry = out;
 }
 
 // a (NP planes, one dword each) += b (NP planes); the sum takes NP + 1 planes
@@ -490,11 +499,7 @@ __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint
                 csa32(t2b, pl[i][0], pl[i][0], y[2].d[i], y[3].d[i]);
                 csa32(carry, pl[i][1], pl[i][1], t2a, t2b);
 #pragma unroll
-                for (int p = 2; p < NP0; ++p) {                  // counter += carry * 4
-                    const uint32_t old = pl[i][p];
-                    pl[i][p] = old ^ carry;
-                    carry = old & carry;
-                }
+                for (int p = 2; p < NP0; ++p) half_add32(pl[i][p], carry);   // counter += carry * 4
             }
         }
 #pragma unroll
