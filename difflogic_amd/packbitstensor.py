@@ -14,7 +14,7 @@ from . import difflogic_cuda
 _L2_GATHER_RATE = 31e12      # B/s: row gathers + stores through the L2s when the input tile stays L2-resident
 _FABRIC_RATE = 7.5e12        # B/s: row gathers + stores between the L2s and Infinity Cache / HBM
 _WRITE_RATE = 6.1e12         # B/s: streaming stores to HBM
-_COUNT_RATE = 5.2e12         # B/s of counted rows: what the chained count kernel parks in LDS, sorts by class and adds up
+_COUNT_RATE = 5.6e12         # B/s of counted rows: what the chained count kernel parks in LDS, sorts by class and adds up
 _LIVE_INPUT = 0.75           # share of gate inputs a gate looks at when the gate ids are uniform (10 of 16 gates use both
                              # inputs, 4 one, 2 none); rows that no gate looks at are not fetched
 _TILE_BYTES = 1024           # one wave covers 64 lanes x 16 bytes of a row
@@ -46,7 +46,7 @@ def group_cost(rows_in, out, depth, words, counted):
     # The chip sweeps all output rows of one 1 KB column tile before the next, but a narrow layer
     # does not fill it: several tiles are then in flight and their input rows share the L2s.
     steps_per_workgroup = 1024 if counted else 64
-    resident_workgroups = 512 if counted else 2048
+    resident_workgroups = 256 if counted else 2048
     tiles_in_flight = max(1.0, resident_workgroups * steps_per_workgroup / max(out, 1))
     hit = min(1.0, _L2_RESIDENT_BYTES / (rows_in * _TILE_BYTES * tiles_in_flight))     # share of gathers served by L2
     through_l2 = (hit * gathered + written) / _L2_GATHER_RATE

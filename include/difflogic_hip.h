@@ -404,14 +404,15 @@ int dl_logic_eval_fused_groupbitsum(const void *x, int depth, const int64_t *con
  *       of a block so that they are sorted by class, and each class's run of slots; and *blocks:
  *       how many blocks of steps a workgroup walks (16 at most; fewer where a workgroup would
  *       otherwise count more than 255 neurons of one class).  Returns padded, or a negated
- *       dl_status: -DL_ERR_TOO_LARGE for k > 16 (the caller then uses
+ *       dl_status: -DL_ERR_TOO_LARGE for k > 32 (the caller then uses
  *       dl_logic_eval_fused_groupbitsum).
- *   slot, runs, padded_steps, blocks   that plan (slot, runs: DEVICE copies)
+ *   slot, runs, padded_steps, blocks   that plan (slot, runs: DEVICE copies; runs 4-byte aligned:
+ *       the kernel reads its entries, whose number is even, two at a time)
  *   workspace DEVICE scratch of dl_logic_eval_chained_groupbitsum_workspace_bytes(...) bytes,
  *             16-byte aligned: one 16-byte record per step (composed per call from the schedule
  *             and the current gate ids) and the bit-sliced partial counters.
  * depth is 1 or 2; a, b are read for the layer below the top one only (a[0], b[0] at depth 2).
- * DL_ERR_TOO_LARGE: rows are not whole 64-bit words or k > 16. */
+ * DL_ERR_TOO_LARGE: rows are not whole 64-bit words or k > 32. */
 int dl_count_chain_block(void);
 int64_t dl_count_chain_padded_steps(int64_t steps);
 int64_t dl_count_chain_plan_build(const int32_t *neuron, int64_t steps, int64_t out_dim, int64_t k,

@@ -189,21 +189,22 @@ def test_launch_plan_follows_the_traffic_model():
     assert pbt.plan_groups(headline, True, 16384) == [4, 2] and pbt.lds_tail(headline, 16384) == 0
     assert pbt.plan_groups(c4, True, 4096) == [2, 2] and pbt.lds_tail(c4, 4096) == 0
     assert pbt.lds_tail(c2, 16384) == 6                       # the whole narrow net runs resident in LDS
-    # measured launch times in ms (bench.py on MI355X): 4-layer prefix + 2 layers with the count
-    # (gate ids drawn uniformly: a quarter of all gate inputs are ignored by their gate and not fetched)
-    measured = {"headline": (headline, [4, 2], 16384, 1.79 + 2.32), "C4": (c4, [2, 2], 4096, 2.64 + 2.32)}
+    # measured launch times in ms on MI355X of the groups called on their own (4-layer prefix + 2 layers with the
+    # count), gate ids drawn uniformly (a quarter of all gate inputs are ignored by their gate and not fetched) but
+    # neither folded nor thinned by what the layers above look at, as they are inside PackBitsTensor
+    measured = {"headline": (headline, [4, 2], 16384, 2.18 + 2.20), "C4": (c4, [2, 2], 4096, 2.74 + 2.23)}
     for name, (dims, groups, words, ms) in measured.items():
         model = pbt.plan_cost(dims, groups, True, words) * 1e3
         assert abs(model - ms) <= 0.25 * ms, (name, model, ms)
     assert abs(pbt.lds_cost(c2, 16384) * 1e3 - 0.75) <= 0.25 * 0.75
     # single groups against their measured times: 784 -> 64000 prefixes of depth 2, 3, 4 and square 64000-wide groups
-    for depth, ms in ((2, 1.56), (3, 1.55), (4, 1.79)):
+    for depth, ms in ((2, 1.56), (3, 1.68), (4, 2.18)):
         assert abs(pbt.group_cost(784, 64000, depth, 16384, False) * 1e3 - ms) <= 0.25 * ms, depth
-    assert abs(pbt.group_cost(64000, 64000, 1, 16384, False) * 1e3 - 2.97) <= 0.25 * 2.97
-    assert abs(pbt.group_cost(64000, 64000, 2, 16384, False) * 1e3 - 3.23) <= 0.25 * 3.23
+    assert abs(pbt.group_cost(64000, 64000, 1, 16384, False) * 1e3 - 2.99) <= 0.25 * 2.99
+    assert abs(pbt.group_cost(64000, 64000, 2, 16384, False) * 1e3 - 3.00) <= 0.25 * 3.00
     # the last layers with the count, one and two layers deep
-    assert abs(pbt.group_cost(64000, 64000, 1, 16384, True) * 1e3 - 1.93) <= 0.25 * 1.93
-    assert abs(pbt.group_cost(64000, 64000, 2, 16384, True) * 1e3 - 2.32) <= 0.25 * 2.32
+    assert abs(pbt.group_cost(64000, 64000, 1, 16384, True) * 1e3 - 1.82) <= 0.25 * 1.82
+    assert abs(pbt.group_cost(64000, 64000, 2, 16384, True) * 1e3 - 2.20) <= 0.25 * 2.20
     # the model scales with the row length: the plan of a 16x shorter batch is the same, its cost 16x lower (up to
     # the per-launch overhead: 6 kernels x 3 us)
     assert pbt.plan_groups(headline, True, 1024) == [4, 2]
