@@ -489,31 +489,34 @@ __global__ __launch_bounds__(DL_BLOCK) void eval_steps_kernel(const V *__restric
                 if (r.leaf[g] != DL_STEP_DEAD) leaves0[g] = row(r.leaf[g]);
             prev = fold_record<V, DS>(leaves0, r);
         }
+        // NB steps at a time, so that the rows of up to 16 leaves are requested together whatever the subtrees' depth
+        constexpr int NB = DS >= 3 ? 2 : DS == 2 ? 4 : 8;
+        static_assert(STEPS % NB == 0 && 8 % NB == 0, "the schedule is a whole number of batches (of chunks of 8 steps)");
 #pragma unroll 1
-        for (int j = 0; j < STEPS; j += 2) {
-            if (first + j >= nsteps) break;                // the schedule is a whole number of step pairs
-            const StepRec<DS> ra = wrec[1 + j], rb = wrec[2 + j];
+        for (int j = 0; j < STEPS; j += NB) {
+            if (first + j >= nsteps) break;
+            StepRec<DS> r[NB];
+#pragma unroll
+            for (int i = 0; i < NB; ++i) r[i] = wrec[1 + j + i];
             // a row that no gate looks at (wave-uniform marker) is not fetched, and nothing is executed in its place:
-            // the registers are "defined" here, before any request of this pair of steps is in flight
-            V la[G], lb[G];
+            // the registers are "defined" here, before any request of this batch of steps is in flight
+            V leaf[NB][G];
 #pragma unroll
-            for (int g = 0; g < G; ++g) {
-                la[g] = any_value<V>();
-                lb[g] = any_value<V>();
+            for (int i = 0; i < NB; ++i)
+#pragma unroll
+                for (int g = 0; g < G; ++g) leaf[i][g] = any_value<V>();
+#pragma unroll
+            for (int i = 0; i < NB; ++i)
+#pragma unroll
+                for (int g = 0; g < G; ++g)
+                    if (r[i].leaf[g] != DL_STEP_DEAD) leaf[i][g] = row(r[i].leaf[g]);
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {
+                const V v = fold_record<V, DS>(leaf[i], r[i]);
+                if (r[i].out != 0xffffffffu)
+                    __builtin_nontemporal_store(gate_apply<V>(prev, v, gate_masks(r[i].gates >> 28)), (y + r[i].out) + col);
+                prev = v;
             }
-#pragma unroll
-            for (int g = 0; g < G; ++g)
-                if (ra.leaf[g] != DL_STEP_DEAD) la[g] = row(ra.leaf[g]);
-#pragma unroll
-            for (int g = 0; g < G; ++g)
-                if (rb.leaf[g] != DL_STEP_DEAD) lb[g] = row(rb.leaf[g]);
-            const V va = fold_record<V, DS>(la, ra);
-            const V vb = fold_record<V, DS>(lb, rb);
-            if (ra.out != 0xffffffffu)
-                __builtin_nontemporal_store(gate_apply<V>(prev, va, gate_masks(ra.gates >> 28)), (y + ra.out) + col);
-            if (rb.out != 0xffffffffu)
-                __builtin_nontemporal_store(gate_apply<V>(va, vb, gate_masks(rb.gates >> 28)), (y + rb.out) + col);
-            prev = vb;
         }
     }
 }
@@ -1807,6 +1810,7 @@ extern "C" int64_t dl_logic_eval_fused_groupbitsum_workspace_bytes(int depth, in
 }
 
 #define DL_EVAL_SCHEDULE_CHUNK 8
+static_assert(DL_EVAL_SCHEDULE_CHUNK % 8 == 0, "eval_steps_kernel walks up to 8 steps at a time");
 
 extern "C" int dl_eval_schedule_chunk(void) { return DL_EVAL_SCHEDULE_CHUNK; }
 
