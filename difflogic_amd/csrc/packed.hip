@@ -853,12 +853,12 @@ template <> struct Words<dl_u32x4> {
 template <typename V, int NP, int NQ>
 __device__ __forceinline__ void expand_counts(const uint32_t (*planes)[NP][Words<V>::n][DL_WAVE], int wave, int lane,
                                               int64_t col, bool live, int64_t cls, int64_t k, int64_t batch,
-                                              int32_t *__restrict__ out) {
+                                              int32_t *__restrict__ out, int32_t base = 0) {
     constexpr int NC = Words<V>::n;
     constexpr int BITS = 8 * NC;
     int32_t cnt[BITS];
 #pragma unroll
-    for (int s = 0; s < BITS; ++s) cnt[s] = 0;
+    for (int s = 0; s < BITS; ++s) cnt[s] = base;
     const int first_bit = BITS * wave;
     const int comp = first_bit >> 5, shift = first_bit & 31;
 #pragma unroll 1
@@ -1099,6 +1099,70 @@ __global__ __launch_bounds__(DL_BLOCK) void count_partial_kernel(const V *__rest
 //   rec[i + 1] = { la, lb, sub gate | top gate << 4 | slot << 8 } for step i, rec[0] for the
 //   vertex before step 0; a wave that starts at step f seeds its chain from rec[f].
 // ------------------------------------------------------------------------------------------
+// Neurons of the top layer whose gate is constant (0 or 15, as it stands after constants were folded into it)
+// output the same word for every sample: they are not parked and not counted.  What the ones among them add to
+// every sample's count of their class goes into the result at the very end (count_finish_kernel's base).
+__global__ __launch_bounds__(DL_BLOCK) void count_constant_ones_kernel(const uint8_t *__restrict__ w_top, int64_t per_class,
+                                                                       int32_t *__restrict__ ones) {
+    __shared__ int32_t part[DL_BLOCK / DL_WAVE];
+    const int64_t cls = blockIdx.x;
+    int32_t n = 0;
+    for (int64_t i = threadIdx.x; i < per_class; i += DL_BLOCK) n += (w_top[cls * per_class + i] & 15u) == 15u;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) n += __shfl_xor(n, off);
+    if (dl_lane() == 0) part[dl_wave_in_block()] = n;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int32_t total = 0;
+        for (int i = 0; i < DL_BLOCK / DL_WAVE; ++i) total += part[i];
+        ones[cls] = total;
+    }
+}
+
+// The plan of a wiring (slot, runs: every neuron parked, a block's outputs sorted by class) thinned for this call:
+// one wave per block takes the constant neurons out, moves the others of their class up and shortens the
+// class's run.  Steps are numbered as the count kernel walks them (workgroup, wave, block, step); lane c keeps
+// count of the constant neurons of class c met so far.
+static_assert(DL_CC_BLOCK % DL_WAVE == 0 && DL_CC_MAX_CLASSES <= DL_WAVE, "a wave covers a block in whole rounds, a lane per class");
+__global__ __launch_bounds__(DL_BLOCK) void count_chain_thin_kernel(const int32_t *__restrict__ neuron,
+                                                                    const uint8_t *__restrict__ w_top,
+                                                                    const uint8_t *__restrict__ slot,
+                                                                    const uint16_t *__restrict__ runs, int64_t steps,
+                                                                    int64_t per_class, int64_t k, int blocks,
+                                                                    int64_t nblocks, uint8_t *__restrict__ slot_call,
+                                                                    uint16_t *__restrict__ runs_call) {
+    const int lane = dl_lane();
+    const int64_t gb = (int64_t) blockIdx.x * (DL_BLOCK / DL_WAVE) + dl_wave_in_block();      // (workgroup g, block b)
+    if (gb >= nblocks) return;
+    const int64_t g = gb / blocks, b = gb % blocks;
+    const int64_t wg_steps = (int64_t) DL_CC_BLOCK * blocks, span = (int64_t) DL_CC_WAVE_STEPS * blocks;
+    uint32_t gone = 0;
+    for (int first = 0; first < DL_CC_BLOCK; first += DL_WAVE) {
+        const int i = first + lane;                           // the order in which the plan numbered a class's slots
+        const int64_t s = g * wg_steps + (i / DL_CC_WAVE_STEPS) * span + b * DL_CC_WAVE_STEPS + i % DL_CC_WAVE_STEPS;
+        const int32_t n = s < steps ? neuron[s] : -1;
+        int cls = -1;
+        bool constant = false;
+        if (n >= 0) {
+            cls = (int) (n / per_class);
+            const uint32_t gate = w_top[n] & 15u;
+            constant = gate == 0u || gate == 15u;
+        }
+        uint32_t before = 0;
+        for (int c = 0; c < (int) k; ++c) {
+            const uint64_t met = __ballot(cls == c && constant);
+            const uint32_t carried = (uint32_t) __builtin_amdgcn_readlane((int) gone, c);
+            if (cls == c) before = carried + (uint32_t) __popcll(met & ((1ull << lane) - 1ull));
+            if (lane == c) gone += (uint32_t) __popcll(met);
+        }
+        slot_call[s] = n >= 0 && !constant ? (uint8_t) (slot[s] - before) : (uint8_t) 255;
+    }
+    if (lane < k) {
+        const uint32_t run = runs[gb * k + lane];
+        runs_call[gb * k + lane] = (uint16_t) ((run & 255u) | (((run >> 8) - gone) << 8));
+    }
+}
+
 template <int DS>
 __global__ __launch_bounds__(DL_BLOCK) void compose_count_chain_kernel(TreeTables t, const int32_t *__restrict__ verts,
                                                                        const int32_t *__restrict__ neuron,
@@ -1259,7 +1323,7 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
 template <typename V, int NP>
 __global__ __launch_bounds__(DL_BLOCK) void count_finish_kernel(const V *__restrict__ partial, int32_t *__restrict__ out,
                                                                 int64_t ncols, int64_t chunks_per_class, int64_t k,
-                                                                int64_t batch) {
+                                                                int64_t batch, const int32_t *__restrict__ base) {
     constexpr int NC = Words<V>::n;
     __shared__ uint32_t planes_lds[4][NP][NC][DL_WAVE];
     const int wave = dl_wave_in_block();
@@ -1285,7 +1349,8 @@ __global__ __launch_bounds__(DL_BLOCK) void count_finish_kernel(const V *__restr
         for (int p = 0; p < NP; ++p) planes_lds[wave][p][c][lane] = Words<V>::get(acc[p], c);
     }
     __syncthreads();
-    expand_counts<V, NP, 4>(planes_lds, wave, lane, col, live, cls, k, batch, out);
+    // (base: what the class's neurons that were left out of the partial counters add to every sample)
+    expand_counts<V, NP, 4>(planes_lds, wave, lane, col, live, cls, k, batch, out, base ? base[cls] : 0);
 }
 
 // Any word width / row length: one thread per (sample, class), like the reference, but with
@@ -1355,13 +1420,13 @@ int launch_count_fused_v(const void *x, const int32_t *leaves, const uint64_t *g
     const int64_t top = chunks_per_class * DL_COUNT_ROWS;
     if (top < (1LL << 13))
         DL_LAUNCH((count_finish_kernel<V, 13>), grid, dim3(DL_BLOCK), 0, s, (const V *) scratch, out, ncols,
-                           chunks_per_class, k, batch);
+                           chunks_per_class, k, batch, (const int32_t *) nullptr);
     else if (top < (1LL << 18))
         DL_LAUNCH((count_finish_kernel<V, 18>), grid, dim3(DL_BLOCK), 0, s, (const V *) scratch, out, ncols,
-                           chunks_per_class, k, batch);
+                           chunks_per_class, k, batch, (const int32_t *) nullptr);
     else
         DL_LAUNCH((count_finish_kernel<V, 31>), grid, dim3(DL_BLOCK), 0, s, (const V *) scratch, out, ncols,
-                           chunks_per_class, k, batch);
+                           chunks_per_class, k, batch, (const int32_t *) nullptr);
     return dl_launch_status();
 }
 
@@ -1933,12 +1998,18 @@ int64_t count_chain_partial_bytes(int64_t padded_steps, int blocks, int64_t k, i
     return tiles * k * (padded_steps / (DL_CC_BLOCK * blocks)) * DL_CC_PLANES * DL_WAVE * vec;
 }
 
+// the plan as thinned per call: slot [padded], runs [blocks of the whole schedule x k], ones [k]; each 16-byte aligned
+int64_t count_chain_call_plan_bytes(int64_t padded_steps, int64_t k) {
+    const int64_t nblocks = padded_steps / DL_CC_BLOCK;
+    return dl_ceil_div(padded_steps, 16) * 16 + dl_ceil_div(nblocks * k * 2, 16) * 16 + dl_ceil_div(k * 4, 16) * 16;
+}
+
 bool valid_cc_blocks(int blocks) { return blocks == 1 || blocks == 2 || blocks == 4 || blocks == 8 || blocks == 16; }
 
 template <typename V, int DS>
 int launch_count_chain(const void *x, const dl_u32x4 *rec, const uint16_t *runs, void *partial, int32_t *out,
-                       int64_t row_bytes, int64_t padded_steps, int blocks, int64_t per_class, int64_t k, int64_t batch,
-                       hipStream_t s) {
+                       const int32_t *ones, int64_t row_bytes, int64_t padded_steps, int blocks, int64_t per_class,
+                       int64_t k, int64_t batch, hipStream_t s) {
     const int64_t ncols = row_bytes / (int64_t) sizeof(V);
     const int64_t tiles = dl_ceil_div(ncols, DL_WAVE);
     const int64_t nwg = padded_steps / (DL_CC_BLOCK * blocks);
@@ -1954,11 +2025,14 @@ int launch_count_chain(const void *x, const dl_u32x4 *rec, const uint16_t *runs,
     if (st != DL_OK) return st;
     const dim3 fgrid((unsigned) tiles, (unsigned) k);
     if (per_class < (1LL << 13))
-        DL_LAUNCH((count_finish_kernel<V, 13>), fgrid, dim3(DL_BLOCK), 0, s, (const V *) partial, out, ncols, nwg, k, batch);
+        DL_LAUNCH((count_finish_kernel<V, 13>), fgrid, dim3(DL_BLOCK), 0, s, (const V *) partial, out, ncols, nwg, k, batch,
+                  ones);
     else if (per_class < (1LL << 18))
-        DL_LAUNCH((count_finish_kernel<V, 18>), fgrid, dim3(DL_BLOCK), 0, s, (const V *) partial, out, ncols, nwg, k, batch);
+        DL_LAUNCH((count_finish_kernel<V, 18>), fgrid, dim3(DL_BLOCK), 0, s, (const V *) partial, out, ncols, nwg, k, batch,
+                  ones);
     else
-        DL_LAUNCH((count_finish_kernel<V, 31>), fgrid, dim3(DL_BLOCK), 0, s, (const V *) partial, out, ncols, nwg, k, batch);
+        DL_LAUNCH((count_finish_kernel<V, 31>), fgrid, dim3(DL_BLOCK), 0, s, (const V *) partial, out, ncols, nwg, k, batch,
+                  ones);
     return dl_launch_status();
 }
 
@@ -1971,7 +2045,8 @@ extern "C" int64_t dl_logic_eval_chained_groupbitsum_workspace_bytes(int64_t pad
         return 0;
     const int64_t row_bytes = words * (bit_count / 8);
     if (row_bytes % 8 != 0) return 0;
-    return (padded_steps + 1) * 16 + count_chain_partial_bytes(padded_steps, blocks, k, row_bytes);
+    return (padded_steps + 1) * 16 + count_chain_partial_bytes(padded_steps, blocks, k, row_bytes) +
+           count_chain_call_plan_bytes(padded_steps, k);
 }
 
 extern "C" int dl_logic_eval_chained_groupbitsum(const void *x, int depth, const int64_t *const *a, const int64_t *const *b,
@@ -2010,21 +2085,33 @@ extern "C" int dl_logic_eval_chained_groupbitsum(const void *x, int depth, const
         t.w[l] = w[l];
     }
     dl_u32x4 *rec = (dl_u32x4 *) workspace;
-    void *partial = (char *) workspace + (padded_steps + 1) * 16;
+    char *partial = (char *) workspace + (padded_steps + 1) * 16;
+    const int64_t nblocks = padded_steps / DL_CC_BLOCK;
+    uint8_t *slot_call = (uint8_t *) (partial + count_chain_partial_bytes(padded_steps, blocks, k, row_bytes));
+    uint16_t *runs_call = (uint16_t *) (slot_call + dl_ceil_div(padded_steps, 16) * 16);
+    int32_t *ones = (int32_t *) ((char *) runs_call + dl_ceil_div(nblocks * k * 2, 16) * 16);
+    const uint8_t *w_top = w[depth - 1];
+    DL_LAUNCH(count_constant_ones_kernel, dim3((unsigned) k), dim3(DL_BLOCK), 0, s, w_top, per_class, ones);
+    int st = dl_launch_status();
+    if (st != DL_OK) return st;
+    DL_LAUNCH(count_chain_thin_kernel, dim3((unsigned) dl_ceil_div(nblocks, DL_BLOCK / DL_WAVE)), dim3(DL_BLOCK), 0, s, neuron, w_top,
+              slot, runs, steps, per_class, k, blocks, nblocks, slot_call, runs_call);
+    st = dl_launch_status();
+    if (st != DL_OK) return st;
     const dim3 cgrid((unsigned) dl_ceil_div(padded_steps + 1, DL_BLOCK));
     if (depth == 2)
-        DL_LAUNCH(compose_count_chain_kernel<1>, cgrid, dim3(DL_BLOCK), 0, s, t, verts, neuron, flip, slot, steps,
+        DL_LAUNCH(compose_count_chain_kernel<1>, cgrid, dim3(DL_BLOCK), 0, s, t, verts, neuron, flip, slot_call, steps,
                   padded_steps, rec);
     else
-        DL_LAUNCH(compose_count_chain_kernel<0>, cgrid, dim3(DL_BLOCK), 0, s, t, verts, neuron, flip, slot, steps,
+        DL_LAUNCH(compose_count_chain_kernel<0>, cgrid, dim3(DL_BLOCK), 0, s, t, verts, neuron, flip, slot_call, steps,
                   padded_steps, rec);
-    const int st = dl_launch_status();
+    st = dl_launch_status();
     if (st != DL_OK) return st;
     const bool wide = row_bytes % 16 == 0 && dl_aligned(x, 16);
     if (depth == 2) {
-        if (wide) return launch_count_chain<dl_u32x4, 1>(x, rec, runs, partial, out, row_bytes, padded_steps, blocks, per_class, k, batch, s);
-        return launch_count_chain<uint64_t, 1>(x, rec, runs, partial, out, row_bytes, padded_steps, blocks, per_class, k, batch, s);
+        if (wide) return launch_count_chain<dl_u32x4, 1>(x, rec, runs_call, partial, out, ones, row_bytes, padded_steps, blocks, per_class, k, batch, s);
+        return launch_count_chain<uint64_t, 1>(x, rec, runs_call, partial, out, ones, row_bytes, padded_steps, blocks, per_class, k, batch, s);
     }
-    if (wide) return launch_count_chain<dl_u32x4, 0>(x, rec, runs, partial, out, row_bytes, padded_steps, blocks, per_class, k, batch, s);
-    return launch_count_chain<uint64_t, 0>(x, rec, runs, partial, out, row_bytes, padded_steps, blocks, per_class, k, batch, s);
+    if (wide) return launch_count_chain<dl_u32x4, 0>(x, rec, runs_call, partial, out, ones, row_bytes, padded_steps, blocks, per_class, k, batch, s);
+    return launch_count_chain<uint64_t, 0>(x, rec, runs_call, partial, out, ones, row_bytes, padded_steps, blocks, per_class, k, batch, s);
 }

@@ -674,6 +674,38 @@ def test_chained_groupbitsum(ext, in_dim, widths, W, k, pad, kind):
     assert torch.equal(got, ext.eval_fused_groupbitsum(_dev(x), dev_layers, pad, k))
 
 
+@pytest.mark.parametrize("top", ["ones", "zeros", "mixed", "one class constant"])
+def test_chained_groupbitsum_leaves_constant_neurons_out(ext, top):
+    """Neurons of the top layer whose gate is constant are neither parked nor counted; the ones among them are added
+    to every sample's count at the end.  All of them constant, none of a class, or every other one: the oracle's counts."""
+    rng = np.random.default_rng(5)
+    in_dim, widths, W, k, pad = 90, [300, 2400], 5, 12, 9
+    x = rng.integers(np.iinfo(np.int64).min, np.iinfo(np.int64).max, (in_dim, W), dtype=np.int64, endpoint=True)
+    layers = random_layers(rng, in_dim, widths)
+    a, b, op = layers[-1]
+    op = op.copy()
+    if top == "ones":
+        op[:] = 15
+    elif top == "zeros":
+        op[:] = 0
+    elif top == "mixed":
+        op[::2] = np.where(np.arange(len(op[::2])) % 3 == 0, 0, 15)
+    else:
+        op[200:400] = 15                                     # class 1 of 12 (200 neurons each)
+    layers[-1] = (a, b, op)
+    dev_layers = [tuple(_dev(t) for t in l) for l in layers]
+    y = x
+    for la, lb, lop in layers:
+        y = po.eval_layer(y, la, lb, lop)
+    want = po.groupbitsum(y, pad, k)
+    for depth in (2, 1):
+        xin = x if depth == 2 else po.eval_layer(x, *layers[0])
+        got = ext.eval_chained_groupbitsum(_dev(xin), dev_layers[-depth:], pad, k)
+        assert got is not None and np.array_equal(got.cpu().numpy(), want), depth
+    if top == "ones":
+        assert (want == widths[-1] // k).all()
+
+
 def test_chained_groupbitsum_declines_where_it_does_not_apply(ext):
     rng = np.random.default_rng(3)
     layers, dev_layers = _chain(rng, 30, [60, 170])
