@@ -410,7 +410,9 @@ int dl_logic_eval_fused_groupbitsum(const void *x, int depth, const int64_t *con
  *       the kernel reads its entries, whose number is even, two at a time)
  *   workspace DEVICE scratch of dl_logic_eval_chained_groupbitsum_workspace_bytes(...) bytes,
  *             16-byte aligned: one 16-byte record per step (composed per call from the schedule
- *             and the current gate ids) and the bit-sliced partial counters.
+ *             and the current gate ids), the bit-sliced partial counters, and the plan as
+ *             thinned for this call (neurons of the top layer whose gate is constant, 0 or 15,
+ *             are neither parked nor counted; what the ones add is put into the result at the end).
  * depth is 1 or 2; a, b are read for the layer below the top one only (a[0], b[0] at depth 2).
  * DL_ERR_TOO_LARGE: rows are not whole 64-bit words or k > 32. */
 int dl_count_chain_block(void);
