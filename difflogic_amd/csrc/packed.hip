@@ -1182,7 +1182,7 @@ __global__ __launch_bounds__(DL_BLOCK) void compose_count_chain_kernel(TreeTable
     }
     uint32_t where = 255;
     // the vertex is the second input of step i - 1's neuron and the first input of step i's; rows that no gate
-    // looks at are not fetched (.w: bit 0 = skip la, bit 1 = skip lb)
+    // looks at are not fetched (.w: bit 0 = skip la, bit 1 = skip lb, bit 2 = the vertex itself is not looked at)
     bool needed = false;
     if (i >= 1) {
         const int64_t s = i - 1;
@@ -1202,6 +1202,7 @@ __global__ __launch_bounds__(DL_BLOCK) void compose_count_chain_kernel(TreeTable
     uint32_t skip = 0;
     if (!needed || (DS == 1 && !gate_uses_a(bits & 15u))) skip |= 1u;
     if (DS == 1 && (!needed || !gate_uses_b(bits & 15u))) skip |= 2u;
+    if (!needed) skip |= 4u;                                  // nobody looks at the vertex: not evaluated either
     rec[i] = dl_u32x4{la, lb, bits | (where << 8), skip};
 }
 
@@ -1260,7 +1261,8 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
     auto walk = [&](auto count, const dl_u32x4 *r, const V *ra, const V *rb) {
 #pragma unroll
         for (int j = 0; j < decltype(count)::value; ++j) {
-            const V cur = vertex(ra[j], DS == 1 ? rb[j] : ra[j], r[j].z);
+            V cur = ra[j];
+            if (DS == 1 && !(r[j].w & 4u)) cur = vertex(ra[j], rb[j], r[j].z);
             const uint32_t where = (r[j].z >> 8) & 255u;
             if (where != 255u) stage[where][lane] = gate_apply<V>(prev, cur, gate_masks((r[j].z >> 4) & 15u));
             prev = cur;
