@@ -22,8 +22,10 @@ moves fewer bytes than their algorithmic sum, so two figures are kept apart:
 When the committed traffic summary was taken from other kernel sources than the built ones,
 `traffic` is null, a warning goes to stderr, and `achieved`/`frac` fall back to null.
 
-`cpu_baseline` times the CPU oracle (single thread, like the reference's generated C) on a bounded
-sample.  `extra.configs` holds the other BASELINE configurations: C2 and C4 (packed inference,
+`cpu_baseline` is the reference's CPU inference path: the C text CompiledLogicNet generates for the
+headline net, gcc-compiled as the reference's driver does and timed single-threaded on a bounded sample.
+gcc needs minutes for 384 000 gates, so it is started as a child process before anything touches the GPU
+and collected after the GPU work; the table interpreter's figure is kept beside it.  `extra.configs` holds the other BASELINE configurations: C2 and C4 (packed inference,
 checked bit-exactly against the CPU interpreter on the first 4096 samples of the full-batch
 result), C3 and C5 (fp32 training forward+backward, with and without the Adam step, eager and as a
 replayed HIP graph) and C1 on the GPU next to the CPU python-implementation step.
@@ -67,12 +69,16 @@ def parse():
     ap.add_argument("--only", default="", help="comma list out of c1,c2,c3,c4,c5: run only these extra configurations")
     ap.add_argument("--skip-headline", action="store_true",
                     help="profiling aid: run only the configurations selected with --only and print their results")
+    ap.add_argument("--gate-mix", default="uniform", choices=("uniform", "two_input_gates_only", "half_pass_through"),
+                    help="profiling aid: run the headline with this gate mix (see GATE_MIXES) instead of the BASELINE config's")
     ap.add_argument("--cpu-sample-log2", type=int, default=18)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 4 plain device copies of 1 GiB (for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE)")
-    ap.add_argument("--cpu-generated-c", action="store_true",
-                    help="also time the reference's own CPU inference path on the host: the generated C of the headline "
-                         "net and of C2, gcc-compiled as experiments/main.py:362 does (minutes of compile time)")
+    ap.add_argument("--no-cpu-generated-c", action="store_true",
+                    help="do not compile and time the reference's own CPU inference path (the generated C of the headline "
+                         "net and of C2, gcc-compiled as experiments/main.py:362 does: minutes of gcc next to the GPU work); "
+                         "cpu_baseline is then the table interpreter")
+    ap.add_argument("--cpu-generated-c-sample-log2", type=int, default=18)
     ap.add_argument("--ceilings", action="store_true",
                     help="measure streaming read/write/copy and row-gather ceilings instead of the benchmark")
     return ap.parse_args()
@@ -113,16 +119,54 @@ def thresholded_input(torch, B, seed, as_float=False):
     return out
 
 
+LOGIT_SEED_OFFSET = 1000
+
+
 def packed_model(torch, dl, F, widths, k, seed=0, connections="random"):
+    """Flatten -> LogicLayer x L -> GroupSum as a user of the reference writes it.  The wiring is what LogicLayer
+    draws after torch.manual_seed(seed); the gate logits are N(0,1) from a CPU generator of their own (seed +
+    LOGIT_SEED_OFFSET) copied into the layers, so that the same net can be made without a GPU (cpu_side_net)."""
     torch.manual_seed(seed)
     mods, d = [torch.nn.Flatten()], F
     for w in widths:
         mods.append(dl.LogicLayer(d, w, connections=connections))
         d = w
+    g = torch.Generator().manual_seed(seed + LOGIT_SEED_OFFSET)
+    with torch.no_grad():
+        for m in mods[1:]:
+            m.weights.copy_(torch.randn(m.out_dim, 16, generator=g))
     return torch.nn.Sequential(*mods, dl.GroupSum(k, 30.0)).eval()
 
 
-def packed_run(torch, dl, model, x, k, steps, warmup):
+def cpu_side_net(torch, F, widths, seed=0, connections="random"):
+    """[(a, b, gate ids)] (numpy) of the net packed_model builds from the same arguments, made on the CPU alone, so
+    that the compile of its generated C can start before anything touches the GPU: the wiring as LogicLayer draws it
+    (oracle.connections: the CPU default generator after torch.manual_seed(seed); the layers' initial weights come
+    from the device's generator and do not advance it), the gate ids as the argmax of packed_model's logits.
+    Part of the CPU-baseline leg; main() checks the GPU model's own tables against these."""
+    import numpy as np
+    from oracle import connections as oc
+    draw = {"random": oc.random_connections, "unique": oc.unique_connections}[connections]
+    torch.manual_seed(seed)
+    wiring, d = [], F
+    for w in widths:
+        wiring.append(draw(d, w))
+        d = w
+    g = torch.Generator().manual_seed(seed + LOGIT_SEED_OFFSET)
+    return [(a.numpy(), b.numpy(), torch.randn(len(a), 16, generator=g).argmax(-1).numpy().astype(np.uint8))
+            for a, b in wiring]
+
+
+def gate_mix(layers):
+    """Share of gate ids, over all layers, that look at both inputs / one input / none."""
+    import numpy as np
+    ids = np.concatenate([np.asarray(l[2]) for l in layers])
+    one = np.isin(ids, (3, 5, 10, 12)).mean()
+    none = np.isin(ids, (0, 15)).mean()
+    return {"two_input": round(float(1 - one - none), 4), "one_input": round(float(one), 4), "constant": round(float(none), 4)}
+
+
+def packed_run(torch, dl, model, x, k, steps, warmup, graph=True):
     """Times `steps` passes of pack -> layers -> counts over x; returns (samples/s, ms per step,
     per-launch table, last output).  Every binding call of the path is bracketed by events on the
     launch stream."""
@@ -210,21 +254,23 @@ def packed_run(torch, dl, model, x, k, steps, warmup):
             setattr(ext, n, real[n])
         record["on"] = False
 
-    # the same step captured once into a HIP graph and replayed (difflogic_amd.graphs.GraphedPackedInference;
-    # the batch sits in the graph's static input buffer, as the eager step's sits in x)
-    from difflogic_amd.graphs import GraphedPackedInference
-    graphed = GraphedPackedInference(model, x, bit_count=64)
-    graphed()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        replayed = graphed()
-    torch.cuda.synchronize()
-    graph_ms = (time.perf_counter() - t0) / steps * 1e3
-    graph_info = {"ms_per_step": round(graph_ms, 4), "samples_per_s": round(B / graph_ms * 1e3, 1),
-                  "equal_to_eager": bool(torch.equal(replayed, out)),
-                  "eager_ms_per_step_with_launch_events": round(elapsed_with_events / steps * 1e3, 4)}
-    del graphed, replayed
+    graph_info = None
+    if graph:
+        # the same step captured once into a HIP graph and replayed (difflogic_amd.graphs.GraphedPackedInference;
+        # the batch sits in the graph's static input buffer, as the eager step's sits in x)
+        from difflogic_amd.graphs import GraphedPackedInference
+        graphed = GraphedPackedInference(model, x, bit_count=64)
+        graphed()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            replayed = graphed()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t0) / steps * 1e3
+        graph_info = {"ms_per_step": round(graph_ms, 4), "samples_per_s": round(B / graph_ms * 1e3, 1),
+                      "equal_to_eager": bool(torch.equal(replayed, out)),
+                      "eager_ms_per_step_with_launch_events": round(elapsed_with_events / steps * 1e3, 4)}
+        del graphed, replayed
 
     per_kernel = {}
     for label, by, s, e in launches:
@@ -261,43 +307,22 @@ def packed_headline(args, torch, dl):
     F, width, L, k = args.features, args.width, args.layers, 10
     B = 1 << args.batch_log2
     model = packed_model(torch, dl, F, [width] * L, k)
+    if args.gate_mix != "uniform":
+        apply_gate_mix(torch, dl, model, args.gate_mix)
     x = bernoulli_input(torch, B, F, 1)
     value, ms_per_step, per_kernel, out, first_ms, graph_info = packed_run(torch, dl, model, x, k, args.steps, args.warmup)
 
-    # dominant kernel = the launch kind that takes the most time in a step
-    dom = max(per_kernel, key=lambda kk: per_kernel[kk]["ms"])
-    avg_ms = per_kernel[dom]["ms"] / per_kernel[dom]["n"]
-    alg = per_kernel[dom]["bytes"]
-    alg_gbps = alg / (avg_ms * 1e-3) / 1e9
     table, note = load_traffic()
-    entry = table.get(dom) or {}
-    traffic = entry.get("hbm_bytes_per_launch")
-    achieved = traffic / (avg_ms * 1e-3) / 1e9 if traffic else None
-    roofline = {
-        "bound": entry.get("bound", "hbm") if traffic else "hbm (traffic of this build not measured)",
-        "kernel": dom,
-        "achieved": round(achieved, 1) if achieved else None, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4) if achieved else None,
-        "traffic": traffic,
-        "achieved_is": "measured L2<->fabric bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a plain "
-                       "copy) / launch time; reads served by the Infinity Cache are included",
-        "algorithmic_bytes_per_launch": int(alg), "alg_GBps": round(alg_gbps, 1),
-        "alg_over_peak": round(alg_gbps / HBM_PEAK_GBS, 4),
-        "avg_launch_ms": round(avg_ms, 4), "launches_timed": per_kernel[dom]["n"],
-        "launches_timed_in": "a second pass of the same steps with HIP events around every launch; the pass that yields "
-                             "`value` runs without them (timing events drain the queue between kernels)",
-        "fully_fused_floor_bytes_per_sample": F // 8 + 4 * k,
-    }
+    prefix = "" if args.gate_mix == "uniform" else args.gate_mix + ": "
+    kernels, roofline = launch_rooflines(per_kernel, args.steps, table, prefix)
+    roofline["achieved_is"] = ("measured L2<->fabric bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a plain "
+                               "copy) / launch time; reads served by the Infinity Cache are included")
+    roofline["launches_timed_in"] = ("a second pass of the same steps with HIP events around every launch; the pass that "
+                                     "yields `value` runs without them (timing events drain the queue between kernels)")
+    roofline["fully_fused_floor_bytes_per_sample"] = F // 8 + 4 * k
     if note:
         roofline["traffic_note"] = note
     total_alg = sum(v["bytes"] * v["n"] for v in per_kernel.values()) / args.steps
-    kernels = kernel_table(per_kernel, args.steps)
-    for label, row in kernels.items():
-        e = table.get(label)
-        if e and e.get("hbm_bytes_per_launch"):
-            row["traffic_GB"] = round(e["hbm_bytes_per_launch"] / 1e9, 3)
-            row["traffic_GBps"] = round(e["hbm_bytes_per_launch"] / (row["avg_ms"] * 1e-3) / 1e9, 1)
-            row["bound"] = e.get("bound")
     info = {
         "kernels": kernels,
         "path_algorithmic_GB_per_step": round(total_alg / 1e9, 2),
@@ -308,35 +333,88 @@ def packed_headline(args, torch, dl):
     }
     if not args.no_configs:
         info["other_word_widths"] = word_width_variants(torch, dl, model, x, out)
-        info["two_input_gates_only"] = two_input_gates_variant(torch, dl, model, x)
+        if args.gate_mix == "uniform":
+            info["other_gate_mixes"] = gate_mix_variants(torch, dl, model, x, table, not args.no_cpu_baseline)
     return value, ms_per_step, roofline, info, model, x, out
 
 
-def two_input_gates_variant(torch, dl, model, x):
-    """The same net with every gate drawn from the ten that look at both of their inputs.  The packed kernels do
-    not fetch rows that no gate looks at (six of the sixteen gates ignore an input), so the headline, whose gate
-    ids are uniform over all sixteen, moves fewer bytes than a net without such gates: this is that net."""
-    import copy
-    two_input = torch.tensor([1, 2, 4, 6, 7, 8, 9, 11, 13, 14], device="cuda")
-    net = copy.deepcopy(model)
-    g = torch.Generator(device="cuda").manual_seed(3)
+GATE_MIXES = {
+    # name: (pool the gate ids are drawn from uniformly, what it stands for)
+    "uniform": (list(range(16)), "N(0,1) gate logits: ids uniform over the 16 gates (the BASELINE config)"),
+    "two_input_gates_only": ([1, 2, 4, 6, 7, 8, 9, 11, 13, 14],
+                             "every gate looks at both of its inputs: nothing for the packed kernels to skip"),
+    "half_pass_through": ([3, 5, 10, 12] * 4 + list(range(16)),
+                          "half of the ids from {a, b, not a, not b}, the other half uniform over all 16: the "
+                          "pass-through-rich end that trained nets are reported to lie towards"),
+}
+
+
+def apply_gate_mix(torch, dl, model, mix, seed=3):
+    """Overwrites the gate logits of `model` with one-hot rows whose ids are drawn from GATE_MIXES[mix]."""
+    pool = torch.tensor(GATE_MIXES[mix][0], device="cuda")
+    g = torch.Generator(device="cuda").manual_seed(seed)
     with torch.no_grad():
-        for m in net:
+        for m in model:
             if isinstance(m, dl.LogicLayer):
-                ids = two_input[torch.randint(0, 10, (m.out_dim,), device="cuda", generator=g)]
+                ids = pool[torch.randint(0, len(pool), (m.out_dim,), device="cuda", generator=g)]
                 m.weights.copy_(torch.nn.functional.one_hot(ids, 16).float())
 
-    def step():
-        with torch.no_grad():
-            return net(dl.PackBitsTensor(x, bit_count=64))
-    step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(5):
-        step()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) / 5 * 1e3
-    return {"ms_per_step": round(ms, 4), "samples_per_s": round(x.shape[0] / ms * 1e3, 1)}
+
+def launch_rooflines(per_kernel, steps, table, prefix=""):
+    """Per-launch table of a packed run, with the measured traffic of each launch where the committed --pmc summary
+    has it (keys of profiles/packed_kernel_traffic.json: `prefix` + the launch label), and the roofline block of
+    the launch kind that takes the most time."""
+    kernels = kernel_table(per_kernel, steps)
+    for label, row in kernels.items():
+        e = table.get(prefix + label)
+        if e and e.get("hbm_bytes_per_launch"):
+            row["traffic_GB"] = round(e["hbm_bytes_per_launch"] / 1e9, 3)
+            row["traffic_GBps"] = round(e["hbm_bytes_per_launch"] / (row["avg_ms"] * 1e-3) / 1e9, 1)
+            row["frac_hbm_traffic"] = round(row["traffic_GBps"] / HBM_PEAK_GBS, 4)
+            row["bound"] = e.get("bound")
+    dom = max(per_kernel, key=lambda kk: per_kernel[kk]["ms"])
+    avg_ms = per_kernel[dom]["ms"] / per_kernel[dom]["n"]
+    alg = per_kernel[dom]["bytes"]
+    alg_gbps = alg / (avg_ms * 1e-3) / 1e9
+    entry = table.get(prefix + dom) or {}
+    traffic = entry.get("hbm_bytes_per_launch")
+    achieved = traffic / (avg_ms * 1e-3) / 1e9 if traffic else None
+    roofline = {
+        "bound": entry.get("bound", "hbm") if traffic else "hbm (traffic of this build not measured)",
+        "kernel": dom,
+        "achieved": round(achieved, 1) if achieved else None, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4) if achieved else None,
+        "traffic": traffic,
+        "algorithmic_bytes_per_launch": int(alg), "alg_GBps": round(alg_gbps, 1),
+        "alg_over_peak": round(alg_gbps / HBM_PEAK_GBS, 4),
+        "avg_launch_ms": round(avg_ms, 4), "launches_timed": per_kernel[dom]["n"],
+    }
+    return kernels, roofline
+
+
+def gate_mix_variants(torch, dl, model, x, table, check_cpu):
+    """The headline net and batch with other gate mixes.  The packed kernels fetch, evaluate and write nothing that
+    no gate looks at (six of the sixteen gates ignore an input, constants fold upwards), so the headline, whose gate
+    ids are uniform over all sixteen, moves fewer bytes than a net without such gates.  Each variant gets the
+    headline's treatment: samples/s, per-launch table with measured traffic, the roofline of its dominant launch,
+    and the first 4096 samples of the full-batch result compared with the CPU interpreter."""
+    import copy
+    res = {}
+    for mix in ("two_input_gates_only", "half_pass_through"):
+        net = copy.deepcopy(model)
+        apply_gate_mix(torch, dl, net, mix)
+        value, ms, per_kernel, out, _, _ = packed_run(torch, dl, net, x, 10, steps=5, warmup=2, graph=False)
+        kernels, roofline = launch_rooflines(per_kernel, 5, table, prefix=mix + ": ")
+        r = {"gate_ids": GATE_MIXES[mix][1], "gate_mix": gate_mix(net_tables(net, dl)), "samples_per_s": round(value, 1),
+             "ms_per_step": round(ms, 4), "kernels": kernels, "roofline": roofline, "checksum": int(out.sum().item())}
+        if check_cpu:
+            from oracle import interp
+            n = 4096
+            want = interp.net_eval(x[:n].cpu().numpy(), net_tables(net, dl), 10, threads=1)
+            r["bit_exact_vs_cpu_interpreter"] = {"samples": n, "equal": bool((out[:n].cpu().numpy() == want).all())}
+        res[mix] = r
+        del net, out
+    return res
 
 
 def word_width_variants(torch, dl, model, x, want):
@@ -367,7 +445,7 @@ def net_tables(model, dl):
              m.weights.argmax(-1).to("cpu").numpy().astype(np.uint8)) for m in model if isinstance(m, dl.LogicLayer)]
 
 
-def cpu_baseline(args, model, x, out, dl):
+def cpu_interpreter(args, model, x, out, dl):
     """The oracle's table-driven C interpreter (same per-word arithmetic as the C the reference
     generates), one thread, on the first 2^cpu_sample_log2 samples of the batch; the GPU's
     full-batch result is compared with it on those samples."""
@@ -381,56 +459,97 @@ def cpu_baseline(args, model, x, out, dl):
     dt = time.perf_counter() - t0
     got = out[:n].cpu().numpy()
     return {"value": round(n / dt, 1), "unit": "samples/s", "cores": 1, "kind": "port",
-            "sample": "first %d of %d samples, same net; oracle/c/packed_interp.c, 1 thread, %.1f s (the reference's "
-                      "generated C itself: --cpu-generated-c, minutes of gcc)" % (n, x.shape[0], dt),
+            "sample": "first %d of %d samples, same net; oracle/c/packed_interp.c (table interpreter), 1 thread, %.1f s"
+                      % (n, x.shape[0], dt),
             "gpu_matches_cpu_on_sample": bool((got == want).all())}
 
 
-def cpu_generated_c(model, x, out, dl, sample_log2=16):
-    """The reference's CPU inference path for `model` on this host: the C text CompiledLogicNet generates
-    (difflogic/compiled_model.py:159-239, restated by oracle/cgen.py), compiled the way the reference's
-    driver does (experiments/main.py:362: gcc -O1 below 50 000 gates, else -O0), 64-bit words, one thread,
-    the whole apply_logic_gate_net call (bool packing, gates, adders) on the first 2^sample_log2 samples."""
-    import subprocess
-    import tempfile
-    from oracle import cgen
-    layers = net_tables(model, dl)
-    gates = sum(len(l[2]) for l in layers)
-    opt = 1 if gates < 50000 else 0
-    work = tempfile.mkdtemp(prefix="dl_bench_cgen_")
-    c_path, so_path = os.path.join(work, "net.c"), os.path.join(work, "net.so")
-    with open(c_path, "w") as f:
-        f.write(cgen.generate_c(layers, x.shape[1], 10, 64))
-    t0 = time.perf_counter()
-    proc = subprocess.Popen(["gcc", "-shared", "-fPIC", "-O%d" % opt, "-o", so_path, c_path])
-    while proc.poll() is None:
-        try:
-            proc.wait(timeout=30)
-        except subprocess.TimeoutExpired:
-            print("bench.py: gcc -O%d on %d gates, %.0f s so far" % (opt, gates, time.perf_counter() - t0),
-                  file=sys.stderr, flush=True)
-    if proc.returncode:
-        return {"error": "gcc exited with %d" % proc.returncode}
-    compile_s = time.perf_counter() - t0
-    fn = cgen.load_apply_fn(so_path)
-    n = min(1 << sample_log2, x.shape[0])
-    xs = x[:n].cpu().numpy()
-    cgen.call_apply_fn(fn, xs[:64], 10, 64)
-    t0 = time.perf_counter()
-    want = cgen.call_apply_fn(fn, xs, 10, 64)
-    dt = time.perf_counter() - t0
-    for path in (c_path, so_path):
-        os.remove(path)
-    os.rmdir(work)
-    return {"value": round(n / dt, 1), "unit": "samples/s", "cores": 1, "kind": "reference's generated C (restated text)",
-            "gates": gates, "compiler": "gcc -shared -fPIC -O%d" % opt, "compile_s": round(compile_s, 1),
-            "sample": "first %d samples, %.1f s" % (n, dt),
-            "gpu_matches_cpu_on_sample": bool((out[:n].cpu().numpy() == want).all())}
+def cpu_baseline(interpreter, compiled, xs, got, sample_note):
+    """`cpu_baseline` of the line: the gcc-compiled generated C where it was started (and built), with the table
+    interpreter's figure beside it; else the interpreter."""
+    if compiled is None:
+        return interpreter
+    res = compiled.collect(xs, got, sample_note)
+    if "error" in res:
+        return dict(interpreter, generated_c_error=res["error"])
+    res["table_interpreter"] = {kk: interpreter[kk] for kk in ("value", "unit", "cores", "sample", "gpu_matches_cpu_on_sample")}
+    return res
 
 
-def packed_config(torch, dl, name, F, widths, B, x, check_cpu, generated_c=False):
+class GeneratedC:
+    """The reference's CPU inference path for one net on this host: the C text CompiledLogicNet generates
+    (difflogic/compiled_model.py:159-239, restated by oracle/cgen.py), compiled the way the reference's driver does
+    (experiments/main.py:362: gcc -O1 below 50 000 gates, else -O0), 64-bit words, one thread.  The constructor
+    writes the text and starts gcc as a child process (minutes for 384 000 gates: call it before the GPU is
+    initialised, so that the child is started from a process that has not touched it); collect() waits for the
+    compiler and times the whole apply_logic_gate_net call (bool packing, gates, adders)."""
+
+    def __init__(self, name, layers, num_inputs, k=10):
+        import subprocess
+        import tempfile
+        import threading
+        from oracle import cgen
+        self.name, self.layers, self.k = name, layers, k
+        self.gates = sum(len(l[2]) for l in layers)
+        self.opt = 1 if self.gates < 50000 else 0
+        self.work = tempfile.mkdtemp(prefix="dl_bench_cgen_")
+        self.c_path, self.so_path = os.path.join(self.work, "net.c"), os.path.join(self.work, "net.so")
+        with open(self.c_path, "w") as f:
+            f.write(cgen.generate_c(layers, num_inputs, k, 64))
+        self.t0 = time.perf_counter()
+        self.t_end = None
+        self.proc = subprocess.Popen(["gcc", "-shared", "-fPIC", "-O%d" % self.opt, "-o", self.so_path, self.c_path])
+
+        def wait():
+            self.proc.wait()
+            self.t_end = time.perf_counter()
+        self._waiter = threading.Thread(target=wait, daemon=True)
+        self._waiter.start()
+
+    def same_net(self, tables):
+        import numpy as np
+        return len(tables) == len(self.layers) and all(
+            np.array_equal(u, v) for mine, theirs in zip(self.layers, tables) for u, v in zip(mine, theirs))
+
+    def collect(self, xs, got, sample_note):
+        """xs bool [n, F] (numpy): the sample; got int32 [n, k]: what the GPU computed for it."""
+        from oracle import cgen
+        while self._waiter.is_alive():
+            self._waiter.join(timeout=30)
+            if self._waiter.is_alive():
+                print("bench.py: waiting for gcc -O%d on the %d gates of %s, %.0f s so far"
+                      % (self.opt, self.gates, self.name, time.perf_counter() - self.t0), file=sys.stderr, flush=True)
+        if self.proc.returncode:
+            return {"error": "gcc exited with %d" % self.proc.returncode}
+        fn = cgen.load_apply_fn(self.so_path)
+        cgen.call_apply_fn(fn, xs[:64], self.k, 64)
+        t0 = time.perf_counter()
+        want = cgen.call_apply_fn(fn, xs, self.k, 64)
+        dt = time.perf_counter() - t0
+        n = xs.shape[0]
+        return {"value": round(n / dt, 1), "unit": "samples/s", "cores": 1, "kind": "generated-c",
+                "gates": self.gates, "compiler": "gcc -shared -fPIC -O%d" % self.opt,
+                "compile_s": round(self.t_end - self.t0, 1),
+                "sample": "%s; the C text CompiledLogicNet generates for this net (restated by oracle/cgen.py), compiled as "
+                          "experiments/main.py:362 does, one apply_logic_gate_net call, 1 thread, %.1f s; gcc ran as a child "
+                          "process next to the GPU work" % (sample_note, dt),
+                "gpu_matches_cpu_on_sample": bool((got == want).all())}
+
+    def close(self):
+        if self._waiter.is_alive():
+            self.proc.kill()
+            self._waiter.join()
+        for path in (self.c_path, self.so_path):
+            if os.path.exists(path):
+                os.remove(path)
+        if os.path.isdir(self.work):
+            os.rmdir(self.work)
+
+
+def packed_config(torch, dl, name, F, widths, B, x, check_cpu, compiled=None):
     """One of the other packed configurations: samples/s, per-launch times, and the first 4096
-    samples of the full-batch result compared with the CPU interpreter."""
+    samples of the full-batch result compared with the CPU interpreter.  ``compiled``: the GeneratedC of this
+    net started by main(), timed on the first 2^16 samples."""
     k = 10
     model = packed_model(torch, dl, F, widths, k)
     value, ms, per_kernel, out, first_ms, graph_info = packed_run(torch, dl, model, x, k, steps=5, warmup=2)
@@ -450,8 +569,14 @@ def packed_config(torch, dl, name, F, widths, B, x, check_cpu, generated_c=False
         dt = time.perf_counter() - t0
         res["bit_exact_vs_cpu_interpreter"] = {"samples": n, "equal": bool((out[:n].cpu().numpy() == want).all()),
                                                "cpu_samples_per_s": round(n / dt, 1)}
-    if generated_c:
-        res["cpu_generated_c"] = cpu_generated_c(model, x, out, dl)
+    res["gate_mix"] = gate_mix(net_tables(model, dl))
+    if compiled is not None:
+        n = min(1 << 16, B)
+        if compiled.same_net(net_tables(model, dl)):
+            res["cpu_generated_c"] = compiled.collect(x[:n].cpu().numpy(), out[:n].cpu().numpy(), "first %d samples" % n)
+        else:
+            res["cpu_generated_c"] = {"error": "the net made on the CPU differs from the model's"}
+        compiled.close()
     del model, out
     return res
 
@@ -733,17 +858,21 @@ def ceilings(torch):
     return res
 
 
-def extra_configs(args, torch, dl):
-    """The other BASELINE configurations (C1 .. C5), each optional."""
+def wanted(args, c, group_off):
     only = {c for c in args.only.lower().split(",") if c}
-    want = lambda c, group_off: (c in only) if only else not group_off      # noqa: E731
+    return (c in only) if only else not group_off
+
+
+def extra_configs(args, torch, dl, started):
+    """The other BASELINE configurations (C1 .. C5), each optional.  ``started``: GeneratedC objects by name."""
+    want = lambda c, group_off: wanted(args, c, group_off)      # noqa: E731
     configs = {}
     check = not args.no_cpu_baseline
     if want("c2", args.no_configs):
         B = 1 << 20
         configs["C2"] = packed_config(torch, dl, "packed inference 784->6x8000->GroupSum(10), batch 2^20, int64 words",
                                       784, [8000] * 6, B, bernoulli_input(torch, B, 784, 1), check,
-                                      generated_c=args.cpu_generated_c)
+                                      compiled=started.get("C2"))
         torch.cuda.empty_cache()
     if want("c4", args.no_configs):
         B = 1 << 18
@@ -789,8 +918,25 @@ def main():
         print("bench.py: this build runs on one GPU only (the path shards along the batch without "
               "communication); --gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
-    import torch
+    import torch                      # (importing it does not initialise the GPU)
 
+    # The reference's CPU inference path (gcc on the generated C) takes minutes to compile: started here, as child
+    # processes of a process that has not touched the GPU yet, and collected after the GPU work.
+    started = {}
+    if not (args.no_cpu_baseline or args.no_cpu_generated_c or args.ceilings):
+        if not args.skip_headline and args.gate_mix == "uniform":
+            started["headline"] = GeneratedC("the headline net", cpu_side_net(torch, args.features, [args.width] * args.layers),
+                                             args.features)
+        if wanted(args, "c2", args.no_configs):
+            started["C2"] = GeneratedC("C2", cpu_side_net(torch, 784, [8000] * 6), 784)
+    try:
+        run(args, torch, started)
+    finally:
+        for c in started.values():
+            c.close()
+
+
+def run(args, torch, started):
     import difflogic_amd as dl
     assert torch.cuda.is_available(), "bench.py needs the GPU"
 
@@ -807,7 +953,8 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     if args.skip_headline:
-        print(json.dumps({"metric": "extra configurations only (--skip-headline)", "extra": {"configs": extra_configs(args, torch, dl)}}))
+        print(json.dumps({"metric": "extra configurations only (--skip-headline)",
+                          "extra": {"configs": extra_configs(args, torch, dl, started)}}))
         return
     value, ms, roofline, info, model, x, out = packed_headline(args, torch, dl)
     result = {
@@ -817,18 +964,27 @@ def main():
         "config": {"workload": "packed inference %d->%dx%d->GroupSum(10), batch 2^%d, int64 words, bool input "
                                "resident in HBM; step = pack + %d gate layers + groupbitsum"
                                % (args.features, args.layers, args.width, args.batch_log2, args.layers),
-                   "connections": "random", "seed": 0},
+                   "connections": "random", "seed": 0, "gate_ids": GATE_MIXES[args.gate_mix][1],
+                   "gate_mix": gate_mix(net_tables(model, dl))},
         "roofline": roofline,
     }
-    result["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(args, model, x, out, dl)
+    interpreter, compiled, sample = None, None, None
+    if not args.no_cpu_baseline:
+        interpreter = cpu_interpreter(args, model, x, out, dl)
+        compiled = started.get("headline")
+        if compiled is not None and not compiled.same_net(net_tables(model, dl)):
+            interpreter["generated_c_error"] = "the net made on the CPU differs from the model's"
+            compiled = None
+        n = min(1 << args.cpu_generated_c_sample_log2, x.shape[0])
+        sample = (x[:n].cpu().numpy(), out[:n].cpu().numpy(), "first %d of %d samples, same net" % (n, x.shape[0]))
     extra = dict(info)
-    if args.cpu_generated_c:
-        extra["cpu_generated_c"] = cpu_generated_c(model, x, out, dl)
     del model, x, out
     gc.collect()
     torch.cuda.empty_cache()
 
-    extra["configs"] = extra_configs(args, torch, dl)
+    extra["configs"] = extra_configs(args, torch, dl, started)
+    # last, so that gcc's minutes on the headline net's C overlap with everything above
+    result["cpu_baseline"] = None if interpreter is None else cpu_baseline(interpreter, compiled, *sample)
     result["extra"] = extra
     print(json.dumps(result))
 

@@ -76,6 +76,50 @@ def test_full_size_packed_inference(name, F, widths, log2b, thresholds):
     assert torch.equal(out_r, out[:B - 37]), name
 
 
+def _set_gate_ids(dl, model, rng, kinds):
+    """Overwrites the model's gate logits with one-hot rows: layer i draws its gate ids from kinds[i]."""
+    pools = {"two-input": [1, 2, 4, 6, 7, 8, 9, 11, 13, 14], "pass-through": [3, 5, 10, 12], "constant": [0, 15],
+             "uniform": list(range(16)), "half pass-through": [3, 5, 10, 12] * 4 + list(range(16))}
+    logic = [m for m in model if isinstance(m, dl.LogicLayer)]
+    with torch.no_grad():
+        for m, kind in zip(logic, kinds):
+            ids = torch.as_tensor(rng.choice(np.array(pools[kind]), m.out_dim)).cuda()
+            m.weights.copy_(torch.nn.functional.one_hot(ids.long(), 16).float())
+
+
+@pytest.mark.parametrize("mix,kinds", [
+    ("two-input gates only", ["two-input"] * 6),                 # nothing to skip anywhere
+    ("pass-through gates only", ["pass-through"] * 6),           # one live leaf per tree
+    ("half pass-through", ["half pass-through"] * 6),
+    ("constant middle layer", ["uniform", "uniform", "constant", "uniform", "uniform", "uniform"]),
+    ("constant first layer", ["constant"] + ["uniform"] * 5),
+    ("constant layer below the top", ["two-input"] * 4 + ["constant", "two-input"]),
+])
+def test_full_size_gate_mixes(mix, kinds):
+    """The headline net (784 -> 6 x 64000, batch 2^20) with gate mixes at the extremes of what the packed kernels
+    skip, through PackBitsTensor on the streaming plan: the oracle on slices of the batch and the per-layer
+    kernels (which skip nothing but ignored rows) on the whole batch."""
+    import difflogic_amd as dl
+    B, F, widths = 1 << 20, 784, [64000] * 6
+    model = _build(dl, F, widths, 0)
+    _set_gate_ids(dl, model, np.random.default_rng(len(mix)), kinds)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.rand(B, F, device="cuda", generator=g) < 0.2
+    with torch.no_grad():
+        out = model(dl.PackBitsTensor(x, bit_count=64))
+    assert out.shape == (B, 10) and out.dtype == torch.int32
+    idx = torch.cat([torch.arange(0, 128), torch.arange(B // 2 - 64, B // 2 + 64), torch.arange(B - 128, B)]).cuda()
+    want = interp.net_eval(x[idx].cpu().numpy(), _tables(dl, model), 10, threads=16)
+    assert np.array_equal(out[idx].cpu().numpy(), want), mix
+    with torch.no_grad():
+        ref = _per_layer(dl, model, x)
+    assert torch.equal(out, ref), mix
+    del ref
+    with torch.no_grad():                                        # a second call reuses the cached schedules and plans
+        again = model(dl.PackBitsTensor(x[:B - 37], bit_count=64))
+    assert torch.equal(again, out[:B - 37]), mix
+
+
 # ------------------------------------------------------------------------------------------
 # fp32 training at BASELINE.json's full sizes (C3: 64000-wide, B = 512, 'unique';
 # C5: 128000-wide, B = 1024, 'random', grad_factor 2; C1: 784 -> 4 x 8000, B = 128, 'random', with

@@ -1,0 +1,100 @@
+"""The packed path on nets whose gate mix is at an extreme of what the skipping machinery (constant folding,
+ignored inputs not fetched, output rows nobody looks at not written, constant neurons left out of the count)
+can meet: nothing to skip at all, pass-through gates only, layers that are constant as a whole.  Through
+PackBitsTensor and GroupSum as a user runs them, on the streaming plan (layers too wide for the LDS-resident
+kernel) and on the LDS-resident kernel, against the oracle's interpreter.  Bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import interp
+from oracle import packed_oracle as po
+from tests.helpers import build_model, random_layers
+
+pytestmark = pytest.mark.gpu
+
+TWO_INPUT = np.array([1, 2, 4, 6, 7, 8, 9, 11, 13, 14], np.uint8)     # the ten gates that look at both inputs
+PASS_THROUGH = np.array([3, 5, 10, 12], np.uint8)                      # a, b, not b, not a
+CONSTANT = np.array([0, 15], np.uint8)
+
+
+def _draw(rng, n, kind):
+    """Gate ids of one layer of `n` neurons."""
+    if kind == "two-input":
+        return rng.choice(TWO_INPUT, n)
+    if kind == "pass-through":
+        return rng.choice(PASS_THROUGH, n)
+    if kind == "constant":
+        return rng.choice(CONSTANT, n)
+    if kind == "zeros":
+        return np.zeros(n, np.uint8)
+    if kind == "ones":
+        return np.full(n, 15, np.uint8)
+    if kind == "half pass-through":
+        return np.where(rng.random(n) < 0.5, rng.choice(PASS_THROUGH, n), rng.integers(0, 16, n)).astype(np.uint8)
+    if kind == "uniform":
+        return rng.integers(0, 16, n).astype(np.uint8)
+    raise ValueError(kind)
+
+
+MIXES = {
+    # name: the kind of every layer in turn (shorter lists repeat their last entry)
+    "two-input gates only": ["two-input"],
+    "pass-through gates only": ["pass-through"],
+    "half pass-through": ["half pass-through"],
+    "constant first layer": ["constant", "uniform"],
+    "constant middle layer": ["uniform", "uniform", "constant", "uniform"],
+    "all-zero middle layer": ["two-input", "two-input", "zeros", "two-input"],
+    "all-ones layer below the top": ["uniform", "uniform", "uniform", "uniform", "ones", "uniform"],
+    "constant top layer": ["uniform", "uniform", "uniform", "uniform", "uniform", "constant"],
+    "pass-through below two-input": ["pass-through", "two-input", "pass-through", "two-input", "pass-through", "two-input"],
+    "everything constant": ["constant"],
+}
+
+
+def _net(rng, F, widths, mix):
+    kinds = MIXES[mix]
+    layers = random_layers(rng, F, widths)
+    return [(a, b, _draw(rng, len(a), kinds[min(i, len(kinds) - 1)]).astype(np.uint8)) for i, (a, b, _) in enumerate(layers)]
+
+
+@pytest.mark.parametrize("mix", sorted(MIXES))
+@pytest.mark.parametrize("shape", ["streaming", "streaming, narrow input", "lds"])
+def test_gate_mix_extremes(mix, shape):
+    import difflogic_amd as dl
+    from difflogic_amd import packbitstensor as pbt
+    rng = np.random.default_rng(sum(map(ord, mix + shape)))
+    k = 10
+    if shape == "lds":
+        F, widths, B = 64, [500, 700, 640, 900, 500, 640], 1000
+    elif shape == "streaming":
+        F, widths, B = 96, [12000, 11000, 12000, 11500, 12000, 10500], 700
+    else:
+        F, widths, B = 16, [12000, 11000, 12000, 11500, 12000, 10500], 129
+    layers = _net(rng, F, widths, mix)
+    dims = [F] + widths
+    if shape == "lds":
+        assert pbt.lds_tail(dims, 16) == len(widths)
+    else:
+        assert pbt.lds_tail(dims, 16) == 0 and len(pbt.plan_groups(dims, True, 16)) >= 2
+    x = rng.random((B, F)) < 0.5
+    want = interp.net_eval(x, layers, k)
+    model = build_model(F, layers, k).eval()
+    for bits in (64, 32):
+        with torch.no_grad():
+            p = dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=bits)
+            got = model(p)
+        assert got.dtype == torch.int32 and np.array_equal(got.cpu().numpy(), want), (mix, shape, bits)
+    # `.t` after the layers alone holds every row of the last layer, constant and unobserved ones included
+    logic = [m for m in model if isinstance(m, dl.LogicLayer)]
+    with torch.no_grad():
+        p = dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=64)
+        for m in logic:
+            p = m(p)
+        words = p.t.cpu().numpy()
+    y, _ = po.packbits(x.T, 64)
+    for a, b, op in layers:
+        y = po.eval_layer(y, a, b, op)
+    assert words.shape == y.shape
+    assert np.array_equal(po.groupbitsum(words, words.shape[1] * 64 - B, k), want)
+    assert np.array_equal(po.unpackbits(words, B), po.unpackbits(y, B)), (mix, shape)
