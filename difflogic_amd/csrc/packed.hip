@@ -455,6 +455,9 @@ __global__ __launch_bounds__(DL_BLOCK) void compose_steps_kernel(const int32_t *
 // One wave = STEPS consecutive steps x 64 vectors; dispatch order as eval_kernel.  BUF: x is at
 // most 4 GiB and is read through a buffer resource, whose loads take the row's byte offset as a
 // scalar operand next to the lane's constant offset: no vector instruction per gather.
+#ifndef DL_STEPS_PER_WAVE
+#define DL_STEPS_PER_WAVE 32           // steps a wave of eval_steps_kernel walks (its first vertex is evaluated on top)
+#endif
 template <typename V, int DS, int STEPS, bool BUF>
 __global__ __launch_bounds__(DL_BLOCK) void eval_steps_kernel(const V *__restrict__ x, const StepRec<DS> *__restrict__ rec,
                                                               V *__restrict__ y, int64_t nsteps, int64_t ncols,
@@ -1123,7 +1126,7 @@ __global__ __launch_bounds__(DL_BLOCK) void count_constant_ones_kernel(const uin
 // one wave per block takes the constant neurons out, moves the others of their class up and shortens the
 // class's run.  Steps are numbered as the count kernel walks them (workgroup, wave, block, step); lane c keeps
 // count of the constant neurons of class c met so far.
-static_assert(DL_CC_BLOCK % DL_WAVE == 0 && DL_CC_MAX_CLASSES <= DL_WAVE, "a wave covers a block in whole rounds, a lane per class");
+static_assert(DL_CC_MAX_CLASSES <= DL_WAVE, "a lane per class");
 __global__ __launch_bounds__(DL_BLOCK) void count_chain_thin_kernel(const int32_t *__restrict__ neuron,
                                                                     const uint8_t *__restrict__ w_top,
                                                                     const uint8_t *__restrict__ slot,
@@ -1140,7 +1143,7 @@ __global__ __launch_bounds__(DL_BLOCK) void count_chain_thin_kernel(const int32_
     for (int first = 0; first < DL_CC_BLOCK; first += DL_WAVE) {
         const int i = first + lane;                           // the order in which the plan numbered a class's slots
         const int64_t s = g * wg_steps + (i / DL_CC_WAVE_STEPS) * span + b * DL_CC_WAVE_STEPS + i % DL_CC_WAVE_STEPS;
-        const int32_t n = s < steps ? neuron[s] : -1;
+        const int32_t n = i < DL_CC_BLOCK && s < steps ? neuron[s] : -1;
         int cls = -1;
         bool constant = false;
         if (n >= 0) {
@@ -1155,7 +1158,7 @@ __global__ __launch_bounds__(DL_BLOCK) void count_chain_thin_kernel(const int32_
             if (cls == c) before = carried + (uint32_t) __popcll(met & ((1ull << lane) - 1ull));
             if (lane == c) gone += (uint32_t) __popcll(met);
         }
-        slot_call[s] = n >= 0 && !constant ? (uint8_t) (slot[s] - before) : (uint8_t) 255;
+        if (i < DL_CC_BLOCK) slot_call[s] = n >= 0 && !constant ? (uint8_t) (slot[s] - before) : (uint8_t) 255;
     }
     if (lane < k) {
         const uint32_t run = runs[gb * k + lane];
@@ -1234,11 +1237,18 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
         const V rb = DS != 1 ? ra : (r.w & 2u) ? any_value<V>() : xcol[(int64_t) r.y * ncols];
         prev = vertex(ra, rb, r.z);
     }
-    V cnt[CPW][DL_CC_PLANES];
+    // counter planes; carries of weight 4 and (with one set of counters, where the registers allow it) 8 waiting for a partner
+    constexpr bool WAIT8 = CPW == 1;
+    V cnt[CPW][DL_CC_PLANES], wait4[CPW], wait8[WAIT8 ? CPW : 1];
+    uint32_t quads[CPW];
 #pragma unroll
-    for (int i = 0; i < CPW; ++i)
+    for (int i = 0; i < CPW; ++i) {
 #pragma unroll
         for (int p = 0; p < DL_CC_PLANES; ++p) cnt[i][p] = Words<V>::zero();
+        wait4[i] = Words<V>::zero();
+        if (WAIT8) wait8[i] = Words<V>::zero();
+        quads[i] = 0;
+    }
 
     // Phase A walks the wave's DL_CC_WAVE_STEPS steps of the block.  With one class per wave the registers hold the
     // rows of all of them, and they are requested before the block before is counted, so that the counting phase
@@ -1301,13 +1311,46 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
                     V v[4];
 #pragma unroll
                     for (int u = 0; u < 4; ++u) v[u] = stage[q + u < n ? start + q + u : DL_CC_BLOCK][lane];
-                    V carry = csa_quad(cnt[i][0], cnt[i][1], v);          // weight 4
+                    const V c4 = csa_quad(cnt[i][0], cnt[i][1], v);       // weight 4
+                    // A carry waits for the next one of its weight instead of rippling through the planes alone:
+                    // every second quad a full adder at weight 4, every fourth one at weight 8 and the ripple
+                    // (quads[i]: how many quads this counter has taken, wave-uniform).
+                    if (!(quads[i] & 1u)) {
+                        wait4[i] = c4;
+                    } else {
+                        V c8;
+                        csa(c8, cnt[i][2], cnt[i][2], wait4[i], c4);
+                        if (WAIT8 && !(quads[i] & 2u)) {
+                            wait8[i] = c8;
+                        } else if (WAIT8) {
+                            V c16;
+                            csa(c16, cnt[i][3], cnt[i][3], wait8[i], c8);
 #pragma unroll
-                    for (int p = 2; p < DL_CC_PLANES; ++p) HalfAdd<V>::run(cnt[i][p], carry);
+                            for (int p = 4; p < DL_CC_PLANES; ++p) HalfAdd<V>::run(cnt[i][p], c16);
+                        } else {
+#pragma unroll
+                            for (int p = 3; p < DL_CC_PLANES; ++p) HalfAdd<V>::run(cnt[i][p], c8);
+                        }
+                    }
+                    ++quads[i];
                 }
             }
         }
         __syncthreads();
+    }
+    // the carries still waiting join the planes
+#pragma unroll
+    for (int i = 0; i < CPW; ++i) {
+        if (quads[i] & 1u) {
+            V c = wait4[i];
+#pragma unroll
+            for (int p = 2; p < DL_CC_PLANES; ++p) HalfAdd<V>::run(cnt[i][p], c);
+        }
+        if (WAIT8 && (quads[i] & 2u)) {
+            V c = wait8[i];
+#pragma unroll
+            for (int p = 3; p < DL_CC_PLANES; ++p) HalfAdd<V>::run(cnt[i][p], c);
+        }
     }
     if (live) {
 #pragma unroll
@@ -1918,7 +1961,7 @@ template <typename V, int DS>
 int launch_eval_steps(const void *x, const int32_t *sub_leaves, const uint64_t *sub_gates, const int32_t *verts,
                       const int32_t *neuron, const uint8_t *flip, const uint8_t *w_top, const uint8_t *out_live, void *y,
                       void *records, int64_t steps, int64_t row_bytes, int64_t x_bytes, hipStream_t s) {
-    constexpr int STEPS = 16;
+    constexpr int STEPS = DL_STEPS_PER_WAVE;
     const int64_t ncols = row_bytes / (int64_t) sizeof(V);
     StepRec<DS> *rec = (StepRec<DS> *) records;
     DL_LAUNCH(compose_steps_kernel<DS>, dim3((unsigned) dl_ceil_div(steps + 1, DL_BLOCK)), dim3(DL_BLOCK), 0, s, sub_leaves,

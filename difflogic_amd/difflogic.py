@@ -311,8 +311,8 @@ class FusedLogicLayerGroupSum(torch.nn.Module):
         layer, gs = self.layer, self.group_sum
         if (isinstance(x, PackBitsTensor) or not self.training or layer.implementation != "cuda" or not x.is_cuda
                 or x.ndim != 2 or x.dtype != layer.weights.dtype or x.shape[0] == 0 or layer.out_dim % gs.k != 0
-                or gs.k > GroupSum._HIP_MAX_K):
-            return gs(layer(x))
+                or gs.k > GroupSum._HIP_MAX_K or layer.out_dim > GroupSum._HIP_MAX_OUT_DIM):
+            return gs(layer(x))                                         # (the limits GroupSum itself falls back beyond)
         xt = x.transpose(0, 1).contiguous()
         assert xt.shape[0] == layer.in_dim, (xt.shape, layer.in_dim)
         a, b = layer.indices

@@ -64,6 +64,57 @@ def test_fused_adam_skips_parameters_without_gradient_and_rejects_other_dtypes()
         dl.FusedAdam([a], lr=-1.0)
 
 
+def test_fused_adam_counter_steps_for_all_of_its_members_or_none():
+    """Parameters updated by one launch share a step counter.  A step on which only some of them have a gradient
+    would advance the count of the others as well (torch keeps a step per parameter): that raises; a step on which
+    none of them has one is skipped as in torch."""
+    import difflogic_amd as dl
+    a, b = _params(1, [(10,), (10,)])
+    opt = dl.FusedAdam([a, b], lr=0.1)
+    a.grad, b.grad = torch.ones_like(a), torch.ones_like(b)
+    opt.step()
+    b.grad = None
+    with pytest.raises(RuntimeError, match="step counter"):
+        opt.step()
+    a.grad = None
+    before = (a.detach().clone(), b.detach().clone())
+    opt.step()                                                  # nothing to do
+    assert torch.equal(a.detach(), before[0]) and torch.equal(b.detach(), before[1])
+    assert float(opt.state[a]["step"]) == 1.0
+
+
+@pytest.mark.parametrize("saved_by", ["torch.optim.Adam", "FusedAdam"])
+def test_fused_adam_resumes_from_a_saved_state(saved_by):
+    """load_state_dict of a state saved by torch.optim.Adam (a step per parameter, no shared counter) or by
+    FusedAdam itself: training goes on as torch.optim.Adam's does (bias correction from the restored count)."""
+    import difflogic_amd as dl
+    shapes = [(300, 16), (7,), (4100,)]
+    ref = _params(5, shapes)
+    first = [p.detach().clone().requires_grad_() for p in ref]
+    opt_r = torch.optim.Adam(ref, lr=0.01)
+    opt_f = (torch.optim.Adam if saved_by == "torch.optim.Adam" else dl.FusedAdam)(first, lr=0.01)
+    g = torch.Generator(device="cuda").manual_seed(9)
+    grads = [[torch.randn(s, device="cuda", generator=g) for s in shapes] for _ in range(7)]
+    for step in range(3):
+        for pr, pf, gr in zip(ref, first, grads[step]):
+            pr.grad, pf.grad = gr.clone(), gr.clone()
+        opt_r.step()
+        opt_f.step()
+    ours = [p.detach().clone().requires_grad_() for p in first]
+    opt_o = dl.FusedAdam(ours, lr=0.01)
+    opt_o.load_state_dict(copy.deepcopy(opt_f.state_dict()))
+    for step in range(3, 7):
+        for pr, po, gr in zip(ref, ours, grads[step]):
+            pr.grad, po.grad = gr.clone(), gr.clone()
+        opt_r.step()
+        opt_o.step()
+        for i, (po, pr) in enumerate(zip(ours, ref)):
+            assert _close(po.detach(), pr.detach(), 4e-6), (step, i)
+    assert float(opt_o.state[ours[0]]["step"]) == 7.0
+    # the three tensors share one rebuilt counter again: one launch
+    assert len({opt_o.state[p]["_counter"].data_ptr() for p in ours}) == 1
+
+
 def test_fused_adam_more_tensors_than_one_launch_takes():
     import difflogic_amd as dl
     n = dl._lib.load().dl_adam_max_tensors() + 5
