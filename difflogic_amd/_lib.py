@@ -14,6 +14,7 @@ DL_ERR_DTYPE = 4
 DL_ERR_LAUNCH = 5
 DL_ERR_TOO_LARGE = 6
 DL_ERR_SCRATCH_LIMIT = 7
+DL_ERR_CAPTURING = 8
 
 DL_F16, DL_F32, DL_F64 = 0, 1, 2
 

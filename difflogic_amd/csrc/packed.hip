@@ -1867,8 +1867,9 @@ static __device__ __align__(256) unsigned char scratch[DL_STATIC_SCRATCH_BYTES];
 static void *scratch_address[DL_MAX_DEVICES];      // per device: where that GPU's copy of `scratch` lives
 static std::mutex scratch_mutex;
 
-// Address of the current device's copy of `scratch` (looked up on the first call per device).
-static int static_scratch(void **ptr) {
+// Address of the current device's copy of `scratch` (looked up on the first call per device; that lookup is a
+// runtime call that must not run while `stream` is being captured into a graph: refused then).
+static int static_scratch(void **ptr, hipStream_t stream) {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) {
@@ -1878,6 +1879,13 @@ static int static_scratch(void **ptr) {
     if (dev < 0 || dev >= DL_MAX_DEVICES) return DL_ERR_TOO_LARGE;
     std::lock_guard<std::mutex> lock(scratch_mutex);
     if (!scratch_address[dev]) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        e = hipStreamIsCapturing(stream, &capturing);
+        if (e != hipSuccess) {
+            dl_last_hip_error_code = (int) e;
+            return DL_ERR_LAUNCH;
+        }
+        if (capturing != hipStreamCaptureStatusNone) return DL_ERR_CAPTURING;
         void *p = nullptr;
         e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
         if (e != hipSuccess || !p) {
@@ -1904,7 +1912,7 @@ extern "C" int dl_logic_eval_fused_groupbitsum_noalloc(const void *x, int depth,
     const int64_t need = dl_logic_eval_fused_groupbitsum_workspace_bytes(depth, out_dim, words, bit_count, k);
     if (need > (int64_t) DL_STATIC_SCRATCH_BYTES) return DL_ERR_SCRATCH_LIMIT;
     void *ws = nullptr;
-    const int st = static_scratch(&ws);
+    const int st = static_scratch(&ws, (hipStream_t) stream);
     if (st != DL_OK) return st;
     return dl_logic_eval_fused_groupbitsum(x, depth, a, b, w, dims, out, words, bit_count, pad_len, k, order, ws, stream);
 }

@@ -1928,6 +1928,7 @@ extern "C" const char *dl_status_string(int status) {
     case DL_ERR_LAUNCH: return "HIP refused the kernel launch";
     case DL_ERR_TOO_LARGE: return "size exceeds what this entry point supports";
     case DL_ERR_SCRATCH_LIMIT: return "the call needs more than the library's static scratch array (DL_STATIC_SCRATCH_BYTES)";
+    case DL_ERR_CAPTURING: return "the first call on a device must be made outside a graph capture";
     default: return "unknown status";
     }
 }

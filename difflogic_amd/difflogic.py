@@ -55,10 +55,24 @@ class LogicLayer(torch.nn.Module):
                              f"{tuple(b.shape)}")
         if self.out_dim and (min(int(a.min()), int(b.min())) < 0 or max(int(a.max()), int(b.max())) >= self.in_dim):
             raise ValueError(f"connection indices have to lie in [0, {self.in_dim})")
+        if getattr(self, "indices", None) is not None:
+            difflogic_cuda.invalidate_wiring(*self.indices)     # what was derived from the wiring being replaced
         self.indices = (a, b)
         if self.implementation == "cuda":
             # reverse index for backward_x (difflogic.py:56-69)
             start, idx = build_reverse_index(a, b, self.in_dim)
+            self.given_x_indices_of_y_start = start.to(self.device)
+            self.given_x_indices_of_y = idx.to(self.device)
+
+    def invalidate_wiring(self):
+        """Drops what is derived from the wiring (evaluation schedules, count plans, the reverse index that
+        backward_x walks) and rebuilds the reverse index from the current contents of ``indices``.  Call it after
+        changing the index tensors in any way other than ``set_connections``.  (The schedule caches notice
+        in-place operations that bump the tensors' version counter by themselves; a write through
+        ``indices[i].data`` bumps nothing, and the reverse index follows neither.)"""
+        difflogic_cuda.invalidate_wiring(*self.indices)
+        if self.implementation == "cuda" and hasattr(self, "given_x_indices_of_y"):
+            start, idx = build_reverse_index(self.indices[0], self.indices[1], self.in_dim)
             self.given_x_indices_of_y_start = start.to(self.device)
             self.given_x_indices_of_y = idx.to(self.device)
 

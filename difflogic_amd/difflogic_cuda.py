@@ -691,7 +691,8 @@ class _WiringCache:
     them is collected, so a freed tensor's address can never be mistaken for a new tensor at the
     same address, and nothing is pinned beyond the wiring's own lifetime.  The key also carries
     the tensors' version counters, so in-place edits of the wiring rebuild the entry (writes
-    through ``.data`` are invisible to the counter: replace the tensors instead).  Thread-safe."""
+    through ``.data`` are invisible to the counter: replace the tensors, or call
+    ``invalidate_wiring`` / ``LogicLayer.invalidate_wiring`` after such a write).  Thread-safe."""
 
     def __init__(self):
         import threading
@@ -726,6 +727,13 @@ class _WiringCache:
     def __len__(self):
         return len(self._entries)
 
+    def drop(self, tensors):
+        """Forgets every entry built from one of ``tensors`` (matched by storage address)."""
+        ptrs = {t.data_ptr() for t in tensors}
+        with self._lock:
+            for key in [k for k, (refs, _) in self._entries.items() if any(k[i][0] in ptrs for i in range(len(refs)))]:
+                del self._entries[key]
+
 
 _SCHEDULES = _WiringCache()
 
@@ -734,6 +742,15 @@ def schedule_for(a, b, in_dim):
     """The cached EvalSchedule of the wiring (a, b): lives as long as the tensors do, rebuilt when
     they are replaced or modified in place."""
     return _SCHEDULES.get((a, b), (int(in_dim),), lambda: EvalSchedule(a, b, in_dim))
+
+
+def invalidate_wiring(*tensors):
+    """Forgets everything derived from the index tensors ``tensors`` (evaluation schedules, count plans and
+    orders), so that the next call rebuilds it from their current contents.  Needed after writing into index
+    tensors through ``.data`` (or any other way that leaves their version counter alone): in-place
+    operations that autograd sees and replaced tensors are noticed without it."""
+    _SCHEDULES.drop(tensors)
+    _COUNT_ORDERS.drop(tensors)
 
 
 def live_inputs(layers, live_out=None):

@@ -39,7 +39,8 @@ typedef enum dl_status {
     DL_ERR_DTYPE = 4,            /* dtype not one of dl_dtype                                 */
     DL_ERR_LAUNCH = 5,           /* the HIP runtime refused the launch (see dl_last_hip_error) */
     DL_ERR_TOO_LARGE = 6,        /* a size exceeds what the entry point supports              */
-    DL_ERR_SCRATCH_LIMIT = 7     /* the call needs more than DL_STATIC_SCRATCH_BYTES of scratch */
+    DL_ERR_SCRATCH_LIMIT = 7,    /* the call needs more than DL_STATIC_SCRATCH_BYTES of scratch */
+    DL_ERR_CAPTURING = 8         /* a first call per device that must not run under graph capture  */
 } dl_status;
 
 typedef enum dl_dtype { DL_F16 = 0, DL_F32 = 1, DL_F64 = 2 } dl_dtype;
@@ -484,7 +485,11 @@ int dl_logic_net_lds_groupbitsum_bool(const uint8_t *x, int64_t batch, int depth
  *   DL_ERR_SCRATCH_LIMIT  dl_logic_eval_fused_groupbitsum_workspace_bytes(depth, dims[depth],
  *                         words, bit_count, k) exceeds DL_STATIC_SCRATCH_BYTES (split the batch);
  *   DL_ERR_TOO_LARGE      rows are not whole 64-bit words (no per-layer fallback exists here).
- * The first call on a device looks the array's address up (make it outside a graph capture).
+ *   DL_ERR_CAPTURING      the first call on a device, which looks the array's address up with a
+ *                         runtime call, was made while `stream` is being captured into a graph
+ *                         (make one call on the device before capturing).
+ * The array takes DL_STATIC_SCRATCH_BYTES of device memory in every process that loads the
+ * library, on every GPU it uses, whether or not this entry point is ever called.
  * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different
  * streams or threads) race; calls ordered on one stream do not.  Nothing in the array needs to be
  * cleared between calls. */

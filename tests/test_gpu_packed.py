@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 import torch
 
+from oracle import connections as oc
 from oracle import interp
 from oracle import packed_oracle as po
 from tests.helpers import build_model, random_layers
@@ -542,6 +543,51 @@ def test_packed_inference_follows_weight_writes_through_data():
     with torch.no_grad():
         got2 = model(dl.PackBitsTensor(xd, bit_count=64)).cpu().numpy()
     assert np.array_equal(got2, interp.net_eval(x, layers2, 10))
+
+
+@pytest.mark.parametrize("shape", ["streaming", "lds"])
+def test_packed_inference_follows_wiring_writes_after_invalidate_wiring(shape):
+    """The schedules and plans cached per wiring follow the index tensors' version counters.  A write through
+    ``indices[i].data`` leaves the counter alone: LogicLayer.invalidate_wiring() after it makes the next packed
+    evaluation (and the training kernels' schedules, and the reverse index) use the new wiring.  In-place
+    operations that do bump the version are noticed by the schedule caches themselves; set_connections needs no call."""
+    import difflogic_amd as dl
+    rng = np.random.default_rng(31)
+    F, widths, B = (64, [12000, 11000, 10500], 300) if shape == "streaming" else (48, [600, 700, 640], 300)
+    layers = random_layers(rng, F, widths)
+    x = rng.random((B, F)) < 0.5
+    model = build_model(F, layers, 10).eval()
+    xd = torch.as_tensor(x).cuda()
+    with torch.no_grad():
+        got = model(dl.PackBitsTensor(xd, bit_count=64)).cpu().numpy()
+    assert np.array_equal(got, interp.net_eval(x, layers, 10))
+    logic = [m for m in model if isinstance(m, dl.LogicLayer)]
+    # (1) through .data, then invalidate_wiring
+    layers2 = [(np.roll(a, 3), b[::-1].copy(), op) for a, b, op in layers]
+    for m, (a, b, _) in zip(logic, layers2):
+        m.indices[0].data.copy_(torch.as_tensor(a))
+        m.indices[1].data.copy_(torch.as_tensor(b))
+        m.invalidate_wiring()
+    with torch.no_grad():
+        got2 = model(dl.PackBitsTensor(xd, bit_count=64)).cpu().numpy()
+    assert np.array_equal(got2, interp.net_eval(x, layers2, 10))
+    start, idx = oc.reverse_index(layers2[1][0], layers2[1][1], widths[0])
+    assert np.array_equal(logic[1].given_x_indices_of_y_start.cpu().numpy(), start)
+    assert np.array_equal(logic[1].given_x_indices_of_y.cpu().numpy(), idx)
+    # (2) an in-place operation (version bump): nothing to call
+    layers3 = [(b, a, op) for a, b, op in layers2]
+    for m, (a, b, _) in zip(logic, layers3):
+        m.indices[0].copy_(torch.as_tensor(a))
+        m.indices[1].copy_(torch.as_tensor(b))
+    with torch.no_grad():
+        got3 = model(dl.PackBitsTensor(xd, bit_count=64)).cpu().numpy()
+    assert np.array_equal(got3, interp.net_eval(x, layers3, 10))
+    # (3) set_connections
+    for m, (a, b, _) in zip(logic, layers):
+        m.set_connections(torch.as_tensor(a), torch.as_tensor(b))
+    with torch.no_grad():
+        got4 = model(dl.PackBitsTensor(xd, bit_count=64)).cpu().numpy()
+    assert np.array_equal(got4, got)
 
 
 @pytest.mark.parametrize("bits,in_dim,widths,W,k,pad", [

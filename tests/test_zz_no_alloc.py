@@ -43,14 +43,18 @@ def test_noalloc_matches_allocating_entry_point_twice_in_a_row():
         xd = _dev(x)
         want = ext.eval_fused_groupbitsum(xd, dev_layers, pad, k)
         order = ext.count_order_for(dev_layers, in_dim, k)
+        out = torch.full((W * 64 - pad, k), -1, dtype=torch.int32, device="cuda")
+        out2 = torch.empty_like(out)
+        # one call ahead of the measurement: the first call on a device looks the scratch array's address up
+        ext.eval_fused_groupbitsum_noalloc(xd, dev_layers, pad, k, out2)
         torch.cuda.synchronize()
         before = torch.cuda.memory_stats()["allocation.all.allocated"]
-        out = torch.full((W * 64 - pad, k), -1, dtype=torch.int32, device="cuda")
-        mid = torch.cuda.memory_stats()["allocation.all.allocated"]
+        free_before = torch.cuda.mem_get_info()[0]              # the driver's view: sees a hipMalloc inside the library too
         got = ext.eval_fused_groupbitsum_noalloc(xd, dev_layers, pad, k, out)
-        got2 = ext.eval_fused_groupbitsum_noalloc(xd, dev_layers, pad, k, torch.empty_like(out), order)
-        after = torch.cuda.memory_stats()["allocation.all.allocated"]
-        assert mid - before == 1 and after - mid == 1          # torch allocated only the two `out` tensors
+        got2 = ext.eval_fused_groupbitsum_noalloc(xd, dev_layers, pad, k, out2, order)
+        torch.cuda.synchronize()
+        assert torch.cuda.memory_stats()["allocation.all.allocated"] == before      # nothing through torch's allocator
+        assert torch.cuda.mem_get_info()[0] == free_before                          # and nothing behind its back
         assert got is out and torch.equal(got, want) and torch.equal(got2, want)
         assert np.array_equal(got.cpu().numpy(), _oracle(x, layers, pad, k))
 
@@ -75,3 +79,45 @@ def test_noalloc_rejects_what_does_not_fit():
     null = ctypes.c_void_p(0)
     assert lib.dl_logic_eval_fused_groupbitsum_noalloc(null, 3, null, null, null, null, null, 1, 64, 0, 10, null,
                                                        null) == _lib.DL_ERR_INVALID_ARGUMENT
+
+
+def test_noalloc_first_call_on_a_device_is_refused_under_graph_capture():
+    """The first call on a device looks the scratch array's address up with a runtime call, which must not happen
+    while the stream is being captured: DL_ERR_CAPTURING then, and the same call works once one call was made
+    outside a capture.  In a process of its own, where no call has been made yet."""
+    import os
+    import subprocess
+    import sys
+    code = r'''
+import numpy as np, torch
+from difflogic_amd import difflogic_cuda as ext
+rng = np.random.default_rng(1)
+dev = lambda a: torch.as_tensor(np.ascontiguousarray(a)).cuda()
+layers = [(dev(rng.integers(0, 50, 640)), dev(rng.integers(0, 50, 640)), dev(rng.integers(0, 16, 640).astype(np.uint8)))]
+x = dev(rng.integers(0, 1 << 62, (50, 4), dtype=np.int64))
+out = torch.empty((256, 10), dtype=torch.int32, device="cuda")
+want = ext.eval_fused_groupbitsum(x, layers, 0, 10)
+torch.cuda.synchronize()
+stream = torch.cuda.Stream()
+graph = torch.cuda.CUDAGraph()
+try:
+    with torch.cuda.graph(graph, stream=stream):
+        ext.eval_fused_groupbitsum_noalloc(x, layers, 0, 10, out)
+    print("NOT REFUSED")
+except RuntimeError as e:
+    print("REFUSED:", e)
+torch.cuda.synchronize()
+ext.eval_fused_groupbitsum_noalloc(x, layers, 0, 10, out)          # outside a capture: looks the address up
+graph = torch.cuda.CUDAGraph()
+out.fill_(-1)
+with torch.cuda.graph(graph, stream=stream):
+    ext.eval_fused_groupbitsum_noalloc(x, layers, 0, 10, out)
+graph.replay()
+torch.cuda.synchronize()
+print("REPLAY EQUAL:", bool(torch.equal(out, want)))
+'''
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True, timeout=110)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "REFUSED: " in proc.stdout and "graph capture" in proc.stdout, proc.stdout
+    assert "REPLAY EQUAL: True" in proc.stdout, proc.stdout
