@@ -16,7 +16,7 @@ DL_ERR_TOO_LARGE = 6
 DL_ERR_SCRATCH_LIMIT = 7
 DL_ERR_CAPTURING = 8
 
-DL_F16, DL_F32, DL_F64 = 0, 1, 2
+DL_F16, DL_F32, DL_F64, DL_F16_W32, DL_F64_W32 = 0, 1, 2, 3, 4
 
 DL_STATIC_SCRATCH_BYTES = 64 << 20      # include/difflogic_hip.h
 

@@ -28,6 +28,21 @@ template <> __device__ __forceinline__ __half down<__half, float>(float v) { ret
 __device__ __forceinline__ float dl_fma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 __device__ __forceinline__ double dl_fma(double a, double b, double c) { return __builtin_fma(a, b, c); }
 
+// Gate weights (probabilities or logits) and their gradients sit next to activations of type T either in T as well
+// or, `w32`, in fp32 whatever T is: what a layer with fp32 weights needs for half / double activations (the
+// reference's --training-bit-count 16 / 64).  The pointers keep the type T* and are reinterpreted.
+template <typename T> __device__ __forceinline__ typename Acc<T>::type wload(const T *__restrict__ w, int64_t at, bool w32) {
+    typedef typename Acc<T>::type C;
+    if constexpr (sizeof(T) == sizeof(float)) return w[at];
+    else return w32 ? (C) reinterpret_cast<const float *>(w)[at] : up<T>(w[at]);
+}
+template <typename T> __device__ __forceinline__ void wstore(T *__restrict__ w, int64_t at, typename Acc<T>::type v, bool w32) {
+    typedef typename Acc<T>::type C;
+    if constexpr (sizeof(T) == sizeof(float)) w[at] = v;
+    else if (w32) reinterpret_cast<float *>(w)[at] = (float) v;
+    else w[at] = down<T, C>(v);
+}
+
 // y = lerp(lerp(P00, P01, b), lerp(P10, P11, b), a), three fused multiply-adds.
 template <typename C> __device__ __forceinline__ C mix(C av, C bv, C p00, C p10, C d0, C d1) {
     const C lo = dl_fma(bv, d0, p00);
@@ -47,11 +62,12 @@ template <typename C> __device__ __forceinline__ Corners<C> corners_of(const C (
     return c;
 }
 
-template <typename T> __device__ __forceinline__ Corners<typename Acc<T>::type> corners(const T *__restrict__ w, int64_t n) {
+template <typename T>
+__device__ __forceinline__ Corners<typename Acc<T>::type> corners(const T *__restrict__ w, int64_t n, bool w32) {
     typedef typename Acc<T>::type C;
     C g[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) g[i] = up<T>(w[n * 16 + i]);
+    for (int i = 0; i < 16; ++i) g[i] = wload<T>(w, n * 16 + i, w32);
     return corners_of<C>(g);
 }
 
@@ -168,17 +184,17 @@ template <typename T, bool LOGITS>
 __device__ __forceinline__ void corners4(const T *__restrict__ w, const int32_t (&n)[4], int lane, bool store_probs,
                                          T *__restrict__ probs, typename Acc<T>::type (&p00)[4],
                                          typename Acc<T>::type (&p10)[4], typename Acc<T>::type (&d0)[4],
-                                         typename Acc<T>::type (&d1)[4]) {
+                                         typename Acc<T>::type (&d1)[4], bool w32 = false) {
     typedef typename Acc<T>::type C;
     const int row = lane >> 4, gate = lane & 15;
     const int32_t mine = row == 0 ? n[0] : row == 1 ? n[1] : row == 2 ? n[2] : n[3];
     const bool valid = mine >= 0;
     const int64_t at = (int64_t) (valid ? mine : 0) * 16 + gate;
-    C p = up<T>(w[at]);
+    C p = wload<T>(w, at, w32);
     if (LOGITS) {
         const C e = dl_exp(p - row16_max(p));
         p = e / row16_sum(e);
-        if (store_probs && valid) probs[at] = down<T, C>(p);
+        if (store_probs && valid) wstore<T>(probs, at, p, w32);
     }
     const C zero = (C) 0;
     const C q00 = row16_sum((gate & 8) ? p : zero), q01 = row16_sum((gate & 4) ? p : zero);
@@ -202,7 +218,7 @@ template <typename T, int VEC, int NPW, bool LOGITS>
 __global__ __launch_bounds__(DL_BLOCK) void forward_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
                                                            const int64_t *__restrict__ b, const T *__restrict__ w,
                                                            T *__restrict__ y, T *__restrict__ probs, int64_t out_dim,
-                                                           int64_t ncols) {
+                                                           int64_t ncols, bool w32) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
     const int wave = dl_wave_in_block();
@@ -221,7 +237,7 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_kernel(const T *__restrict__
         ib[j] = b[n];
         ids[j] = n0 + j < out_dim ? (int32_t) (n0 + j) : -1;
     }
-    corners4<T, LOGITS>(w, ids, lane, blockIdx.y == 0, probs, p00, p10, d0, d1);
+    corners4<T, LOGITS>(w, ids, lane, blockIdx.y == 0, probs, p00, p10, d0, d1, w32);
     const P *xv = reinterpret_cast<const P *>(x);
     P *yv = reinterpret_cast<P *>(y);
     for (int64_t col = (int64_t) blockIdx.y * DL_WAVE + lane; col < ncols; col += (int64_t) gridDim.y * DL_WAVE) {
@@ -252,7 +268,7 @@ template <typename T>
 __device__ __forceinline__ void store_grad_w(int lane, bool neuron_valid, int64_t n, typename Acc<T>::type s00,
                                              typename Acc<T>::type s01, typename Acc<T>::type s10,
                                              typename Acc<T>::type s11, const T *__restrict__ probs,
-                                             T *__restrict__ gw) {
+                                             T *__restrict__ gw, bool w32 = false) {
     typedef typename Acc<T>::type C;
     const bool valid = lane < 16 && neuron_valid;
     C r = (C) 0;
@@ -261,11 +277,11 @@ __device__ __forceinline__ void store_grad_w(int lane, bool neuron_valid, int64_
     if (lane & 2) r += s10;
     if (lane & 1) r += s11;
     if (probs != nullptr) {
-        const C p = valid ? up<T>(probs[n * 16 + lane]) : (C) 0;
+        const C p = valid ? wload<T>(probs, n * 16 + lane, w32) : (C) 0;
         const C dot = row16_sum(p * r);
         r = p * (r - dot);
     }
-    if (valid) gw[n * 16 + lane] = down<T, C>(r);
+    if (valid) wstore<T>(gw, n * 16 + lane, r, w32);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -282,7 +298,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_w_kernel(const T *__restric
                                                               const int64_t *__restrict__ b,
                                                               const T *__restrict__ gy, const T *__restrict__ probs,
                                                               T *__restrict__ gw, int64_t out_dim, int64_t ncols,
-                                                              int64_t gdiv) {
+                                                              int64_t gdiv, bool w32) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
     __shared__ C partial[4][NPW][4];
@@ -361,7 +377,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_w_kernel(const T *__restric
 
 #pragma unroll
     for (int j = 0; j < NPW; ++j)
-        store_grad_w<T>(lane, n0 + j < out_dim, n0 + j, s00[j], s01[j], s10[j], s11[j], probs, gw);
+        store_grad_w<T>(lane, n0 + j < out_dim, n0 + j, s00[j], s01[j], s10[j], s11[j], probs, gw, w32);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -379,7 +395,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_x_kernel(const T *__restric
                                                               const int64_t *__restrict__ start,
                                                               const int64_t *__restrict__ idx, T *__restrict__ gx,
                                                               int64_t in_dim, int64_t ncols,
-                                                              typename Acc<T>::type scale, int64_t gdiv) {
+                                                              typename Acc<T>::type scale, int64_t gdiv, bool w32) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
     const int wave = dl_wave_in_block();
@@ -403,7 +419,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_x_kernel(const T *__restric
             const bool isaA = iaA == c, isaB = iaB == c;
             const P gA = gv[grad_row(nA, gdiv) * ncols + col], oA = xv[(isaA ? ibA : iaA) * ncols + col];
             const P gB = gv[grad_row(nB, gdiv) * ncols + col], oB = xv[(isaB ? ibB : iaB) * ncols + col];
-            const Corners<C> kA = corners<T>(w, nA), kB = corners<T>(w, nB);
+            const Corners<C> kA = corners<T>(w, nA, w32), kB = corners<T>(w, nB, w32);
             {
                 const C d0 = kA.p01 - kA.p00, d1 = kA.p11 - kA.p10, dd = d1 - d0, da = kA.p10 - kA.p00;
                 const C k0 = (isaA && ibA == c) ? (C) 0.5 * (da + d0) : (isaA ? da : d0);
@@ -439,7 +455,8 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_chain_kernel(const T *__rest
                                                                  const int32_t *__restrict__ neuron,
                                                                  const uint8_t *__restrict__ flip,
                                                                  const T *__restrict__ w, T *__restrict__ y,
-                                                                 T *__restrict__ probs, int64_t nchunks, int64_t ncols) {
+                                                                 T *__restrict__ probs, int64_t nchunks, int64_t ncols,
+                                                                 bool w32) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
     const int wave = dl_wave_in_block();
@@ -465,7 +482,7 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_chain_kernel(const T *__rest
 #pragma unroll
             for (int i = 0; i < 4; ++i) n[i] = neuron[s0 + j0 + i];
             C p00[4], p10[4], d0[4], d1[4];
-            corners4<T, LOGITS>(w, n, lane, ct == 0, probs, p00, p10, d0, d1);
+            corners4<T, LOGITS>(w, n, lane, ct == 0, probs, p00, p10, d0, d1, w32);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int j = j0 + i;
@@ -584,7 +601,7 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_chain_rows_kernel(const T *_
                                                                       const uint8_t *__restrict__ flip,
                                                                       const T *__restrict__ w, T *__restrict__ y,
                                                                       T *__restrict__ probs, int64_t steps, int chunk,
-                                                                      int64_t ncols) {
+                                                                      int64_t ncols, bool w32) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
     const int wave = dl_wave_in_block();
@@ -614,7 +631,7 @@ __global__ __launch_bounds__(DL_BLOCK) void forward_chain_rows_kernel(const T *_
 #pragma unroll
         for (int i = 0; i < 4; ++i) n[i] = g + i < s1 ? neuron[g + i] : -1;
         C p00[4], p10[4], d0[4], d1[4];
-        corners4<T, LOGITS>(w, n, lane, col0 == 0, probs, p00, p10, d0, d1);
+        corners4<T, LOGITS>(w, n, lane, col0 == 0, probs, p00, p10, d0, d1, w32);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int64_t s = g + i;
@@ -650,7 +667,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_w_chain_kernel(const T *__r
                                                                     const uint8_t *__restrict__ flip,
                                                                     const T *__restrict__ gy,
                                                                     const T *__restrict__ probs, T *__restrict__ gw,
-                                                                    int64_t nchunks, int64_t ncols, int64_t gdiv) {
+                                                                    int64_t nchunks, int64_t ncols, int64_t gdiv, bool w32) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
     const int wave = dl_wave_in_block();
@@ -696,7 +713,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_w_chain_kernel(const T *__r
             }
         }
         wave_sum4(s00, s01, s10, s11, lane);
-        store_grad_w<T>(lane, n >= 0, n >= 0 ? n : 0, s00, s01, s10, s11, probs, gw);
+        store_grad_w<T>(lane, n >= 0, n >= 0 ? n : 0, s00, s01, s10, s11, probs, gw, w32);
 #pragma unroll
         for (int q = 0; q < CPL; ++q) prev[q] = cur[q];
     }
@@ -739,7 +756,8 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
     const uint8_t *__restrict__ flip, const int32_t *__restrict__ dst, const T *__restrict__ w,
     const T *__restrict__ gy, const T *__restrict__ probs, T *__restrict__ gw,
     typename Acc<T>::type *__restrict__ partial, T *__restrict__ gx, T *__restrict__ overflow, int64_t steps, int chunk,
-    int64_t in_dim, int64_t out_dim, int64_t ncols, typename Acc<T>::type scale, int64_t gdiv, LowerLayer<T> low) {
+    int64_t in_dim, int64_t out_dim, int64_t ncols, typename Acc<T>::type scale, int64_t gdiv, LowerLayer<T> low,
+    bool w32) {
     typedef typename Acc<T>::type C;
     typedef Pack<T, VEC> P;
     constexpr bool RECOMPUTE = LOWER == 2;
@@ -851,7 +869,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
             load_row(xv, verts[s0 - 1], true, before);
         }
         load_row(gv, grad_row(n, gdiv), true, g);
-        const Corners<C> k = corners<T>(w, n);
+        const Corners<C> k = corners<T>(w, n, w32);
         const C d0 = k.p01 - k.p00, dd = (k.p11 - k.p10) - d0, da = k.p10 - k.p00;
         const C kv = f ? da : d0;
 #pragma unroll
@@ -888,7 +906,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
             }
         }
         load_row(gv, grad_row(nn, gdiv), valid, grad);
-        prob = up<T>(w[nn * 16 + gate]);
+        prob = wload<T>(w, nn * 16 + gate, w32);
     };
     P cur[CPL], g[CPL], la[LCPL], lb[LCPL];
     C pw, lpw = (C) 0;
@@ -940,7 +958,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_chain_kernel(
                 const C dot = row16_sum(pr * r);
                 r = pr * (r - dot);
             }
-            if (valid && lane < 16) gw[nn * 16 + lane] = down<T, C>(r);
+            if (valid && lane < 16) wstore<T>(gw, nn * 16 + lane, r, w32);
         } else if (valid && lane < 4) {              // several segments: backward_w_finish_kernel adds them
             const C mine = lane == 0 ? s00 : lane == 1 ? s01 : lane == 2 ? s10 : s11;
             partial[((int64_t) blockIdx.y * out_dim + nn) * 4 + lane] = mine;
@@ -1045,7 +1063,7 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_w_rows_kernel(LowerLayer<T>
 template <typename T>
 __global__ __launch_bounds__(DL_BLOCK) void backward_w_finish_kernel(const typename Acc<T>::type *__restrict__ partial,
                                                                      const T *__restrict__ probs, T *__restrict__ gw,
-                                                                     int64_t out_dim, int segments) {
+                                                                     int64_t out_dim, int segments, bool w32) {
     typedef typename Acc<T>::type C;
     const int lane = dl_lane();
     const int64_t n = ((int64_t) blockIdx.x * 4 + dl_wave_in_block()) * 4 + (lane >> 4);
@@ -1062,11 +1080,11 @@ __global__ __launch_bounds__(DL_BLOCK) void backward_w_finish_kernel(const typen
     if (gate & 2) r += sum[2];
     if (gate & 1) r += sum[3];
     if (probs != nullptr) {
-        const C p = valid ? up<T>(probs[n * 16 + gate]) : (C) 0;
+        const C p = valid ? wload<T>(probs, n * 16 + gate, w32) : (C) 0;
         const C dot = row16_sum(p * r);
         r = p * (r - dot);
     }
-    if (valid) gw[n * 16 + gate] = down<T, C>(r);
+    if (valid) wstore<T>(gw, n * 16 + gate, r, w32);
 }
 
 template <typename T> struct Vec16 { static constexpr int n = 16 / (int) sizeof(T); };
@@ -1078,7 +1096,7 @@ unsigned col_tiles(int64_t ncols) {
 
 template <typename T, bool LOGITS>
 int forward_t(const void *x, const int64_t *a, const int64_t *b, const void *w, void *y, void *probs, int64_t out_dim,
-              int64_t batch, hipStream_t s) {
+              int64_t batch, hipStream_t s, bool w32 = false) {
     constexpr int NPW = 4;
     const int64_t blocks = dl_ceil_div(out_dim, 4 * NPW);
     if (out_dim > 0x7fffffffLL) return DL_ERR_TOO_LARGE;     // neuron ids travel as int32 inside the kernel
@@ -1086,17 +1104,17 @@ int forward_t(const void *x, const int64_t *a, const int64_t *b, const void *w, 
     if (batch % V == 0 && dl_aligned(x, 16) && dl_aligned(y, 16)) {
         DL_LAUNCH((forward_kernel<T, V, NPW, LOGITS>), dim3((unsigned) blocks, col_tiles(batch / V)),
                            dim3(DL_BLOCK), 0, s, (const T *) x, a, b, (const T *) w, (T *) y, (T *) probs, out_dim,
-                           batch / V);
+                           batch / V, w32);
     } else {
         DL_LAUNCH((forward_kernel<T, 1, NPW, LOGITS>), dim3((unsigned) blocks, col_tiles(batch)), dim3(DL_BLOCK),
-                           0, s, (const T *) x, a, b, (const T *) w, (T *) y, (T *) probs, out_dim, batch);
+                           0, s, (const T *) x, a, b, (const T *) w, (T *) y, (T *) probs, out_dim, batch, w32);
     }
     return dl_launch_status();
 }
 
 template <typename T>
 int backward_w_t(const void *x, const int64_t *a, const int64_t *b, const void *gy, const void *probs, void *gw,
-                 int64_t out_dim, int64_t batch, hipStream_t s, int64_t gdiv = 0) {
+                 int64_t out_dim, int64_t batch, hipStream_t s, int64_t gdiv = 0, bool w32 = false) {
     constexpr int NPW = 2;       // neurons per wave when the workgroup's waves split a neuron's batch
     constexpr int NPW1 = 2;      // ... when a wave owns whole rows: short rows, more neurons' loads in flight per wave
     constexpr int V = Vec16<T>::n;
@@ -1110,20 +1128,20 @@ int backward_w_t(const void *x, const int64_t *a, const int64_t *b, const void *
     const T *xp = (const T *) x, *gp = (const T *) gy, *pp = (const T *) probs;
     T *wp = (T *) gw;
     if (vec && split)
-        DL_LAUNCH((backward_w_kernel<T, V, NPW, 4>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv);
+        DL_LAUNCH((backward_w_kernel<T, V, NPW, 4>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv, w32);
     else if (vec)
-        DL_LAUNCH((backward_w_kernel<T, V, NPW1, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv);
+        DL_LAUNCH((backward_w_kernel<T, V, NPW1, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv, w32);
     else if (split)
-        DL_LAUNCH((backward_w_kernel<T, 1, NPW, 4>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv);
+        DL_LAUNCH((backward_w_kernel<T, 1, NPW, 4>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv, w32);
     else
-        DL_LAUNCH((backward_w_kernel<T, 1, NPW1, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv);
+        DL_LAUNCH((backward_w_kernel<T, 1, NPW1, 1>), grid, block, 0, s, xp, a, b, gp, pp, wp, out_dim, ncols, gdiv, w32);
     return dl_launch_status();
 }
 
 template <typename T>
 int backward_x_t(const void *x, const int64_t *a, const int64_t *b, const void *w, const void *gy,
                  const int64_t *start, const int64_t *idx, void *gx, int64_t in_dim, int64_t batch, double scale,
-                 hipStream_t s, int64_t gdiv = 0) {
+                 hipStream_t s, int64_t gdiv = 0, bool w32 = false) {
     typedef typename Acc<T>::type C;
     constexpr int V = Vec16<T>::n;
     const int64_t blocks = dl_ceil_div(in_dim, 4);
@@ -1131,11 +1149,11 @@ int backward_x_t(const void *x, const int64_t *a, const int64_t *b, const void *
     if (batch % V == 0 && dl_aligned(x, 16) && dl_aligned(gy, 16) && dl_aligned(gx, 16)) {
         DL_LAUNCH((backward_x_kernel<T, V>), dim3((unsigned) blocks, col_tiles(batch / V)), dim3(DL_BLOCK), 0, s,
                            (const T *) x, a, b, (const T *) w, (const T *) gy, start, idx, (T *) gx, in_dim, batch / V,
-                           (C) scale, gdiv);
+                           (C) scale, gdiv, w32);
     } else {
         DL_LAUNCH((backward_x_kernel<T, 1>), dim3((unsigned) blocks, col_tiles(batch)), dim3(DL_BLOCK), 0, s,
                            (const T *) x, a, b, (const T *) w, (const T *) gy, start, idx, (T *) gx, in_dim, batch,
-                           (C) scale, gdiv);
+                           (C) scale, gdiv, w32);
     }
     return dl_launch_status();
 }
@@ -1418,7 +1436,7 @@ int chain_chunk(int64_t steps) {
 
 template <typename T, bool LOGITS>
 int forward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, const uint8_t *flip, int64_t steps,
-                    const void *w, void *y, void *probs, int64_t batch, hipStream_t s) {
+                    const void *w, void *y, void *probs, int64_t batch, hipStream_t s, bool w32 = false) {
     constexpr int V = Vec16<T>::n;
     if (batch % V != 0 || !dl_aligned(x, 16) || !dl_aligned(y, 16)) return DL_ERR_TOO_LARGE;
     const int64_t nchunks = steps / DL_TRAIN_CHUNK, ncols = batch / V;
@@ -1432,10 +1450,10 @@ int forward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, 
         const dim3 grid((unsigned) blocks, (unsigned) segments), block(DL_BLOCK);
         if (ncols <= 2 * DL_WAVE)
             DL_LAUNCH((forward_chain_rows_kernel<T, V, 2, LOGITS>), grid, block, 0, s, xp, verts, neuron, flip, wp,
-                               (T *) y, (T *) probs, steps, chunk, ncols);
+                               (T *) y, (T *) probs, steps, chunk, ncols, w32);
         else
             DL_LAUNCH((forward_chain_rows_kernel<T, V, 4, LOGITS>), grid, block, 0, s, xp, verts, neuron, flip, wp,
-                               (T *) y, (T *) probs, steps, chunk, ncols);
+                               (T *) y, (T *) probs, steps, chunk, ncols, w32);
         return dl_launch_status();
     }
     const int64_t blocks = dl_ceil_div(nchunks, 4);
@@ -1444,11 +1462,11 @@ int forward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, 
         // short rows: 8-byte vectors put a row on all 64 lanes instead of half of them
         constexpr int H = V >= 2 ? V / 2 : 1;
         DL_LAUNCH((forward_chain_kernel<T, H, DL_TRAIN_CHUNK, LOGITS>), dim3((unsigned) blocks, 1), dim3(DL_BLOCK), 0, s, xp,
-                  verts, neuron, flip, wp, (T *) y, (T *) probs, nchunks, 2 * ncols);
+                  verts, neuron, flip, wp, (T *) y, (T *) probs, nchunks, 2 * ncols, w32);
         return dl_launch_status();
     }
     DL_LAUNCH((forward_chain_kernel<T, V, DL_TRAIN_CHUNK, LOGITS>), dim3((unsigned) blocks, col_tiles(ncols)),
-                       dim3(DL_BLOCK), 0, s, xp, verts, neuron, flip, wp, (T *) y, (T *) probs, nchunks, ncols);
+                       dim3(DL_BLOCK), 0, s, xp, verts, neuron, flip, wp, (T *) y, (T *) probs, nchunks, ncols, w32);
     return dl_launch_status();
 }
 
@@ -1471,7 +1489,8 @@ int forward_chain_lower_t(const void *lx, const int64_t *la, const int64_t *lb, 
 
 template <typename T>
 int backward_w_chain_t(const void *x, const int32_t *verts, const int32_t *neuron, const uint8_t *flip, int64_t steps,
-                       const void *gy, const void *probs, void *gw, int64_t batch, hipStream_t s, int64_t gdiv = 0) {
+                       const void *gy, const void *probs, void *gw, int64_t batch, hipStream_t s, int64_t gdiv = 0,
+                       bool w32 = false) {
     constexpr int V = Vec16<T>::n;
     if (batch % V != 0 || !dl_aligned(x, 16) || !dl_aligned(gy, 16)) return DL_ERR_TOO_LARGE;
     const int64_t nchunks = steps / DL_TRAIN_CHUNK, ncols = batch / V;
@@ -1481,13 +1500,13 @@ int backward_w_chain_t(const void *x, const int32_t *verts, const int32_t *neuro
     const T *xp = (const T *) x, *gp = (const T *) gy, *pp = (const T *) probs;
     if (ncols <= DL_WAVE)
         DL_LAUNCH((backward_w_chain_kernel<T, V, 1, DL_TRAIN_CHUNK>), grid, block, 0, s, xp, verts, neuron, flip,
-                           gp, pp, (T *) gw, nchunks, ncols, gdiv);
+                           gp, pp, (T *) gw, nchunks, ncols, gdiv, w32);
     else if (ncols <= 2 * DL_WAVE)
         DL_LAUNCH((backward_w_chain_kernel<T, V, 2, DL_TRAIN_CHUNK>), grid, block, 0, s, xp, verts, neuron, flip,
-                           gp, pp, (T *) gw, nchunks, ncols, gdiv);
+                           gp, pp, (T *) gw, nchunks, ncols, gdiv, w32);
     else
         DL_LAUNCH((backward_w_chain_kernel<T, V, 4, DL_TRAIN_CHUNK>), grid, block, 0, s, xp, verts, neuron, flip,
-                           gp, pp, (T *) gw, nchunks, ncols, gdiv);
+                           gp, pp, (T *) gw, nchunks, ncols, gdiv, w32);
     return dl_launch_status();
 }
 
@@ -1502,7 +1521,7 @@ int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron,
                      int64_t steps, const void *w, const void *gy, bool softmax_backward, const int32_t *fix_vertex,
                      const int32_t *fix_start, int64_t n_fix, int64_t overflow_rows, void *gw, void *gx, void *workspace,
                      int64_t in_dim, int64_t out_dim, int64_t batch, double scale, hipStream_t s, int64_t gdiv = 0,
-                     const LowerLayer<T> *lower = nullptr) {
+                     const LowerLayer<T> *lower = nullptr, bool w32 = false) {
     typedef typename Acc<T>::type C;
     constexpr int V = Vec16<T>::n;
     if (batch % V != 0 || !dl_aligned(x, 16) || !dl_aligned(gy, 16) || !dl_aligned(gx, 16) || !dl_aligned(workspace, 16))
@@ -1512,7 +1531,7 @@ int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron,
     if (ncols > DL_ROWS_MAX_VECTORS) return DL_ERR_TOO_LARGE;
     const int segments = row_segments(ncols);
     // with `lower`: whole rows per wave only, and gx holds the n_fix rows that finish after the pass
-    if (lower && (segments > 1 || !dl_aligned(lower->x, 16))) return DL_ERR_TOO_LARGE;
+    if (lower && (segments > 1 || !dl_aligned(lower->x, 16) || w32)) return DL_ERR_TOO_LARGE;
     const LowerLayer<T> none = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
     // workspace: [segments x out x 4 corner sums (only with several segments)] [overflow rows]
     const int64_t partial_bytes = backward_partial_bytes<T>(out_dim, batch);
@@ -1529,13 +1548,16 @@ int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron,
     do {                                                                                                                    \
         if (lower && !x)                                                                                                    \
             DL_LAUNCH((backward_chain_kernel<T, VV, CPL, 2>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp,     \
-                      pp, (T *) gw, partial, (T *) gx, overflow, steps, chunk, in_dim, out_dim, NC, (C) scale, gdiv, *lower); \
+                      pp, (T *) gw, partial, (T *) gx, overflow, steps, chunk, in_dim, out_dim, NC, (C) scale, gdiv, *lower, \
+                      false);                                                                                               \
         else if (lower)                                                                                                     \
             DL_LAUNCH((backward_chain_kernel<T, VV, CPL, 1>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp,     \
-                      pp, (T *) gw, partial, (T *) gx, overflow, steps, chunk, in_dim, out_dim, NC, (C) scale, gdiv, *lower); \
+                      pp, (T *) gw, partial, (T *) gx, overflow, steps, chunk, in_dim, out_dim, NC, (C) scale, gdiv, *lower, \
+                      false);                                                                                               \
         else                                                                                                                \
             DL_LAUNCH((backward_chain_kernel<T, VV, CPL, 0>), grid, block, 0, s, xp, verts, neuron, flip, dst, wp, gp,     \
-                      pp, (T *) gw, partial, (T *) gx, overflow, steps, chunk, in_dim, out_dim, NC, (C) scale, gdiv, none);  \
+                      pp, (T *) gw, partial, (T *) gx, overflow, steps, chunk, in_dim, out_dim, NC, (C) scale, gdiv, none,   \
+                      w32);                                                                                                 \
     } while (0)
     if (V >= 2 && ncols <= DL_WAVE / 2)
         DL_LAUNCH_BACKWARD_CHAIN(H, 1, 2 * ncols);   // short rows: 8-byte vectors use all 64 lanes
@@ -1552,7 +1574,7 @@ int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron,
         const int64_t fin_blocks = dl_ceil_div(out_dim, 16);
         if (fin_blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
         DL_LAUNCH(backward_w_finish_kernel<T>, dim3((unsigned) fin_blocks), block, 0, s, (const C *) partial, pp, (T *) gw,
-                  out_dim, segments);
+                  out_dim, segments, w32);
         st = dl_launch_status();
         if (st != DL_OK) return st;
     }
@@ -1566,11 +1588,26 @@ int backward_chain_t(const void *x, const int32_t *verts, const int32_t *neuron,
     return dl_launch_status();
 }
 
+// DL_F16_W32 / DL_F64_W32 (activations in half / double, gate weights and their gradients in fp32) -> the
+// activations' dtype; returns whether the weights are fp32
+bool weights_fp32(int &dtype) {
+    if (dtype == DL_F16_W32) {
+        dtype = DL_F16;
+        return true;
+    }
+    if (dtype == DL_F64_W32) {
+        dtype = DL_F64;
+        return true;
+    }
+    return false;
+}
+
 }  // namespace
 
 extern "C" int64_t dl_logic_backward_chained_workspace_bytes(int64_t overflow_rows, int64_t out_dim, int64_t batch,
                                                              int dtype) {
     if (overflow_rows < 0 || out_dim < 0 || batch < 0) return -DL_ERR_INVALID_ARGUMENT;
+    weights_fp32(dtype);
     switch (dtype) {
     case DL_F16: return backward_partial_bytes<__half>(out_dim, batch) + overflow_rows * batch * 2;
     case DL_F32: return backward_partial_bytes<float>(out_dim, batch) + overflow_rows * batch * 4;
@@ -1585,6 +1622,7 @@ extern "C" int dl_logic_backward_chained(const void *x, const int32_t *verts, co
                                          int64_t n_fix, int64_t overflow_rows, void *grad_w, void *grad_x,
                                          void *workspace, int64_t in_dim, int64_t out_dim, int64_t batch, double scale,
                                          int dtype, void *stream) {
+    const bool w32 = weights_fp32(dtype);
     if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
     if (in_dim <= 0 || out_dim <= 0 || batch <= 0 || steps < out_dim || n_fix < 0 || n_fix > in_dim || overflow_rows < 0)
         return DL_ERR_INVALID_ARGUMENT;
@@ -1595,13 +1633,15 @@ extern "C" int dl_logic_backward_chained(const void *x, const int32_t *verts, co
     switch (dtype) {
     case DL_F16:
         return backward_chain_t<__half>(x, verts, neuron, flip, dst, steps, w, grad_y, sb, fix_vertex, fix_start, n_fix,
-                                        overflow_rows, grad_w, grad_x, workspace, in_dim, out_dim, batch, scale, s);
+                                        overflow_rows, grad_w, grad_x, workspace, in_dim, out_dim, batch, scale, s, 0, nullptr,
+                                        w32);
     case DL_F32:
         return backward_chain_t<float>(x, verts, neuron, flip, dst, steps, w, grad_y, sb, fix_vertex, fix_start, n_fix,
                                        overflow_rows, grad_w, grad_x, workspace, in_dim, out_dim, batch, scale, s);
     default:
         return backward_chain_t<double>(x, verts, neuron, flip, dst, steps, w, grad_y, sb, fix_vertex, fix_start, n_fix,
-                                        overflow_rows, grad_w, grad_x, workspace, in_dim, out_dim, batch, scale, s);
+                                        overflow_rows, grad_w, grad_x, workspace, in_dim, out_dim, batch, scale, s, 0, nullptr,
+                                        w32);
     }
 }
 
@@ -1650,6 +1690,7 @@ extern "C" int dl_logic_backward_chained_lower(const void *x, const int32_t *ver
 extern "C" int dl_logic_forward_chained(const void *x, const int32_t *verts, const int32_t *neuron, const uint8_t *flip,
                                         int64_t steps, const void *w, void *y, void *probs, int64_t in_dim,
                                         int64_t out_dim, int64_t batch, int dtype, void *stream) {
+    const bool w32 = weights_fp32(dtype);
     if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
     if (in_dim < 0 || out_dim < 0 || batch <= 0 || steps < out_dim || steps % DL_TRAIN_CHUNK != 0)
         return DL_ERR_INVALID_ARGUMENT;
@@ -1658,15 +1699,15 @@ extern "C" int dl_logic_forward_chained(const void *x, const int32_t *verts, con
     hipStream_t s = (hipStream_t) stream;
     if (probs) {
         switch (dtype) {
-        case DL_F16: return forward_chain_t<__half, true>(x, verts, neuron, flip, steps, w, y, probs, batch, s);
+        case DL_F16: return forward_chain_t<__half, true>(x, verts, neuron, flip, steps, w, y, probs, batch, s, w32);
         case DL_F32: return forward_chain_t<float, true>(x, verts, neuron, flip, steps, w, y, probs, batch, s);
-        default: return forward_chain_t<double, true>(x, verts, neuron, flip, steps, w, y, probs, batch, s);
+        default: return forward_chain_t<double, true>(x, verts, neuron, flip, steps, w, y, probs, batch, s, w32);
         }
     }
     switch (dtype) {
-    case DL_F16: return forward_chain_t<__half, false>(x, verts, neuron, flip, steps, w, y, nullptr, batch, s);
+    case DL_F16: return forward_chain_t<__half, false>(x, verts, neuron, flip, steps, w, y, nullptr, batch, s, w32);
     case DL_F32: return forward_chain_t<float, false>(x, verts, neuron, flip, steps, w, y, nullptr, batch, s);
-    default: return forward_chain_t<double, false>(x, verts, neuron, flip, steps, w, y, nullptr, batch, s);
+    default: return forward_chain_t<double, false>(x, verts, neuron, flip, steps, w, y, nullptr, batch, s, w32);
     }
 }
 
@@ -1704,6 +1745,7 @@ extern "C" int dl_logic_backward_w_chained(const void *x, const int32_t *verts, 
                                            const uint8_t *flip, int64_t steps, const void *grad_y, const void *probs,
                                            void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch, int dtype,
                                            void *stream) {
+    const bool w32 = weights_fp32(dtype);
     if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
     if (in_dim < 0 || out_dim < 0 || batch <= 0 || steps < out_dim || steps % DL_TRAIN_CHUNK != 0)
         return DL_ERR_INVALID_ARGUMENT;
@@ -1711,44 +1753,47 @@ extern "C" int dl_logic_backward_w_chained(const void *x, const int32_t *verts, 
     if (!x || !verts || !neuron || !flip || !grad_y || !grad_w || in_dim == 0) return DL_ERR_INVALID_ARGUMENT;
     hipStream_t s = (hipStream_t) stream;
     switch (dtype) {
-    case DL_F16: return backward_w_chain_t<__half>(x, verts, neuron, flip, steps, grad_y, probs, grad_w, batch, s);
+    case DL_F16: return backward_w_chain_t<__half>(x, verts, neuron, flip, steps, grad_y, probs, grad_w, batch, s, 0, w32);
     case DL_F32: return backward_w_chain_t<float>(x, verts, neuron, flip, steps, grad_y, probs, grad_w, batch, s);
-    default: return backward_w_chain_t<double>(x, verts, neuron, flip, steps, grad_y, probs, grad_w, batch, s);
+    default: return backward_w_chain_t<double>(x, verts, neuron, flip, steps, grad_y, probs, grad_w, batch, s, 0, w32);
     }
 }
 
 extern "C" int dl_logic_forward(const void *x, const int64_t *a, const int64_t *b, const void *w, void *y,
                                 int64_t in_dim, int64_t out_dim, int64_t batch, int dtype, void *stream) {
+    const bool w32 = weights_fp32(dtype);
     if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
     if (in_dim < 0 || out_dim < 0 || batch < 0) return DL_ERR_INVALID_ARGUMENT;
     if (out_dim == 0 || batch == 0) return DL_OK;
     if (!x || !a || !b || !w || !y || in_dim == 0) return DL_ERR_INVALID_ARGUMENT;
     hipStream_t s = (hipStream_t) stream;
     switch (dtype) {
-    case DL_F16: return forward_t<__half, false>(x, a, b, w, y, nullptr, out_dim, batch, s);
+    case DL_F16: return forward_t<__half, false>(x, a, b, w, y, nullptr, out_dim, batch, s, w32);
     case DL_F32: return forward_t<float, false>(x, a, b, w, y, nullptr, out_dim, batch, s);
-    default: return forward_t<double, false>(x, a, b, w, y, nullptr, out_dim, batch, s);
+    default: return forward_t<double, false>(x, a, b, w, y, nullptr, out_dim, batch, s, w32);
     }
 }
 
 extern "C" int dl_logic_forward_logits(const void *x, const int64_t *a, const int64_t *b, const void *logits, void *y,
                                        void *probs, int64_t in_dim, int64_t out_dim, int64_t batch, int dtype,
                                        void *stream) {
+    const bool w32 = weights_fp32(dtype);
     if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
     if (in_dim < 0 || out_dim < 0 || batch <= 0) return DL_ERR_INVALID_ARGUMENT;   // probs are written by column tile 0
     if (out_dim == 0) return DL_OK;
     if (!x || !a || !b || !logits || !y || !probs || in_dim == 0) return DL_ERR_INVALID_ARGUMENT;
     hipStream_t s = (hipStream_t) stream;
     switch (dtype) {
-    case DL_F16: return forward_t<__half, true>(x, a, b, logits, y, probs, out_dim, batch, s);
+    case DL_F16: return forward_t<__half, true>(x, a, b, logits, y, probs, out_dim, batch, s, w32);
     case DL_F32: return forward_t<float, true>(x, a, b, logits, y, probs, out_dim, batch, s);
-    default: return forward_t<double, true>(x, a, b, logits, y, probs, out_dim, batch, s);
+    default: return forward_t<double, true>(x, a, b, logits, y, probs, out_dim, batch, s, w32);
     }
 }
 
 extern "C" int dl_logic_backward_w(const void *x, const int64_t *a, const int64_t *b, const void *grad_y,
                                    void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch, int dtype,
                                    void *stream) {
+    const bool w32 = weights_fp32(dtype);
     if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
     if (in_dim < 0 || out_dim < 0 || batch < 0) return DL_ERR_INVALID_ARGUMENT;
     if (out_dim == 0) return DL_OK;
@@ -1756,15 +1801,16 @@ extern "C" int dl_logic_backward_w(const void *x, const int64_t *a, const int64_
     if (batch > 0 && (!x || !grad_y)) return DL_ERR_INVALID_ARGUMENT;
     hipStream_t s = (hipStream_t) stream;
     switch (dtype) {
-    case DL_F16: return backward_w_t<__half>(x, a, b, grad_y, nullptr, grad_w, out_dim, batch, s);
+    case DL_F16: return backward_w_t<__half>(x, a, b, grad_y, nullptr, grad_w, out_dim, batch, s, 0, w32);
     case DL_F32: return backward_w_t<float>(x, a, b, grad_y, nullptr, grad_w, out_dim, batch, s);
-    default: return backward_w_t<double>(x, a, b, grad_y, nullptr, grad_w, out_dim, batch, s);
+    default: return backward_w_t<double>(x, a, b, grad_y, nullptr, grad_w, out_dim, batch, s, 0, w32);
     }
 }
 
 extern "C" int dl_logic_backward_logits(const void *x, const int64_t *a, const int64_t *b, const void *grad_y,
                                         const void *probs, void *grad_logits, int64_t in_dim, int64_t out_dim,
                                         int64_t batch, int dtype, void *stream) {
+    const bool w32 = weights_fp32(dtype);
     if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
     if (in_dim < 0 || out_dim < 0 || batch < 0) return DL_ERR_INVALID_ARGUMENT;
     if (out_dim == 0) return DL_OK;
@@ -1772,9 +1818,9 @@ extern "C" int dl_logic_backward_logits(const void *x, const int64_t *a, const i
     if (batch > 0 && (!x || !grad_y)) return DL_ERR_INVALID_ARGUMENT;
     hipStream_t s = (hipStream_t) stream;
     switch (dtype) {
-    case DL_F16: return backward_w_t<__half>(x, a, b, grad_y, probs, grad_logits, out_dim, batch, s);
+    case DL_F16: return backward_w_t<__half>(x, a, b, grad_y, probs, grad_logits, out_dim, batch, s, 0, w32);
     case DL_F32: return backward_w_t<float>(x, a, b, grad_y, probs, grad_logits, out_dim, batch, s);
-    default: return backward_w_t<double>(x, a, b, grad_y, probs, grad_logits, out_dim, batch, s);
+    default: return backward_w_t<double>(x, a, b, grad_y, probs, grad_logits, out_dim, batch, s, 0, w32);
     }
 }
 
@@ -1782,6 +1828,7 @@ extern "C" int dl_logic_backward_x(const void *x, const int64_t *a, const int64_
                                    const void *grad_y, const int64_t *start, const int64_t *idx, void *grad_x,
                                    int64_t in_dim, int64_t out_dim, int64_t batch, double scale, int dtype,
                                    void *stream) {
+    const bool w32 = weights_fp32(dtype);
     if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
     if (in_dim < 0 || out_dim < 0 || batch < 0) return DL_ERR_INVALID_ARGUMENT;
     if (in_dim == 0 || batch == 0) return DL_OK;
@@ -1789,9 +1836,9 @@ extern "C" int dl_logic_backward_x(const void *x, const int64_t *a, const int64_
     if (out_dim > 0 && (!a || !b || !w || !grad_y || !idx)) return DL_ERR_INVALID_ARGUMENT;
     hipStream_t s = (hipStream_t) stream;
     switch (dtype) {
-    case DL_F16: return backward_x_t<__half>(x, a, b, w, grad_y, start, idx, grad_x, in_dim, batch, scale, s);
+    case DL_F16: return backward_x_t<__half>(x, a, b, w, grad_y, start, idx, grad_x, in_dim, batch, scale, s, 0, w32);
     case DL_F32: return backward_x_t<float>(x, a, b, w, grad_y, start, idx, grad_x, in_dim, batch, scale, s);
-    default: return backward_x_t<double>(x, a, b, w, grad_y, start, idx, grad_x, in_dim, batch, scale, s);
+    default: return backward_x_t<double>(x, a, b, w, grad_y, start, idx, grad_x, in_dim, batch, scale, s, 0, w32);
     }
 }
 

@@ -110,8 +110,11 @@ class LogicLayer(torch.nn.Module):
         a, b = self.indices
         tail = (self.given_x_indices_of_y_start, self.given_x_indices_of_y, float(self.grad_factor))
         if self.training:
-            if self.weights.dtype == x.dtype and x.shape[1] > 0:
-                # softmax and its backward run inside the layer kernels
+            same = self.weights.dtype == x.dtype
+            mixed = self.weights.dtype == torch.float32 and x.dtype in (torch.float16, torch.float64)
+            if (same or mixed) and x.shape[1] > 0:
+                # softmax and its backward run inside the layer kernels; fp32 weights next to half / double
+                # activations (the reference's --training-bit-count 16 / 64) are read as they are
                 return LogicLayerLogitsFunction.apply(x, a, b, self.weights, *tail,
                                                       self._train_schedule()).transpose(0, 1)
             w = torch.nn.functional.softmax(self.weights, dim=-1).to(x.dtype)

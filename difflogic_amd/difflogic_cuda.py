@@ -45,6 +45,20 @@ def _float_code(t, name):
     return code
 
 
+_MIXED_CODES = {torch.float16: _lib.DL_F16_W32, torch.float64: _lib.DL_F64_W32}
+
+
+def _layer_code(x, w, name):
+    """dtype code of a layer call: activations ``x`` and gate weights / logits / probabilities ``w`` of one float
+    dtype (the reference's functions), or fp32 ``w`` next to half / double ``x`` (a layer with fp32 weights on
+    half / double inputs: experiments/main.py:19-23,286)."""
+    if w.dtype == x.dtype:
+        return _float_code(x, name)
+    if w.dtype == torch.float32 and x.dtype in _MIXED_CODES:
+        return _MIXED_CODES[x.dtype]
+    raise RuntimeError(f"{name}: expected weights of the activations' dtype ({x.dtype}) or float32, got {w.dtype}")
+
+
 def _same_device(*tensors):
     dev = tensors[0].device
     for t in tensors[1:]:
@@ -98,10 +112,10 @@ def forward(x, a, b, w, schedule=None):
     same result, one gathered input row per neuron instead of two."""
     for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w")):
         _check_input(t, n)
-    code = _float_code(x, "logic_layer_cuda_forward")
-    if x.dim() != 2 or w.dim() != 2 or w.shape[1] != 16 or w.dtype != x.dtype:
-        raise RuntimeError(f"expected x [in,B] and w [out,16] of one dtype, got {tuple(x.shape)} {x.dtype}, "
+    if x.dim() != 2 or w.dim() != 2 or w.shape[1] != 16:
+        raise RuntimeError(f"expected x [in,B] and w [out,16], got {tuple(x.shape)} {x.dtype}, "
                            f"{tuple(w.shape)} {w.dtype}")
+    code = _layer_code(x, w, "logic_layer_cuda_forward")
     out_dim = w.shape[0]
     _check_index(a, "a", out_dim)
     _check_index(b, "b", out_dim)
@@ -161,11 +175,11 @@ def backward_x(x, a, b, w, grad_y, given_x_indices_of_y_start, given_x_indices_o
                  (given_x_indices_of_y_start, "given_x_indices_of_y_start"),
                  (given_x_indices_of_y, "given_x_indices_of_y")):
         _check_input(t, n)
-    code = _float_code(x, "logic_layer_cuda_backward_x")
     if (x.dim() != 2 or grad_y.dim() != 2 or grad_y.shape[1] != x.shape[1] or grad_y.dtype != x.dtype
-            or w.dim() != 2 or w.shape != (grad_y.shape[0], 16) or w.dtype != x.dtype):
+            or w.dim() != 2 or w.shape != (grad_y.shape[0], 16)):
         raise RuntimeError(f"expected x [in,B], w [out,16], grad_y [out,B] of one dtype, got {tuple(x.shape)}, "
                            f"{tuple(w.shape)}, {tuple(grad_y.shape)}")
+    code = _layer_code(x, w, "logic_layer_cuda_backward_x")
     in_dim, batch = x.shape
     out_dim = grad_y.shape[0]
     _check_index(a, "a", out_dim)
@@ -187,21 +201,23 @@ def forward_logits(x, a, b, logits, schedule=None):
     """``forward(x, a, b, softmax(logits, -1))`` with the softmax computed inside the kernel.
     Returns (y [out,B], probs [out,16]); ``probs`` feeds backward_x / backward_logits.  Not part of
     the reference's extension (difflogic/difflogic.py:123-126 runs the softmax in torch).
+    ``logits`` have x's dtype, or are float32 next to a half / double x (``probs`` are float32 then,
+    and so is what backward_logits / backward_chained return for them).
     ``schedule`` (an EvalSchedule of (a, b)) selects the chained kernel: same result, one
     gathered input row per neuron instead of two."""
     for t, n in ((x, "x"), (a, "a"), (b, "b"), (logits, "logits")):
         _check_input(t, n)
-    code = _float_code(x, "logic_layer_cuda_forward")
-    if x.dim() != 2 or logits.dim() != 2 or logits.shape[1] != 16 or logits.dtype != x.dtype or x.shape[1] == 0:
-        raise RuntimeError(f"expected x [in,B>0] and logits [out,16] of one dtype, got {tuple(x.shape)} {x.dtype}, "
+    if x.dim() != 2 or logits.dim() != 2 or logits.shape[1] != 16 or x.shape[1] == 0:
+        raise RuntimeError(f"expected x [in,B>0] and logits [out,16], got {tuple(x.shape)} {x.dtype}, "
                            f"{tuple(logits.shape)} {logits.dtype}")
+    code = _layer_code(x, logits, "logic_layer_cuda_forward")
     out_dim = logits.shape[0]
     _check_index(a, "a", out_dim)
     _check_index(b, "b", out_dim)
     dev = _same_device(x, a, b, logits)
     in_dim, batch = x.shape
     y = torch.empty((out_dim, batch), dtype=x.dtype, device=dev)
-    probs = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
+    probs = torch.empty((out_dim, 16), dtype=logits.dtype, device=dev)
     lib = _lib.load()
     with _on(dev):
         st = _lib.DL_ERR_TOO_LARGE
@@ -230,17 +246,17 @@ def backward_logits(x, a, b, grad_y, probs, schedule=None):
     ``schedule`` selects the chained kernel (bit-identical result)."""
     for t, n in ((x, "x"), (a, "a"), (b, "b"), (grad_y, "grad_y"), (probs, "probs")):
         _check_input(t, n)
-    code = _float_code(x, "logic_layer_cuda_backward_w")
     if (x.dim() != 2 or grad_y.dim() != 2 or grad_y.shape[1] != x.shape[1] or grad_y.dtype != x.dtype
-            or probs.shape != (grad_y.shape[0], 16) or probs.dtype != x.dtype):
+            or probs.shape != (grad_y.shape[0], 16)):
         raise RuntimeError(f"expected x [in,B], grad_y [out,B], probs [out,16] of one dtype, got {tuple(x.shape)}, "
                            f"{tuple(grad_y.shape)}, {tuple(probs.shape)}")
+    code = _layer_code(x, probs, "logic_layer_cuda_backward_w")
     out_dim = grad_y.shape[0]
     _check_index(a, "a", out_dim)
     _check_index(b, "b", out_dim)
     dev = _same_device(x, a, b, grad_y, probs)
     in_dim, batch = x.shape
-    grad_logits = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
+    grad_logits = torch.empty((out_dim, 16), dtype=probs.dtype, device=dev)
     lib = _lib.load()
     with _on(dev):
         st = _lib.DL_ERR_TOO_LARGE
@@ -264,11 +280,11 @@ def backward_chained(x, w, grad_y, schedule, scale=1.0, softmax_backward=False):
     then uses the separate functions).  Not part of the reference's extension."""
     for t, n in ((x, "x"), (w, "w"), (grad_y, "grad_y")):
         _check_input(t, n)
-    code = _float_code(x, "logic_layer_cuda_backward")
     if (x.dim() != 2 or grad_y.dim() != 2 or grad_y.shape[1] != x.shape[1] or grad_y.dtype != x.dtype
-            or w.shape != (grad_y.shape[0], 16) or w.dtype != x.dtype):
+            or w.shape != (grad_y.shape[0], 16)):
         raise RuntimeError(f"expected x [in,B], w [out,16], grad_y [out,B] of one dtype, got {tuple(x.shape)}, "
                            f"{tuple(w.shape)}, {tuple(grad_y.shape)}")
+    code = _layer_code(x, w, "logic_layer_cuda_backward")
     dev = _same_device(x, w, grad_y)
     in_dim, batch = x.shape
     out_dim = grad_y.shape[0]
@@ -278,7 +294,7 @@ def backward_chained(x, w, grad_y, schedule, scale=1.0, softmax_backward=False):
     dst, fix_vertex, fix_start, n_fix, rows = schedule.backward_plan()
     if rows > in_dim * BACKWARD_CHAIN_MAX_OVERFLOW:
         return None
-    grad_w = torch.empty((out_dim, 16), dtype=x.dtype, device=dev)
+    grad_w = torch.empty((out_dim, 16), dtype=w.dtype, device=dev)
     grad_x = torch.empty_like(x)
     lib = _lib.load()
     ws_bytes = lib.dl_logic_backward_chained_workspace_bytes(rows, out_dim, batch, code)

@@ -43,7 +43,14 @@ typedef enum dl_status {
     DL_ERR_CAPTURING = 8         /* a first call per device that must not run under graph capture  */
 } dl_status;
 
-typedef enum dl_dtype { DL_F16 = 0, DL_F32 = 1, DL_F64 = 2 } dl_dtype;
+/* DL_F16_W32 / DL_F64_W32: activations and their gradients (x, y, grad_y, grad_x) in half / double, everything of
+ * shape [out, 16] (gate weights, logits, probabilities, grad_w, grad_logits) in fp32: a layer with fp32 weights on
+ * half / double inputs (the reference's --training-bit-count 16 / 64, experiments/main.py:19-23,286, casts the
+ * probabilities instead, difflogic/difflogic.py:123-126).  Accepted by dl_logic_forward, dl_logic_forward_logits,
+ * dl_logic_forward_chained, dl_logic_backward_w, dl_logic_backward_logits, dl_logic_backward_w_chained,
+ * dl_logic_backward_x, dl_logic_backward_chained and dl_logic_backward_chained_workspace_bytes; every other
+ * entry point answers DL_ERR_DTYPE. */
+typedef enum dl_dtype { DL_F16 = 0, DL_F32 = 1, DL_F64 = 2, DL_F16_W32 = 3, DL_F64_W32 = 4 } dl_dtype;
 
 /* Library version (major*10000 + minor*100 + patch) and a static message per status. */
 int dl_version(void);

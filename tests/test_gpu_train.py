@@ -511,6 +511,53 @@ def test_layer_module_with_half_and_double_activations(dtype, rtol, along_schedu
     assert ok, err
 
 
+@pytest.mark.parametrize("dtype,rtol", [(torch.float16, 4e-3), (torch.float64, 1e-5)])
+@pytest.mark.parametrize("in_dim,out_dim,batch", [(20, 50, 37), (48, 120, 264), (64, 200, 1040), (30, 64, 4104), (16, 24, 8)])
+def test_kernels_take_fp32_weights_beside_half_and_double_activations(ext, dtype, rtol, in_dim, out_dim, batch):
+    """DL_F16_W32 / DL_F64_W32 through the bindings: half / double activations and gradients, fp32 logits,
+    probabilities and logit gradients, with the softmax and its backward inside the kernels (the reference casts
+    the fp32 softmax to the activations' dtype in torch, difflogic/difflogic.py:123-126).  Plain kernels, the kernels
+    along the schedule and the one-pass backward, against fp64 arithmetic on the values as rounded to ``dtype``."""
+    x, a, b, _, gy = _case(in_dim + batch, in_dim, out_dim, batch, dtype=dtype)
+    g = torch.Generator().manual_seed(batch)
+    logits = torch.randn(out_dim, 16, generator=g)
+    xd, ad, bd, ld, gd = x.cuda(), a.cuda(), b.cuda(), logits.cuda(), gy.cuda()
+    sched = ext.schedule_for(ad, bd, in_dim)
+    start, idx = _csr(a, b, in_dim)
+
+    l64 = logits.double().requires_grad_()
+    x64 = x.double().t().contiguous().requires_grad_()
+    y64 = fo.layer_forward_sequential(x64, a, b, torch.softmax(l64, -1))           # [B, out]
+    (y64 * gy.double().t()).sum().backward()
+
+    for schedule in (None, sched):
+        y, probs = ext.forward_logits(xd, ad, bd, ld, schedule)
+        assert y.dtype == dtype and probs.dtype == torch.float32
+        assert close(probs, torch.softmax(logits.double(), -1), 2e-6)[0]
+        ok, err = close(y, y64.t().to(dtype), rtol)
+        assert ok, (schedule is not None, err)
+        gl = ext.backward_logits(xd, ad, bd, gd, probs, schedule)
+        assert gl.dtype == torch.float32
+        ok, err = close(gl, l64.grad, rtol)
+        assert ok, (schedule is not None, err)
+    gx = ext.backward_x(xd, ad, bd, probs, gd, start.cuda(), idx.cuda(), 1.5)
+    assert gx.dtype == dtype
+    ok, err = close(gx, 1.5 * x64.grad.t(), rtol)
+    assert ok, err
+    both = ext.backward_chained(xd, probs, gd, sched, 1.5, softmax_backward=True)
+    if both is not None:
+        assert both[0].dtype == torch.float32 and both[1].dtype == dtype
+        ok, err = close(both[0], l64.grad, rtol)
+        assert ok, err
+        ok, err = close(both[1], 1.5 * x64.grad.t(), rtol)
+        assert ok, err
+    # probabilities given instead of logits (the reference's forward), fp32 beside the activations
+    ok, err = close(ext.forward(xd, ad, bd, probs), y64.t().to(dtype), rtol)
+    assert ok, err
+    with pytest.raises(RuntimeError):
+        ext.forward(xd.float(), ad, bd, probs.double())           # only fp32 weights may differ from the activations
+
+
 @pytest.mark.parametrize("in_dim,out_dim,batch,k", [(12, 30, 7, 3), (33, 100, 256, 10), (50, 77, 513, 7), (16, 40, 2048, 2),
                                                     (64, 1300, 260, 10), (20, 64, 64, 1)])
 def test_forward_and_backward_fused_with_group_sum(ext, in_dim, out_dim, batch, k):
