@@ -132,7 +132,7 @@ class LogicLayer(torch.nn.Module):
         assert isinstance(x, PackBitsTensor)
         assert x.features == self.in_dim, (x.features, self.in_dim)
         a, b = self.indices
-        return x.defer_layer(a, b, self._gate_ids())
+        return x.defer_layer(a, b, self._gate_ids(), key=(self.weights.data_ptr(), self.weights._version, self.out_dim))
 
     # Below this many inputs a 1 KB column tile of the whole input stays in the L2 caches and the
     # second gather of a row hits there; above it the chained kernels halve the gathered rows.

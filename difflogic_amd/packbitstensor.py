@@ -16,10 +16,15 @@ _FABRIC_RATE = 7.5e12        # B/s: row gathers + stores between the L2s and Inf
 _WRITE_RATE = 6.1e12         # B/s: streaming stores to HBM
 _COUNT_RATE = 5.6e12         # B/s of counted rows: what the chained count kernel parks in LDS, sorts by class and adds up
 _LIVE_INPUT = 0.75           # share of gate inputs a gate looks at when the gate ids are uniform (10 of 16 gates use both
-                             # inputs, 4 one, 2 none); rows that no gate looks at are not fetched
+                             # inputs, 4 one, 2 none); rows that no gate looks at are not fetched.  The default where
+                             # the net's own share has not been measured (PackBitsTensor._live_share)
 _TILE_BYTES = 1024           # one wave covers 64 lanes x 16 bytes of a row
 _L2_RESIDENT_BYTES = 4 << 20     # input tiles (rows x 1 KB each) in flight up to this size are re-read from L2 (4 MB per XCD)
-_LDS_GATE_WORD_SECONDS = 9.4e-13     # LDS-resident whole-net kernel: seconds per gate and 64-sample word
+_LDS_GATE_WORD_SECONDS = 7.9e-13     # LDS-resident whole-net kernel: seconds per gate and 64-sample word
+_BOOL_STAGE_RATE = 5.2e12    # B/s of bool input bytes that the LDS kernel packs on their way into LDS
+_PACKED_STAGE_RATE = 1.5e12  # B/s of packed input rows on their way into LDS (16 or 32 bytes of every row per workgroup)
+_PACK_RATE = 4.8e12          # B/s (bool bytes read + words written) of the transpose-and-pack kernel
+_STREAM_CALL_SECONDS = 6e-5  # per call of the streaming path: constant folding, liveness and record kernels
 _LAUNCH_SECONDS = 3e-6       # per kernel on the stream; decides between plans for small batches only
 
 
@@ -28,19 +33,20 @@ def _chained(depth):
     return depth >= 2
 
 
-def group_cost(rows_in, out, depth, words, counted):
+def group_cost(rows_in, out, depth, words, counted, live=_LIVE_INPUT):
     """Modelled seconds of one fused group: `depth` layers from `rows_in` input rows to `out` output
-    rows of `words` 64-bit words, ending in the per-class count when `counted`."""
+    rows of `words` 64-bit words, ending in the per-class count when `counted`.  ``live``: share of the gate
+    inputs that their gate looks at (1.0: two-input gates only)."""
     row_bytes = 8.0 * words
     # rows gathered per output row: the leaves of a tree of gates that are looked at.  Along a schedule the tree is
     # the subtree under the vertex two consecutive neurons share (needed unless both ignore it).
-    shared_needed = 1 - (1 - _LIVE_INPUT) ** 2
+    shared_needed = 1 - (1 - live) ** 2
     if counted:                                    # walked along the schedule: one seed per 128 steps
-        gathers = (2 * _LIVE_INPUT) ** (depth - 1) * shared_needed * (1 + 1 / 128) * out
-    elif _chained(depth):                          # one seed per 16 steps
-        gathers = (2 * _LIVE_INPUT) ** (depth - 1) * shared_needed * (1 + 1 / 16) * out
+        gathers = (2 * live) ** (depth - 1) * shared_needed * (1 + 1 / 128) * out
+    elif _chained(depth):                          # one seed per 32 steps
+        gathers = (2 * live) ** (depth - 1) * shared_needed * (1 + 1 / 32) * out
     else:
-        gathers = (2 * _LIVE_INPUT) ** depth * out
+        gathers = (2 * live) ** depth * out
     gathered = gathers * row_bytes
     written = 0.0 if counted else out * row_bytes
     # The chip sweeps all output rows of one 1 KB column tile before the next, but a narrow layer
@@ -60,7 +66,7 @@ def group_cost(rows_in, out, depth, words, counted):
     return t + _LAUNCH_SECONDS * (3 if counted or _chained(depth) else 1)
 
 
-def plan_groups(dims, count_at_end, words=16384):
+def plan_groups(dims, count_at_end, words=16384, live=_LIVE_INPUT):
     """Splits consecutive layers into fused groups.
 
     ``dims`` = [in_dim, width_1, ..., width_L]; ``words`` = 64-bit words per row.  Returns a list of
@@ -76,31 +82,36 @@ def plan_groups(dims, count_at_end, words=16384):
             if counted and depth > difflogic_cuda.MAX_FUSE_DEPTH_COUNT:
                 continue
             prev = best[i - depth]
-            c = prev[0] + group_cost(dims[i - depth], dims[i], depth, words, counted)
+            c = prev[0] + group_cost(dims[i - depth], dims[i], depth, words, counted, live)
             if best[i] is None or c < best[i][0]:
                 best[i] = (c, prev[1] + [depth])
     return best[n][1]
 
 
-def plan_cost(dims, groups, count_at_end, words=16384):
+def plan_cost(dims, groups, count_at_end, words=16384, live=_LIVE_INPUT):
     """Modelled seconds of running ``groups`` (as plan_groups returns them) over ``dims``."""
     t, pos = 0.0, 0
     for j, depth in enumerate(groups):
-        t += group_cost(dims[pos], dims[pos + depth], depth, words, count_at_end and j == len(groups) - 1)
+        t += group_cost(dims[pos], dims[pos + depth], depth, words, count_at_end and j == len(groups) - 1, live)
         pos += depth
     return t
 
 
-def lds_cost(dims, words):
-    """Modelled seconds of the LDS-resident whole-net kernel over all of ``dims``."""
-    return sum(dims[1:]) * words * _LDS_GATE_WORD_SECONDS + 2 * _LAUNCH_SECONDS
+def lds_cost(dims, words, from_bool=False):
+    """Modelled seconds of the LDS-resident whole-net kernel over all of ``dims``; ``from_bool``: it reads the bool
+    input itself (64 bytes per word and feature) instead of packed words."""
+    staging = dims[0] * words * (64 / _BOOL_STAGE_RATE if from_bool else 8 / _PACKED_STAGE_RATE)
+    return sum(dims[1:]) * words * _LDS_GATE_WORD_SECONDS + staging + 2 * _LAUNCH_SECONDS
 
 
-def lds_tail(dims, words=16384):
+def lds_tail(dims, words=16384, live=_LIVE_INPUT, from_bool=False):
     """Number of layers at the end of the net (``dims`` = [in_dim, width_1, ..., width_L]) to run
     in the LDS-resident whole-net kernel together with the count: the longest run of trailing
     layers whose input and widths all fit its buffer, if the model prices it below the streaming
-    plan for the same layers (0 otherwise)."""
+    plan for the same layers (0 otherwise).  The LDS kernel evaluates every gate; the streaming kernels
+    skip what no gate looks at, so a net rich in pass-through gates (low ``live``) may stream faster.
+    ``from_bool``: the input has not been packed yet; if the whole net runs in LDS it never is, while the
+    streaming kernels need the pack kernel first."""
     limit = difflogic_cuda.net_lds_max_width()
     n = 0
     while n < len(dims) - 1 and n < difflogic_cuda.MAX_NET_DEPTH and max(dims[len(dims) - 2 - n:]) <= limit:
@@ -108,8 +119,25 @@ def lds_tail(dims, words=16384):
     if n == 0:
         return 0
     tail = dims[len(dims) - 1 - n:]
-    streaming = plan_cost(tail, plan_groups(tail, True, words), True, words)
-    return n if lds_cost(tail, words) < streaming else 0
+    whole = from_bool and n == len(dims) - 1
+    streaming = plan_cost(tail, plan_groups(tail, True, words, live), True, words, live) + _STREAM_CALL_SECONDS
+    if whole:
+        streaming += dims[0] * words * 72 / _PACK_RATE
+    return n if lds_cost(tail, words, whole) < streaming else 0
+
+
+# share of the gate inputs that their gate looks at, per set of weight tensors (see PackBitsTensor._live_share)
+_LIVE_SHARES = {}
+_USES_INPUTS = (0, 2, 2, 1, 2, 1, 2, 2, 2, 2, 1, 2, 1, 2, 2, 0)      # inputs gate id i looks at
+
+
+def measured_live_share(layers):
+    """Share of the gate inputs of ``layers`` = [(a, b, gate ids), ...] that their gate looks at (0.75 for uniformly
+    drawn ids, 1.0 for two-input gates only, 0.5 for pass-through gates only).  Reads the device: one
+    synchronisation."""
+    ids = torch.cat([w.reshape(-1) for _, _, w in layers]).long()
+    uses = torch.tensor(_USES_INPUTS, dtype=torch.float32, device=ids.device)
+    return float(uses[ids].mean().item()) / 2 if ids.numel() else _LIVE_INPUT
 
 
 class PackBitsTensor:
@@ -134,6 +162,7 @@ class PackBitsTensor:
         self._rows = None             # int64 [features, 2 * ceil(B / 128)]: the padded rows
         self._public = None           # what `.t` handed out or was set to, while it is current
         self._pending = []            # [(a, b, w)] applied to the rows but not yet evaluated
+        self._keys = []               # per pending layer: what identifies the weights its gate ids came from, or None
         self._folded = True           # constants folded through the pending layers' gate ids (_fold_pending)
         if device == "cuda":
             if bit_count not in (8, 16, 32, 64):
@@ -209,6 +238,24 @@ class PackBitsTensor:
             self._pending = difflogic_cuda.fold_gate_constants(self._pending)
         self._folded = True
 
+    def _live_share(self):
+        """Share of the pending layers' gate inputs that their gate looks at, for the launch planner.  Measured
+        once per set of weight tensors (and their version counters) and remembered: a stale or default value
+        changes the plan, never the result.  The default where it cannot be measured without disturbing the
+        caller (weights of unknown origin, a stream being captured into a graph)."""
+        if not self._pending or any(k is None for k in self._keys):
+            return _LIVE_INPUT
+        key = tuple(self._keys)
+        share = _LIVE_SHARES.get(key)
+        if share is None:
+            if torch.cuda.is_current_stream_capturing():
+                return _LIVE_INPUT
+            share = measured_live_share(self._pending)
+            if len(_LIVE_SHARES) >= 256:
+                _LIVE_SHARES.clear()
+            _LIVE_SHARES[key] = share
+        return share
+
     def _run_groups(self, groups, live=None):
         """Evaluates the first sum(groups) pending layers group by group.  ``live`` (difflogic_cuda.live_inputs of
         the pending layers): rows that the layers still pending afterwards do not look at need not be written; the
@@ -226,11 +273,12 @@ class PackBitsTensor:
         if pos:
             self._rows, self._public = rows, None
         self._pending = self._pending[pos:]
+        self._keys = self._keys[pos:]
 
     @property
     def t(self):
         if self._pending:
-            self._run_groups(plan_groups(self._dims(), False, self._words64()))
+            self._run_groups(plan_groups(self._dims(), False, self._words64(), self._live_share()))
         if self._public is None:
             rows = self._words()
             dtype = difflogic_cuda._BITS_TO_DTYPE[self.bit_count]
@@ -245,6 +293,7 @@ class PackBitsTensor:
     @t.setter
     def t(self, value):
         self._pending = []
+        self._keys = []
         self._folded = True
         self._src = None
         self._rows = None
@@ -252,9 +301,11 @@ class PackBitsTensor:
         bits = difflogic_cuda._WORD_BITS.get(value.dtype, self.bit_count)
         self._batch = max(0, value.shape[1] * bits - self.pad_len)
 
-    def defer_layer(self, a, b, w):
-        """Applies the gate layer (a, b, w) lazily."""
+    def defer_layer(self, a, b, w, key=None):
+        """Applies the gate layer (a, b, w) lazily.  ``key``: a hashable that changes whenever the gate ids ``w`` may
+        have (the weights' address and version counter); lets the planner remember what it measured for them."""
         self._pending.append((a, b, w))
+        self._keys.append(key)
         self._folded = False
         return self
 
@@ -264,7 +315,8 @@ class PackBitsTensor:
             if self.features % k != 0:
                 raise ValueError(f"in_dim ({self.features}) has to be divisible by k ({k}) but it is not")
             dims = self._dims()
-            tail = lds_tail(dims, self._words64())
+            share = self._live_share()
+            tail = lds_tail(dims, self._words64(), share, from_bool=self._src is not None)
             if tail:
                 # the narrow end of the net runs resident in LDS; what lies before it streams
                 head = len(self._pending) - tail
@@ -274,13 +326,13 @@ class PackBitsTensor:
                     if out is not None:
                         return out
                 if head:
-                    self._run_groups(plan_groups(dims[:head + 1], False, self._words64()))
+                    self._run_groups(plan_groups(dims[:head + 1], False, self._words64(), share))
                 rows = self._words()
                 out = difflogic_cuda.eval_net_lds(rows, self._pending, self._pad(rows), k)
                 if out is not None:
                     return out
             self._fold_pending()
-            groups = plan_groups(self._dims(), True, self._words64())
+            groups = plan_groups(self._dims(), True, self._words64(), share)
             # output rows of the groups before the last that no gate above them looks at are not computed
             live = difflogic_cuda.live_inputs(self._pending) if len(groups) > 1 else None
             self._run_groups(groups[:-1], live)
