@@ -49,6 +49,10 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 TRAFFIC_JSON = os.path.join(ROOT, "profiles", "packed_kernel_traffic.json")
+TRAIN_TRAFFIC_JSON = os.path.join(ROOT, "profiles", "train_step_traffic.json")
+# what the measured traffic of a training step depends on
+TRAIN_TRAFFIC_SOURCES = ("difflogic_amd/csrc/train.hip", "difflogic_amd/csrc/schedule.cpp", "difflogic_amd/csrc/dl_common.h",
+                         "difflogic_amd/difflogic.py")
 # what the measured traffic of the packed launches depends on: the kernels and the launch plan
 TRAFFIC_SOURCES = ("difflogic_amd/csrc/packed.hip", "difflogic_amd/csrc/count_chain.h", "difflogic_amd/csrc/schedule.cpp",
                    "difflogic_amd/csrc/dl_common.h", "difflogic_amd/packbitstensor.py")
@@ -71,6 +75,9 @@ def parse():
                     help="profiling aid: run only the configurations selected with --only and print their results")
     ap.add_argument("--gate-mix", default="uniform", choices=("uniform", "two_input_gates_only", "half_pass_through"),
                     help="profiling aid: run the headline with this gate mix (see GATE_MIXES) instead of the BASELINE config's")
+    ap.add_argument("--train-eager-only", default="", choices=("", "written", "fused"),
+                    help="profiling aid: of a training configuration run only the eager forward+backward loop of the model "
+                         "as written for the reference, or of the fuse_for_training model (for whole-step counters)")
     ap.add_argument("--cpu-sample-log2", type=int, default=18)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 4 plain device copies of 1 GiB (for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE)")
@@ -84,10 +91,10 @@ def parse():
     return ap.parse_args()
 
 
-def source_hash():
-    """sha256 over the sources the packed launches' traffic depends on."""
+def source_hash(sources=TRAFFIC_SOURCES):
+    """sha256 over the sources the measured traffic depends on (default: the packed launches')."""
     h = hashlib.sha256()
-    for rel in TRAFFIC_SOURCES:
+    for rel in sources:
         with open(os.path.join(ROOT, rel), "rb") as f:
             h.update(rel.encode() + b"\0" + f.read() + b"\0")
     return h.hexdigest()[:16]
@@ -287,9 +294,19 @@ def kernel_table(per_kernel, steps):
             for kk, v in per_kernel.items()}
 
 
+_TRAFFIC = None
+
+
 def load_traffic():
     """The committed rocprofv3 --pmc summary of the packed launches, or ({}, note) when it was
     taken from other kernel sources than the ones in the tree."""
+    global _TRAFFIC
+    if _TRAFFIC is None:
+        _TRAFFIC = read_traffic()
+    return _TRAFFIC
+
+
+def read_traffic():
     if not os.path.exists(TRAFFIC_JSON):
         return {}, "no traffic summary committed"
     with open(TRAFFIC_JSON) as f:
@@ -546,7 +563,7 @@ class GeneratedC:
             os.rmdir(self.work)
 
 
-def packed_config(torch, dl, name, F, widths, B, x, check_cpu, compiled=None):
+def packed_config(torch, dl, tag, name, F, widths, B, x, check_cpu, compiled=None):
     """One of the other packed configurations: samples/s, per-launch times, and the first 4096
     samples of the full-batch result compared with the CPU interpreter.  ``compiled``: the GeneratedC of this
     net started by main(), timed on the first 2^16 samples."""
@@ -556,10 +573,12 @@ def packed_config(torch, dl, name, F, widths, B, x, check_cpu, compiled=None):
     W = B // 64
     dims = [F] + list(widths)
     alg = sum(eval_layer_bytes(i, o, W) for i, o in zip(dims[:-1], dims[1:])) + 8 * W * dims[-1] + 4 * k * B
+    table, _ = load_traffic()
+    kernels, roofline = launch_rooflines(per_kernel, 5, table, prefix=tag + ": ")
     res = {"workload": name, "dtype": "int64", "samples_per_s": round(value, 1), "ms_per_step": round(ms, 4),
            "algorithmic_GB_per_step_without_pack": round(alg / 1e9, 2),
            "alg_over_peak": round(alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-           "first_call_ms": round(first_ms, 1), "hip_graph_replay": graph_info, "kernels": kernel_table(per_kernel, 5),
+           "first_call_ms": round(first_ms, 1), "hip_graph_replay": graph_info, "kernels": kernels, "roofline": roofline,
            "checksum": int(out.sum().item())}
     if check_cpu:
         from oracle import interp
@@ -592,7 +611,22 @@ def train_alg_bytes(dims, B):
     return alg + sum(4 * B * (2 * i + o) + 64 * o for i, o in zip(dims[1:-1], dims[2:]))
 
 
-def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor, x, steps, warmup, other_dtypes=False):
+def load_train_traffic(config):
+    """{variant: measured bytes between the L2s and the fabric per eager forward+backward step} of `config` from the
+    committed rocprofv3 --pmc summary, or {} when it was taken from other kernel sources than the ones in the tree."""
+    if not os.path.exists(TRAIN_TRAFFIC_JSON):
+        return {}
+    with open(TRAIN_TRAFFIC_JSON) as f:
+        table = json.load(f)
+    if table.get("_source_hash") != source_hash(TRAIN_TRAFFIC_SOURCES):
+        print("bench.py: WARNING: profiles/train_step_traffic.json was measured on other kernel sources than the tree's: "
+              "frac_hbm_traffic not reported", file=sys.stderr)
+        return {}
+    return table.get(config, {})
+
+
+def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor, x, steps, warmup, other_dtypes=False,
+                 eager_only="", config=""):
     """fp32 training step of one configuration with CrossEntropy: forward+backward and
     forward+backward+Adam(lr 0.01), each eager and replayed as one HIP graph; once for the model as
     the reference's user writes it (torch's fused Adam) and once with the training epilogue of this
@@ -620,14 +654,25 @@ def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps, last
 
-    def report(sec, loss):
-        return {"neuron_samples_per_s": round(neuron_samples / sec, 1), "ms_per_step": round(sec * 1e3, 4),
-                "alg_GBps": round(alg / sec / 1e9, 1), "frac_hbm_algorithmic": round(alg / sec / 1e9 / HBM_PEAK_GBS, 4),
-                "loss": round(float(loss), 6)}
+    traffic = load_train_traffic(config)
+
+    def report(sec, loss, variant=None):
+        r = {"neuron_samples_per_s": round(neuron_samples / sec, 1), "ms_per_step": round(sec * 1e3, 4),
+             "alg_GBps": round(alg / sec / 1e9, 1), "frac_hbm_algorithmic": round(alg / sec / 1e9 / HBM_PEAK_GBS, 4),
+             "loss": round(float(loss), 6)}
+        t = traffic.get(variant)
+        if t:
+            # measured bytes between the L2 caches and the fabric per step (rocprofv3 FETCH_SIZE + WRITE_SIZE over the
+            # same eager loop) over this run's time: the bandwidth; frac_hbm_algorithmic above is a ratio to compare
+            # against the per-layer formula, not a bandwidth
+            r["traffic_GB_per_step"] = round(t["hbm_bytes_per_step"] / 1e9, 3)
+            r["traffic_GBps"] = round(t["hbm_bytes_per_step"] / sec / 1e9, 1)
+            r["frac_hbm_traffic"] = round(t["hbm_bytes_per_step"] / sec / 1e9 / HBM_PEAK_GBS, 4)
+        return r
 
     res = {"workload": name, "dtype": "f32", "algorithmic_GB_per_step": round(alg / 1e9, 3)}
 
-    def measure(net, out, make_opt):
+    def measure(net, out, make_opt, variant):
         """forward+backward and forward+backward+Adam of `net`, eager and as a replayed HIP graph."""
         def fwd_bwd():
             net.zero_grad(set_to_none=True)
@@ -636,7 +681,9 @@ def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor
             return loss
 
         sec, loss = timeit(fwd_bwd)
-        out["fwd_bwd_eager"] = report(sec, loss.item())
+        out["fwd_bwd_eager"] = report(sec, loss.item(), variant)
+        if eager_only:
+            return
         # Drop every reference to the eager autograd graph before capturing: gradient-accumulation
         # nodes kept alive by `loss` belong to the default stream and would be replayed into the
         # capture stream's backward.
@@ -675,12 +722,14 @@ def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor
     # the model as a user of the reference writes it, then with the last LogicLayer and GroupSum merged
     # and the first two layers merged (difflogic_amd.fuse_for_training: same parameters; the Adam steps above moved
     # them, so the losses differ)
-    measure(model, res, lambda ps: torch.optim.Adam(ps, lr=0.01, fused=True, capturable=True))
-    res["optimizer"] = "torch.optim.Adam(fused=True, capturable=True)"
-    res["fused_for_training"] = {"optimizer": "difflogic_amd.FusedAdam (one launch over all weight tensors)"}
-    measure(dl.fuse_for_training(model).train(), res["fused_for_training"], lambda ps: dl.FusedAdam(ps, lr=0.01))
+    if eager_only != "fused":
+        measure(model, res, lambda ps: torch.optim.Adam(ps, lr=0.01, fused=True, capturable=True), "written")
+        res["optimizer"] = "torch.optim.Adam(fused=True, capturable=True)"
+    if eager_only != "written":
+        res["fused_for_training"] = {"optimizer": "difflogic_amd.FusedAdam (one launch over all weight tensors)"}
+        measure(dl.fuse_for_training(model).train(), res["fused_for_training"], lambda ps: dl.FusedAdam(ps, lr=0.01), "fused")
 
-    if other_dtypes:
+    if other_dtypes and not eager_only:
         # experiments/main.py:19-23,286 (--training-bit-count 16 / 64): the input is cast, the weights stay fp32
         res["other_input_dtypes"] = {}
         for key, dtype, size in (("f16", torch.float16, 2), ("f64", torch.float64, 8)):
@@ -870,13 +919,13 @@ def extra_configs(args, torch, dl, started):
     check = not args.no_cpu_baseline
     if want("c2", args.no_configs):
         B = 1 << 20
-        configs["C2"] = packed_config(torch, dl, "packed inference 784->6x8000->GroupSum(10), batch 2^20, int64 words",
+        configs["C2"] = packed_config(torch, dl, "C2", "packed inference 784->6x8000->GroupSum(10), batch 2^20, int64 words",
                                       784, [8000] * 6, B, bernoulli_input(torch, B, 784, 1), check,
                                       compiled=started.get("C2"))
         torch.cuda.empty_cache()
     if want("c4", args.no_configs):
         B = 1 << 18
-        configs["C4"] = packed_config(torch, dl, "packed inference 9216->4x256000->GroupSum(10), batch 2^18, int64 words, "
+        configs["C4"] = packed_config(torch, dl, "C4", "packed inference 9216->4x256000->GroupSum(10), batch 2^18, int64 words, "
                                       "thresholded-uniform input", 9216, [256000] * 4, B, thresholded_input(torch, B, 1),
                                       check)
         torch.cuda.empty_cache()
@@ -886,8 +935,10 @@ def extra_configs(args, torch, dl, started):
         x = bernoulli_input(torch, B, 784, 2).float()
         configs["C3"], model = train_config(
             torch, dl, "fp32 train 784->6x64000->GroupSum(10,tau=30), B=512, connections=unique, CrossEntropy",
-            784, [64000] * 6, 10, 30.0, B, "unique", 1.0, x, steps, warmup, other_dtypes=True)
-        configs["C3"]["kernels_alone_64000x64000"] = train_kernels_alone(torch, dl, model, B, 64000)
+            784, [64000] * 6, 10, 30.0, B, "unique", 1.0, x, steps, warmup, other_dtypes=True,
+            eager_only=args.train_eager_only, config="C3")
+        if not args.train_eager_only:
+            configs["C3"]["kernels_alone_64000x64000"] = train_kernels_alone(torch, dl, model, B, 64000)
         del model, x
         gc.collect()
         torch.cuda.empty_cache()
@@ -896,7 +947,8 @@ def extra_configs(args, torch, dl, started):
         x = thresholded_input(torch, B, 2, as_float=True)
         configs["C5"], model = train_config(
             torch, dl, "fp32 train 9216->12x128000->GroupSum(10,tau=100), B=1024, connections=random, grad_factor=2, "
-            "thresholded-uniform input, CrossEntropy", 9216, [128000] * 12, 10, 100.0, B, "random", 2.0, x, steps, warmup)
+            "thresholded-uniform input, CrossEntropy", 9216, [128000] * 12, 10, 100.0, B, "random", 2.0, x, steps, warmup,
+            eager_only=args.train_eager_only, config="C5")
         del model, x
         gc.collect()
         torch.cuda.empty_cache()
@@ -905,7 +957,8 @@ def extra_configs(args, torch, dl, started):
         x = bernoulli_input(torch, B, 784, 2).float()
         configs["C1"], model = train_config(
             torch, dl, "fp32 train 784->4x8000->GroupSum(10,tau=10), B=128, connections=random, CrossEntropy",
-            784, [8000] * 4, 10, 10.0, B, "random", 1.0, x, max(steps, 50), warmup)
+            784, [8000] * 4, 10, 10.0, B, "random", 1.0, x, max(steps, 50), warmup, eager_only=args.train_eager_only,
+            config="C1")
         del model, x
         if not args.no_cpu_baseline:
             configs["C1"]["cpu_baseline"] = train_cpu_baseline(torch)
