@@ -1281,8 +1281,27 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
     const std::integral_constant<int, FIRST> first_batch;
     const std::integral_constant<int, REST> second_batch;
     if constexpr (AHEAD) request(first_batch, 0, r0, ra0, rb0);
+    // this block's runs of parked outputs per owned class: read a block ahead (a scalar load: a vector load in the
+    // counting phase would have to wait for the rows requested above, which return in order), so that the counting
+    // phase starts without waiting for it
+    auto run_of = [&](int b, int i) -> uint32_t {
+        const int64_t cls = wave + i * DL_CC_WAVES;
+        if (cls >= k || b >= blocks) return 0u;
+        const int64_t at = (g * blocks + b) * k + cls;
+        const uint32_t pair = reinterpret_cast<const uint32_t *>(runs)[at >> 1];
+        return (at & 1) ? pair >> 16 : pair & 0xffffu;
+    };
+    uint32_t run_next[CPW];
+#pragma unroll
+    for (int i = 0; i < CPW; ++i) run_next[i] = run_of(0, i);
 #pragma unroll 1
     for (int b = 0; b < blocks; ++b) {
+        uint32_t run_now[CPW];
+#pragma unroll
+        for (int i = 0; i < CPW; ++i) {
+            run_now[i] = run_next[i];
+            run_next[i] = run_of(b + 1, i);
+        }
         if constexpr (!AHEAD) request(first_batch, b * DL_CC_WAVE_STEPS, r0, ra0, rb0);
         walk(first_batch, r0, ra0, rb0);
         if constexpr (REST > 0) {
@@ -1300,11 +1319,7 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
         for (int i = 0; i < CPW; ++i) {
             const int64_t cls = wave + i * DL_CC_WAVES;
             if (cls < k) {
-                // (a scalar load of the pair of entries that holds this one: a vector load here would have to wait
-                // for the rows requested above, which return in order)
-                const int64_t at = (g * blocks + b) * k + cls;
-                const uint32_t pair = reinterpret_cast<const uint32_t *>(runs)[at >> 1];
-                const uint32_t run = (at & 1) ? pair >> 16 : pair & 0xffffu;
+                const uint32_t run = run_now[i];
                 const int start = (int) (run & 255u), n = (int) (run >> 8);
 #pragma unroll 1
                 for (int q = 0; q < n; q += 4) {

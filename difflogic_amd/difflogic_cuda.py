@@ -777,16 +777,21 @@ def live_inputs(layers, live_out=None):
     produces the input of ``layers[i]``.  Not part of the reference's extension."""
     lib = _lib.load()
     res = [None] * len(layers)
+    # one cleared buffer for all layers' vectors (each starts on a 16-byte boundary): one fill instead of one per layer
+    starts, total = [0] * len(layers), 0
+    for i in range(1, len(layers)):
+        starts[i], total = total, total + -(-int(layers[i - 1][2].shape[0]) // 16) * 16
+    pool = torch.zeros(max(1, total), dtype=torch.uint8, device=layers[0][2].device) if layers else None
     for i in range(len(layers) - 1, -1, -1):
         a, b, w = layers[i]
         _check_input(w, "w")
         _check_index(a, "a", w.shape[0])
         _check_index(b, "b", w.shape[0])
-        dev = _same_device(a, b, w)
+        dev = _same_device(a, b, w, pool)
         in_dim = int(layers[i - 1][2].shape[0]) if i > 0 else None
         if in_dim is None:
             break                                     # the first layer's input rows are the caller's data
-        live_in = torch.zeros(in_dim, dtype=torch.uint8, device=dev)
+        live_in = pool[starts[i]:starts[i] + in_dim]
         with _on(dev):
             st = lib.dl_mark_live_inputs(_p(a), _p(b), _p(w), _p(live_out) if live_out is not None else None, _p(live_in),
                                          w.shape[0], _stream(dev))
