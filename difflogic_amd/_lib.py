@@ -76,6 +76,7 @@ SIGNATURES = {
     "dl_logic_net_lds_groupbitsum_scheduled": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _i64,
                                                _i64, _vp, _vp],
     "dl_logic_net_lds_groupbitsum_bool": [_vp, _i64, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp],
+    "dl_logic_net_lds_groupbitsum_thinned": [_vp, _int, _i64, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _i64, _vp, _vp],
     "dl_count_chain_block": [],
     "dl_count_chain_padded_steps": [_i64],
     "dl_count_chain_plan_build": [_vp, _i64, _i64, _i64, _vp, _vp, ctypes.POINTER(_int)],

@@ -115,6 +115,167 @@ __global__ __launch_bounds__(DL_BLOCK) void compose_net_kernel(NetWiring t, uint
     rec[t.offset[l] + i] = row(t.a[l][i]) | (row(t.b[l][i]) << DL_NET_ID_BITS) | ((t.w[l][i] & 15u) << (2 * DL_NET_ID_BITS));
 }
 
+// ------------------------------------------------------------------------------------------
+// The net thinned for one call.  Constants are folded through the gate ids (a gate that reads a constant neuron is
+// replaced by the one-input gate it amounts to), the neurons that some gate above still looks at are marked from the
+// last layer downwards, and everything else is neither evaluated nor stored: a hidden layer keeps its marked neurons
+// only, renumbered 0, 1, ... in their order (their rank is the row their output is stored at), the last layer's
+// classes keep their non-constant neurons, and what the constant ones among them add to every sample's count goes
+// into the result at the end.  The kernel reads the numbers of neurons left from `thin`:
+//   thin[l], l < depth - 1        neurons left of hidden layer l
+//   thin[depth - 1 + c]           neurons left of class c of the last layer
+//   thin[depth - 1 + k + c]       constant-one neurons of class c
+// ------------------------------------------------------------------------------------------
+struct ThinTables {
+    uint8_t *folded[DL_NET_MAX_DEPTH];          // gate ids of layer l with the constants below folded in
+    uint8_t *live[DL_NET_MAX_DEPTH];            // hidden layer l: neuron n is looked at (the last layer: null)
+    int32_t *rank[DL_NET_MAX_DEPTH];            // rank of neuron n among the neurons left (of its class, in the last layer)
+    int32_t *thin;
+    int32_t k;
+};
+
+__device__ __forceinline__ bool net_gate_uses_a(uint32_t op) { return (((op >> 3) ^ (op >> 1)) & 1u) || (((op >> 2) ^ op) & 1u); }
+__device__ __forceinline__ bool net_gate_uses_b(uint32_t op) { return (((op >> 3) ^ (op >> 2)) & 1u) || (((op >> 1) ^ op) & 1u); }
+
+#define DL_NET_RANK_ITEMS (DL_NET_MAX_WIDTH / DL_NET_THREADS)        // consecutive neurons per thread
+
+// Gate ids of layer l with the constants of the layer below folded in (launched layer by layer, upwards); clears
+// the layer's marks.  Gate ids are (f(0,0) f(0,1) f(1,0) f(1,1)), most significant bit first.
+__global__ __launch_bounds__(DL_BLOCK) void net_thin_fold_kernel(NetWiring t, ThinTables thin, int l, int depth) {
+    const int n = (int) (blockIdx.x * DL_BLOCK + threadIdx.x);
+    if (n >= t.width[l]) return;
+    uint32_t op = t.w[l][n] & 15u;
+    if (l > 0) {
+        const uint32_t ga = thin.folded[l - 1][t.a[l][n]], gb = thin.folded[l - 1][t.b[l][n]];
+        if (ga == 0u || ga == 15u) {                             // a is constant: f'(a, b) = f(that constant, b)
+            const uint32_t f0 = ga ? (op >> 1) & 1u : (op >> 3) & 1u, f1 = ga ? op & 1u : (op >> 2) & 1u;
+            op = f0 << 3 | f1 << 2 | f0 << 1 | f1;
+        }
+        if (gb == 0u || gb == 15u) {
+            const uint32_t f0 = gb ? (op >> 2) & 1u : (op >> 3) & 1u, f1 = gb ? op & 1u : (op >> 1) & 1u;
+            op = f0 << 3 | f0 << 2 | f1 << 1 | f1;
+        }
+    }
+    thin.folded[l][n] = (uint8_t) op;
+    if (l + 1 < depth) thin.live[l][n] = 0;
+}
+
+// Marks the neurons of layer l - 1 that a neuron of layer l which is itself looked at (the last layer: every neuron)
+// looks at (launched layer by layer, downwards).  A constant neuron marks nothing and, its readers having been
+// folded, is marked by nobody.
+__global__ __launch_bounds__(DL_BLOCK) void net_thin_mark_kernel(NetWiring t, ThinTables thin, int l, int depth) {
+    const int n = (int) (blockIdx.x * DL_BLOCK + threadIdx.x);
+    if (n >= t.width[l] || (l + 1 < depth && !thin.live[l][n])) return;
+    const uint32_t op = thin.folded[l][n];
+    if (net_gate_uses_a(op)) thin.live[l - 1][t.a[l][n]] = 1;
+    if (net_gate_uses_b(op)) thin.live[l - 1][t.b[l][n]] = 1;
+}
+
+// blockIdx.x = layer: exclusive prefix sums of "this neuron is left" over the layer's neurons
+__global__ __launch_bounds__(DL_NET_THREADS) void net_thin_rank_kernel(NetWiring t, ThinTables thin, int depth) {
+    __shared__ int32_t wave_total[DL_NET_THREADS / DL_WAVE];
+    const int l = blockIdx.x, tid = (int) threadIdx.x, lane = dl_lane(), wave = dl_wave_in_block();
+    const int width = t.width[l];
+    const bool last = l == depth - 1;
+    const uint8_t *flag_src = last ? thin.folded[l] : thin.live[l];
+    int32_t local[DL_NET_RANK_ITEMS], sum = 0;
+#pragma unroll
+    for (int i = 0; i < DL_NET_RANK_ITEMS; ++i) {
+        const int n = tid * DL_NET_RANK_ITEMS + i;
+        int32_t f = 0;
+        if (n < width) {
+            const uint32_t v = flag_src[n];
+            f = last ? (v != 0u && v != 15u) : v != 0u;
+        }
+        local[i] = sum;
+        sum += f;
+    }
+    int32_t incl = sum;                                      // inclusive scan of the threads' sums within the wave
+#pragma unroll
+    for (int off = 1; off < DL_WAVE; off <<= 1) {
+        const int32_t up = __shfl_up(incl, off, DL_WAVE);
+        if (lane >= off) incl += up;
+    }
+    if (lane == DL_WAVE - 1) wave_total[wave] = incl;
+    __syncthreads();
+    int32_t before = 0, total = 0;
+    for (int w = 0; w < DL_NET_THREADS / DL_WAVE; ++w) {
+        if (w < wave) before += wave_total[w];
+        total += wave_total[w];
+    }
+    const int32_t mine = before + incl - sum;                // neurons left before this thread's first
+    int32_t *rank = thin.rank[l];
+    if (!last) {
+#pragma unroll
+        for (int i = 0; i < DL_NET_RANK_ITEMS; ++i) {
+            const int n = tid * DL_NET_RANK_ITEMS + i;
+            if (n < width) rank[n] = mine + local[i];
+        }
+        if (tid == 0) thin.thin[l] = total;
+        return;
+    }
+    // the last layer: ranks within each class, the classes' numbers of neurons left and of constant ones
+    const int per_class = width / thin.k;
+#pragma unroll
+    for (int i = 0; i < DL_NET_RANK_ITEMS; ++i) {
+        const int n = tid * DL_NET_RANK_ITEMS + i;
+        if (n < width && n % per_class == 0) rank[n] = mine + local[i];      // neurons left before the class
+    }
+    __threadfence_block();
+    __syncthreads();
+    int32_t at_start[DL_NET_RANK_ITEMS];
+#pragma unroll
+    for (int i = 0; i < DL_NET_RANK_ITEMS; ++i) {
+        const int n = tid * DL_NET_RANK_ITEMS + i;
+        at_start[i] = n < width ? rank[(n / per_class) * per_class] : 0;
+    }
+    __syncthreads();                                         // every class start has been read before any rank changes
+#pragma unroll
+    for (int i = 0; i < DL_NET_RANK_ITEMS; ++i) {
+        const int n = tid * DL_NET_RANK_ITEMS + i;
+        if (n < width) rank[n] = mine + local[i] - at_start[i];
+    }
+    for (int c = wave; c < thin.k; c += DL_NET_THREADS / DL_WAVE) {      // a wave per class
+        int32_t left = 0, ones = 0;
+        for (int i = lane; i < per_class; i += DL_WAVE) {
+            const uint32_t g = thin.folded[l][c * per_class + i];
+            left += g != 0u && g != 15u;
+            ones += g == 15u;
+        }
+#pragma unroll
+        for (int off = DL_WAVE / 2; off > 0; off >>= 1) {
+            left += __shfl_xor(left, off, DL_WAVE);
+            ones += __shfl_xor(ones, off, DL_WAVE);
+        }
+        if (lane == 0) {
+            thin.thin[depth - 1 + c] = left;
+            thin.thin[depth - 1 + thin.k + c] = ones;
+        }
+    }
+}
+
+// records of the neurons left (layer blockIdx.y): a | b << 14 | gate << 28 at the neuron's rank, the inputs' rows being
+// the ranks of the layer below (an input that the gate does not look at: row 0)
+__global__ __launch_bounds__(DL_BLOCK) void compose_net_thin_kernel(NetWiring t, ThinTables thin, int depth,
+                                                                    uint32_t *__restrict__ rec) {
+    const int l = blockIdx.y;
+    const int n = (int) (blockIdx.x * DL_BLOCK + threadIdx.x);
+    if (n >= t.width[l]) return;
+    const uint32_t gate = thin.folded[l][n];
+    int64_t at;
+    if (l < depth - 1) {
+        if (!thin.live[l][n]) return;
+        at = thin.rank[l][n];
+    } else {
+        if (gate == 0u || gate == 15u) return;
+        const int per_class = t.width[l] / thin.k;
+        at = (int64_t) (n / per_class) * per_class + thin.rank[l][n];
+    }
+    auto row = [&](int64_t v) -> uint32_t { return (uint32_t) (l == 0 ? v + t.in_base : thin.rank[l - 1][v]); };
+    const uint32_t ra = net_gate_uses_a(gate) ? row(t.a[l][n]) : 0u, rb = net_gate_uses_b(gate) ? row(t.b[l][n]) : 0u;
+    rec[t.offset[l] + at] = ra | (rb << DL_NET_ID_BITS) | (gate << (2 * DL_NET_ID_BITS));
+}
+
 // COLS 64-bit words as 2 * COLS dwords
 template <int COLS> struct Row { uint32_t d[2 * COLS]; };
 
@@ -289,20 +450,22 @@ __device__ __forceinline__ void load_class_records(uint32_t *r4, const uint32_t 
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         const int64_t i = i0 + u * DL_WAVE;
-        r4[u] = ctab[i < per_class ? i : per_class - 1];
+        r4[u] = ctab[i < per_class ? i : (per_class > 0 ? per_class - 1 : 0)];
     }
 }
 
 // BOOLIN: the input is the bool matrix [batch, in_dim] itself (sample-major, as the user holds it) and is
 // packed on the way into LDS, so neither the pack kernel nor the packed input exist: the workgroup reads
 // the COLS * 64 sample rows of its columns (one contiguous region) and folds them into the input rows.
-template <int COLS, int GPT, int NP0, bool BOOLIN>
+// THIN: the net thinned for this call (ThinTables): numbers of neurons from `thin`, no schedules.
+template <int COLS, int GPT, int NP0, bool BOOLIN, bool THIN>
 __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint64_t *__restrict__ x,
                                                                       const uint8_t *__restrict__ xb,
                                                                       const uint32_t *__restrict__ rec, NetShape net,
                                                                       int32_t *__restrict__ out, int64_t ncols,
                                                                       int64_t per_class, int64_t k, int64_t batch,
-                                                                      uint32_t grouped_blocks) {
+                                                                      uint32_t grouped_blocks,
+                                                                      const int32_t *__restrict__ thin) {
     extern __shared__ __align__(16) uint8_t act[];             // [rows][COLS] 64-bit words
     const int tid = (int) threadIdx.x;
     const int wave = dl_wave_in_block(), lane = dl_lane();
@@ -320,15 +483,15 @@ __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint
     const int64_t col0 = group * COLS;
 
     // records a thread needs for layer l, requested one layer ahead of their use
-    constexpr int NR = GPT > DL_NET_CHUNK + 2 ? GPT : DL_NET_CHUNK + 2;
+    constexpr int NR = THIN || GPT > DL_NET_CHUNK + 2 ? GPT : DL_NET_CHUNK + 2;
     const int rt = tid;
     auto load_records = [&](int l, uint32_t *r) __attribute__((always_inline)) {
         const uint32_t *tab = rec + net.offset[l];
         // scheduled: entry 8 tid + i sits at tab[i * stride + tid], i = 0..8, and the record of step 8192 + tid at
         // tab[9 * stride + tid]; else neuron tid + 1024 i at tab[tid + 1024 i]
-        const bool sched = net.steps[l] > 0;
+        const bool sched = !THIN && net.steps[l] > 0;
         const int chunks = net.steps[l] / DL_NET_CHUNK;
-        const int limit = sched ? (chunks < DL_NET_THREADS ? chunks : DL_NET_THREADS) : net.width[l];
+        const int limit = sched ? (chunks < DL_NET_THREADS ? chunks : DL_NET_THREADS) : THIN ? thin[l] : net.width[l];
         const int extra = net.steps[l] - DL_NET_CHUNK * limit;
         const int step = sched ? net.stride[l] : DL_NET_THREADS;
         const int entries = sched ? DL_NET_CHUNK + 2 : GPT;
@@ -396,8 +559,10 @@ __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint
     uint32_t r[NR];
     if (net.depth > 1) load_records(0, r);
     // the class phase's first records (wave = class)
+    // (thinned for this call: a class keeps `left` of its per_class records, and `base` constant ones count for every sample)
+    auto class_left = [&](int64_t cls) -> int64_t { return THIN ? (int64_t) thin[net.depth - 1 + cls] : per_class; };
     uint32_t rc[4] = {0, 0, 0, 0};
-    if (wave < k) load_class_records(rc, ltab + wave * per_class, lane, per_class);
+    if (wave < k) load_class_records(rc, ltab + wave * per_class, lane, class_left(wave));
 
     if (BOOLIN) {
         stage_bool(group, tid, DL_NET_THREADS);
@@ -431,7 +596,7 @@ __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint
     for (int l = 0; l + 1 < net.depth; ++l) {
         uint32_t rn[NR];
         if (l + 2 < net.depth) load_records(l + 1, rn);
-        if (net.steps[l] > 0) {
+        if (!THIN && net.steps[l] > 0) {
             // along the schedule: this thread's chunk of 8 steps, 9 rows read, outputs in schedule order
             // (and, of a schedule of more than 1024 chunks, one of the remaining steps)
             const int stride = net.stride[l];
@@ -454,10 +619,11 @@ __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint
             if (tid < extra)                                    // step 8192 + tid
                 lds_store<COLS>(act, (uint32_t) ((tid % DL_NET_CHUNK) * stride + DL_NET_THREADS + tid / DL_NET_CHUNK), ye);
         } else {
-            const int width = net.width[l];
+            const int width = THIN ? thin[l] : net.width[l];    // (thinned: the neurons left, at rows 0, 1, ...)
             Row<COLS> y[GPT];
 #pragma unroll
-            for (int g = 0; g < GPT; ++g) y[g] = gate_rows<COLS>(act, r[g]);
+            for (int g = 0; g < GPT; ++g)
+                if (!THIN || g * DL_NET_THREADS + wave * DL_WAVE < width) y[g] = gate_rows<COLS>(act, r[g]);   // (a wave skips rounds in which it has no neuron)
             __syncthreads();                                    // every thread has read its inputs
 #pragma unroll
             for (int g = 0; g < GPT; ++g) {
@@ -482,13 +648,15 @@ __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint
         // What is left of the class after the whole quads (fewer than 256 neurons) goes row by row: 64 neurons,
         // lanes past the end of the class contributing zero words, rippled in with weight 1.
         const uint32_t *ctab = ltab + cls * per_class;
-        if (cls != wave) load_class_records(rc, ctab, lane, per_class);
-        const int64_t quads = per_class / (4 * DL_WAVE);
+        const int64_t left = class_left(cls);
+        const int32_t base = THIN ? thin[net.depth - 1 + k + cls] : 0;
+        if (cls != wave) load_class_records(rc, ctab, lane, left);
+        const int64_t quads = left / (4 * DL_WAVE);
         for (int64_t q = 0; q < quads; ++q) {
             uint32_t r4[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) r4[u] = rc[u];
-            load_class_records(rc, ctab, (q + 1) * 4 * DL_WAVE + lane, per_class);   // next quad, or the rest
+            load_class_records(rc, ctab, (q + 1) * 4 * DL_WAVE + lane, left);   // next quad, or the rest
             Row<COLS> y[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) y[u] = gate_rows<COLS>(act, r4[u]);
@@ -505,9 +673,9 @@ __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int64_t i = (quads * 4 + u) * DL_WAVE;          // first neuron of this row
-            if (i >= per_class) break;                            // uniform
+            if (i >= left) break;                                 // uniform
             Row<COLS> y = gate_rows<COLS>(act, rc[u]);
-            const uint32_t live = i + lane < per_class ? ~0u : 0u;
+            const uint32_t live = i + lane < left ? ~0u : 0u;
 #pragma unroll
             for (int d = 0; d < 2 * COLS; ++d) {
                 uint32_t carry = y.d[d] & live;
@@ -524,39 +692,36 @@ __global__ __launch_bounds__(DL_NET_THREADS) void eval_net_lds_kernel(const uint
 #pragma unroll
         for (int t = 0; t < COLS; ++t) {
             const int64_t sample = col0 * 64 + lane * COLS + t;
-            if (sample < batch && sample < ncols * 64) out[sample * k + cls] = count[t];
+            if (sample < batch && sample < ncols * 64) out[sample * k + cls] = count[t] + base;
         }
     }
 }
 
 template <int COLS, int GPT>
 int launch_net(const void *x, bool bool_input, const uint32_t *rec, const NetShape &net, int32_t *out, int64_t ncols,
-               int64_t per_class, int64_t k, int64_t batch, int64_t rows, hipStream_t s) {
+               int64_t per_class, int64_t k, int64_t batch, int64_t rows, const int32_t *thin, hipStream_t s) {
     const int64_t groups = dl_ceil_div(ncols, COLS);
     if (groups > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     const size_t lds = (size_t) rows * 8 * COLS;
     const dim3 block(DL_NET_THREADS);
     // a lane counts ceil(per_class / 64) neurons: NP0 planes hold up to 2^NP0 - 1
     const bool small = dl_ceil_div(per_class, DL_WAVE) < 16;
-    if (bool_input) {
-        const dim3 grid((unsigned) groups);
-        if (small)
-            DL_LAUNCH((eval_net_lds_kernel<COLS, GPT, 4, true>), grid, block, lds, s, (const uint64_t *) nullptr,
-                      (const uint8_t *) x, rec, net, out, ncols, per_class, k, batch, 0u);
-        else
-            DL_LAUNCH((eval_net_lds_kernel<COLS, GPT, 8, true>), grid, block, lds, s, (const uint64_t *) nullptr,
-                      (const uint8_t *) x, rec, net, out, ncols, per_class, k, batch, 0u);
-        return dl_launch_status();
-    }
     const dim3 grid((unsigned) groups);
     const uint32_t share = 8 * (16 / COLS);                    // workgroups sharing input lines, one set per XCD
-    const uint32_t grouped = (uint32_t) groups / share * share;
-    if (small)
-        DL_LAUNCH((eval_net_lds_kernel<COLS, GPT, 4, false>), grid, block, lds, s, (const uint64_t *) x,
-                  (const uint8_t *) nullptr, rec, net, out, ncols, per_class, k, batch, grouped);
-    else
-        DL_LAUNCH((eval_net_lds_kernel<COLS, GPT, 8, false>), grid, block, lds, s, (const uint64_t *) x,
-                  (const uint8_t *) nullptr, rec, net, out, ncols, per_class, k, batch, grouped);
+    const uint32_t grouped = bool_input ? 0u : (uint32_t) groups / share * share;
+    const uint64_t *words = bool_input ? nullptr : (const uint64_t *) x;
+    const uint8_t *bools = bool_input ? (const uint8_t *) x : nullptr;
+#define DL_NET_LAUNCH(NP0, BOOLIN, THIN)                                                                                \
+    DL_LAUNCH((eval_net_lds_kernel<COLS, GPT, NP0, BOOLIN, THIN>), grid, block, lds, s, words, bools, rec, net, out, ncols,    \
+              per_class, k, batch, grouped, thin)
+    if (bool_input) {
+        if (thin) { if (small) DL_NET_LAUNCH(4, true, true); else DL_NET_LAUNCH(8, true, true); }
+        else { if (small) DL_NET_LAUNCH(4, true, false); else DL_NET_LAUNCH(8, true, false); }
+    } else {
+        if (thin) { if (small) DL_NET_LAUNCH(4, false, true); else DL_NET_LAUNCH(8, false, true); }
+        else { if (small) DL_NET_LAUNCH(4, false, false); else DL_NET_LAUNCH(8, false, false); }
+    }
+#undef DL_NET_LAUNCH
     return dl_launch_status();
 }
 
@@ -575,19 +740,23 @@ extern "C" int64_t dl_logic_net_lds_workspace_bytes(int depth, const int64_t *di
     if (depth < 1 || depth > DL_NET_MAX_DEPTH || !dims) return 0;
     // per layer: the records (9 per chunk of a schedule of at most width + width / 4 + 32 steps, chunks
     // rounded up to whole waves) and width row ids
+    // (thinned: a record, a rank, a folded gate id and a mark per neuron = 10 bytes, and three numbers per layer /
+    // class: fits the same bound with the last term, k <= dims[depth])
     int64_t bytes = 0;
     for (int l = 1; l <= depth; ++l) {
         const int64_t w = dims[l] > 0 ? dims[l] : 0;
         bytes += 4 * (w + w / 2 + 640 + DL_NET_THREADS) + 4 * w;
     }
-    return bytes;
+    return bytes + 8 * (dims[depth] > 0 ? dims[depth] : 0);
 }
 
 // bool_input: x is the bool matrix [batch, dims[0]] (sample-major); words, bit_count and pad_len are then unused.
+// thinned: the net thinned for this call (see ThinTables); the schedules are not used then.
 static int net_lds_run(const void *x, bool bool_input, int64_t batch, int depth, const int64_t *const *a,
                        const int64_t *const *b, const uint8_t *const *w, const int64_t *dims, const int32_t *const *verts,
                        const int32_t *const *neuron, const uint8_t *const *flip, const int64_t *steps, int32_t *out,
-                       int64_t words, int bit_count, int64_t pad_len, int64_t k, void *workspace, void *stream) {
+                       int64_t words, int bit_count, int64_t pad_len, int64_t k, void *workspace, void *stream,
+                       bool thinned = false) {
     if (!bool_input && bit_count != 8 && bit_count != 16 && bit_count != 32 && bit_count != 64) return DL_ERR_BIT_COUNT;
     if (depth < 1 || !dims || !a || !b || !w || words < 0 || k <= 0 || pad_len < 0) return DL_ERR_INVALID_ARGUMENT;
     if (depth > DL_NET_MAX_DEPTH) return DL_ERR_TOO_LARGE;
@@ -641,8 +810,8 @@ static int net_lds_run(const void *x, bool bool_input, int64_t batch, int depth,
         int64_t count = dims[l + 1];
         // A hidden layer is walked along its schedule when one is given, every chunk finds a thread, its outputs in
         // schedule order fit the buffer, and the schedule is not much longer than the layer (few, long trails).
-        if (l + 1 < depth && steps && verts && neuron && flip && verts[l] && neuron[l] && flip[l] && steps[l] >= dims[l + 1] &&
-            steps[l] % DL_NET_CHUNK == 0) {
+        if (!thinned && l + 1 < depth && steps && verts && neuron && flip && verts[l] && neuron[l] && flip[l] &&
+            steps[l] >= dims[l + 1] && steps[l] % DL_NET_CHUNK == 0) {
             const int64_t nchunks = steps[l] / DL_NET_CHUNK;
             const int64_t stride = dl_ceil_div(nchunks, DL_WAVE) * DL_WAVE;
             const int64_t extra = steps[l] > DL_NET_CHUNK * DL_NET_THREADS ? steps[l] - DL_NET_CHUNK * DL_NET_THREADS : 0;
@@ -675,15 +844,48 @@ static int net_lds_run(const void *x, bool bool_input, int64_t batch, int depth,
         if (st != DL_OK) return st;
     }
     net.in_base = wiring.in_base = (int32_t) (bool_input ? rows : 0);      // the input's rows follow the layers'
-    DL_LAUNCH(compose_net_kernel, dim3((unsigned) dl_ceil_div(entries, DL_BLOCK), (unsigned) depth), dim3(DL_BLOCK), 0, s,
-              wiring, rec);
-    int st = dl_launch_status();
+    const int32_t *thin = nullptr;
+    int st;
+    if (thinned) {
+        // ranks follow the records, then the numbers of neurons left, the folded gate ids and the marks
+        ThinTables th;
+        int32_t *rank = (int32_t *) workspace + offset;
+        for (int l = 0; l < DL_NET_MAX_DEPTH; ++l) th.folded[l] = th.live[l] = nullptr, th.rank[l] = nullptr;
+        for (int l = 0; l < depth; ++l) {
+            th.rank[l] = rank;
+            rank += dims[l + 1];
+        }
+        th.thin = rank;
+        th.k = (int32_t) k;
+        uint8_t *bytes = (uint8_t *) (rank + depth + 2 * k);
+        for (int l = 0; l < depth; ++l) {
+            th.folded[l] = bytes, bytes += dims[l + 1];
+            if (l + 1 < depth) th.live[l] = bytes, bytes += dims[l + 1];
+        }
+        if ((char *) bytes - (char *) workspace > dl_logic_net_lds_workspace_bytes(depth, dims)) return DL_ERR_INVALID_ARGUMENT;
+        for (int l = 0; l < depth; ++l)
+            DL_LAUNCH(net_thin_fold_kernel, dim3((unsigned) dl_ceil_div(dims[l + 1], DL_BLOCK)), dim3(DL_BLOCK), 0, s, wiring, th, l,
+                      depth);
+        for (int l = depth - 1; l >= 1; --l)
+            DL_LAUNCH(net_thin_mark_kernel, dim3((unsigned) dl_ceil_div(dims[l + 1], DL_BLOCK)), dim3(DL_BLOCK), 0, s, wiring, th, l,
+                      depth);
+        DL_LAUNCH(net_thin_rank_kernel, dim3((unsigned) depth), dim3(DL_NET_THREADS), 0, s, wiring, th, depth);
+        st = dl_launch_status();
+        if (st != DL_OK) return st;
+        DL_LAUNCH(compose_net_thin_kernel, dim3((unsigned) dl_ceil_div(entries, DL_BLOCK), (unsigned) depth), dim3(DL_BLOCK), 0, s,
+                  wiring, th, depth, rec);
+        thin = th.thin;
+    } else {
+        DL_LAUNCH(compose_net_kernel, dim3((unsigned) dl_ceil_div(entries, DL_BLOCK), (unsigned) depth), dim3(DL_BLOCK), 0, s,
+                  wiring, rec);
+    }
+    st = dl_launch_status();
     if (st != DL_OK) return st;
 
     const int64_t ncols = row_bytes / 8;
     const int64_t per_class = dims[depth] / k;
-    if (four) return launch_net<4, 5>(x, bool_input, rec, net, out, ncols, per_class, k, batch, rows + input_rows, s);
-    return launch_net<2, 10>(x, bool_input, rec, net, out, ncols, per_class, k, batch, rows + input_rows, s);
+    if (four) return launch_net<4, 5>(x, bool_input, rec, net, out, ncols, per_class, k, batch, rows + input_rows, thin, s);
+    return launch_net<2, 10>(x, bool_input, rec, net, out, ncols, per_class, k, batch, rows + input_rows, thin, s);
 }
 
 extern "C" int dl_logic_net_lds_groupbitsum(const void *x, int depth, const int64_t *const *a, const int64_t *const *b,
@@ -701,6 +903,17 @@ extern "C" int dl_logic_net_lds_groupbitsum_scheduled(const void *x, int depth, 
                                                       int64_t pad_len, int64_t k, void *workspace, void *stream) {
     return net_lds_run(x, false, 0, depth, a, b, w, dims, verts, neuron, flip, steps, out, words, bit_count, pad_len, k,
                        workspace, stream);
+}
+
+extern "C" int dl_logic_net_lds_groupbitsum_thinned(const void *x, int bool_input, int64_t batch, int depth,
+                                                    const int64_t *const *a, const int64_t *const *b,
+                                                    const uint8_t *const *w, const int64_t *dims, int32_t *out,
+                                                    int64_t words, int bit_count, int64_t pad_len, int64_t k,
+                                                    void *workspace, void *stream) {
+    if (batch < 0) return DL_ERR_INVALID_ARGUMENT;
+    return net_lds_run(x, bool_input != 0, batch, depth, a, b, w, dims, nullptr, nullptr, nullptr, nullptr, out,
+                       bool_input ? 0 : words, bool_input ? 64 : bit_count, bool_input ? 0 : pad_len, k, workspace, stream,
+                       true);
 }
 
 extern "C" int dl_logic_net_lds_groupbitsum_bool(const uint8_t *x, int64_t batch, int depth, const int64_t *const *a,

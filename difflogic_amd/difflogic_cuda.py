@@ -950,13 +950,26 @@ def net_lds_max_width():
     return int(_lib.load().dl_logic_net_lds_max_width())
 
 
-def eval_net_lds(x, layers, pad_len, k, scheduled=True):
+def _net_lds_thinned(x, bool_input, batch, layers, dims, k, words, bits, pad_len, out, dev):
+    lib = _lib.load()
+    depth = len(layers)
+    ptrs = lambda i: (ctypes.c_void_p * depth)(*[l[i].data_ptr() for l in layers])  # noqa: E731
+    pdims = (ctypes.c_int64 * (depth + 1))(*dims)
+    ws = torch.empty(max(1, lib.dl_logic_net_lds_workspace_bytes(depth, pdims) // 4), dtype=torch.int32, device=dev)
+    with _on(dev):
+        return lib.dl_logic_net_lds_groupbitsum_thinned(_p(x), 1 if bool_input else 0, batch, depth, ptrs(0), ptrs(1), ptrs(2),
+                                                        pdims, _p(out), words, bits, int(pad_len), int(k), _p(ws), _stream(dev))
+
+
+def eval_net_lds(x, layers, pad_len, k, scheduled=True, thin=False):
     """groupbitsum(eval(... eval(x, layer 0) ..., last layer), pad_len, k) for a whole narrow net
     (every layer and the input at most net_lds_max_width() wide, at most MAX_NET_DEPTH layers) in
     one kernel that keeps the activations in LDS.  ``scheduled``: hidden layers are walked along
     their (cached) evaluation schedules where that fits, which nearly halves their LDS reads; the
-    result is the same.  Returns None where the kernel does not apply (the caller then uses the
-    streaming kernels).  Not part of the reference's extension."""
+    result is the same.  ``thin``: instead, the net is thinned for this call (constants folded, neurons that
+    no gate looks at neither evaluated nor stored; pays where many gates ignore an input).  Returns None where
+    the kernel does not apply (the caller then uses the streaming kernels).  Not part of the reference's
+    extension."""
     dev, bits, depth, pa, pb, pw, pdims, dims = _fused_args(x, layers)
     out_dim, words = dims[-1], x.shape[1]
     if k <= 0 or out_dim % k != 0:
@@ -968,6 +981,13 @@ def eval_net_lds(x, layers, pad_len, k, scheduled=True):
         return None
     lib = _lib.load()
     out = torch.empty((batch, k), dtype=torch.int32, device=dev)
+    if thin:
+        st = _net_lds_thinned(x, False, batch, layers, dims, k, words, bits, pad_len, out, dev)
+        if st == _lib.DL_ERR_TOO_LARGE:
+            return None
+        if st:
+            _raise(st, "logic_net_lds_groupbitsum_thinned")
+        return out
     ws = torch.empty(max(1, lib.dl_logic_net_lds_workspace_bytes(depth, pdims) // 4), dtype=torch.int32, device=dev)
     scheds = [schedule_for(a, b, dims[i]) for i, (a, b, _) in enumerate(layers[:-1])] if scheduled else []
     with _on(dev):
@@ -989,7 +1009,7 @@ def eval_net_lds(x, layers, pad_len, k, scheduled=True):
     return out
 
 
-def eval_net_lds_bool(x, layers, k, scheduled=True):
+def eval_net_lds_bool(x, layers, k, scheduled=True, thin=False):
     """eval_net_lds on the bool input itself: ``x`` [B, in] bool (sample-major, as PackBitsTensor
     receives it) -> int32 [B, k], the result of packing x with 64-bit words, evaluating every layer
     and groupbitsum, in one kernel that packs the input on its way into LDS (no pack kernel, no
@@ -1020,6 +1040,13 @@ def eval_net_lds_bool(x, layers, k, scheduled=True):
     lib = _lib.load()
     out = torch.empty((batch, k), dtype=torch.int32, device=dev)
     if batch == 0:
+        return out
+    if thin:
+        st = _net_lds_thinned(x, True, batch, layers, dims, k, 0, 64, 0, out, dev)
+        if st == _lib.DL_ERR_TOO_LARGE:
+            return None
+        if st:
+            _raise(st, "logic_net_lds_groupbitsum_thinned")
         return out
     ws = torch.empty(max(1, lib.dl_logic_net_lds_workspace_bytes(depth, pdims) // 4), dtype=torch.int32, device=dev)
     scheds = [schedule_for(a, b, dims[i]) for i, (a, b, _) in enumerate(layers[:-1])] if scheduled else []

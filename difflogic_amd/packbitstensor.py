@@ -21,6 +21,10 @@ _LIVE_INPUT = 0.75           # share of gate inputs a gate looks at when the gat
 _TILE_BYTES = 1024           # one wave covers 64 lanes x 16 bytes of a row
 _L2_RESIDENT_BYTES = 4 << 20     # input tiles (rows x 1 KB each) in flight up to this size are re-read from L2 (4 MB per XCD)
 _LDS_GATE_WORD_SECONDS = 7.9e-13     # LDS-resident whole-net kernel: seconds per gate and 64-sample word
+_LDS_THIN_BELOW = 0.9        # share of looked-at gate inputs below which the LDS kernel runs the net thinned for the call
+                             # (neuron by neuron over the neurons left) instead of whole along its schedules
+_LDS_THIN_GAIN = 0.78        # what thinning leaves of the gates' time: measured 0.61-0.63 ms against 0.74 ms on
+                             # 784 -> 6 x 8000 for shares of 0.5 to 0.75 (all looked at: 0.77 ms, hence the threshold)
 _BOOL_STAGE_RATE = 5.2e12    # B/s of bool input bytes that the LDS kernel packs on their way into LDS
 _PACKED_STAGE_RATE = 1.5e12  # B/s of packed input rows on their way into LDS (16 or 32 bytes of every row per workgroup)
 _PACK_RATE = 4.8e12          # B/s (bool bytes read + words written) of the transpose-and-pack kernel
@@ -97,19 +101,21 @@ def plan_cost(dims, groups, count_at_end, words=16384, live=_LIVE_INPUT):
     return t
 
 
-def lds_cost(dims, words, from_bool=False):
+def lds_cost(dims, words, from_bool=False, live=1.0):
     """Modelled seconds of the LDS-resident whole-net kernel over all of ``dims``; ``from_bool``: it reads the bool
-    input itself (64 bytes per word and feature) instead of packed words."""
+    input itself (64 bytes per word and feature) instead of packed words; ``live``: the share of gate inputs that
+    are looked at (decides whether the net is thinned for the call)."""
     staging = dims[0] * words * (64 / _BOOL_STAGE_RATE if from_bool else 8 / _PACKED_STAGE_RATE)
-    return sum(dims[1:]) * words * _LDS_GATE_WORD_SECONDS + staging + 2 * _LAUNCH_SECONDS
+    gates = sum(dims[1:]) * words * _LDS_GATE_WORD_SECONDS * (_LDS_THIN_GAIN if live < _LDS_THIN_BELOW else 1.0)
+    return gates + staging + 2 * _LAUNCH_SECONDS
 
 
 def lds_tail(dims, words=16384, live=_LIVE_INPUT, from_bool=False):
     """Number of layers at the end of the net (``dims`` = [in_dim, width_1, ..., width_L]) to run
     in the LDS-resident whole-net kernel together with the count: the longest run of trailing
     layers whose input and widths all fit its buffer, if the model prices it below the streaming
-    plan for the same layers (0 otherwise).  The LDS kernel evaluates every gate; the streaming kernels
-    skip what no gate looks at, so a net rich in pass-through gates (low ``live``) may stream faster.
+    plan for the same layers (0 otherwise).  Both skip what no gate looks at (the LDS kernel by thinning the net
+    for the call when ``live`` is low enough to pay for it).
     ``from_bool``: the input has not been packed yet; if the whole net runs in LDS it never is, while the
     streaming kernels need the pack kernel first."""
     limit = difflogic_cuda.net_lds_max_width()
@@ -123,7 +129,7 @@ def lds_tail(dims, words=16384, live=_LIVE_INPUT, from_bool=False):
     streaming = plan_cost(tail, plan_groups(tail, True, words, live), True, words, live) + _STREAM_CALL_SECONDS
     if whole:
         streaming += dims[0] * words * 72 / _PACK_RATE
-    return n if lds_cost(tail, words, whole) < streaming else 0
+    return n if lds_cost(tail, words, whole, live) < streaming else 0
 
 
 # share of the gate inputs that their gate looks at, per set of weight tensors (see PackBitsTensor._live_share)
@@ -322,13 +328,13 @@ class PackBitsTensor:
                 head = len(self._pending) - tail
                 if head == 0 and self._src is not None:
                     # the whole net, straight from the bool input: packing happens on the way into LDS
-                    out = difflogic_cuda.eval_net_lds_bool(self._src, self._pending, k)
+                    out = difflogic_cuda.eval_net_lds_bool(self._src, self._pending, k, thin=share < _LDS_THIN_BELOW)
                     if out is not None:
                         return out
                 if head:
                     self._run_groups(plan_groups(dims[:head + 1], False, self._words64(), share))
                 rows = self._words()
-                out = difflogic_cuda.eval_net_lds(rows, self._pending, self._pad(rows), k)
+                out = difflogic_cuda.eval_net_lds(rows, self._pending, self._pad(rows), k, thin=share < _LDS_THIN_BELOW)
                 if out is not None:
                     return out
             self._fold_pending()

@@ -481,6 +481,23 @@ int dl_logic_net_lds_groupbitsum_bool(const uint8_t *x, int64_t batch, int depth
                                       const uint8_t *const *flip, const int64_t *steps, int32_t *out,
                                       int64_t k, void *workspace, void *stream);
 
+/* dl_logic_net_lds_groupbitsum / _bool with the net thinned for this call: what no gate looks at is neither
+ * evaluated nor stored (the reference evaluates every gate of every layer, difflogic/difflogic.py:147; its
+ * generated C leaves the same pruning to gcc).  Before the net runs, one small kernel folds constants through the
+ * gate ids `w` (a gate that reads a constant neuron becomes the one-input gate it amounts to) and marks, from the
+ * last layer downwards, the neurons that some gate above still looks at; the net kernel then evaluates, per hidden
+ * layer, the marked neurons only (renumbered in their order, neuron by neuron: two row reads per gate, no
+ * schedules), per class the non-constant neurons of the last layer, and adds the constant ones of a class to every
+ * sample's count.  Same result as the other entry points, bit for bit; pays where well below all of the neurons are
+ * looked at (uniformly drawn ids: about 55 %).
+ *   bool_input != 0: x is the bool matrix [batch, dims[0]] as for dl_logic_net_lds_groupbitsum_bool (words,
+ *   bit_count, pad_len unused); else packed words as for dl_logic_net_lds_groupbitsum (batch unused).
+ *   workspace, limits and status codes as for those. */
+int dl_logic_net_lds_groupbitsum_thinned(const void *x, int bool_input, int64_t batch, int depth,
+                                         const int64_t *const *a, const int64_t *const *b, const uint8_t *const *w,
+                                         const int64_t *dims, int32_t *out, int64_t words, int bit_count,
+                                         int64_t pad_len, int64_t k, void *workspace, void *stream);
+
 /* dl_logic_eval_fused_groupbitsum without a workspace argument, for callers that cannot allocate
  * device memory: code under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc.  It has no counterpart in the reference (whose functions allocate their outputs and

@@ -98,3 +98,45 @@ def test_gate_mix_extremes(mix, shape):
     assert words.shape == y.shape
     assert np.array_equal(po.groupbitsum(words, words.shape[1] * 64 - B, k), want)
     assert np.array_equal(po.unpackbits(words, B), po.unpackbits(y, B)), (mix, shape)
+
+
+@pytest.mark.parametrize("mix", sorted(MIXES))
+@pytest.mark.parametrize("from_bool", [False, True])
+def test_lds_resident_kernel_thinned_and_whole(mix, from_bool):
+    """The LDS-resident kernel called directly, with the net thinned for the call (layers that shrink to nothing,
+    classes without a neuron left, constants added to the counts) and whole (along the schedules and neuron by
+    neuron), on the packed words and on the bool matrix."""
+    from difflogic_amd import difflogic_cuda as ext
+    rng = np.random.default_rng(sum(map(ord, mix)) + from_bool)
+    F, widths, B, k = 48, [300, 1100, 640, 2100, 500, 1280], 64 * 5 + (17 if from_bool else 0), 10
+    layers = _net(rng, F, widths, mix)
+    x = rng.random((B, F)) < 0.5
+    want = interp.net_eval(x, layers, k)
+    dev = [tuple(torch.as_tensor(v).cuda() for v in l) for l in layers]
+    for kw in (dict(thin=True), dict(), dict(scheduled=False)):
+        if from_bool:
+            got = ext.eval_net_lds_bool(torch.as_tensor(x).cuda(), dev, k, **kw)
+        else:
+            words, pad = po.packbits(x.T, 64)
+            got = ext.eval_net_lds(torch.as_tensor(words).cuda(), dev, pad, k, **kw)
+        assert got is not None and np.array_equal(got.cpu().numpy(), want), (mix, from_bool, kw)
+
+
+def test_pack_tensor_thins_the_lds_net_by_the_measured_share(monkeypatch):
+    """PackBitsTensor runs a net that is resident in LDS thinned when a good part of its gate inputs is ignored
+    (uniformly drawn ids) and whole along the schedules when every gate looks at both inputs."""
+    import difflogic_amd as dl
+    from difflogic_amd import difflogic_cuda as ext
+    rng = np.random.default_rng(5)
+    F, widths, B, k = 64, [500, 700, 640], 300, 10
+    seen = []
+    real = ext.eval_net_lds_bool
+    monkeypatch.setattr(ext, "eval_net_lds_bool", lambda *a, **kw: seen.append(kw.get("thin")) or real(*a, **kw))
+    for mix, thin in (("half pass-through", True), ("two-input gates only", False)):
+        layers = _net(rng, F, widths, mix)
+        x = rng.random((B, F)) < 0.5
+        model = build_model(F, layers, k).eval()
+        with torch.no_grad():
+            got = model(dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=64))
+        assert np.array_equal(got.cpu().numpy(), interp.net_eval(x, layers, k))
+        assert seen and seen[-1] is thin, (mix, seen)

@@ -625,6 +625,8 @@ def test_net_lds_groupbitsum(ext, bits, in_dim, widths, W, k, pad):
     assert np.array_equal(got.cpu().numpy(), want)
     # hidden layers evaluated neuron by neuron instead of along their schedules: the same counts
     assert torch.equal(got, ext.eval_net_lds(_dev(x), dev_layers, pad, k, scheduled=False))
+    # the net thinned for the call (constants folded, neurons that nothing looks at left out): the same counts
+    assert torch.equal(got, ext.eval_net_lds(_dev(x), dev_layers, pad, k, thin=True))
     t = _dev(x)
     for lay in dev_layers:
         t = ext.eval(t, *lay)
@@ -821,6 +823,7 @@ def test_net_lds_from_the_bool_input(ext, in_dim, widths, B, k):
     packed, pad2 = ext.tensor_packbits_batch_major(xb, 64)
     assert torch.equal(got, ext.eval_net_lds(packed, dev_layers, pad2, k))
     assert torch.equal(got, ext.eval_net_lds_bool(xb, dev_layers, k, scheduled=False))
+    assert torch.equal(got, ext.eval_net_lds_bool(xb, dev_layers, k, thin=True))
 
 
 def test_net_lds_from_the_bool_input_declines_what_does_not_fit(ext):

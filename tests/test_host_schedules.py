@@ -218,6 +218,9 @@ def test_launch_plan_follows_the_traffic_model():
     assert pbt.lds_tail(c2, 16384, from_bool=True) == 6 and pbt.lds_tail(c2, 16384, 1.0, from_bool=True) == 6
     assert abs(pbt.lds_cost(c2, 16384, True) * 1e3 - 0.78) <= 0.25 * 0.78
     assert abs((pbt.plan_cost(c2, pbt.plan_groups(c2, True, 16384), True, 16384) + pbt._STREAM_CALL_SECONDS) * 1e3 + 0.19 - 0.88) <= 0.25 * 0.88
-    # pass-through gates only (half of all gate inputs ignored): streaming C2 wins, 0.71 against 0.78 ms
-    assert pbt.lds_tail(c2, 16384, 0.5, from_bool=True) == 0
+    # where a good part of the gate inputs is ignored the LDS kernel runs the net thinned: 0.61-0.63 ms for shares of
+    # 0.5 to 0.75 against 0.74 whole, which also beats streaming for pass-through gates only (0.71 ms)
+    assert abs(pbt.lds_cost(c2, 16384, True, 0.75) * 1e3 - 0.62) <= 0.15 * 0.62
+    assert pbt.lds_cost(c2, 16384, True, 0.95) == pbt.lds_cost(c2, 16384, True)
+    assert pbt.lds_tail(c2, 16384, 0.5, from_bool=True) == 6
     assert pbt.plan_groups([784], True) == []
