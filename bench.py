@@ -54,7 +54,7 @@ TRAIN_TRAFFIC_JSON = os.path.join(ROOT, "profiles", "train_step_traffic.json")
 TRAIN_TRAFFIC_SOURCES = ("difflogic_amd/csrc/train.hip", "difflogic_amd/csrc/schedule.cpp", "difflogic_amd/csrc/dl_common.h",
                          "difflogic_amd/difflogic.py")
 # what the measured traffic of the packed launches depends on: the kernels and the launch plan
-TRAFFIC_SOURCES = ("difflogic_amd/csrc/packed.hip", "difflogic_amd/csrc/count_chain.h", "difflogic_amd/csrc/schedule.cpp",
+TRAFFIC_SOURCES = ("difflogic_amd/csrc/packed.hip", "difflogic_amd/csrc/lds_net.hip", "difflogic_amd/csrc/count_chain.h", "difflogic_amd/csrc/schedule.cpp",
                    "difflogic_amd/csrc/dl_common.h", "difflogic_amd/packbitstensor.py")
 
 

@@ -389,8 +389,18 @@ template <int D, int NP, int BIT, int NPMAX> __device__ __forceinline__ void fol
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
             const uint32_t lo = q[i][p], hi = q[D / 2 + i][p];
-            other[p] = lane_partner<BIT>(up ? lo : hi);
-            q[i][p] = up ? hi : lo;
+            if constexpr (BIT == 5 || BIT == 4) {
+                // gfx950's swaps exchange the upper half (odd rows of 16) of the first operand with the lower half
+                // (even rows) of the second: afterwards one holds the lane's own dword of the half it keeps and the
+                // other its partner's, which one being the same to the sum
+                const auto r = BIT == 5 ? __builtin_amdgcn_permlane32_swap(lo, hi, false, false)
+                                        : __builtin_amdgcn_permlane16_swap(lo, hi, false, false);
+                q[i][p] = (uint32_t) r[0];
+                other[p] = (uint32_t) r[1];
+            } else {
+                other[p] = lane_partner<BIT>(up ? lo : hi);
+                q[i][p] = up ? hi : lo;
+            }
         }
         planes_add<NP>(q[i], other);
     }
