@@ -34,6 +34,11 @@ __device__ __forceinline__ GateMasks gate_masks(uint32_t op) {
 // What stands in for an operand that no gate looks at: whatever the registers hold (an empty statement that the
 // compiler takes to define them), so that nothing is executed to make a value up.  Not for a place where loads
 // into the same registers may still be in flight: the compiler then waits for them before the statement.
+// The language promises nothing about an output-only empty asm; what it relies on is that the value is never looked
+// at by a gate (the records' liveness marks see to that) and that the compiler neither reads nor reorders around
+// it in a way that changes results.  The guard is empirical: the bit-exact comparisons with the per-layer kernels
+// and the CPU oracle at full size, for every gate mix (tests/test_gpu_fullsize.py, tests/test_gpu_gate_mixes.py),
+// which a build with another compiler has to pass before its numbers mean anything.
 template <typename V> __device__ __forceinline__ V any_value() {
     if constexpr (sizeof(V) < 4) {
         uint32_t v;
