@@ -1393,7 +1393,12 @@ __global__ __launch_bounds__(DL_BLOCK) void count_finish_kernel(const V *__restr
     __shared__ uint32_t planes_lds[4][NP][NC][DL_WAVE];
     const int wave = dl_wave_in_block();
     const int lane = dl_lane();
-    const int64_t tile = blockIdx.x, cls = blockIdx.y;
+    // A sample's k counts are 4k consecutive bytes of the output, written by k workgroups.  Workgroups are dealt
+    // round-robin to the 8 XCDs; the k of a column tile get consecutive places on ONE of them, so that they run at
+    // about the same time and their 4-byte stores meet in that XCD's L2 before the lines are written back.
+    const int64_t place = blockIdx.x / 8, xcd = blockIdx.x % 8;
+    const int64_t tile = (place / k) * 8 + xcd, cls = place % k;
+    if (tile * DL_WAVE >= ncols) return;
     const int64_t col = tile * DL_WAVE + lane;
     const bool live = col < ncols;
 
@@ -1416,6 +1421,88 @@ __global__ __launch_bounds__(DL_BLOCK) void count_finish_kernel(const V *__restr
     __syncthreads();
     // (base: what the class's neurons that were left out of the partial counters add to every sample)
     expand_counts<V, NP, 4>(planes_lds, wave, lane, col, live, cls, k, batch, out, base ? base[cls] : 0);
+}
+
+// count_finish_kernel for 16-byte lanes and k <= 16 with whole-line stores.  A sample's k counts are 4k consecutive
+// bytes of the output; one workgroup per (column tile, class) writes them as 4-byte stores 4k bytes apart, which
+// costs half of that kernel's time.  Here a workgroup owns 16 columns of a tile (2048 consecutive samples) and ALL
+// classes, wave c summing class c: a lane is (column l = lane % 16, chunk slot q = lane / 16) and adds up every
+// fourth chunk; the four slots (rows of 16 lanes) are added bit-sliced with gfx950's row and half swaps; row q then
+// expands the 32 samples of dword q, half of them per round, into an LDS stage laid out as the output is
+// ([column][dword][sample][class], a pad per run so that a wave's stores spread over the banks), which the
+// workgroup writes out in 256-byte pieces.
+#define DL_FINISH_COLS 16
+template <int NP>
+__global__ __launch_bounds__(16 * DL_WAVE) void count_finish_rows_kernel(const dl_u32x4 *__restrict__ partial,
+                                                                         int32_t *__restrict__ out, int64_t ncols,
+                                                                         int64_t chunks_per_class, int k, int64_t batch,
+                                                                         const int32_t *__restrict__ base) {
+    using V = dl_u32x4;
+    extern __shared__ int32_t finish_stage[];                  // [64 runs][16 samples * k + 1]
+    const int wave = dl_wave_in_block(), lane = dl_lane();
+    const int l = lane & (DL_FINISH_COLS - 1), q = lane / DL_FINISH_COLS;
+    constexpr int GROUPS = DL_WAVE / DL_FINISH_COLS;
+    const int64_t tile = blockIdx.x / GROUPS, group = blockIdx.x % GROUPS;
+    const int64_t col0 = tile * DL_WAVE + group * DL_FINISH_COLS;              // first column of the workgroup
+    const bool live = col0 + l < ncols;
+    const int cls = wave;                                      // (the launch has k waves)
+
+    V acc[NP + 1];
+#pragma unroll
+    for (int p = 0; p <= NP; ++p) acc[p] = V{0, 0, 0, 0};
+    const V *src = partial + ((tile * ((int64_t) k * chunks_per_class) + (int64_t) cls * chunks_per_class) * DL_COUNT_PLANES) * DL_WAVE +
+                   group * DL_FINISH_COLS + l;
+    for (int64_t c = q; c < chunks_per_class; c += GROUPS) {
+        V part[DL_COUNT_PLANES];
+#pragma unroll
+        for (int p = 0; p < DL_COUNT_PLANES; ++p)
+            part[p] = live ? __builtin_nontemporal_load(src + (c * DL_COUNT_PLANES + p) * DL_WAVE) : V{0, 0, 0, 0};
+        sliced_add<V, NP, DL_COUNT_PLANES>(acc, part);         // the carry out of plane NP-1 is zero by construction
+    }
+    // rows 0 + 1 and 2 + 3, then the two halves: every row ends up with the total
+#pragma unroll
+    for (int round = 0; round < 2; ++round) {
+        V other[NP];
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const auto r = round == 0 ? __builtin_amdgcn_permlane16_swap(acc[p][d], acc[p][d], false, false)
+                                          : __builtin_amdgcn_permlane32_swap(acc[p][d], acc[p][d], false, false);
+                acc[p][d] = (uint32_t) r[0];
+                other[p][d] = (uint32_t) r[1];
+            }
+        }
+        sliced_add<V, NP, NP>(acc, other);
+    }
+    uint32_t slice[NP];
+#pragma unroll
+    for (int p = 0; p < NP; ++p) slice[p] = q == 0 ? acc[p][0] : q == 1 ? acc[p][1] : q == 2 ? acc[p][2] : acc[p][3];
+
+    const int run = 16 * k + 1;                                // ints per (column, dword, half) run of the stage
+    const int32_t add = base ? base[cls] : 0;
+    const int64_t sample_group = col0 * 128;                   // first sample of the workgroup
+    const int nwaves = k;
+#pragma unroll 1
+    for (int half = 0; half < 2; ++half) {
+        int32_t *mine = finish_stage + (l * 4 + q) * run + cls;
+#pragma unroll
+        for (int s = 0; s < 16; ++s) {
+            int32_t cnt = add;
+#pragma unroll
+            for (int p = 0; p < NP; ++p) cnt += (int32_t) (((slice[p] >> (16 * half + s)) & 1u) << p);
+            mine[s * k] = cnt;
+        }
+        __syncthreads();
+        // run m = 4 l + q holds samples 128 l + 32 q + 16 half .. + 15 of the workgroup, k counts each
+        for (int m = wave; m < 4 * DL_FINISH_COLS; m += nwaves) {
+            const int64_t first = sample_group + (m >> 2) * 128 + (m & 3) * 32 + 16 * half;
+            const int64_t limit = first < batch ? (batch - first < 16 ? (batch - first) * k : 16 * k) : 0;
+            for (int i = lane; i < 16 * k; i += DL_WAVE)
+                if (i < limit) out[first * k + i] = finish_stage[m * run + i];
+        }
+        __syncthreads();
+    }
 }
 
 // Any word width / row length: one thread per (sample, class), like the reference, but with
@@ -1474,13 +1561,13 @@ int launch_count_fused_v(const void *x, const int32_t *leaves, const uint64_t *g
     const int64_t ncols = row_bytes / (int64_t) sizeof(V);
     const int64_t tiles = dl_ceil_div(ncols, DL_WAVE);
     const int64_t chunks_per_class = dl_ceil_div(per_class, DL_COUNT_ROWS);
-    if (k * chunks_per_class > 0x7fffffffLL || tiles > 65535) return DL_ERR_TOO_LARGE;
+    if (k * chunks_per_class > 0x7fffffffLL || tiles > 65535 || dl_ceil_div(tiles, 8) * 8 * k > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     DL_LAUNCH((count_partial_kernel<V, TREE>), dim3((unsigned) (k * chunks_per_class), (unsigned) tiles),
                        dim3(DL_BLOCK), 0, s, (const V *) x, leaves, gates, (V *) scratch, ncols, per_class,
                        chunks_per_class);
     int st = dl_launch_status();
     if (st != DL_OK) return st;
-    const dim3 grid((unsigned) tiles, (unsigned) k);
+    const dim3 grid((unsigned) (dl_ceil_div(tiles, 8) * 8 * k));
     // planes needed for counts up to per_class (pass 1 rounds a class up to whole chunks of 128)
     const int64_t top = chunks_per_class * DL_COUNT_ROWS;
     if (top < (1LL << 13))
@@ -2086,7 +2173,7 @@ int launch_count_chain(const void *x, const dl_u32x4 *rec, const uint16_t *runs,
     const int64_t ncols = row_bytes / (int64_t) sizeof(V);
     const int64_t tiles = dl_ceil_div(ncols, DL_WAVE);
     const int64_t nwg = padded_steps / (DL_CC_BLOCK * blocks);
-    if (nwg > 0x7fffffffLL || tiles > 65535) return DL_ERR_TOO_LARGE;
+    if (nwg > 0x7fffffffLL || tiles > 65535 || dl_ceil_div(tiles, 8) * 8 * k > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     const dim3 grid((unsigned) nwg, (unsigned) tiles), block(DL_CC_WAVES * DL_WAVE);
     if (k <= DL_CC_WAVES)
         DL_LAUNCH((count_chain_kernel<V, DS, 1>), grid, block, 0, s, (const V *) x, rec, runs, (V *) partial, ncols, k, nwg,
@@ -2096,7 +2183,17 @@ int launch_count_chain(const void *x, const dl_u32x4 *rec, const uint16_t *runs,
                   blocks);
     int st = dl_launch_status();
     if (st != DL_OK) return st;
-    const dim3 fgrid((unsigned) tiles, (unsigned) k);
+    if constexpr (sizeof(V) == 16) {
+        // whole-line stores where a wave per class fits a workgroup
+        const size_t lds = (size_t) 64 * (16 * k + 1) * 4;
+        if (k <= 16 && per_class < (1LL << 13) && tiles * 4 <= 0x7fffffffLL) {
+            const dim3 rgrid((unsigned) (tiles * 4)), rblock((unsigned) (k * DL_WAVE));
+            DL_LAUNCH((count_finish_rows_kernel<13>), rgrid, rblock, lds, s, (const dl_u32x4 *) partial, out, ncols, nwg, (int) k, batch,
+                      ones);
+            return dl_launch_status();
+        }
+    }
+    const dim3 fgrid((unsigned) (dl_ceil_div(tiles, 8) * 8 * k));
     if (per_class < (1LL << 13))
         DL_LAUNCH((count_finish_kernel<V, 13>), fgrid, dim3(DL_BLOCK), 0, s, (const V *) partial, out, ncols, nwg, k, batch,
                   ones);
