@@ -501,6 +501,10 @@ class GeneratedC:
     initialised, so that the child is started from a process that has not touched it); collect() waits for the
     compiler and times the whole apply_logic_gate_net call (bool packing, gates, adders)."""
 
+    # collect() gives the compiler this long, counted from its start (about 130 s for the headline's 384 000 gates on
+    # the GPU box's host); a host that needs longer gets the table interpreter's figure instead of a run without end
+    MAX_WAIT_S = 420.0
+
     def __init__(self, name, layers, num_inputs, k=10):
         import subprocess
         import tempfile
@@ -534,8 +538,13 @@ class GeneratedC:
         while self._waiter.is_alive():
             self._waiter.join(timeout=30)
             if self._waiter.is_alive():
+                waited = time.perf_counter() - self.t0
                 print("bench.py: waiting for gcc -O%d on the %d gates of %s, %.0f s so far"
-                      % (self.opt, self.gates, self.name, time.perf_counter() - self.t0), file=sys.stderr, flush=True)
+                      % (self.opt, self.gates, self.name, waited), file=sys.stderr, flush=True)
+                if waited > self.MAX_WAIT_S:
+                    self.proc.kill()
+                    self._waiter.join()
+                    return {"error": "gcc -O%d on %d gates not finished after %.0f s: stopped" % (self.opt, self.gates, waited)}
         if self.proc.returncode:
             return {"error": "gcc exited with %d" % self.proc.returncode}
         fn = cgen.load_apply_fn(self.so_path)
