@@ -460,6 +460,9 @@ __global__ __launch_bounds__(DL_BLOCK) void compose_steps_kernel(const int32_t *
 // One wave = STEPS consecutive steps x 64 vectors; dispatch order as eval_kernel.  BUF: x is at
 // most 4 GiB and is read through a buffer resource, whose loads take the row's byte offset as a
 // scalar operand next to the lane's constant offset: no vector instruction per gather.
+#ifndef DL_CC_REQUEST_PARTS
+#define DL_CC_REQUEST_PARTS 2          // count_chain_kernel: a block's rows are requested in this many parts along the walk before
+#endif
 #ifndef DL_STEPS_PER_WAVE
 #define DL_STEPS_PER_WAVE 32           // steps a wave of eval_steps_kernel walks (its first vertex is evaluated on top)
 #endif
@@ -1265,13 +1268,17 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
     constexpr bool AHEAD = CPW == 1;
     dl_u32x4 r0[FIRST];
     V ra0[FIRST], rb0[FIRST];
-    auto request = [&](auto count, int first, dl_u32x4 *r, V *ra, V *rb) {
+    auto issue = [&](auto count, const dl_u32x4 *r, V *ra, V *rb) {
 #pragma unroll
         for (int j = 0; j < decltype(count)::value; ++j) {
-            r[j] = wrec[1 + first + j];
             ra[j] = (r[j].w & 1u) ? any_value<V>() : xcol[(int64_t) r[j].x * ncols];
             if (DS == 1) rb[j] = (r[j].w & 2u) ? any_value<V>() : xcol[(int64_t) r[j].y * ncols];
         }
+    };
+    auto request = [&](auto count, int first, dl_u32x4 *r, V *ra, V *rb) {
+#pragma unroll
+        for (int j = 0; j < decltype(count)::value; ++j) r[j] = wrec[1 + first + j];
+        issue(count, r, ra, rb);
     };
     auto walk = [&](auto count, const dl_u32x4 *r, const V *ra, const V *rb) {
 #pragma unroll
@@ -1308,7 +1315,23 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
             run_next[i] = run_of(b + 1, i);
         }
         if constexpr (!AHEAD) request(first_batch, b * DL_CC_WAVE_STEPS, r0, ra0, rb0);
-        walk(first_batch, r0, ra0, rb0);
+        if constexpr (AHEAD) {
+            // The next block's rows are requested as soon as registers are free for them: part by part, right after
+            // this block's steps that held those registers have been walked (the rows have a whole block's time to
+            // arrive either way; asked for earlier, more of that time has requests in flight).
+            constexpr int PART = FIRST / DL_CC_REQUEST_PARTS;
+            const std::integral_constant<int, PART> part;
+            const bool more = b + 1 < blocks;
+#pragma unroll
+            for (int i = 0; i < DL_CC_REQUEST_PARTS; ++i) {
+                walk(part, r0 + i * PART, ra0 + i * PART, rb0 + i * PART);
+                __builtin_amdgcn_sched_barrier(0);
+                if (more) request(part, (b + 1) * DL_CC_WAVE_STEPS + i * PART, r0 + i * PART, ra0 + i * PART, rb0 + i * PART);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+            walk(first_batch, r0, ra0, rb0);
+        }
         if constexpr (REST > 0) {
             dl_u32x4 r[REST > 0 ? REST : 1];
             V ra[REST > 0 ? REST : 1], rb[REST > 0 ? REST : 1];
@@ -1316,8 +1339,6 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
             walk(second_batch, r, ra, rb);
         }
         __builtin_amdgcn_sched_barrier(0);          // (requests moved up into the walk would not fit the registers)
-        if constexpr (AHEAD)
-            if (b + 1 < blocks) request(first_batch, (b + 1) * DL_CC_WAVE_STEPS, r0, ra0, rb0);
         __syncthreads();
         // phase B: the owner of a class adds that class's run of parked outputs to its counters
 #pragma unroll
