@@ -480,7 +480,7 @@ __global__ __launch_bounds__(DL_BLOCK) void eval_steps_kernel(const V *__restric
     // Workgroups are dealt round-robin to the 8 XCDs, each with an L2 of its own.  xcd_owns_tiles (the grid's
     // second dimension is then a multiple of 8): XCD j takes the column tiles j, j + 8, ... one after the other, so
     // that a tile of the input is fetched into one L2 instead of eight and stays there while the tile is swept
-    // (headline prefix: fetched 2.08 -> 0.3 GB per launch, 1.13 -> 1.06 ms).
+    // (headline prefix: fetched 2.08 -> 0.97 GB per launch, 1.13 -> 1.07 ms).
     int64_t bx = blockIdx.x, by = blockIdx.y;
     if (xcd_owns_tiles) {
         const int64_t id = (int64_t) blockIdx.y * gridDim.x + blockIdx.x, xcd = id % 8, place = id / 8;
