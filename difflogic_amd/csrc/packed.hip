@@ -2139,7 +2139,8 @@ int launch_eval_steps(const void *x, const int32_t *sub_leaves, const uint64_t *
     int64_t ctiles = dl_ceil_div(ncols, DL_WAVE);
     // an input whose column tile (rows x 64 lanes) fits an XCD's 4 MB L2 with room to spare: one XCD per column tile
     const int64_t in_rows = ncols > 0 ? x_bytes / (ncols * (int64_t) sizeof(V)) : 0;
-    const bool own = in_rows * DL_WAVE * (int64_t) sizeof(V) <= DL_XCD_TILE_BYTES;
+    // (and enough column tiles to keep the eight XCDs evenly busy: a whole number each, or many)
+    const bool own = in_rows * DL_WAVE * (int64_t) sizeof(V) <= DL_XCD_TILE_BYTES && (ctiles % 8 == 0 || ctiles >= 64);
     if (own) ctiles = dl_ceil_div(ctiles, 8) * 8;                // (tiles past the last column do nothing)
     if (ctiles > 65528) ctiles = 65528;
     const int64_t gx = dl_ceil_div(steps, 4 * STEPS);

@@ -362,6 +362,9 @@ def test_lazy_pack_tensor_keeps_t_current():
     (32, 50, [60, 70], 7, "unique"), (8, 7, [20, 20], 16, "any"), (64, 5, [3, 3], 5, "self"),
     (64, 784, [6000, 6000, 6000, 6000], 64, "random"), (64, 3000, [3000, 3000], 128, "random"),
     (64, 40, [80, 80, 80, 80], 9, "any"), (64, 500, [64000], 16, "random"),
+    # 8, 9 and 65 column tiles of 128 words: each XCD sweeps whole column tiles (a whole number each; not with 9;
+    # with 65 the grid is padded to 72 and the tiles past the last column do nothing)
+    (64, 784, [2000, 2000], 1024, "random"), (64, 784, [2000, 2000], 1100, "random"), (64, 100, [300, 300], 8197, "random"),
 ])
 def test_eval_chained_equals_eval_fused(ext, bits, in_dim, widths, W, kind):
     from oracle import connections as oc
@@ -694,6 +697,8 @@ def test_pack_tensor_runs_narrow_tail_in_lds(monkeypatch):
     # more classes than a workgroup has waves: two sets of counters per wave
     (50, [100, 640], 70, 20, 63, "any"), (784, [8000, 8000], 32, 32, 0, "random"), (40, [96], 5, 24, 7, "any"),
     (30, [60, 3200], 3, 25, 0, "any"), (300, [6800], 16, 17, 0, "random"),
+    # 8 and 16 column tiles: the workgroups of a column tile share an XCD (count and finishing kernels)
+    (784, [2000, 2000], 1024, 10, 3, "random"), (100, [2560], 2048, 10, 0, "any"),
 ])
 def test_chained_groupbitsum(ext, in_dim, widths, W, k, pad, kind):
     """The count walked along the evaluation schedule against the oracle and the unchained
