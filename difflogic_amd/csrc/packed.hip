@@ -1246,9 +1246,10 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
     const int lane = dl_lane();
     if (wave == 0) stage[DL_CC_BLOCK][lane] = Words<V>::zero();   // (visible after the first block's barrier)
     // Workgroups are dealt round-robin to the 8 XCDs.  With a whole number of column tiles per XCD, XCD j takes the
-    // tiles j, j + 8, ...: the workgroups that gather from one column tile then share an L2, which serves some of
-    // the second reads of a row (every row has two readers when no gate ignores an input: count group 2.71 -> 2.62
-    // ms on such a net; no change where many rows are skipped).
+    // tiles j, j + 8, ...: the workgroups that gather from one column tile then share an L2 and an XCD works on one
+    // column tile at a time.  Measured: count group 2.71 -> 2.62 ms on a net where no gate ignores an input (every
+    // row is fetched, twice), no change where many rows are skipped; the L2 hit rate hardly moves (3 -> 4 %), so
+    // it is not second reads served by the L2 that is gained.
     int64_t g = blockIdx.x, tile = blockIdx.y;
     if (gridDim.y % 8 == 0) {
         const int64_t id = (int64_t) blockIdx.y * gridDim.x + blockIdx.x, xcd = id % 8, place = id / 8;
