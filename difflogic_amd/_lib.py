@@ -54,6 +54,7 @@ SIGNATURES = {
     "dl_adam_step": [_int, _vp, _vp, _vp, _vp, _vp, _vp, _dbl, _dbl, _dbl, _dbl, _dbl, _vp],
     "dl_gate_ids": [_vp, _vp, _i64, _int, _vp],
     "dl_fold_gate_constants": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp],
+    "dl_gate_ids_folded": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _i64, _vp],
     "dl_mark_live_inputs": [_vp, _vp, _vp, _vp, _vp, _i64, _vp],
     "dl_logic_eval": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "dl_tensor_packbits": [_vp, _vp, _i64, _i64, _int, ctypes.POINTER(_i64), _vp],
@@ -76,7 +77,7 @@ SIGNATURES = {
     "dl_logic_net_lds_groupbitsum_scheduled": [_vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _i64,
                                                _i64, _vp, _vp],
     "dl_logic_net_lds_groupbitsum_bool": [_vp, _i64, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp],
-    "dl_logic_net_lds_groupbitsum_thinned": [_vp, _int, _i64, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _i64, _vp, _vp],
+    "dl_logic_net_lds_groupbitsum_thinned": [_vp, _int, _i64, _int, _vp, _vp, _vp, _int, _vp, _vp, _i64, _int, _i64, _i64, _vp, _vp],
     "dl_count_chain_block": [],
     "dl_count_chain_padded_steps": [_i64],
     "dl_count_chain_plan_build": [_vp, _i64, _i64, _i64, _vp, _vp, ctypes.POINTER(_int)],

@@ -160,6 +160,13 @@ __global__ __launch_bounds__(DL_BLOCK) void net_thin_fold_kernel(NetWiring t, Th
     if (l + 1 < depth) thin.live[l][n] = 0;
 }
 
+// Where the caller's gate ids are folded already: only the marks of the hidden layers are cleared (in one launch;
+// `marks` is the first layer's, the others follow it, `total` bytes in all).
+__global__ __launch_bounds__(DL_BLOCK) void net_thin_clear_kernel(uint8_t *__restrict__ marks, int64_t total) {
+    const int64_t i = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x;
+    if (i < total) marks[i] = 0;
+}
+
 // Marks the neurons of layer l - 1 that a neuron of layer l which is itself looked at (the last layer: every neuron)
 // looks at (launched layer by layer, downwards).  A constant neuron marks nothing and, its readers having been
 // folded, is marked by nobody.
@@ -766,7 +773,7 @@ static int net_lds_run(const void *x, bool bool_input, int64_t batch, int depth,
                        const int64_t *const *b, const uint8_t *const *w, const int64_t *dims, const int32_t *const *verts,
                        const int32_t *const *neuron, const uint8_t *const *flip, const int64_t *steps, int32_t *out,
                        int64_t words, int bit_count, int64_t pad_len, int64_t k, void *workspace, void *stream,
-                       bool thinned = false) {
+                       bool thinned = false, bool folded = false) {
     if (!bool_input && bit_count != 8 && bit_count != 16 && bit_count != 32 && bit_count != 64) return DL_ERR_BIT_COUNT;
     if (depth < 1 || !dims || !a || !b || !w || words < 0 || k <= 0 || pad_len < 0) return DL_ERR_INVALID_ARGUMENT;
     if (depth > DL_NET_MAX_DEPTH) return DL_ERR_TOO_LARGE;
@@ -868,14 +875,22 @@ static int net_lds_run(const void *x, bool bool_input, int64_t batch, int depth,
         th.thin = rank;
         th.k = (int32_t) k;
         uint8_t *bytes = (uint8_t *) (rank + depth + 2 * k);
+        uint8_t *marks = bytes;                                  // the hidden layers' marks, one after the other
+        int64_t nmarks = 0;
+        for (int l = 0; l + 1 < depth; ++l) th.live[l] = bytes, bytes += dims[l + 1], nmarks += dims[l + 1];
         for (int l = 0; l < depth; ++l) {
-            th.folded[l] = bytes, bytes += dims[l + 1];
-            if (l + 1 < depth) th.live[l] = bytes, bytes += dims[l + 1];
+            // (folded already: the caller's gate ids are read where the folded ones would be; nothing writes them)
+            if (folded) th.folded[l] = const_cast<uint8_t *>(w[l]);
+            else th.folded[l] = bytes, bytes += dims[l + 1];
         }
         if ((char *) bytes - (char *) workspace > dl_logic_net_lds_workspace_bytes(depth, dims)) return DL_ERR_INVALID_ARGUMENT;
-        for (int l = 0; l < depth; ++l)
-            DL_LAUNCH(net_thin_fold_kernel, dim3((unsigned) dl_ceil_div(dims[l + 1], DL_BLOCK)), dim3(DL_BLOCK), 0, s, wiring, th, l,
-                      depth);
+        if (folded) {
+            if (nmarks > 0) DL_LAUNCH(net_thin_clear_kernel, dim3((unsigned) dl_ceil_div(nmarks, DL_BLOCK)), dim3(DL_BLOCK), 0, s, marks, nmarks);
+        } else {
+            for (int l = 0; l < depth; ++l)
+                DL_LAUNCH(net_thin_fold_kernel, dim3((unsigned) dl_ceil_div(dims[l + 1], DL_BLOCK)), dim3(DL_BLOCK), 0, s, wiring, th,
+                          l, depth);
+        }
         for (int l = depth - 1; l >= 1; --l)
             DL_LAUNCH(net_thin_mark_kernel, dim3((unsigned) dl_ceil_div(dims[l + 1], DL_BLOCK)), dim3(DL_BLOCK), 0, s, wiring, th, l,
                       depth);
@@ -917,13 +932,13 @@ extern "C" int dl_logic_net_lds_groupbitsum_scheduled(const void *x, int depth, 
 
 extern "C" int dl_logic_net_lds_groupbitsum_thinned(const void *x, int bool_input, int64_t batch, int depth,
                                                     const int64_t *const *a, const int64_t *const *b,
-                                                    const uint8_t *const *w, const int64_t *dims, int32_t *out,
+                                                    const uint8_t *const *w, int folded, const int64_t *dims, int32_t *out,
                                                     int64_t words, int bit_count, int64_t pad_len, int64_t k,
                                                     void *workspace, void *stream) {
     if (batch < 0) return DL_ERR_INVALID_ARGUMENT;
     return net_lds_run(x, bool_input != 0, batch, depth, a, b, w, dims, nullptr, nullptr, nullptr, nullptr, out,
                        bool_input ? 0 : words, bool_input ? 64 : bit_count, bool_input ? 0 : pad_len, k, workspace, stream,
-                       true);
+                       true, folded != 0);
 }
 
 extern "C" int dl_logic_net_lds_groupbitsum_bool(const uint8_t *x, int64_t batch, int depth, const int64_t *const *a,

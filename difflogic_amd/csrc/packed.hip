@@ -1753,17 +1753,13 @@ extern "C" int dl_tensor_packbits(const uint8_t *t, void *out, int64_t features,
 
 // Gate ids of a layer for packed inference: argmax over each neuron's 16 weights, as
 // weights.argmax(-1).to(uint8): the first maximal value wins, a NaN counts as maximal.
-template <typename T>
-__global__ __launch_bounds__(DL_BLOCK) void gate_ids_kernel(const T *__restrict__ w, uint8_t *__restrict__ ids,
-                                                            int64_t out_dim) {
-    const int64_t n = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x;
-    if (n >= out_dim) return;
-    float best = (float) w[n * 16];
-    int at = 0;
+template <typename T, typename C> __device__ __forceinline__ uint32_t argmax16(const T *__restrict__ w) {
+    C best = (C) w[0];
+    uint32_t at = 0;
     if (best == best) {                                   // not NaN: look on
 #pragma unroll
         for (int i = 1; i < 16; ++i) {
-            const float v = (float) w[n * 16 + i];
+            const C v = (C) w[i];
             if (v != v) {                                 // the first NaN
                 at = i;
                 break;
@@ -1771,27 +1767,45 @@ __global__ __launch_bounds__(DL_BLOCK) void gate_ids_kernel(const T *__restrict_
             if (v > best) best = v, at = i;
         }
     }
-    ids[n] = (uint8_t) at;
+    return at;
 }
 
-__global__ __launch_bounds__(DL_BLOCK) void gate_ids_f64_kernel(const double *__restrict__ w, uint8_t *__restrict__ ids,
-                                                                int64_t out_dim) {
+template <typename T, typename C>
+__global__ __launch_bounds__(DL_BLOCK) void gate_ids_kernel(const T *__restrict__ w, uint8_t *__restrict__ ids,
+                                                            int64_t out_dim) {
     const int64_t n = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x;
     if (n >= out_dim) return;
-    double best = w[n * 16];
-    int at = 0;
-    if (best == best) {
-#pragma unroll
-        for (int i = 1; i < 16; ++i) {
-            const double v = w[n * 16 + i];
-            if (v != v) {
-                at = i;
-                break;
-            }
-            if (v > best) best = v, at = i;
-        }
+    ids[n] = (uint8_t) argmax16<T, C>(w + n * 16);
+}
+
+// f'(a, b) = f(a, b) with the inputs that are constant (state 1: all zeros, 2: all ones; 0: varies) put in: the
+// gate the neuron amounts to on the inputs that vary.  Gate ids are (f(0,0) f(0,1) f(1,0) f(1,1)), MSB first.
+__device__ __forceinline__ uint32_t fold_gate(uint32_t op, uint32_t sa, uint32_t sb) {
+    if (sa) {                                                   // a is the constant sa - 1
+        const uint32_t f0 = sa == 2 ? (op >> 1) & 1u : (op >> 3) & 1u, f1 = sa == 2 ? op & 1u : (op >> 2) & 1u;
+        op = f0 << 3 | f1 << 2 | f0 << 1 | f1;
     }
-    ids[n] = (uint8_t) at;
+    if (sb) {
+        const uint32_t f0 = sb == 2 ? (op >> 2) & 1u : (op >> 3) & 1u, f1 = sb == 2 ? op & 1u : (op >> 1) & 1u;
+        op = f0 << 3 | f0 << 2 | f1 << 1 | f1;
+    }
+    return op;
+}
+
+// gate_ids_kernel and fold_gate_constants_kernel in one: the argmax gate with the constants among the layer's input
+// rows folded in, and which of the layer's own outputs are constant
+template <typename T, typename C>
+__global__ __launch_bounds__(DL_BLOCK) void gate_ids_folded_kernel(const T *__restrict__ w, const int64_t *__restrict__ a,
+                                                                   const int64_t *__restrict__ b,
+                                                                   const uint8_t *__restrict__ state_in,
+                                                                   uint8_t *__restrict__ ids, uint8_t *__restrict__ state_out,
+                                                                   int64_t out_dim) {
+    const int64_t n = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x;
+    if (n >= out_dim) return;
+    const uint32_t sa = state_in ? state_in[a[n]] : 0u, sb = state_in ? state_in[b[n]] : 0u;
+    const uint32_t op = fold_gate(argmax16<T, C>(w + n * 16), sa, sb);
+    ids[n] = (uint8_t) op;
+    state_out[n] = op == 0u ? 1 : op == 15u ? 2 : 0;
 }
 
 extern "C" int dl_gate_ids(const void *w, uint8_t *ids, int64_t out_dim, int dtype, void *stream) {
@@ -1803,9 +1817,31 @@ extern "C" int dl_gate_ids(const void *w, uint8_t *ids, int64_t out_dim, int dty
     if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     hipStream_t s = (hipStream_t) stream;
     const dim3 grid((unsigned) blocks), block(DL_BLOCK);
-    if (dtype == DL_F16) DL_LAUNCH(gate_ids_kernel<__half>, grid, block, 0, s, (const __half *) w, ids, out_dim);
-    else if (dtype == DL_F32) DL_LAUNCH(gate_ids_kernel<float>, grid, block, 0, s, (const float *) w, ids, out_dim);
-    else DL_LAUNCH(gate_ids_f64_kernel, grid, block, 0, s, (const double *) w, ids, out_dim);
+    if (dtype == DL_F16) DL_LAUNCH((gate_ids_kernel<__half, float>), grid, block, 0, s, (const __half *) w, ids, out_dim);
+    else if (dtype == DL_F32) DL_LAUNCH((gate_ids_kernel<float, float>), grid, block, 0, s, (const float *) w, ids, out_dim);
+    else DL_LAUNCH((gate_ids_kernel<double, double>), grid, block, 0, s, (const double *) w, ids, out_dim);
+    return dl_launch_status();
+}
+
+extern "C" int dl_gate_ids_folded(const void *w, int dtype, const int64_t *a, const int64_t *b, const uint8_t *state_in,
+                                  uint8_t *ids, uint8_t *state_out, int64_t out_dim, void *stream) {
+    if (dtype != DL_F16 && dtype != DL_F32 && dtype != DL_F64) return DL_ERR_DTYPE;
+    if (out_dim < 0) return DL_ERR_INVALID_ARGUMENT;
+    if (out_dim == 0) return DL_OK;
+    if (!w || !a || !b || !ids || !state_out) return DL_ERR_INVALID_ARGUMENT;
+    const int64_t blocks = dl_ceil_div(out_dim, DL_BLOCK);
+    if (blocks > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
+    hipStream_t s = (hipStream_t) stream;
+    const dim3 grid((unsigned) blocks), block(DL_BLOCK);
+    if (dtype == DL_F16)
+        DL_LAUNCH((gate_ids_folded_kernel<__half, float>), grid, block, 0, s, (const __half *) w, a, b, state_in, ids, state_out,
+                  out_dim);
+    else if (dtype == DL_F32)
+        DL_LAUNCH((gate_ids_folded_kernel<float, float>), grid, block, 0, s, (const float *) w, a, b, state_in, ids, state_out,
+                  out_dim);
+    else
+        DL_LAUNCH((gate_ids_folded_kernel<double, double>), grid, block, 0, s, (const double *) w, a, b, state_in, ids,
+                  state_out, out_dim);
     return dl_launch_status();
 }
 
@@ -1823,16 +1859,8 @@ __global__ __launch_bounds__(DL_BLOCK) void fold_gate_constants_kernel(const int
                                                                        uint8_t *__restrict__ state_out, int64_t out_dim) {
     const int64_t n = (int64_t) blockIdx.x * DL_BLOCK + threadIdx.x;
     if (n >= out_dim) return;
-    uint32_t op = w[n] & 15u;                                   // (f(0,0) f(0,1) f(1,0) f(1,1)), MSB first
     const uint32_t sa = state_in ? state_in[a[n]] : 0u, sb = state_in ? state_in[b[n]] : 0u;
-    if (sa) {                                                   // a is the constant sa - 1
-        const uint32_t f0 = sa == 2 ? (op >> 1) & 1u : (op >> 3) & 1u, f1 = sa == 2 ? op & 1u : (op >> 2) & 1u;
-        op = f0 << 3 | f1 << 2 | f0 << 1 | f1;
-    }
-    if (sb) {
-        const uint32_t f0 = sb == 2 ? (op >> 2) & 1u : (op >> 3) & 1u, f1 = sb == 2 ? op & 1u : (op >> 1) & 1u;
-        op = f0 << 3 | f0 << 2 | f1 << 1 | f1;
-    }
+    const uint32_t op = fold_gate(w[n] & 15u, sa, sb);
     w_out[n] = (uint8_t) op;
     state_out[n] = op == 0u ? 1 : op == 15u ? 2 : 0;
 }

@@ -132,7 +132,13 @@ class LogicLayer(torch.nn.Module):
         assert isinstance(x, PackBitsTensor)
         assert x.features == self.in_dim, (x.features, self.in_dim)
         a, b = self.indices
-        return x.defer_layer(a, b, self._gate_ids(), key=(self.weights.data_ptr(), self.weights._version, self.out_dim))
+        key = (self.weights.data_ptr(), self.weights._version, self.out_dim)
+        w = self.weights.detach()
+        if w.is_cuda and w.is_contiguous() and w.dtype in (torch.float16, torch.float32, torch.float64):
+            # the argmax gates with the constants among x's rows folded in, in one kernel (x tracks which rows those are)
+            ids, state = difflogic_cuda.gate_ids_folded(w, a, b, x.row_state(a.device))
+            return x.defer_layer(a, b, ids, key=key, state=state)
+        return x.defer_layer(a, b, self._gate_ids(), key=key)
 
     # Below this many inputs a 1 KB column tile of the whole input stays in the L2 caches and the
     # second gather of a row hits there; above it the chained kernels halve the gathered rows.

@@ -457,6 +457,32 @@ def gate_ids(weights):
     return ids
 
 
+def gate_ids_folded(weights, a, b, state=None):
+    """gate_ids and one step of fold_gate_constants in one kernel: (ids, state_out) for a layer with wiring
+    ``a``, ``b`` whose input rows are constant where ``state`` says so (uint8 [in]: 0 varies, 1 all zeros, 2 all
+    ones; None: all vary).  ``ids`` uint8 [out] are the argmax gates with those constants folded in, ``state_out``
+    uint8 [out] the constants among the layer's outputs.  Not part of the reference's extension."""
+    _check_input(weights, "weights")
+    code = _float_code(weights, "gate_ids")
+    if weights.dim() != 2 or weights.shape[1] != 16:
+        raise RuntimeError(f"expected weights [out,16], got {tuple(weights.shape)}")
+    out_dim = weights.shape[0]
+    _check_index(a, "a", out_dim)
+    _check_index(b, "b", out_dim)
+    dev = _same_device(weights, a, b) if state is None else _same_device(weights, a, b, state)
+    if state is not None:
+        _check_input(state, "state")
+        if state.dtype != torch.uint8 or state.dim() != 1:
+            raise RuntimeError(f"expected state [in] uint8, got {tuple(state.shape)} {state.dtype}")
+    both = torch.empty((2, out_dim), dtype=torch.uint8, device=dev)
+    with _on(dev):
+        st = _lib.load().dl_gate_ids_folded(_p(weights), code, _p(a), _p(b), _p(state) if state is not None else None,
+                                            _p(both[0]), _p(both[1]), out_dim, _stream(dev))
+    if st:
+        _raise(st, "gate_ids_folded")
+    return both[0], both[1]
+
+
 def fold_gate_constants(layers):
     """``layers`` = [(a, b, w), ...] applied one after the other to rows that vary -> the same list
     with gate ids in which constants are folded: a neuron that reads a constant neuron (gate id 0 or
@@ -950,7 +976,7 @@ def net_lds_max_width():
     return int(_lib.load().dl_logic_net_lds_max_width())
 
 
-def _net_lds_thinned(x, bool_input, batch, layers, dims, k, words, bits, pad_len, out, dev):
+def _net_lds_thinned(x, bool_input, batch, layers, dims, k, words, bits, pad_len, out, dev, folded=False):
     lib = _lib.load()
     depth = len(layers)
     ptrs = lambda i: (ctypes.c_void_p * depth)(*[l[i].data_ptr() for l in layers])  # noqa: E731
@@ -958,16 +984,18 @@ def _net_lds_thinned(x, bool_input, batch, layers, dims, k, words, bits, pad_len
     ws = torch.empty(max(1, lib.dl_logic_net_lds_workspace_bytes(depth, pdims) // 4), dtype=torch.int32, device=dev)
     with _on(dev):
         return lib.dl_logic_net_lds_groupbitsum_thinned(_p(x), 1 if bool_input else 0, batch, depth, ptrs(0), ptrs(1), ptrs(2),
-                                                        pdims, _p(out), words, bits, int(pad_len), int(k), _p(ws), _stream(dev))
+                                                        1 if folded else 0, pdims, _p(out), words, bits, int(pad_len), int(k),
+                                                        _p(ws), _stream(dev))
 
 
-def eval_net_lds(x, layers, pad_len, k, scheduled=True, thin=False):
+def eval_net_lds(x, layers, pad_len, k, scheduled=True, thin=False, folded=False):
     """groupbitsum(eval(... eval(x, layer 0) ..., last layer), pad_len, k) for a whole narrow net
     (every layer and the input at most net_lds_max_width() wide, at most MAX_NET_DEPTH layers) in
     one kernel that keeps the activations in LDS.  ``scheduled``: hidden layers are walked along
     their (cached) evaluation schedules where that fits, which nearly halves their LDS reads; the
     result is the same.  ``thin``: instead, the net is thinned for this call (constants folded, neurons that
-    no gate looks at neither evaluated nor stored; pays where many gates ignore an input).  Returns None where
+    no gate looks at neither evaluated nor stored; pays where many gates ignore an input; ``folded``: the gate ids
+    have the constants folded in already, so the kernels that would do it are left out).  Returns None where
     the kernel does not apply (the caller then uses the streaming kernels).  Not part of the reference's
     extension."""
     dev, bits, depth, pa, pb, pw, pdims, dims = _fused_args(x, layers)
@@ -982,7 +1010,7 @@ def eval_net_lds(x, layers, pad_len, k, scheduled=True, thin=False):
     lib = _lib.load()
     out = torch.empty((batch, k), dtype=torch.int32, device=dev)
     if thin:
-        st = _net_lds_thinned(x, False, batch, layers, dims, k, words, bits, pad_len, out, dev)
+        st = _net_lds_thinned(x, False, batch, layers, dims, k, words, bits, pad_len, out, dev, folded)
         if st == _lib.DL_ERR_TOO_LARGE:
             return None
         if st:
@@ -1009,7 +1037,7 @@ def eval_net_lds(x, layers, pad_len, k, scheduled=True, thin=False):
     return out
 
 
-def eval_net_lds_bool(x, layers, k, scheduled=True, thin=False):
+def eval_net_lds_bool(x, layers, k, scheduled=True, thin=False, folded=False):
     """eval_net_lds on the bool input itself: ``x`` [B, in] bool (sample-major, as PackBitsTensor
     receives it) -> int32 [B, k], the result of packing x with 64-bit words, evaluating every layer
     and groupbitsum, in one kernel that packs the input on its way into LDS (no pack kernel, no
@@ -1042,7 +1070,7 @@ def eval_net_lds_bool(x, layers, k, scheduled=True, thin=False):
     if batch == 0:
         return out
     if thin:
-        st = _net_lds_thinned(x, True, batch, layers, dims, k, 0, 64, 0, out, dev)
+        st = _net_lds_thinned(x, True, batch, layers, dims, k, 0, 64, 0, out, dev, folded)
         if st == _lib.DL_ERR_TOO_LARGE:
             return None
         if st:

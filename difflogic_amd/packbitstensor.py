@@ -170,6 +170,8 @@ class PackBitsTensor:
         self._pending = []            # [(a, b, w)] applied to the rows but not yet evaluated
         self._keys = []               # per pending layer: what identifies the weights its gate ids came from, or None
         self._folded = True           # constants folded through the pending layers' gate ids (_fold_pending)
+        self._state = None            # which rows of the deferred result are constant (uint8 [features]: 0 varies, 1 all
+                                      # zeros, 2 all ones), where the layers that made it said so; None: not known
         if device == "cuda":
             if bit_count not in (8, 16, 32, 64):
                 raise ValueError("`bit_count` has to be in { 8, 16, 32, 64 }")
@@ -301,18 +303,30 @@ class PackBitsTensor:
         self._pending = []
         self._keys = []
         self._folded = True
+        self._state = None
         self._src = None
         self._rows = None
         self._public = value
         bits = difflogic_cuda._WORD_BITS.get(value.dtype, self.bit_count)
         self._batch = max(0, value.shape[1] * bits - self.pad_len)
 
-    def defer_layer(self, a, b, w, key=None):
+    def row_state(self, device):
+        """What a layer applied next may assume about the rows it reads: uint8 [features] (0 varies, 1 all zeros,
+        2 all ones) or None (every row may vary).  See defer_layer."""
+        state = self._state
+        return state if state is not None and state.device == device else None
+
+    def defer_layer(self, a, b, w, key=None, state=None):
         """Applies the gate layer (a, b, w) lazily.  ``key``: a hashable that changes whenever the gate ids ``w`` may
-        have (the weights' address and version counter); lets the planner remember what it measured for them."""
+        have (the weights' address and version counter); lets the planner remember what it measured for them.
+        ``state``: the caller folded the constants among the rows it reads (row_state) into ``w`` already and says
+        which of the layer's own outputs are constant (difflogic_cuda.gate_ids_folded); without it the folding is
+        done before the layers run."""
         self._pending.append((a, b, w))
         self._keys.append(key)
-        self._folded = False
+        if state is None:
+            self._folded = False
+        self._state = state
         return self
 
     def group_sum(self, k):
@@ -328,13 +342,15 @@ class PackBitsTensor:
                 head = len(self._pending) - tail
                 if head == 0 and self._src is not None:
                     # the whole net, straight from the bool input: packing happens on the way into LDS
-                    out = difflogic_cuda.eval_net_lds_bool(self._src, self._pending, k, thin=share < _LDS_THIN_BELOW)
+                    out = difflogic_cuda.eval_net_lds_bool(self._src, self._pending, k, thin=share < _LDS_THIN_BELOW,
+                                                           folded=self._folded)
                     if out is not None:
                         return out
                 if head:
                     self._run_groups(plan_groups(dims[:head + 1], False, self._words64(), share))
                 rows = self._words()
-                out = difflogic_cuda.eval_net_lds(rows, self._pending, self._pad(rows), k, thin=share < _LDS_THIN_BELOW)
+                out = difflogic_cuda.eval_net_lds(rows, self._pending, self._pad(rows), k, thin=share < _LDS_THIN_BELOW,
+                                                  folded=self._folded)
                 if out is not None:
                     return out
             self._fold_pending()

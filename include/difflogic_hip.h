@@ -284,6 +284,12 @@ int dl_gate_ids(const void *w, uint8_t *ids, int64_t out_dim, int dtype, void *s
 int dl_fold_gate_constants(const int64_t *a, const int64_t *b, const uint8_t *w, const uint8_t *state_in,
                            uint8_t *w_out, uint8_t *state_out, int64_t out_dim, void *stream);
 
+/* dl_gate_ids and dl_fold_gate_constants of one layer in one kernel (what a layer in eval mode hands to the packed
+ * path): ids[n] = the argmax gate of neuron n with the constants among its input rows folded in, state_out[n] =
+ * whether the neuron is constant itself.  w [out_dim, 16] of `dtype`; a, b, state_in, state_out as above. */
+int dl_gate_ids_folded(const void *w, int dtype, const int64_t *a, const int64_t *b, const uint8_t *state_in,
+                       uint8_t *ids, uint8_t *state_out, int64_t out_dim, void *stream);
+
 /* Which input rows a layer looks at, for packed inference across fused groups (no counterpart in the
  * reference): live_in[r] is set to 1 where some neuron n with live_out[n] != 0 (live_out NULL: every
  * neuron) reads row r through an input its gate does not ignore.  live_in [in_dim] is cleared by the
@@ -492,10 +498,13 @@ int dl_logic_net_lds_groupbitsum_bool(const uint8_t *x, int64_t batch, int depth
  * looked at (uniformly drawn ids: about 55 %).
  *   bool_input != 0: x is the bool matrix [batch, dims[0]] as for dl_logic_net_lds_groupbitsum_bool (words,
  *   bit_count, pad_len unused); else packed words as for dl_logic_net_lds_groupbitsum (batch unused).
+ *   folded != 0: the gate ids `w` have the constants folded in already (dl_gate_ids_folded layer by layer, or
+ *   dl_fold_gate_constants): the folding kernels are left out.  (Ids that are not folded give the same counts
+ *   passed this way; a constant neuron that a gate still looks at is then kept and evaluated like any other.)
  *   workspace, limits and status codes as for those. */
 int dl_logic_net_lds_groupbitsum_thinned(const void *x, int bool_input, int64_t batch, int depth,
                                          const int64_t *const *a, const int64_t *const *b, const uint8_t *const *w,
-                                         const int64_t *dims, int32_t *out, int64_t words, int bit_count,
+                                         int folded, const int64_t *dims, int32_t *out, int64_t words, int bit_count,
                                          int64_t pad_len, int64_t k, void *workspace, void *stream);
 
 /* dl_logic_eval_fused_groupbitsum without a workspace argument, for callers that cannot allocate

@@ -428,6 +428,44 @@ def test_fold_gate_constants(ext):
     assert all(torch.equal(u[2], v[2]) for u, v in zip(folded, again))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.float64])
+def test_gate_ids_folded_is_gate_ids_then_fold(ext, dtype):
+    """dl_gate_ids_folded against dl_gate_ids followed by dl_fold_gate_constants, layer by layer (ties, NaNs and
+    constant gates included), and LogicLayer in eval mode hands PackBitsTensor exactly those ids."""
+    import difflogic_amd as dl
+    rng = np.random.default_rng(23)
+    torch.manual_seed(23)
+    in_dim, widths = 50, [400, 300, 500]
+    layers = random_layers(rng, in_dim, widths)
+    state, plain = None, []
+    for a, b, _ in layers:
+        w = torch.randn(len(a), 16, dtype=dtype)
+        w[rng.random(len(a)) < 0.2, 0] = 30.0                     # constant-zero gates
+        w[rng.random(len(a)) < 0.1, 15] = 40.0                    # constant-one gates
+        w[rng.random(len(a)) < 0.1, :] = 1.0                      # ties: the first wins
+        w[rng.random(len(a)) < 0.05, 7] = float("nan")            # a NaN counts as maximal
+        w = w.cuda()
+        ids = ext.gate_ids(w)
+        assert torch.equal(ids.cpu(), w.cpu().argmax(-1).to(torch.uint8))
+        plain.append((_dev(a), _dev(b), ids))
+        got_ids, state = ext.gate_ids_folded(w, _dev(a), _dev(b), state)
+        want = ext.fold_gate_constants(plain)[-1][2]
+        assert torch.equal(got_ids, want)
+        assert torch.equal(state, torch.where(want == 0, 1, torch.where(want == 15, 2, 0)).to(torch.uint8))
+    assert int((state != 0).sum()) > 100
+    # through the modules: the deferred layers hold the folded ids, and nothing is folded again before they run
+    model = build_model(in_dim, [(a, b, w.cpu().numpy()) for a, b, w in plain], 10).eval()
+    p = dl.PackBitsTensor(torch.as_tensor(rng.random((70, in_dim)) < 0.5).cuda(), bit_count=64)
+    with torch.no_grad():
+        for m in model:
+            if isinstance(m, dl.LogicLayer):
+                p = m(p)
+    assert p._folded and len(p._pending) == 3
+    want = ext.fold_gate_constants([(a, b, m.weights.argmax(-1).to(torch.uint8)) for (a, b, _), m in
+                                    zip(plain, [m for m in model if isinstance(m, dl.LogicLayer)])])
+    assert all(torch.equal(u[2], v[2]) for u, v in zip(p._pending, want))
+
+
 def test_pack_tensor_after_counting_with_rows_left_unwritten():
     """A net too wide for the LDS kernel streams in several groups; group_sum leaves rows of the inner groups unwritten
     that no gate above looks at.  The object stays usable: counting again, reading `.t` (every row of the last layer)
