@@ -466,6 +466,9 @@ __global__ __launch_bounds__(DL_BLOCK) void compose_steps_kernel(const int32_t *
 #ifndef DL_PACK_SHARE
 #define DL_PACK_SHARE 16               // pack kernel: neighbouring workgroups (64 output bytes per row each) that share an XCD
 #endif
+#ifndef DL_CC_XCD_TILE_BYTES
+#define DL_CC_XCD_TILE_BYTES (64 << 20)    // count_chain_kernel: input column tiles up to this size get an XCD of their own
+#endif
 #ifndef DL_XCD_TILE_BYTES
 #define DL_XCD_TILE_BYTES (2 << 20)    // eval_steps_kernel: input column tiles up to this size get an XCD (an L2) of their own
 #endif
@@ -1240,18 +1243,21 @@ __global__ __launch_bounds__(DL_CC_WAVES * DL_WAVE) void count_chain_kernel(cons
                                                                             const dl_u32x4 *__restrict__ rec,
                                                                             const uint16_t *__restrict__ runs,
                                                                             V *__restrict__ partial, int64_t ncols,
-                                                                            int64_t k, int64_t nwg, int blocks) {
+                                                                            int64_t k, int64_t nwg, int blocks,
+                                                                            uint32_t xcd_owns_tiles) {
     __shared__ V stage[DL_CC_BLOCK + 1][DL_WAVE];        // the last slot stays zero: what a run's padding reads
     const int wave = dl_wave_in_block();
     const int lane = dl_lane();
     if (wave == 0) stage[DL_CC_BLOCK][lane] = Words<V>::zero();   // (visible after the first block's barrier)
-    // Workgroups are dealt round-robin to the 8 XCDs.  With a whole number of column tiles per XCD, XCD j takes the
-    // tiles j, j + 8, ...: the workgroups that gather from one column tile then share an L2 and an XCD works on one
-    // column tile at a time.  Measured: count group 2.71 -> 2.62 ms on a net where no gate ignores an input (every
-    // row is fetched, twice), no change where many rows are skipped; the L2 hit rate hardly moves (3 -> 4 %), so
-    // it is not second reads served by the L2 that is gained.
+    // Workgroups are dealt round-robin to the 8 XCDs.  xcd_owns_tiles (a whole number of column tiles per XCD): XCD j
+    // takes the tiles j, j + 8, ...: the workgroups that gather from one column tile then share an L2 and an XCD
+    // works on one column tile at a time.  Measured on 64000-row inputs: count group 2.71 -> 2.62 ms on a net where
+    // no gate ignores an input (every row is fetched, twice), no change where many rows are skipped; the L2 hit rate
+    // hardly moves (3 -> 4 %), so it is not second reads served by the L2 that is gained.  On 256000-row inputs it
+    // loses (1.43 -> 1.58 ms): eight column tiles in flight are 2 GB, far beyond the 256 MB Infinity Cache that
+    // serves a row's second read while the whole chip sweeps one tile; the launcher asks for it up to 64 MB a tile.
     int64_t g = blockIdx.x, tile = blockIdx.y;
-    if (gridDim.y % 8 == 0) {
+    if (xcd_owns_tiles) {
         const int64_t id = (int64_t) blockIdx.y * gridDim.x + blockIdx.x, xcd = id % 8, place = id / 8;
         g = place % gridDim.x;
         tile = (place / gridDim.x) * 8 + xcd;
@@ -2256,18 +2262,19 @@ bool valid_cc_blocks(int blocks) { return blocks == 1 || blocks == 2 || blocks =
 template <typename V, int DS>
 int launch_count_chain(const void *x, const dl_u32x4 *rec, const uint16_t *runs, void *partial, int32_t *out,
                        const int32_t *ones, int64_t row_bytes, int64_t padded_steps, int blocks, int64_t per_class,
-                       int64_t k, int64_t batch, hipStream_t s) {
+                       int64_t k, int64_t batch, int64_t in_rows, hipStream_t s) {
     const int64_t ncols = row_bytes / (int64_t) sizeof(V);
     const int64_t tiles = dl_ceil_div(ncols, DL_WAVE);
     const int64_t nwg = padded_steps / (DL_CC_BLOCK * blocks);
     if (nwg > 0x7fffffffLL || tiles > 65535 || dl_ceil_div(tiles, 8) * 8 * k > 0x7fffffffLL) return DL_ERR_TOO_LARGE;
     const dim3 grid((unsigned) nwg, (unsigned) tiles), block(DL_CC_WAVES * DL_WAVE);
+    const uint32_t own = tiles % 8 == 0 && in_rows * DL_WAVE * (int64_t) sizeof(V) <= DL_CC_XCD_TILE_BYTES ? 1u : 0u;
     if (k <= DL_CC_WAVES)
         DL_LAUNCH((count_chain_kernel<V, DS, 1>), grid, block, 0, s, (const V *) x, rec, runs, (V *) partial, ncols, k, nwg,
-                  blocks);
+                  blocks, own);
     else
         DL_LAUNCH((count_chain_kernel<V, DS, 2>), grid, block, 0, s, (const V *) x, rec, runs, (V *) partial, ncols, k, nwg,
-                  blocks);
+                  blocks, own);
     int st = dl_launch_status();
     if (st != DL_OK) return st;
     if constexpr (sizeof(V) == 16) {
@@ -2366,9 +2373,9 @@ extern "C" int dl_logic_eval_chained_groupbitsum(const void *x, int depth, const
     if (st != DL_OK) return st;
     const bool wide = row_bytes % 16 == 0 && dl_aligned(x, 16);
     if (depth == 2) {
-        if (wide) return launch_count_chain<dl_u32x4, 1>(x, rec, runs_call, partial, out, ones, row_bytes, padded_steps, blocks, per_class, k, batch, s);
-        return launch_count_chain<uint64_t, 1>(x, rec, runs_call, partial, out, ones, row_bytes, padded_steps, blocks, per_class, k, batch, s);
+        if (wide) return launch_count_chain<dl_u32x4, 1>(x, rec, runs_call, partial, out, ones, row_bytes, padded_steps, blocks, per_class, k, batch, dims[0], s);
+        return launch_count_chain<uint64_t, 1>(x, rec, runs_call, partial, out, ones, row_bytes, padded_steps, blocks, per_class, k, batch, dims[0], s);
     }
-    if (wide) return launch_count_chain<dl_u32x4, 0>(x, rec, runs_call, partial, out, ones, row_bytes, padded_steps, blocks, per_class, k, batch, s);
-    return launch_count_chain<uint64_t, 0>(x, rec, runs_call, partial, out, ones, row_bytes, padded_steps, blocks, per_class, k, batch, s);
+    if (wide) return launch_count_chain<dl_u32x4, 0>(x, rec, runs_call, partial, out, ones, row_bytes, padded_steps, blocks, per_class, k, batch, dims[0], s);
+    return launch_count_chain<uint64_t, 0>(x, rec, runs_call, partial, out, ones, row_bytes, padded_steps, blocks, per_class, k, batch, dims[0], s);
 }
