@@ -287,6 +287,7 @@ class PackBitsTensor:
     def t(self):
         if self._pending:
             self._run_groups(plan_groups(self._dims(), False, self._words64(), self._live_share()))
+        self._state = None            # the caller may write into the words: nothing is known about the rows from here on
         if self._public is None:
             rows = self._words()
             dtype = difflogic_cuda._BITS_TO_DTYPE[self.bit_count]

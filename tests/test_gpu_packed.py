@@ -466,6 +466,30 @@ def test_gate_ids_folded_is_gate_ids_then_fold(ext, dtype):
     assert all(torch.equal(u[2], v[2]) for u, v in zip(p._pending, want))
 
 
+def test_rows_written_through_t_are_not_taken_for_constants():
+    """A layer of constant gates makes constant rows, which the next layer's gate ids fold in; once `.t` has been
+    handed out the caller may have written into those rows, and the folding must not rely on them any more."""
+    import difflogic_amd as dl
+    rng = np.random.default_rng(29)
+    F, B = 40, 200
+    layers = random_layers(rng, F, [128, 256])
+    layers[0][2][:] = rng.choice([0, 15], 128)                 # every row of the first layer is constant
+    model = build_model(F, layers, 2).eval()
+    logic = [m for m in model if isinstance(m, dl.LogicLayer)]
+    x = rng.random((B, F)) < 0.5
+    p = dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=64)
+    with torch.no_grad():
+        p = logic[0](p)
+        assert p.row_state(torch.device("cuda", 0)) is not None
+        words = p.t                                            # a view of the rows where their length allows it
+        fresh = torch.as_tensor(rng.integers(-2**62, 2**62, tuple(words.shape), dtype=np.int64)).cuda()
+        words.copy_(fresh)                                     # the rows vary now
+        mid = p.t.cpu().numpy().copy()
+        p = logic[1](p)
+        got = p.t.cpu().numpy()
+    assert np.array_equal(got, po.eval_layer(mid, *layers[1]))
+
+
 def test_pack_tensor_after_counting_with_rows_left_unwritten():
     """A net too wide for the LDS kernel streams in several groups; group_sum leaves rows of the inner groups unwritten
     that no gate above looks at.  The object stays usable: counting again, reading `.t` (every row of the last layer)
