@@ -365,6 +365,7 @@ def test_lazy_pack_tensor_keeps_t_current():
     # 8, 9 and 65 column tiles of 128 words: each XCD sweeps whole column tiles (a whole number each; not with 9;
     # with 65 the grid is padded to 72 and the tiles past the last column do nothing)
     (64, 784, [2000, 2000], 1024, "random"), (64, 784, [2000, 2000], 1100, "random"), (64, 100, [300, 300], 8197, "random"),
+    (64, 784, [1500, 1500, 1500, 1500], 1024, "random"), (64, 200, [600, 600, 600], 2048, "unique"),
 ])
 def test_eval_chained_equals_eval_fused(ext, bits, in_dim, widths, W, kind):
     from oracle import connections as oc
