@@ -831,6 +831,62 @@ def test_fuse_first_layers_trains_like_the_unfused_model(widths, batch, conn, gr
                            model(dl.PackBitsTensor(x.bool().cuda(), bit_count=64)))
 
 
+@pytest.mark.parametrize("widths,wide", [([400, 400, 300], False), ([300, 600, 600, 300], True), ([200, 400], False)])
+def test_fused_sequential_runs_the_logic_layers_as_one_autograd_node(widths, wide, monkeypatch):
+    """fuse_for_training's Sequential: one autograd node from the first logic layer to the class scores, with the
+    scores and every gradient bit for bit those of the same modules run one after the other; inputs that want a
+    gradient are served too; a module the node does not know in between, eval mode and double inputs under float
+    weights fall back to (or are) the modules one by one."""
+    import difflogic_amd as dl
+    if wide:                                                     # layers this narrow walk their schedules too
+        monkeypatch.setattr(dl.LogicLayer, "_CHAIN_MIN_IN_DIM", 0)
+        monkeypatch.setattr(dl.LogicLayer, "_CHAIN_MIN_OUT_DIM", 0)
+        monkeypatch.setattr(dl.difflogic_cuda, "BACKWARD_CHAIN_MAX_OVERFLOW", 1e9)
+    torch.manual_seed(9)
+    F, k, B = 60, 10, 96
+    mods, d = [torch.nn.Flatten()], F
+    for wd in widths:
+        mods.append(dl.LogicLayer(d, wd, grad_factor=1.5))
+        d = wd
+    model = torch.nn.Sequential(*mods, dl.GroupSum(k, 5.0)).train()
+    fused = dl.fuse_for_training(model).train()
+    assert isinstance(fused, dl.difflogic.FusedSequential) and list(fused.state_dict()) == list(model.state_dict())
+    one_by_one = torch.nn.Sequential(*fused)                   # the same modules without the node
+    layers = [m for m in model if isinstance(m, dl.LogicLayer)]
+    x = (torch.rand(B, F) < 0.4).float().cuda()
+    labels = torch.randint(0, k, (B,)).cuda()
+
+    def run(net, inp):
+        net.zero_grad(set_to_none=True)
+        out = net(inp)
+        torch.nn.functional.cross_entropy(out, labels).backward()
+        return out, [l.weights.grad.clone() for l in layers]
+
+    out, gw = run(fused, x)
+    assert type(out.grad_fn).__name__ == "LogicNetFunctionBackward"
+    ref, gref = run(one_by_one, x)
+    assert type(ref.grad_fn).__name__ != "LogicNetFunctionBackward"
+    assert torch.equal(out, ref) and all(torch.equal(u, v) for u, v in zip(gw, gref))
+    xg = x.clone().requires_grad_()
+    out, gw = run(fused, xg)
+    gx = xg.grad.clone()
+    xg.grad = None
+    ref, gref = run(one_by_one, xg)
+    assert type(out.grad_fn).__name__ == "LogicNetFunctionBackward"
+    assert torch.equal(out, ref) and torch.equal(gx, xg.grad) and all(torch.equal(u, v) for u, v in zip(gw, gref))
+    # double inputs under float weights: the layers take them (fp32 logits beside double activations), the fused
+    # GroupSum does not, so the modules run one by one
+    out = fused(x.double())
+    assert out.dtype == torch.float64 and type(out.grad_fn).__name__ != "LogicNetFunctionBackward"
+    # a module the node does not know
+    odd = dl.difflogic.FusedSequential(*list(fused)[:2], torch.nn.Identity(), *list(fused)[2:]).train()
+    out = odd(x)
+    assert type(out.grad_fn).__name__ != "LogicNetFunctionBackward" and torch.equal(out, ref)
+    fused.eval()
+    with torch.no_grad():
+        assert torch.equal(fused(x), one_by_one.eval()(x))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16])
 @pytest.mark.parametrize("in0,in_dim,out_dim,batch,kind", [(40, 64, 64, 256, "random"), (100, 300, 300, 512, "random"),
                                                            (30, 50, 60, 128, "unique"), (20, 30, 47, 260, "any"),
