@@ -1,5 +1,7 @@
 """PackBitsTensor: a batch of boolean feature vectors packed along the batch into integer
 words, feature-major (reference: difflogic/packbitstensor.py)."""
+import functools
+
 import numpy as np
 import torch
 
@@ -75,7 +77,13 @@ def plan_groups(dims, count_at_end, words=16384, live=_LIVE_INPUT):
 
     ``dims`` = [in_dim, width_1, ..., width_L]; ``words`` = 64-bit words per row.  Returns a list of
     group sizes summing to L; when ``count_at_end`` the last group is the one fused with the bit
-    count.  Chosen by dynamic programming over group_cost."""
+    count.  Chosen by dynamic programming over group_cost (remembered per shape: a call on a small batch is
+    bound by the host)."""
+    return list(_plan_groups(tuple(dims), bool(count_at_end), int(words), float(live)))
+
+
+@functools.lru_cache(maxsize=512)
+def _plan_groups(dims, count_at_end, words, live):
     n = len(dims) - 1
     if n == 0:
         return []
@@ -117,7 +125,12 @@ def lds_tail(dims, words=16384, live=_LIVE_INPUT, from_bool=False):
     plan for the same layers (0 otherwise).  Both skip what no gate looks at (the LDS kernel by thinning the net
     for the call when ``live`` is low enough to pay for it).
     ``from_bool``: the input has not been packed yet; if the whole net runs in LDS it never is, while the
-    streaming kernels need the pack kernel first."""
+    streaming kernels need the pack kernel first.  (Remembered per shape, like plan_groups.)"""
+    return _lds_tail(tuple(dims), int(words), float(live), bool(from_bool))
+
+
+@functools.lru_cache(maxsize=512)
+def _lds_tail(dims, words, live, from_bool):
     limit = difflogic_cuda.net_lds_max_width()
     n = 0
     while n < len(dims) - 1 and n < difflogic_cuda.MAX_NET_DEPTH and max(dims[len(dims) - 2 - n:]) <= limit:
