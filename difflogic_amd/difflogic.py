@@ -544,11 +544,21 @@ class LogicNetFunction(torch.autograd.Function):
             cur = fn.forward(node, cur, *args[1:])
             nodes.append((fn, node, weight_pos))
             needs_x = needs_x or any(needs[pos] for pos in weight_pos)
+        # what the stages saved goes through the node's own save_for_backward, so that autograd frees it after the
+        # backward pass (and notices writes into it) as it does for the stages run as nodes of their own
+        ctx.save_for_backward(*[t for _, node, _ in nodes for t in node.saved_tensors])
+        ctx.saved_counts = [len(node.saved_tensors) for _, node, _ in nodes]
+        for _, node, _ in nodes:
+            node.saved_tensors = ()
         ctx.nodes = nodes
         return cur
 
     @staticmethod
     def backward(ctx, grad):
+        saved, at = ctx.saved_tensors, 0
+        for (_, node, _), count in zip(ctx.nodes, ctx.saved_counts):
+            node.saved_tensors = saved[at:at + count]
+            at += count
         grads = []
         for fn, node, weight_pos in reversed(ctx.nodes):
             if grad is None:                                 # nothing below wants a gradient
@@ -557,6 +567,8 @@ class LogicNetFunction(torch.autograd.Function):
             out = fn.backward(node, grad)
             grads.extend(out[pos] for pos in reversed(weight_pos))
             grad = out[0]
+        for _, node, _ in ctx.nodes:
+            node.saved_tensors = ()
         return (grad, None) + tuple(reversed(grads))
 
 

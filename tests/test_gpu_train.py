@@ -874,6 +874,16 @@ def test_fused_sequential_runs_the_logic_layers_as_one_autograd_node(widths, wid
     ref, gref = run(one_by_one, xg)
     assert type(out.grad_fn).__name__ == "LogicNetFunctionBackward"
     assert torch.equal(out, ref) and torch.equal(gx, xg.grad) and all(torch.equal(u, v) for u, v in zip(gw, gref))
+    # the activations are freed with the graph's buffers, as for any node; a retained graph can be walked twice
+    fused.zero_grad(set_to_none=True)
+    loss = torch.nn.functional.cross_entropy(fused(x), labels)
+    loss.backward(retain_graph=True)
+    first = [l.weights.grad.clone() for l in layers]
+    fused.zero_grad(set_to_none=True)
+    loss.backward()
+    assert all(torch.equal(u, l.weights.grad) for u, l in zip(first, layers))
+    with pytest.raises(RuntimeError):
+        loss.backward()
     # double inputs under float weights: the layers take them (fp32 logits beside double activations), the fused
     # GroupSum does not, so the modules run one by one
     out = fused(x.double())
