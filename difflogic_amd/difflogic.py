@@ -612,19 +612,27 @@ class FusedSequential(torch.nn.Sequential):
                 i += 1
             elif (isinstance(m, FusedLogicLayerGroupSum) and i + 2 == len(mods) and isinstance(mods[i + 1], _GroupSumDone)):
                 layer, gs = m.layer, m.group_sum
-                if (not m.training or layer.implementation != "cuda" or dtype != layer.weights.dtype
-                        or layer.out_dim % gs.k != 0 or gs.k > GroupSum._HIP_MAX_K or layer.out_dim > GroupSum._HIP_MAX_OUT_DIM):
+                if (not m.training or layer.implementation != "cuda" or layer.out_dim % gs.k != 0
+                        or gs.k > GroupSum._HIP_MAX_K or layer.out_dim > GroupSum._HIP_MAX_OUT_DIM):
                     return None
-                stages.append((LogicLayerGroupSumFunction,
-                               (None, layer.indices[0], layer.indices[1], layer.weights, layer.given_x_indices_of_y_start,
-                                layer.given_x_indices_of_y, float(layer.grad_factor), layer._train_schedule(), int(gs.k),
-                                float(gs.tau)), (3,)))
+                if dtype == layer.weights.dtype:
+                    stages.append((LogicLayerGroupSumFunction,
+                                   (None, layer.indices[0], layer.indices[1], layer.weights, layer.given_x_indices_of_y_start,
+                                    layer.given_x_indices_of_y, float(layer.grad_factor), layer._train_schedule(), int(gs.k),
+                                    float(gs.tau)), (3,)))
+                else:
+                    # half / double activations over fp32 weights: the layer takes them, the fused kernels of layer +
+                    # GroupSum do not; the two run as stages of their own on the feature-major activation
+                    st = self._layer_stage(layer, dtype)
+                    if st is None:
+                        return None
+                    stages += [st, (GroupSumCudaFunction, (None, int(gs.k), float(gs.tau)), ())]
                 i += 2
             else:
                 return None
             first = False
         # (a run that does not end in the fused GroupSum would hand a feature-major activation on: not taken)
-        return stages if stages and stages[-1][0] is LogicLayerGroupSumFunction else None
+        return stages if stages and stages[-1][0] in (LogicLayerGroupSumFunction, GroupSumCudaFunction) else None
 
     @staticmethod
     def _layer_stage(layer, dtype):

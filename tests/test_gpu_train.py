@@ -835,8 +835,8 @@ def test_fuse_first_layers_trains_like_the_unfused_model(widths, batch, conn, gr
 def test_fused_sequential_runs_the_logic_layers_as_one_autograd_node(widths, wide, monkeypatch):
     """fuse_for_training's Sequential: one autograd node from the first logic layer to the class scores, with the
     scores and every gradient bit for bit those of the same modules run one after the other; inputs that want a
-    gradient are served too; a module the node does not know in between, eval mode and double inputs under float
-    weights fall back to (or are) the modules one by one."""
+    gradient are served too, and so are half / double inputs under float weights; a module the node does not know in
+    between and eval mode fall back to (or are) the modules one by one."""
     import difflogic_amd as dl
     if wide:                                                     # layers this narrow walk their schedules too
         monkeypatch.setattr(dl.LogicLayer, "_CHAIN_MIN_IN_DIM", 0)
@@ -884,10 +884,14 @@ def test_fused_sequential_runs_the_logic_layers_as_one_autograd_node(widths, wid
     assert all(torch.equal(u, l.weights.grad) for u, l in zip(first, layers))
     with pytest.raises(RuntimeError):
         loss.backward()
-    # double inputs under float weights: the layers take them (fp32 logits beside double activations), the fused
-    # GroupSum does not, so the modules run one by one
-    out = fused(x.double())
-    assert out.dtype == torch.float64 and type(out.grad_fn).__name__ != "LogicNetFunctionBackward"
+    # double / half inputs under float weights: the layers take them (fp32 logits beside the activations), the fused
+    # layer + GroupSum kernels do not: those two run as stages of their own inside the node
+    for dt in (torch.float64, torch.float16):
+        out, gw = run(fused, x.to(dt))
+        assert out.dtype == dt and type(out.grad_fn).__name__ == "LogicNetFunctionBackward"
+        ref, gref = run(one_by_one, x.to(dt))
+        assert torch.equal(out, ref) and all(torch.equal(u, v) for u, v in zip(gw, gref))
+    ref, gref = run(one_by_one, x)
     # a module the node does not know
     odd = dl.difflogic.FusedSequential(*list(fused)[:2], torch.nn.Identity(), *list(fused)[2:]).train()
     out = odd(x)
