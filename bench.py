@@ -761,6 +761,18 @@ def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor
             sec, loss = timeit(fwd_bwd)
             out["fwd_bwd_eager"] = report_dtype(sec, loss.item())
             del loss
+            # the fuse_for_training model: its layers and the GroupSum as one autograd node (less host work per step)
+            fused_model = dl.fuse_for_training(model).train()
+
+            def fwd_bwd_fused():
+                fused_model.zero_grad(set_to_none=True)
+                loss = loss_fn(fused_model(xd), labels)
+                loss.backward()
+                return loss
+
+            sec, loss = timeit(fwd_bwd_fused)
+            out["fused_for_training_fwd_bwd_eager"] = report_dtype(sec, loss.item())
+            del loss, fused_model
             model.zero_grad(set_to_none=True)
             gc.collect()
             torch.cuda.synchronize()
