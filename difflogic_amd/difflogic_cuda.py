@@ -73,8 +73,8 @@ _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 def _stream(dev):
     """torch's current stream on ``dev`` as the void* the C ABI takes."""
     if _raw_stream is not None and dev.index is not None:
-        return ctypes.c_void_p(_raw_stream(dev.index))           # no Stream object on the hot path
-    return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+        return _raw_stream(dev.index)                            # no Stream object on the hot path
+    return torch.cuda.current_stream(dev).cuda_stream
 
 
 class _NoGuard:
@@ -103,7 +103,9 @@ def _raise(status, what):
 
 
 def _p(t):
-    return ctypes.c_void_p(t.data_ptr())
+    """The tensor's device address as the bindings take it (argtypes say void *; a plain int converts without an
+    object of its own, which counts on the paths that are bound by the host)."""
+    return t.data_ptr()
 
 
 def forward(x, a, b, w, schedule=None):
