@@ -140,3 +140,36 @@ def test_pack_tensor_thins_the_lds_net_by_the_measured_share(monkeypatch):
             got = model(dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=64))
         assert np.array_equal(got.cpu().numpy(), interp.net_eval(x, layers, k))
         assert seen and seen[-1] is thin, (mix, seen)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_nets_with_a_gate_family_drawn_per_layer(seed):
+    """Depth, widths (narrow: the LDS-resident kernel, wide: the streaming groups), class count, word width, batch
+    AND every layer's gate family drawn at random, so that constant, pass-through and two-input layers meet in
+    orders the fixed mixes above do not list."""
+    import difflogic_amd as dl
+    kinds = ["uniform", "two-input", "pass-through", "half pass-through", "constant", "uniform"]
+    rng = np.random.default_rng(7000 + seed)
+    for case in range(10):
+        depth = int(rng.integers(1, 7))
+        k = int(rng.choice([1, 2, 3, 5, 10, 16, 20]))
+        F = int(rng.choice([16, 32, 48, 100, 784, 1000]))
+        wide = case % 3 == 0
+        widths, d = [], F
+        for i in range(depth):
+            lo = max(k, (d + 1) // 2)
+            w = int(rng.integers(lo, max(lo + 1, 14000 if wide else 3000)))
+            if i == depth - 1:
+                w = max(k, -(-w // k) * k)
+            widths.append(w)
+            d = w
+        B = int(rng.choice([1, 63, 64, 65, 127, 129, 1000, 4096, 8192 + 5]))
+        layers = [(a, b, _draw(rng, len(a), kinds[int(rng.integers(0, len(kinds)))]).astype(np.uint8))
+                  for a, b, _ in random_layers(rng, F, widths)]
+        x = rng.random((B, F)) < 0.5
+        want = interp.net_eval(x, layers, k)
+        model = build_model(F, layers, k).eval()
+        bits = int(rng.choice([8, 16, 32, 64]))
+        with torch.no_grad():
+            got = model(dl.PackBitsTensor(torch.as_tensor(x).cuda(), bit_count=bits)).cpu().numpy()
+        assert got.shape == want.shape and np.array_equal(got, want), (seed, case, F, widths, k, bits, B)
