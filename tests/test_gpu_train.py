@@ -193,6 +193,66 @@ def test_train_step_matches_python_implementation(conn, grad_factor, batch):
     assert ok, rep
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_random_models_train_like_the_python_implementation(seed, monkeypatch):
+    """Depth, widths, wiring kind, batch, tau, grad_factor, the kernels' route (plain or along the schedules) and the
+    model's form (as written or fuse_for_training) drawn at random: loss and every gradient of one step against the
+    CPU python implementation in fp64, with the fp32 python implementation's own distance as the budget."""
+    import difflogic_amd as dl
+    rng = np.random.default_rng(4200 + seed)
+    torch.manual_seed(seed)
+    if seed % 2:
+        monkeypatch.setattr(dl.LogicLayer, "_CHAIN_MIN_IN_DIM", 0)
+        monkeypatch.setattr(dl.LogicLayer, "_CHAIN_MIN_OUT_DIM", 0)
+    depth = int(rng.integers(1, 6))
+    k = int(rng.choice([2, 5, 10]))
+    F = int(rng.choice([20, 64, 200]))
+    tau = float(rng.choice([1.0, 10.0, 30.0]))
+    grad_factor = float(rng.choice([1.0, 1.5, 2.0]))
+    batch = int(rng.choice([1, 7, 32, 100, 128, 260]))
+    mods, d, widths = [torch.nn.Flatten()], F, []
+    for i in range(depth):
+        w = int(rng.integers((d + 1) // 2 + 1, max((d + 1) // 2 + 2, 500)))
+        if i == depth - 1:
+            w = -(-w // k) * k
+        conn = str(rng.choice(["random", "unique"])) if d * (d - 1) // 2 >= w else "random"
+        mods.append(dl.LogicLayer(d, w, grad_factor=grad_factor, connections=conn))
+        widths.append(w)
+        d = w
+    model = torch.nn.Sequential(*mods, dl.GroupSum(k, tau)).train()
+    layers = [m for m in model if isinstance(m, dl.LogicLayer)]
+    x = (torch.rand(batch, F) < 0.3).float()
+    labels = torch.randint(0, k, (batch,))
+    want_gx = bool(rng.random() < 0.5)
+    net_gpu = dl.fuse_for_training(model).train() if seed % 4 >= 2 else model
+
+    def python_impl(dtype):
+        lg = [l.weights.detach().cpu().to(dtype).requires_grad_(True) for l in layers]
+        net = fo.PythonNet([(l.indices[0].cpu(), l.indices[1].cpu(), w) for l, w in zip(layers, lg)], k, tau, grad_factor)
+        xo = x.detach().clone().to(dtype).requires_grad_(True)
+        out = net(xo, training=True)
+        loss = torch.nn.functional.cross_entropy(out, labels)
+        loss.backward()
+        return out.detach(), loss.detach(), [w.grad for w in lg], xo.grad
+
+    out32, loss32, gw32, gx32 = python_impl(torch.float32)
+    out64, loss64, gw64, gx64 = python_impl(torch.float64)
+    xg = x.detach().cuda().requires_grad_(want_gx)
+    got_out = net_gpu(xg)
+    got_loss = torch.nn.functional.cross_entropy(got_out, labels.cuda())
+    got_loss.backward()
+    what = (seed, F, widths, k, tau, grad_factor, batch)
+    ok, rep = within_budget(got_out, out64, out32)
+    assert ok, (what, rep)
+    assert abs(got_loss.item() - loss64.item()) <= RTOL * abs(loss64.item()) + 1e-7, what
+    for l, w64, w32 in zip(layers, gw64, gw32):
+        ok, rep = within_budget(l.weights.grad, w64, w32)
+        assert ok, (what, rep)
+    if want_gx:
+        ok, rep = within_budget(xg.grad, gx64, gx32)
+        assert ok, (what, rep)
+
+
 def test_eval_mode_and_state_dict_round_trip():
     import difflogic_amd as dl
     torch.manual_seed(1)
