@@ -178,9 +178,14 @@ __global__ __launch_bounds__(DL_BLOCK) void net_thin_mark_kernel(NetWiring t, Th
     if (net_gate_uses_b(op)) thin.live[l - 1][t.b[l][n]] = 1;
 }
 
-// blockIdx.x = layer: exclusive prefix sums of "this neuron is left" over the layer's neurons
+// blockIdx.x = layer: exclusive prefix sums of "this neuron is left" over the layer's neurons.  One scan carries two
+// counts: the neurons left in the low half of the word and, in the last layer, the constant-one neurons in the high
+// half (neither exceeds DL_NET_MAX_WIDTH < 2^16, and both only grow along the layer, so differences of two scan
+// values are the differences of the halves).
 __global__ __launch_bounds__(DL_NET_THREADS) void net_thin_rank_kernel(NetWiring t, ThinTables thin, int depth) {
+    static_assert(DL_NET_MAX_WIDTH < (1 << 16), "two counts per word");
     __shared__ int32_t wave_total[DL_NET_THREADS / DL_WAVE];
+    __shared__ int32_t class_at[DL_NET_MAX_WIDTH + 1];       // last layer: the scan at each class's first neuron, then the total
     const int l = blockIdx.x, tid = (int) threadIdx.x, lane = dl_lane(), wave = dl_wave_in_block();
     const int width = t.width[l];
     const bool last = l == depth - 1;
@@ -192,7 +197,7 @@ __global__ __launch_bounds__(DL_NET_THREADS) void net_thin_rank_kernel(NetWiring
         int32_t f = 0;
         if (n < width) {
             const uint32_t v = flag_src[n];
-            f = last ? (v != 0u && v != 15u) : v != 0u;
+            f = last ? (int32_t) (v != 0u && v != 15u) | ((int32_t) (v == 15u) << 16) : (int32_t) (v != 0u);
         }
         local[i] = sum;
         sum += f;
@@ -210,7 +215,7 @@ __global__ __launch_bounds__(DL_NET_THREADS) void net_thin_rank_kernel(NetWiring
         if (w < wave) before += wave_total[w];
         total += wave_total[w];
     }
-    const int32_t mine = before + incl - sum;                // neurons left before this thread's first
+    const int32_t mine = before + incl - sum;                // the scan before this thread's first neuron
     int32_t *rank = thin.rank[l];
     if (!last) {
 #pragma unroll
@@ -226,38 +231,19 @@ __global__ __launch_bounds__(DL_NET_THREADS) void net_thin_rank_kernel(NetWiring
 #pragma unroll
     for (int i = 0; i < DL_NET_RANK_ITEMS; ++i) {
         const int n = tid * DL_NET_RANK_ITEMS + i;
-        if (n < width && n % per_class == 0) rank[n] = mine + local[i];      // neurons left before the class
+        if (n < width && n % per_class == 0) class_at[n / per_class] = mine + local[i];
     }
-    __threadfence_block();
+    if (tid == 0) class_at[thin.k] = total;
     __syncthreads();
-    int32_t at_start[DL_NET_RANK_ITEMS];
 #pragma unroll
     for (int i = 0; i < DL_NET_RANK_ITEMS; ++i) {
         const int n = tid * DL_NET_RANK_ITEMS + i;
-        at_start[i] = n < width ? rank[(n / per_class) * per_class] : 0;
+        if (n < width) rank[n] = ((mine + local[i]) & 0xffff) - (class_at[n / per_class] & 0xffff);
     }
-    __syncthreads();                                         // every class start has been read before any rank changes
-#pragma unroll
-    for (int i = 0; i < DL_NET_RANK_ITEMS; ++i) {
-        const int n = tid * DL_NET_RANK_ITEMS + i;
-        if (n < width) rank[n] = mine + local[i] - at_start[i];
-    }
-    for (int c = wave; c < thin.k; c += DL_NET_THREADS / DL_WAVE) {      // a wave per class
-        int32_t left = 0, ones = 0;
-        for (int i = lane; i < per_class; i += DL_WAVE) {
-            const uint32_t g = thin.folded[l][c * per_class + i];
-            left += g != 0u && g != 15u;
-            ones += g == 15u;
-        }
-#pragma unroll
-        for (int off = DL_WAVE / 2; off > 0; off >>= 1) {
-            left += __shfl_xor(left, off, DL_WAVE);
-            ones += __shfl_xor(ones, off, DL_WAVE);
-        }
-        if (lane == 0) {
-            thin.thin[depth - 1 + c] = left;
-            thin.thin[depth - 1 + thin.k + c] = ones;
-        }
+    for (int c = tid; c < thin.k; c += DL_NET_THREADS) {
+        const int32_t d = class_at[c + 1] - class_at[c];
+        thin.thin[depth - 1 + c] = d & 0xffff;
+        thin.thin[depth - 1 + thin.k + c] = d >> 16;
     }
 }
 

@@ -1134,19 +1134,31 @@ __global__ __launch_bounds__(DL_BLOCK) void count_partial_kernel(const V *__rest
 // Neurons of the top layer whose gate is constant (0 or 15, as it stands after constants were folded into it)
 // output the same word for every sample: they are not parked and not counted.  What the ones among them add to
 // every sample's count of their class goes into the result at the very end (count_finish_kernel's base).
-__global__ __launch_bounds__(DL_BLOCK) void count_constant_ones_kernel(const uint8_t *__restrict__ w_top, int64_t per_class,
-                                                                       int32_t *__restrict__ ones) {
-    __shared__ int32_t part[DL_BLOCK / DL_WAVE];
+#define DL_ONES_THREADS 1024
+__global__ __launch_bounds__(DL_ONES_THREADS) void count_constant_ones_kernel(const uint8_t *__restrict__ w_top, int64_t per_class,
+                                                                              int32_t *__restrict__ ones) {
+    __shared__ int32_t part[DL_ONES_THREADS / DL_WAVE];
     const int64_t cls = blockIdx.x;
     int32_t n = 0;
-    for (int64_t i = threadIdx.x; i < per_class; i += DL_BLOCK) n += (w_top[cls * per_class + i] & 15u) == 15u;
+    constexpr int AT_ONCE = 8;                                 // loads in flight per thread (one at a time, the kernel
+                                                               // waits out a memory latency per DL_ONES_THREADS neurons)
+    for (int64_t first = threadIdx.x; first < per_class; first += AT_ONCE * DL_ONES_THREADS) {
+        uint32_t v[AT_ONCE];
+#pragma unroll
+        for (int u = 0; u < AT_ONCE; ++u) {
+            const int64_t i = first + u * DL_ONES_THREADS;
+            v[u] = i < per_class ? w_top[cls * per_class + i] : 0u;
+        }
+#pragma unroll
+        for (int u = 0; u < AT_ONCE; ++u) n += (v[u] & 15u) == 15u;
+    }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) n += __shfl_xor(n, off);
     if (dl_lane() == 0) part[dl_wave_in_block()] = n;
     __syncthreads();
     if (threadIdx.x == 0) {
         int32_t total = 0;
-        for (int i = 0; i < DL_BLOCK / DL_WAVE; ++i) total += part[i];
+        for (int i = 0; i < DL_ONES_THREADS / DL_WAVE; ++i) total += part[i];
         ones[cls] = total;
     }
 }
@@ -2355,7 +2367,7 @@ extern "C" int dl_logic_eval_chained_groupbitsum(const void *x, int depth, const
     uint16_t *runs_call = (uint16_t *) (slot_call + dl_ceil_div(padded_steps, 16) * 16);
     int32_t *ones = (int32_t *) ((char *) runs_call + dl_ceil_div(nblocks * k * 2, 16) * 16);
     const uint8_t *w_top = w[depth - 1];
-    DL_LAUNCH(count_constant_ones_kernel, dim3((unsigned) k), dim3(DL_BLOCK), 0, s, w_top, per_class, ones);
+    DL_LAUNCH(count_constant_ones_kernel, dim3((unsigned) k), dim3(DL_ONES_THREADS), 0, s, w_top, per_class, ones);
     int st = dl_launch_status();
     if (st != DL_OK) return st;
     DL_LAUNCH(count_chain_thin_kernel, dim3((unsigned) dl_ceil_div(nblocks, DL_BLOCK / DL_WAVE)), dim3(DL_BLOCK), 0, s, neuron, w_top,
