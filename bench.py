@@ -388,7 +388,7 @@ def launch_rooflines(per_kernel, steps, table, prefix=""):
             row["traffic_GB"] = round(e["hbm_bytes_per_launch"] / 1e9, 3)
             row["traffic_GBps"] = round(e["hbm_bytes_per_launch"] / (row["avg_ms"] * 1e-3) / 1e9, 1)
             row["frac_hbm_traffic"] = round(row["traffic_GBps"] / HBM_PEAK_GBS, 4)
-            row["bound"] = e.get("bound")
+            row["limited_by"] = e.get("bound")
     dom = max(per_kernel, key=lambda kk: per_kernel[kk]["ms"])
     avg_ms = per_kernel[dom]["ms"] / per_kernel[dom]["n"]
     alg = per_kernel[dom]["bytes"]
@@ -397,7 +397,9 @@ def launch_rooflines(per_kernel, steps, table, prefix=""):
     traffic = entry.get("hbm_bytes_per_launch")
     achieved = traffic / (avg_ms * 1e-3) / 1e9 if traffic else None
     roofline = {
-        "bound": entry.get("bound", "hbm") if traffic else "hbm (traffic of this build not measured)",
+        # `achieved`, `peak` and `frac` are HBM figures; what actually limits the launch is said in words beside them
+        "bound": "hbm",
+        "limited_by": entry.get("bound", "hbm") if traffic else "hbm (traffic of this build not measured)",
         "kernel": dom,
         "achieved": round(achieved, 1) if achieved else None, "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4) if achieved else None,
