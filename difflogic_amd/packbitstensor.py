@@ -202,7 +202,11 @@ class PackBitsTensor:
 
     @staticmethod
     def _row_bytes(batch):
-        return 16 * -(-batch // 128)
+        """Length of a padded row: whole 16-byte vectors; from 2 KB on whole 128-byte lines, so that every row starts
+        on a line and the 1 KB piece of a row that a wave reads is 8 lines, not 9 (batch 10^6 on the 784 -> 6 x 64000
+        net: 2.70 -> 2.48 ns per sample; at most 6 % more columns)."""
+        n = 16 * -(-batch // 128)
+        return n if n < 2048 else 128 * -(-n // 128)
 
     def _adopt(self, value):
         """(rows, shared): ``value`` (words as `.t` shows them) as padded int64 rows; ``shared`` says

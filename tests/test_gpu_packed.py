@@ -79,10 +79,11 @@ def test_packbits_batch_major_rows(ext, B, F, row_bytes):
 
 
 @pytest.mark.parametrize("bits", [8, 16, 32, 64])
-@pytest.mark.parametrize("B", [1, 37, 64, 100, 128, 200, 1000, 1024 + 96])
+@pytest.mark.parametrize("B", [1, 37, 64, 100, 128, 200, 1000, 1024 + 96, 16384, 16384 + 128, 3 * 8192 + 100])
 def test_pack_tensor_every_width_and_batch(bits, B):
-    """PackBitsTensor keeps padded rows inside; `.t`, `.pad_len` and the counts are the reference's for every
-    word width and batch size, before, between and after layers, and writes into `.t` are seen."""
+    """PackBitsTensor keeps padded rows inside (whole 16-byte vectors, from 2 KB on whole 128-byte lines); `.t`,
+    `.pad_len` and the counts are the reference's for every word width and batch size, before, between and after
+    layers, and writes into `.t` are seen."""
     import difflogic_amd as dl
     rng = np.random.default_rng(B * 4 + bits)
     layers = random_layers(rng, 24, [48, 48, 30])
