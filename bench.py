@@ -267,7 +267,10 @@ def packed_run(torch, dl, model, x, k, steps, warmup, graph=True):
         # the batch sits in the graph's static input buffer, as the eager step's sits in x)
         from difflogic_amd.graphs import GraphedPackedInference
         graphed = GraphedPackedInference(model, x, bit_count=64)
-        graphed()
+        # (capturing leaves the GPU idle for milliseconds, after which launches run up to 1.3x slower for some twenty
+        # steps: the replays get the warm-up the eager steps had)
+        for _ in range(max(warmup, 20)):
+            graphed()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
