@@ -235,9 +235,12 @@ def packed_run(torch, dl, model, x, k, steps, warmup, graph=True):
         first_call_ms = (time.perf_counter() - t_first) * 1e3       # includes the host-side schedule / order builds
         # untimed: a third of a second of the same steps ahead of the warm-up proper, so that clocks and caches have
         # settled however few warm-up steps were asked for (the first launches of a process run up to 1.5x slower)
+        # (back to back, as the timed steps run: launches that follow an idle GPU run slower for a while, so the host
+        # waits for the stream every eighth step only, which bounds the queue)
         t_settle = time.perf_counter() + 0.3
         while time.perf_counter() < t_settle:
-            out = step()
+            for _ in range(8):
+                out = step()
             torch.cuda.synchronize()
         for _ in range(max(0, warmup - 1)):
             out = step()
@@ -660,6 +663,13 @@ def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor
     alg = train_alg_bytes([F] + list(widths), B)
 
     def timeit(fn):
+        # untimed: a fifth of a second of the same steps, back to back as the timed ones run, ahead of the warm-up
+        # proper (launches that follow an idle GPU run slower for some tens of milliseconds)
+        t_settle = time.perf_counter() + 0.2
+        while time.perf_counter() < t_settle:
+            for _ in range(8):
+                fn()
+            torch.cuda.synchronize()
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
