@@ -58,6 +58,10 @@ TRAFFIC_SOURCES = ("difflogic_amd/csrc/packed.hip", "difflogic_amd/csrc/lds_net.
                    "difflogic_amd/csrc/dl_common.h", "difflogic_amd/packbitstensor.py")
 
 
+# seconds of untimed steps ahead of each warm-up (packed_run, train_config's timeit); --no-settle zeroes them
+SETTLE_S = {"packed": 0.3, "train": 0.2}
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -78,6 +82,9 @@ def parse():
     ap.add_argument("--train-eager-only", default="", choices=("", "written", "fused"),
                     help="profiling aid: of a training configuration run only the eager forward+backward loop of the model "
                          "as written for the reference, or of the fuse_for_training model (for whole-step counters)")
+    ap.add_argument("--no-settle", action="store_true",
+                    help="profiling aid: leave out the untimed steps ahead of each warm-up (counter runs record every "
+                         "dispatch; per-launch figures do not depend on them)")
     ap.add_argument("--cpu-sample-log2", type=int, default=18)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 4 plain device copies of 1 GiB (for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE)")
@@ -237,7 +244,7 @@ def packed_run(torch, dl, model, x, k, steps, warmup, graph=True):
         # settled however few warm-up steps were asked for (the first launches of a process run up to 1.5x slower)
         # (back to back, as the timed steps run: launches that follow an idle GPU run slower for a while, so the host
         # waits for the stream every eighth step only, which bounds the queue)
-        t_settle = time.perf_counter() + 0.3
+        t_settle = time.perf_counter() + SETTLE_S["packed"]
         while time.perf_counter() < t_settle:
             for _ in range(8):
                 out = step()
@@ -665,7 +672,7 @@ def train_config(torch, dl, name, F, widths, k, tau, B, connections, grad_factor
     def timeit(fn):
         # untimed: a fifth of a second of the same steps, back to back as the timed ones run, ahead of the warm-up
         # proper (launches that follow an idle GPU run slower for some tens of milliseconds)
-        t_settle = time.perf_counter() + 0.2
+        t_settle = time.perf_counter() + SETTLE_S["train"]
         while time.perf_counter() < t_settle:
             for _ in range(8):
                 fn()
@@ -1004,6 +1011,8 @@ def extra_configs(args, torch, dl, started):
 
 def main():
     args = parse()
+    if args.no_settle:
+        SETTLE_S.update(packed=0.0, train=0.0)
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the path shards along the batch without "
               "communication); --gpus %d is not supported" % args.gpus, file=sys.stderr)
