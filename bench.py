@@ -460,14 +460,14 @@ def word_width_variants(torch, dl, model, x, want):
         def step():
             with torch.no_grad():
                 return model(dl.PackBitsTensor(inp, bit_count=bits))
-        for _ in range(3):                      # (the first steps after a pause run slower)
+        for _ in range(24):                     # (steps that follow a pause run slower, for some twenty steps)
             step()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(5):
+        for _ in range(10):
             got = step()
         torch.cuda.synchronize()
-        res[name] = {"ms_per_step": round((time.perf_counter() - t0) / 5 * 1e3, 4),
+        res[name] = {"ms_per_step": round((time.perf_counter() - t0) / 10 * 1e3, 4),
                      "equal_to_int64_run": bool(torch.equal(got, want[:inp.shape[0]]))}
     return res
 
